@@ -1,0 +1,130 @@
+"""ctypes binding of the CPU oracle (oracle/cp4_oracle.c).
+
+Test infrastructure only: imported by tests/, by ``__graft_entry__.smoke()``
+and by the ``cpu_baseline`` leg of bench.py as the checker / reported CPU
+baseline.  The shipped package never imports this module.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libcp4oracle.so")
+
+
+class Shape(ctypes.Structure):
+    """Same nine unsigned fields, same order, as the reference's tensor_shape
+    (Cuda_kernels/Tensor.cuh:10-19)."""
+    _fields_ = [(k, ctypes.c_uint) for k in
+                ("N", "H", "W", "pad", "T", "C", "Y", "X", "Rank")]
+
+
+def build(force=False):
+    if force or not os.path.exists(_LIB_PATH):
+        cmd = ["make", "-C", _HERE] + (["-B"] if force else [])
+        subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _lib = ctypes.CDLL(build())
+        _lib.cp4o_count_exceeding.restype = ctypes.c_long
+    return _lib
+
+
+def _fp(a):
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def shape_of(x_shape, FK, FC, FH, FW, pad):
+    """tensor_shape from operand shapes, as CP::Conv2dForward derives it
+    (Cuda_kernels/cp4Conv2d.cu:21-30)."""
+    N, C, H, W = x_shape
+    return Shape(N=N, H=H, W=W, pad=pad, T=FK.shape[0], C=C, Y=FH.shape[0],
+                 X=FW.shape[0], Rank=FK.shape[1])
+
+
+def num_threads():
+    return int(lib().cp4o_num_threads())
+
+
+def recompose(FK, FC, FH, FW):
+    FK, FC, FH, FW = map(_f32, (FK, FC, FH, FW))
+    s = Shape(T=FK.shape[0], C=FC.shape[0], Y=FH.shape[0], X=FW.shape[0],
+              Rank=FK.shape[1])
+    K = np.empty((s.T, s.C, s.Y, s.X), np.float32)
+    lib().cp4o_recompose(ctypes.byref(s), _fp(FK), _fp(FC), _fp(FH), _fp(FW), _fp(K))
+    return K
+
+
+def forward(x, FK, FC, FH, FW, pad, direct=False):
+    x, FK, FC, FH, FW = map(_f32, (x, FK, FC, FH, FW))
+    s = shape_of(x.shape, FK, FC, FH, FW, pad)
+    assert FC.shape == (s.C, s.Rank)
+    y = np.empty((s.N, s.T, s.H, s.W), np.float32)
+    fn = lib().cp4o_forward_direct if direct else lib().cp4o_forward_unfused
+    rc = fn(ctypes.byref(s), _fp(x), _fp(FK), _fp(FC), _fp(FH), _fp(FW), _fp(y))
+    assert direct or rc == 0
+    return y
+
+
+def backward_data(dy, FK, FC, FH, FW, pad, direct=False):
+    dy, FK, FC, FH, FW = map(_f32, (dy, FK, FC, FH, FW))
+    N, T, H, W = dy.shape
+    assert FK.shape[0] == T
+    s = Shape(N=N, H=H, W=W, pad=pad, T=T, C=FC.shape[0], Y=FH.shape[0],
+              X=FW.shape[0], Rank=FK.shape[1])
+    dx = np.empty((N, s.C, H, W), np.float32)
+    fn = (lib().cp4o_backward_data_direct if direct
+          else lib().cp4o_backward_data_unfused)
+    rc = fn(ctypes.byref(s), _fp(dy), _fp(FK), _fp(FC), _fp(FH), _fp(FW), _fp(dx))
+    assert direct or rc == 0
+    return dx
+
+
+def backward_filter(x, dy, FK, FC, FH, FW, pad, direct=False):
+    """Returns (dFK, dFC, dFH, dFW)."""
+    x, dy, FK, FC, FH, FW = map(_f32, (x, dy, FK, FC, FH, FW))
+    s = shape_of(x.shape, FK, FC, FH, FW, pad)
+    assert dy.shape == (s.N, s.T, s.H, s.W)
+    outs = [np.zeros_like(f) for f in (FK, FC, FH, FW)]
+    if direct:
+        for which, o in enumerate(outs):
+            lib().cp4o_backward_filter_factor_direct(
+                ctypes.byref(s), ctypes.c_int(which), _fp(o), _fp(x), _fp(dy),
+                _fp(FK), _fp(FC), _fp(FH), _fp(FW))
+    else:
+        rc = lib().cp4o_backward_filter_unfused(
+            ctypes.byref(s), _fp(x), _fp(dy), _fp(FK), _fp(FC), _fp(FH), _fp(FW),
+            *[_fp(o) for o in outs])
+        assert rc == 0
+    return tuple(outs)
+
+
+def backward_filter_full(x, dy, Y, X, pad):
+    """Dense filter gradient dK[T,C,Y,X] (cp4Conv2dBackwardFilter.cu:23-59)."""
+    x, dy = _f32(x), _f32(dy)
+    N, C, H, W = x.shape
+    s = Shape(N=N, H=H, W=W, pad=pad, T=dy.shape[1], C=C, Y=Y, X=X, Rank=0)
+    dK = np.zeros((s.T, C, Y, X), np.float32)
+    lib().cp4o_backward_filter_full_direct(ctypes.byref(s), _fp(dK), _fp(x), _fp(dy))
+    return dK
+
+
+def count_exceeding(a, b, tol):
+    a, b = _f32(a).ravel(), _f32(b).ravel()
+    assert a.size == b.size
+    return int(lib().cp4o_count_exceeding(_fp(a), _fp(b), ctypes.c_size_t(a.size),
+                                          ctypes.c_float(tol)))
