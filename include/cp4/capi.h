@@ -1,0 +1,175 @@
+/*
+ * C ABI of the MI355X (gfx950) fused CP4-decomposed Conv2d library.
+ *
+ *   y[n,k,h,w] = sum_r FK[k,r] sum_c FC[c,r] sum_{i,j} FH[i,r] FW[j,r]
+ *                x[n,c,h+i-pad,w+j-pad]            (zero padding, stride 1)
+ *
+ * Plain pointers and sizes only.  Every data pointer is a DEVICE pointer to
+ * contiguous fp32; activations are NCHW, the four factor matrices row-major
+ * [dim, Rank] in the reference's argument order (out-channel FK = "FT",
+ * in-channel FC, height FH = "FY", width FW = "FX").  Nothing here keeps global
+ * state between calls, so calls on different streams may overlap.  Functions
+ * return a status code and never exit the process.
+ */
+#ifndef CP4_CAPI_H
+#define CP4_CAPI_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* The nine unsigned fields of the reference's tensor_shape, same order
+ * (Cuda_kernels/Tensor.cuh:10-19).  T = out-channel count K. */
+typedef struct cp4_shape {
+  unsigned N, H, W, pad, T, C, Y, X, Rank;
+} cp4_shape;
+
+typedef enum cp4_status {
+  CP4_OK = 0,
+  CP4_ERR_NULL_POINTER = 1,
+  CP4_ERR_SHAPE = 2,       /* zero dim, Y != X, sizes beyond 2^31 elements ... */
+  CP4_ERR_HIP = 3,         /* a HIP runtime call failed; see cp4_last_error_message */
+  CP4_ERR_WORKSPACE = 4,   /* workspace missing or too small */
+  CP4_ERR_UNSUPPORTED = 5  /* requested kernel variant cannot run this shape */
+} cp4_status;
+
+/* A hipStream_t passed as void*; NULL is the default stream. */
+typedef void* cp4_stream;
+
+const char* cp4_status_string(cp4_status);
+/* Detail of the calling thread's last failure ("" if none). */
+const char* cp4_last_error_message(void);
+
+/* ---- the three passes --------------------------------------------------- */
+
+/* Replaces cp4_conv2d_forward_gpu (Cuda_kernels/cp4Conv2dForward.cuh:7-14,
+ * .cu:187-328): x[N,C,H,W] -> y[N,T,H,W].  Asynchronous on `stream`. */
+cp4_status cp4_conv2d_forward(const cp4_shape* shape, const float* x,
+                              const float* FK, const float* FC,
+                              const float* FH, const float* FW, float* y,
+                              cp4_stream stream);
+
+/* Replaces cp4_conv2d_backward_data_gpu
+ * (Cuda_kernels/cp4Conv2dBackwardData.cuh:7-14, .cu:112-282):
+ * dy[N,T,H,W] -> dx[N,C,H,W] with the reference's flipped taps. */
+cp4_status cp4_conv2d_backward_data(const cp4_shape* shape, const float* dy,
+                                    const float* FK, const float* FC,
+                                    const float* FH, const float* FW,
+                                    float* dx, cp4_stream stream);
+
+/* Replaces the four host loop nests cp4_conv2d_backward_filter_{t,c,y,x}_gpu
+ * (Cuda_kernels/cp4Conv2dBackwardFilter.cuh:13-47, .cu:64-257) with one fused
+ * call producing dFK[T,R], dFC[C,R], dFH[Y,R], dFW[X,R].  Outputs are
+ * OVERWRITTEN (the reference's per-factor functions accumulate; the C++
+ * wrappers of the same names keep that).  `workspace` must hold at least
+ * cp4_conv2d_backward_filter_workspace_bytes(shape) bytes of device memory;
+ * its contents are scratch.  Deterministic: no floating-point atomics. */
+size_t cp4_conv2d_backward_filter_workspace_bytes(const cp4_shape* shape);
+cp4_status cp4_conv2d_backward_filter(const cp4_shape* shape, const float* x,
+                                      const float* dy, const float* FK,
+                                      const float* FC, const float* FH,
+                                      const float* FW, float* dFK, float* dFC,
+                                      float* dFH, float* dFW, void* workspace,
+                                      size_t workspace_bytes,
+                                      cp4_stream stream);
+
+/* Replaces cp4_conv2d_backward_filter_full_gpu
+ * (Cuda_kernels/cp4Conv2dBackwardFilter.cuh:7-11, .cu:23-59): dense filter
+ * gradient dK[T,C,Y,X]; accumulate != 0 adds into dK as the reference does. */
+cp4_status cp4_conv2d_backward_filter_full(const cp4_shape* shape,
+                                           const float* x, const float* dy,
+                                           float* dK, int accumulate,
+                                           cp4_stream stream);
+
+/* ---- timed launches: the reference's PROFCOUNT loop ---------------------- */
+
+/* Replace the event-timed loops of cp4Conv2dForward.cu:245-327 and
+ * cp4Conv2dBackwardData.cu:165-281: `warmup` untimed launches, then
+ * `profcount` launches bracketed by ONE pair of HIP events on `stream` with no
+ * host synchronisation in between; *mean_us = elapsed / profcount. */
+cp4_status cp4_time_forward(const cp4_shape* shape, const float* x,
+                            const float* FK, const float* FC, const float* FH,
+                            const float* FW, float* y, unsigned warmup,
+                            unsigned profcount, float* mean_us,
+                            cp4_stream stream);
+cp4_status cp4_time_backward_data(const cp4_shape* shape, const float* dy,
+                                  const float* FK, const float* FC,
+                                  const float* FH, const float* FW, float* dx,
+                                  unsigned warmup, unsigned profcount,
+                                  float* mean_us, cp4_stream stream);
+cp4_status cp4_time_backward_filter(const cp4_shape* shape, const float* x,
+                                    const float* dy, const float* FK,
+                                    const float* FC, const float* FH,
+                                    const float* FW, float* dFK, float* dFC,
+                                    float* dFH, float* dFW, void* workspace,
+                                    size_t workspace_bytes, unsigned warmup,
+                                    unsigned profcount, float* mean_us,
+                                    cp4_stream stream);
+
+/* ---- kernel variants and the tuner --------------------------------------- */
+
+/* Replaces the reference's tile heuristic (cp4Conv2dForward.cu:228-233).  The
+ * forward / backward-data pass has several kernel variants; variant -1 means
+ * "library's choice" (a tuned entry for this shape if cp4_tune_forward has
+ * run, else a size heuristic). */
+int cp4_forward_variant_count(void);
+const char* cp4_forward_variant_name(int variant);
+/* CP4_OK if `variant` can run `shape`, else CP4_ERR_UNSUPPORTED. */
+cp4_status cp4_forward_variant_supported(const cp4_shape* shape, int variant);
+cp4_status cp4_conv2d_forward_variant(const cp4_shape* shape, const float* x,
+                                      const float* FK, const float* FC,
+                                      const float* FH, const float* FW,
+                                      float* y, int variant,
+                                      cp4_stream stream);
+/* Times every variant that supports `shape` (warmup + profcount launches
+ * each) on the caller's buffers, remembers the fastest for this shape for the
+ * rest of the process and reports it. */
+cp4_status cp4_tune_forward(const cp4_shape* shape, const float* x,
+                            const float* FK, const float* FC, const float* FH,
+                            const float* FW, float* y, unsigned warmup,
+                            unsigned profcount, int* best_variant,
+                            float* best_us, cp4_stream stream);
+void cp4_tune_clear(void);
+
+/* ---- device allocator / copy helpers (the reference's Tensor uses
+ * cudaMallocManaged, Cuda_kernels/Tensor.cu:8-39) ------------------------- */
+cp4_status cp4_set_device(int ordinal);
+cp4_status cp4_device_malloc(void** ptr, size_t bytes);
+cp4_status cp4_device_free(void* ptr);
+cp4_status cp4_host_malloc(void** ptr, size_t bytes); /* pinned */
+cp4_status cp4_host_free(void* ptr);
+cp4_status cp4_memcpy_h2d(void* dst, const void* src, size_t bytes, cp4_stream);
+cp4_status cp4_memcpy_d2h(void* dst, const void* src, size_t bytes, cp4_stream);
+cp4_status cp4_memcpy_d2d(void* dst, const void* src, size_t bytes, cp4_stream);
+cp4_status cp4_memset_zero(void* dst, size_t bytes, cp4_stream);
+cp4_status cp4_stream_synchronize(cp4_stream);
+cp4_status cp4_device_synchronize(void);
+
+/* ---- test / bench utilities (Cuda_kernels/Utils.cuh:9-13) ---------------- */
+
+/* Replaces cp_recompose (Utils.cu:36-98): K[T,C,Y,X] = sum_r FK FC FH FW. */
+cp4_status cp4_recompose(const cp4_shape* shape, const float* FK,
+                         const float* FC, const float* FH, const float* FW,
+                         float* K, cp4_stream stream);
+/* Replaces arrayRelativeDelta / AllClose (Utils.cu:143-180): *count = number
+ * of elements with symmetric relative error > tol (absolute error if either
+ * value is 0).  Synchronises `stream`. */
+cp4_status cp4_count_exceeding(const float* A, const float* B, size_t n,
+                               float tol, long long* count, cp4_stream stream);
+/* Replaces random_fill's generator (Utils.cu:22-33): uniform in (0,1], a
+ * counter-based hash of (seed, index), reproducible on any device. */
+cp4_status cp4_random_uniform(float* dst, size_t n, unsigned long long seed,
+                              cp4_stream stream);
+/* Plain streaming copy (one read + one write per element); the calibration
+ * kernel for bandwidth and for hardware-counter scale factors. */
+cp4_status cp4_copy_f32(float* dst, const float* src, size_t n, cp4_stream);
+cp4_status cp4_time_copy_f32(float* dst, const float* src, size_t n,
+                             unsigned warmup, unsigned profcount,
+                             float* mean_us, cp4_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CP4_CAPI_H */

@@ -1,0 +1,16 @@
+"""MI355X-native fused CP4-decomposed Conv2d (forward, backward-data,
+backward-filter) behind a C ABI.
+
+This Python package is only the loader/binding of ``csrc/libcp4conv.so`` used
+by the tests and the bench; the product is the shared library and the C++ host
+layer under ``csrc/host``.  There is no CPU or PyTorch fallback: importing
+``paralleltnnlayers_amd.capi`` without the built library raises.
+"""
+from .capi import (Shape, Cp4Error, lib, library_path, conv2d_forward,
+                   conv2d_backward_data, conv2d_backward_filter,
+                   conv2d_backward_filter_full, backward_filter_workspace_bytes,
+                   time_forward, time_backward_data, time_backward_filter,
+                   tune_forward, forward_variants, recompose, count_exceeding,
+                   random_uniform, time_copy)
+
+__all__ = [n for n in dir() if not n.startswith("_")]

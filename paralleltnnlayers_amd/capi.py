@@ -1,0 +1,258 @@
+"""ctypes binding of include/cp4/capi.h.
+
+Device memory and streams come from PyTorch (ROCm): every tensor argument must
+be a contiguous float32 CUDA(-HIP) tensor; its ``data_ptr()`` is what crosses
+the C ABI.  Launches go on torch's current stream unless ``stream`` is given.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "csrc", "libcp4conv.so")
+
+
+class Cp4Error(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__(f"cp4 status {status}: {message}")
+        self.status = status
+
+
+class Shape(ctypes.Structure):
+    """cp4_shape: the nine unsigned fields of the reference's tensor_shape
+    (Cuda_kernels/Tensor.cuh:10-19), same order."""
+    _fields_ = [(k, ctypes.c_uint) for k in
+                ("N", "H", "W", "pad", "T", "C", "Y", "X", "Rank")]
+
+    def __repr__(self):
+        return "Shape(" + ", ".join(f"{k}={getattr(self, k)}" for k, _ in self._fields_) + ")"
+
+
+# status codes of cp4_status
+OK, ERR_NULL_POINTER, ERR_SHAPE, ERR_HIP, ERR_WORKSPACE, ERR_UNSUPPORTED = range(6)
+
+_lib = None
+_F = ctypes.c_void_p          # const float* / float* (device)
+_S = ctypes.POINTER(Shape)
+
+
+def library_path():
+    return _LIB
+
+
+def lib():
+    """The loaded shared library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB):
+        raise ImportError(
+            f"{_LIB} is missing: build it with `python -c 'import __graft_entry__ as g; "
+            "g.build()'` (or `make -C paralleltnnlayers_amd/csrc`). There is no fallback path.")
+    L = ctypes.CDLL(_LIB)
+    L.cp4_status_string.restype = ctypes.c_char_p
+    L.cp4_status_string.argtypes = [ctypes.c_int]
+    L.cp4_last_error_message.restype = ctypes.c_char_p
+    L.cp4_forward_variant_name.restype = ctypes.c_char_p
+    L.cp4_forward_variant_name.argtypes = [ctypes.c_int]
+    L.cp4_conv2d_backward_filter_workspace_bytes.restype = ctypes.c_size_t
+    L.cp4_conv2d_backward_filter_workspace_bytes.argtypes = [_S]
+    fwd = [_S, _F, _F, _F, _F, _F, _F]
+    L.cp4_conv2d_forward.argtypes = fwd + [ctypes.c_void_p]
+    L.cp4_conv2d_forward_variant.argtypes = fwd + [ctypes.c_int, ctypes.c_void_p]
+    L.cp4_conv2d_backward_data.argtypes = fwd + [ctypes.c_void_p]
+    bwf = [_S] + [_F] * 10 + [ctypes.c_void_p, ctypes.c_size_t]
+    L.cp4_conv2d_backward_filter.argtypes = bwf + [ctypes.c_void_p]
+    L.cp4_conv2d_backward_filter_full.argtypes = [_S, _F, _F, _F, ctypes.c_int, ctypes.c_void_p]
+    timing = [ctypes.c_uint, ctypes.c_uint, ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
+    L.cp4_time_forward.argtypes = fwd + timing
+    L.cp4_time_backward_data.argtypes = fwd + timing
+    L.cp4_time_backward_filter.argtypes = bwf + timing
+    L.cp4_forward_variant_supported.argtypes = [_S, ctypes.c_int]
+    L.cp4_tune_forward.argtypes = fwd + [ctypes.c_uint, ctypes.c_uint,
+                                         ctypes.POINTER(ctypes.c_int),
+                                         ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
+    L.cp4_tune_clear.restype = None
+    L.cp4_recompose.argtypes = [_S, _F, _F, _F, _F, _F, ctypes.c_void_p]
+    L.cp4_count_exceeding.argtypes = [_F, _F, ctypes.c_size_t, ctypes.c_float,
+                                      ctypes.POINTER(ctypes.c_longlong), ctypes.c_void_p]
+    L.cp4_random_uniform.argtypes = [_F, ctypes.c_size_t, ctypes.c_ulonglong, ctypes.c_void_p]
+    L.cp4_copy_f32.argtypes = [_F, _F, ctypes.c_size_t, ctypes.c_void_p]
+    L.cp4_time_copy_f32.argtypes = [_F, _F, ctypes.c_size_t] + timing
+    L.cp4_device_malloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t]
+    L.cp4_device_free.argtypes = [ctypes.c_void_p]
+    L.cp4_host_malloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t]
+    L.cp4_host_free.argtypes = [ctypes.c_void_p]
+    for name in ("cp4_memcpy_h2d", "cp4_memcpy_d2h", "cp4_memcpy_d2d"):
+        getattr(L, name).argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                                     ctypes.c_void_p]
+    L.cp4_memset_zero.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    L.cp4_stream_synchronize.argtypes = [ctypes.c_void_p]
+    L.cp4_set_device.argtypes = [ctypes.c_int]
+    _lib = L
+    return L
+
+
+def check(status):
+    if status != OK:
+        L = lib()
+        raise Cp4Error(status, f"{L.cp4_status_string(status).decode()}: "
+                               f"{L.cp4_last_error_message().decode()}")
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.dtype == torch.float32 and t.is_contiguous(), \
+        "expected a contiguous float32 device tensor"
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(stream):
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def shape_for(x_or_dy_shape, FK, FC, FH, FW, pad):
+    """tensor_shape as CP::Conv2dForward / Conv2dBackwardData derive it
+    (Cuda_kernels/cp4Conv2d.cu:21-30, 55-64): N,H,W from the activation, T and
+    Rank from FK, C from FC, Y from FH, X from FW."""
+    N, _, H, W = x_or_dy_shape
+    return Shape(N=N, H=H, W=W, pad=pad, T=FK.shape[0], C=FC.shape[0],
+                 Y=FH.shape[0], X=FW.shape[0], Rank=FK.shape[1])
+
+
+def conv2d_forward(x, FK, FC, FH, FW, pad=1, out=None, variant=-1, stream=None):
+    s = shape_for(x.shape, FK, FC, FH, FW, pad)
+    assert x.shape[1] == s.C and FC.shape[1] == s.Rank
+    y = out if out is not None else torch.empty((s.N, s.T, s.H, s.W), device=x.device,
+                                                dtype=torch.float32)
+    check(lib().cp4_conv2d_forward_variant(ctypes.byref(s), _ptr(x), _ptr(FK), _ptr(FC),
+                                           _ptr(FH), _ptr(FW), _ptr(y), variant,
+                                           _stream(stream)))
+    return y
+
+
+def conv2d_backward_data(dy, FK, FC, FH, FW, pad=1, out=None, stream=None):
+    s = shape_for(dy.shape, FK, FC, FH, FW, pad)
+    assert dy.shape[1] == s.T
+    dx = out if out is not None else torch.empty((s.N, s.C, s.H, s.W), device=dy.device,
+                                                 dtype=torch.float32)
+    check(lib().cp4_conv2d_backward_data(ctypes.byref(s), _ptr(dy), _ptr(FK), _ptr(FC),
+                                         _ptr(FH), _ptr(FW), _ptr(dx), _stream(stream)))
+    return dx
+
+
+def backward_filter_workspace_bytes(s):
+    return int(lib().cp4_conv2d_backward_filter_workspace_bytes(ctypes.byref(s)))
+
+
+def _workspace(s, device, workspace):
+    need = backward_filter_workspace_bytes(s)
+    if workspace is None:
+        workspace = torch.empty(max(need, 4) // 4 + 1, device=device, dtype=torch.float32)
+    return workspace, workspace.numel() * 4
+
+
+def conv2d_backward_filter(x, dy, FK, FC, FH, FW, pad=1, workspace=None, stream=None):
+    """Returns (dFK, dFC, dFH, dFW)."""
+    s = shape_for(x.shape, FK, FC, FH, FW, pad)
+    assert tuple(dy.shape) == (s.N, s.T, s.H, s.W) and x.shape[1] == s.C
+    outs = [torch.empty_like(f) for f in (FK, FC, FH, FW)]
+    ws, ws_bytes = _workspace(s, x.device, workspace)
+    check(lib().cp4_conv2d_backward_filter(
+        ctypes.byref(s), _ptr(x), _ptr(dy), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
+        *[_ptr(o) for o in outs], ctypes.c_void_p(ws.data_ptr()), ws_bytes, _stream(stream)))
+    return tuple(outs)
+
+
+def conv2d_backward_filter_full(x, dy, Y, X, pad=1, out=None, stream=None):
+    N, C, H, W = x.shape
+    s = Shape(N=N, H=H, W=W, pad=pad, T=dy.shape[1], C=C, Y=Y, X=X, Rank=0)
+    accumulate = out is not None
+    dK = out if accumulate else torch.empty((s.T, C, Y, X), device=x.device,
+                                            dtype=torch.float32)
+    check(lib().cp4_conv2d_backward_filter_full(ctypes.byref(s), _ptr(x), _ptr(dy), _ptr(dK),
+                                                int(accumulate), _stream(stream)))
+    return dK
+
+
+def time_forward(x, FK, FC, FH, FW, y, pad, warmup=1, profcount=47, stream=None):
+    s = shape_for(x.shape, FK, FC, FH, FW, pad)
+    us = ctypes.c_float()
+    check(lib().cp4_time_forward(ctypes.byref(s), _ptr(x), _ptr(FK), _ptr(FC), _ptr(FH),
+                                 _ptr(FW), _ptr(y), warmup, profcount, ctypes.byref(us),
+                                 _stream(stream)))
+    return us.value
+
+
+def time_backward_data(dy, FK, FC, FH, FW, dx, pad, warmup=1, profcount=47, stream=None):
+    s = shape_for(dy.shape, FK, FC, FH, FW, pad)
+    us = ctypes.c_float()
+    check(lib().cp4_time_backward_data(ctypes.byref(s), _ptr(dy), _ptr(FK), _ptr(FC),
+                                       _ptr(FH), _ptr(FW), _ptr(dx), warmup, profcount,
+                                       ctypes.byref(us), _stream(stream)))
+    return us.value
+
+
+def time_backward_filter(x, dy, FK, FC, FH, FW, pad, warmup=1, profcount=47,
+                         workspace=None, stream=None):
+    s = shape_for(x.shape, FK, FC, FH, FW, pad)
+    outs = [torch.empty_like(f) for f in (FK, FC, FH, FW)]
+    ws, ws_bytes = _workspace(s, x.device, workspace)
+    us = ctypes.c_float()
+    check(lib().cp4_time_backward_filter(
+        ctypes.byref(s), _ptr(x), _ptr(dy), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
+        *[_ptr(o) for o in outs], ctypes.c_void_p(ws.data_ptr()), ws_bytes, warmup,
+        profcount, ctypes.byref(us), _stream(stream)))
+    return us.value
+
+
+def forward_variants(s=None):
+    """[(index, name, supported-for-shape)]"""
+    L = lib()
+    out = []
+    for v in range(L.cp4_forward_variant_count()):
+        ok = None if s is None else L.cp4_forward_variant_supported(ctypes.byref(s), v) == OK
+        out.append((v, L.cp4_forward_variant_name(v).decode(), ok))
+    return out
+
+
+def tune_forward(x, FK, FC, FH, FW, y, pad, warmup=1, profcount=10, stream=None):
+    s = shape_for(x.shape, FK, FC, FH, FW, pad)
+    best, us = ctypes.c_int(-1), ctypes.c_float()
+    check(lib().cp4_tune_forward(ctypes.byref(s), _ptr(x), _ptr(FK), _ptr(FC), _ptr(FH),
+                                 _ptr(FW), _ptr(y), warmup, profcount, ctypes.byref(best),
+                                 ctypes.byref(us), _stream(stream)))
+    return best.value, us.value
+
+
+def recompose(FK, FC, FH, FW, stream=None):
+    s = Shape(T=FK.shape[0], C=FC.shape[0], Y=FH.shape[0], X=FW.shape[0], Rank=FK.shape[1])
+    K = torch.empty((s.T, s.C, s.Y, s.X), device=FK.device, dtype=torch.float32)
+    check(lib().cp4_recompose(ctypes.byref(s), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
+                              _ptr(K), _stream(stream)))
+    return K
+
+
+def count_exceeding(a, b, tol, stream=None):
+    assert a.numel() == b.numel()
+    n = ctypes.c_longlong()
+    check(lib().cp4_count_exceeding(_ptr(a), _ptr(b), a.numel(), tol, ctypes.byref(n),
+                                    _stream(stream)))
+    return n.value
+
+
+def random_uniform(shape, seed, device="cuda", stream=None):
+    t = torch.empty(shape, device=device, dtype=torch.float32)
+    check(lib().cp4_random_uniform(_ptr(t), t.numel(), seed, _stream(stream)))
+    return t
+
+
+def time_copy(dst, src, warmup=1, profcount=47, stream=None):
+    us = ctypes.c_float()
+    check(lib().cp4_time_copy_f32(_ptr(dst), _ptr(src), src.numel(), warmup, profcount,
+                                  ctypes.byref(us), _stream(stream)))
+    return us.value

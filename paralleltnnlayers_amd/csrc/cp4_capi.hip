@@ -1,0 +1,459 @@
+// C ABI entry points: argument checks, kernel-variant choice, the PROFCOUNT
+// timing loops and the device allocator / copy helpers.
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <tuple>
+
+#include "cp4_internal.h"
+
+namespace {
+
+using cp4::FwdArgs;
+
+thread_local char g_err[256] = "";
+
+cp4_status fail(cp4_status st, const char* what) {
+  std::snprintf(g_err, sizeof(g_err), "%s", what);
+  return st;
+}
+cp4_status hip_fail(hipError_t e, const char* where) {
+  std::snprintf(g_err, sizeof(g_err), "%s: %s", where, hipGetErrorString(e));
+  return CP4_ERR_HIP;
+}
+#define CP4_HIP(call)                                  \
+  do {                                                 \
+    hipError_t e_ = (call);                            \
+    if (e_ != hipSuccess) return hip_fail(e_, #call);  \
+  } while (0)
+
+hipStream_t as_stream(cp4_stream s) { return static_cast<hipStream_t>(s); }
+
+// Shape rules shared by the three passes.  N == 0 is a valid empty batch.
+cp4_status check_shape(const cp4_shape* s) {
+  if (!s) return fail(CP4_ERR_NULL_POINTER, "shape is NULL");
+  if (!s->H || !s->W || !s->T || !s->C || !s->Y || !s->X || !s->Rank)
+    return fail(CP4_ERR_SHAPE, "H, W, T, C, Y, X and Rank must be >= 1");
+  if ((unsigned long long)s->H * s->W >= (1ull << 31))
+    return fail(CP4_ERR_SHAPE, "H*W must be below 2^31");
+  if (s->N > 65535u) return fail(CP4_ERR_SHAPE, "N must be <= 65535");
+  if (s->T > 65535u || s->C > 65535u || s->Rank > 65535u)
+    return fail(CP4_ERR_SHAPE, "T, C and Rank must be <= 65535");
+  if (s->Y > 1024u || s->X > 1024u || s->pad > 1024u)
+    return fail(CP4_ERR_SHAPE, "Y, X and pad must be <= 1024");
+  return CP4_OK;
+}
+
+FwdArgs forward_args(const cp4_shape& s, const float* x, const float* FK,
+                     const float* FC, const float* FH, const float* FW,
+                     float* y) {
+  FwdArgs a{};
+  a.x = x; a.Fin = FC; a.Fout = FK; a.FH = FH; a.FW = FW; a.y = y;
+  a.N = s.N; a.Cin = s.C; a.Cout = s.T; a.H = s.H; a.W = s.W; a.pad = s.pad;
+  a.Y = s.Y; a.X = s.X; a.R = s.Rank; a.flip = 0;
+  return a;
+}
+// Backward-data is the forward kernel on dy with the channel factors swapped
+// and the taps read in reverse (cp4Conv2dBackwardData.cu:79-87,98-108).
+FwdArgs backward_data_args(const cp4_shape& s, const float* dy, const float* FK,
+                           const float* FC, const float* FH, const float* FW,
+                           float* dx) {
+  FwdArgs a{};
+  a.x = dy; a.Fin = FK; a.Fout = FC; a.FH = FH; a.FW = FW; a.y = dx;
+  a.N = s.N; a.Cin = s.T; a.Cout = s.C; a.H = s.H; a.W = s.W; a.pad = s.pad;
+  a.Y = s.Y; a.X = s.X; a.R = s.Rank; a.flip = 1;
+  return a;
+}
+
+struct Variant {
+  const char* name;
+  bool (*supported)(const FwdArgs&);
+  hipError_t (*launch)(const FwdArgs&, hipStream_t);
+};
+// Order = preference of the untuned heuristic, last to first.
+const Variant kVariants[] = {
+    {"general_valu", cp4::fwd_general_supported, cp4::fwd_general_launch},
+    {"mfma_strip", cp4::fwd_mfma_supported, cp4::fwd_mfma_launch},
+};
+constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+
+using TuneKey = std::tuple<int, int, int, int, int, int, int, int, int, int>;
+std::mutex g_tune_mu;
+std::map<TuneKey, int> g_tuned;
+
+TuneKey key_of(const FwdArgs& a) {
+  return TuneKey(a.N, a.Cin, a.Cout, a.H, a.W, a.pad, a.Y, a.X, a.R, a.flip);
+}
+
+int choose_variant(const FwdArgs& a) {
+  {
+    std::lock_guard<std::mutex> lk(g_tune_mu);
+    auto it = g_tuned.find(key_of(a));
+    if (it != g_tuned.end()) return it->second;
+  }
+  for (int v = kNumVariants - 1; v >= 0; --v)
+    if (kVariants[v].supported(a)) return v;
+  return -1;
+}
+
+cp4_status run_forward_like(const FwdArgs& a, int variant, hipStream_t st) {
+  if (a.N == 0) return CP4_OK;
+  if (variant < 0) variant = choose_variant(a);
+  if (variant < 0 || variant >= kNumVariants || !kVariants[variant].supported(a))
+    return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape");
+  CP4_HIP(kVariants[variant].launch(a, st));
+  return CP4_OK;
+}
+
+cp4_status check_forward_ptrs(const void* x, const void* FK, const void* FC,
+                              const void* FH, const void* FW, const void* y) {
+  if (!x || !FK || !FC || !FH || !FW || !y)
+    return fail(CP4_ERR_NULL_POINTER, "a data pointer is NULL");
+  return CP4_OK;
+}
+
+// `warmup` untimed launches then `profcount` launches between one event pair.
+template <class Launch>
+cp4_status time_loop(Launch&& launch, unsigned warmup, unsigned profcount,
+                     float* mean_us, hipStream_t st) {
+  if (!mean_us) return fail(CP4_ERR_NULL_POINTER, "mean_us is NULL");
+  if (profcount == 0) return fail(CP4_ERR_SHAPE, "profcount must be >= 1");
+  hipEvent_t e0, e1;
+  CP4_HIP(hipEventCreate(&e0));
+  CP4_HIP(hipEventCreate(&e1));
+  cp4_status rc = CP4_OK;
+  for (unsigned i = 0; i < warmup && rc == CP4_OK; ++i) rc = launch();
+  hipError_t e = hipSuccess;
+  if (rc == CP4_OK) e = hipEventRecord(e0, st);
+  for (unsigned i = 0; i < profcount && rc == CP4_OK && e == hipSuccess; ++i)
+    rc = launch();
+  if (rc == CP4_OK && e == hipSuccess) e = hipEventRecord(e1, st);
+  if (rc == CP4_OK && e == hipSuccess) e = hipEventSynchronize(e1);
+  float ms = 0.f;
+  if (rc == CP4_OK && e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc != CP4_OK) return rc;
+  if (e != hipSuccess) return hip_fail(e, "timing loop");
+  *mean_us = ms * 1e3f / (float)profcount;
+  return CP4_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* cp4_status_string(cp4_status s) {
+  switch (s) {
+    case CP4_OK: return "ok";
+    case CP4_ERR_NULL_POINTER: return "null pointer";
+    case CP4_ERR_SHAPE: return "invalid shape";
+    case CP4_ERR_HIP: return "HIP runtime error";
+    case CP4_ERR_WORKSPACE: return "workspace missing or too small";
+    case CP4_ERR_UNSUPPORTED: return "unsupported kernel variant for this shape";
+  }
+  return "unknown status";
+}
+
+const char* cp4_last_error_message(void) { return g_err; }
+
+cp4_status cp4_conv2d_forward_variant(const cp4_shape* shape, const float* x,
+                                      const float* FK, const float* FC,
+                                      const float* FH, const float* FW,
+                                      float* y, int variant,
+                                      cp4_stream stream) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return CP4_OK;
+  rc = check_forward_ptrs(x, FK, FC, FH, FW, y);
+  if (rc != CP4_OK) return rc;
+  return run_forward_like(forward_args(*shape, x, FK, FC, FH, FW, y), variant,
+                          as_stream(stream));
+}
+
+cp4_status cp4_conv2d_forward(const cp4_shape* shape, const float* x,
+                              const float* FK, const float* FC,
+                              const float* FH, const float* FW, float* y,
+                              cp4_stream stream) {
+  return cp4_conv2d_forward_variant(shape, x, FK, FC, FH, FW, y, -1, stream);
+}
+
+cp4_status cp4_conv2d_backward_data(const cp4_shape* shape, const float* dy,
+                                    const float* FK, const float* FC,
+                                    const float* FH, const float* FW,
+                                    float* dx, cp4_stream stream) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return CP4_OK;
+  rc = check_forward_ptrs(dy, FK, FC, FH, FW, dx);
+  if (rc != CP4_OK) return rc;
+  return run_forward_like(backward_data_args(*shape, dy, FK, FC, FH, FW, dx),
+                          -1, as_stream(stream));
+}
+
+size_t cp4_conv2d_backward_filter_workspace_bytes(const cp4_shape* shape) {
+  if (check_shape(shape) != CP4_OK || shape->N == 0) return 0;
+  return cp4::bwd_filter_workspace_bytes(*shape);
+}
+
+cp4_status cp4_conv2d_backward_filter(const cp4_shape* shape, const float* x,
+                                      const float* dy, const float* FK,
+                                      const float* FC, const float* FH,
+                                      const float* FW, float* dFK, float* dFC,
+                                      float* dFH, float* dFW, void* workspace,
+                                      size_t workspace_bytes,
+                                      cp4_stream stream) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (!FK || !FC || !FH || !FW || !dFK || !dFC || !dFH || !dFW)
+    return fail(CP4_ERR_NULL_POINTER, "a factor or gradient pointer is NULL");
+  const cp4_shape& s = *shape;
+  hipStream_t st = as_stream(stream);
+  if (s.N == 0) {  // empty batch: the gradients are zero
+    CP4_HIP(hipMemsetAsync(dFK, 0, sizeof(float) * s.T * s.Rank, st));
+    CP4_HIP(hipMemsetAsync(dFC, 0, sizeof(float) * s.C * s.Rank, st));
+    CP4_HIP(hipMemsetAsync(dFH, 0, sizeof(float) * s.Y * s.Rank, st));
+    CP4_HIP(hipMemsetAsync(dFW, 0, sizeof(float) * s.X * s.Rank, st));
+    return CP4_OK;
+  }
+  if (!x || !dy) return fail(CP4_ERR_NULL_POINTER, "x or dy is NULL");
+  if (!workspace || workspace_bytes < cp4::bwd_filter_workspace_bytes(s))
+    return fail(CP4_ERR_WORKSPACE,
+                "workspace smaller than cp4_conv2d_backward_filter_workspace_bytes");
+  cp4::BwdFilterArgs a{};
+  a.x = x; a.dy = dy; a.FK = FK; a.FC = FC; a.FH = FH; a.FW = FW;
+  a.dFK = dFK; a.dFC = dFC; a.dFH = dFH; a.dFW = dFW; a.workspace = workspace;
+  a.N = s.N; a.C = s.C; a.T = s.T; a.H = s.H; a.W = s.W; a.pad = s.pad;
+  a.Y = s.Y; a.X = s.X; a.R = s.Rank;
+  CP4_HIP(cp4::bwd_filter_launch(a, st));
+  return CP4_OK;
+}
+
+cp4_status cp4_conv2d_backward_filter_full(const cp4_shape* shape,
+                                           const float* x, const float* dy,
+                                           float* dK, int accumulate,
+                                           cp4_stream stream) {
+  cp4_shape s;
+  if (!shape) return fail(CP4_ERR_NULL_POINTER, "shape is NULL");
+  s = *shape;
+  if (s.Rank == 0) s.Rank = 1;  // the dense gradient does not involve the rank
+  cp4_status rc = check_shape(&s);
+  if (rc != CP4_OK) return rc;
+  if (!dK) return fail(CP4_ERR_NULL_POINTER, "dK is NULL");
+  hipStream_t st = as_stream(stream);
+  if (s.N == 0) {
+    if (!accumulate)
+      CP4_HIP(hipMemsetAsync(dK, 0, sizeof(float) * s.T * s.C * s.Y * s.X, st));
+    return CP4_OK;
+  }
+  if (!x || !dy) return fail(CP4_ERR_NULL_POINTER, "x or dy is NULL");
+  CP4_HIP(cp4::bwd_filter_full_launch(s, x, dy, dK, accumulate, st));
+  return CP4_OK;
+}
+
+cp4_status cp4_time_forward(const cp4_shape* shape, const float* x,
+                            const float* FK, const float* FC, const float* FH,
+                            const float* FW, float* y, unsigned warmup,
+                            unsigned profcount, float* mean_us,
+                            cp4_stream stream) {
+  return time_loop(
+      [&] { return cp4_conv2d_forward(shape, x, FK, FC, FH, FW, y, stream); },
+      warmup, profcount, mean_us, as_stream(stream));
+}
+
+cp4_status cp4_time_backward_data(const cp4_shape* shape, const float* dy,
+                                  const float* FK, const float* FC,
+                                  const float* FH, const float* FW, float* dx,
+                                  unsigned warmup, unsigned profcount,
+                                  float* mean_us, cp4_stream stream) {
+  return time_loop(
+      [&] { return cp4_conv2d_backward_data(shape, dy, FK, FC, FH, FW, dx, stream); },
+      warmup, profcount, mean_us, as_stream(stream));
+}
+
+cp4_status cp4_time_backward_filter(const cp4_shape* shape, const float* x,
+                                    const float* dy, const float* FK,
+                                    const float* FC, const float* FH,
+                                    const float* FW, float* dFK, float* dFC,
+                                    float* dFH, float* dFW, void* workspace,
+                                    size_t workspace_bytes, unsigned warmup,
+                                    unsigned profcount, float* mean_us,
+                                    cp4_stream stream) {
+  return time_loop(
+      [&] {
+        return cp4_conv2d_backward_filter(shape, x, dy, FK, FC, FH, FW, dFK, dFC,
+                                          dFH, dFW, workspace, workspace_bytes,
+                                          stream);
+      },
+      warmup, profcount, mean_us, as_stream(stream));
+}
+
+int cp4_forward_variant_count(void) { return kNumVariants; }
+
+const char* cp4_forward_variant_name(int v) {
+  return (v >= 0 && v < kNumVariants) ? kVariants[v].name : "";
+}
+
+cp4_status cp4_forward_variant_supported(const cp4_shape* shape, int variant) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (variant < 0 || variant >= kNumVariants)
+    return fail(CP4_ERR_UNSUPPORTED, "variant index out of range");
+  const FwdArgs a = forward_args(*shape, nullptr, nullptr, nullptr, nullptr,
+                                 nullptr, nullptr);
+  return kVariants[variant].supported(a)
+             ? CP4_OK
+             : fail(CP4_ERR_UNSUPPORTED, "variant does not support this shape");
+}
+
+cp4_status cp4_tune_forward(const cp4_shape* shape, const float* x,
+                            const float* FK, const float* FC, const float* FH,
+                            const float* FW, float* y, unsigned warmup,
+                            unsigned profcount, int* best_variant,
+                            float* best_us, cp4_stream stream) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  rc = check_forward_ptrs(x, FK, FC, FH, FW, y);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return fail(CP4_ERR_SHAPE, "cannot tune an empty batch");
+  const FwdArgs a = forward_args(*shape, x, FK, FC, FH, FW, y);
+  int best = -1;
+  float best_t = 0.f;
+  for (int v = 0; v < kNumVariants; ++v) {
+    if (!kVariants[v].supported(a)) continue;
+    float us = 0.f;
+    rc = time_loop([&] { return run_forward_like(a, v, as_stream(stream)); },
+                   warmup, profcount, &us, as_stream(stream));
+    if (rc != CP4_OK) return rc;
+    if (best < 0 || us < best_t) { best = v; best_t = us; }
+  }
+  if (best < 0) return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape");
+  {
+    std::lock_guard<std::mutex> lk(g_tune_mu);
+    g_tuned[key_of(a)] = best;
+  }
+  if (best_variant) *best_variant = best;
+  if (best_us) *best_us = best_t;
+  return CP4_OK;
+}
+
+void cp4_tune_clear(void) {
+  std::lock_guard<std::mutex> lk(g_tune_mu);
+  g_tuned.clear();
+}
+
+cp4_status cp4_set_device(int ordinal) {
+  CP4_HIP(hipSetDevice(ordinal));
+  return CP4_OK;
+}
+cp4_status cp4_device_malloc(void** ptr, size_t bytes) {
+  if (!ptr) return fail(CP4_ERR_NULL_POINTER, "ptr is NULL");
+  *ptr = nullptr;
+  if (bytes == 0) return CP4_OK;
+  CP4_HIP(hipMalloc(ptr, bytes));
+  return CP4_OK;
+}
+cp4_status cp4_device_free(void* ptr) {
+  if (ptr) CP4_HIP(hipFree(ptr));
+  return CP4_OK;
+}
+cp4_status cp4_host_malloc(void** ptr, size_t bytes) {
+  if (!ptr) return fail(CP4_ERR_NULL_POINTER, "ptr is NULL");
+  *ptr = nullptr;
+  if (bytes == 0) return CP4_OK;
+  CP4_HIP(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
+  return CP4_OK;
+}
+cp4_status cp4_host_free(void* ptr) {
+  if (ptr) CP4_HIP(hipHostFree(ptr));
+  return CP4_OK;
+}
+cp4_status cp4_memcpy_h2d(void* dst, const void* src, size_t bytes, cp4_stream s) {
+  if (bytes == 0) return CP4_OK;
+  if (!dst || !src) return fail(CP4_ERR_NULL_POINTER, "memcpy pointer is NULL");
+  CP4_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(s)));
+  return CP4_OK;
+}
+cp4_status cp4_memcpy_d2h(void* dst, const void* src, size_t bytes, cp4_stream s) {
+  if (bytes == 0) return CP4_OK;
+  if (!dst || !src) return fail(CP4_ERR_NULL_POINTER, "memcpy pointer is NULL");
+  CP4_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_stream(s)));
+  return CP4_OK;
+}
+cp4_status cp4_memcpy_d2d(void* dst, const void* src, size_t bytes, cp4_stream s) {
+  if (bytes == 0) return CP4_OK;
+  if (!dst || !src) return fail(CP4_ERR_NULL_POINTER, "memcpy pointer is NULL");
+  CP4_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(s)));
+  return CP4_OK;
+}
+cp4_status cp4_memset_zero(void* dst, size_t bytes, cp4_stream s) {
+  if (bytes == 0) return CP4_OK;
+  if (!dst) return fail(CP4_ERR_NULL_POINTER, "memset pointer is NULL");
+  CP4_HIP(hipMemsetAsync(dst, 0, bytes, as_stream(s)));
+  return CP4_OK;
+}
+cp4_status cp4_stream_synchronize(cp4_stream s) {
+  CP4_HIP(hipStreamSynchronize(as_stream(s)));
+  return CP4_OK;
+}
+cp4_status cp4_device_synchronize(void) {
+  CP4_HIP(hipDeviceSynchronize());
+  return CP4_OK;
+}
+
+cp4_status cp4_recompose(const cp4_shape* shape, const float* FK,
+                         const float* FC, const float* FH, const float* FW,
+                         float* K, cp4_stream stream) {
+  if (!shape) return fail(CP4_ERR_NULL_POINTER, "shape is NULL");
+  if (!shape->T || !shape->C || !shape->Y || !shape->X || !shape->Rank)
+    return fail(CP4_ERR_SHAPE, "T, C, Y, X and Rank must be >= 1");
+  if (!FK || !FC || !FH || !FW || !K)
+    return fail(CP4_ERR_NULL_POINTER, "a data pointer is NULL");
+  CP4_HIP(cp4::recompose_launch(*shape, FK, FC, FH, FW, K, as_stream(stream)));
+  return CP4_OK;
+}
+
+cp4_status cp4_count_exceeding(const float* A, const float* B, size_t n,
+                               float tol, long long* count, cp4_stream stream) {
+  if (!count) return fail(CP4_ERR_NULL_POINTER, "count is NULL");
+  *count = 0;
+  if (n == 0) return CP4_OK;
+  if (!A || !B) return fail(CP4_ERR_NULL_POINTER, "a data pointer is NULL");
+  hipStream_t st = as_stream(stream);
+  unsigned long long* d = nullptr;
+  CP4_HIP(hipMalloc(&d, sizeof(*d)));
+  unsigned long long h = 0;
+  hipError_t e = hipMemsetAsync(d, 0, sizeof(*d), st);
+  if (e == hipSuccess) e = cp4::count_exceeding_launch(A, B, n, tol, d, st);
+  if (e == hipSuccess) e = hipMemcpyAsync(&h, d, sizeof(h), hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  (void)hipFree(d);
+  if (e != hipSuccess) return hip_fail(e, "cp4_count_exceeding");
+  *count = (long long)h;
+  return CP4_OK;
+}
+
+cp4_status cp4_random_uniform(float* dst, size_t n, unsigned long long seed,
+                              cp4_stream stream) {
+  if (n == 0) return CP4_OK;
+  if (!dst) return fail(CP4_ERR_NULL_POINTER, "dst is NULL");
+  CP4_HIP(cp4::random_uniform_launch(dst, n, seed, as_stream(stream)));
+  return CP4_OK;
+}
+
+cp4_status cp4_copy_f32(float* dst, const float* src, size_t n, cp4_stream stream) {
+  if (n == 0) return CP4_OK;
+  if (!dst || !src) return fail(CP4_ERR_NULL_POINTER, "a data pointer is NULL");
+  CP4_HIP(cp4::copy_f32_launch(dst, src, n, as_stream(stream)));
+  return CP4_OK;
+}
+
+cp4_status cp4_time_copy_f32(float* dst, const float* src, size_t n,
+                             unsigned warmup, unsigned profcount,
+                             float* mean_us, cp4_stream stream) {
+  return time_loop([&] { return cp4_copy_f32(dst, src, n, stream); }, warmup,
+                   profcount, mean_us, as_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,60 @@
+// Internal interface between the C ABI (cp4_capi.hip) and the kernel
+// translation units.  Every launcher validates nothing: the C ABI has already
+// checked pointers and shape, and each launcher's own `*_supported` predicate
+// says whether its kernel's assumptions hold for a shape.
+#ifndef CP4_INTERNAL_H
+#define CP4_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+
+#include "cp4/capi.h"
+
+namespace cp4 {
+
+// Operands of one forward-shaped launch.  Backward-data is the same kernel
+// with x<-dy, Cin<-T, Cout<-C, Fin<-FK, Fout<-FC and flipped taps
+// (Cuda_kernels/cp4Conv2dBackwardData.cu:79-87,98-108).
+struct FwdArgs {
+  const float* x;     // [N, Cin, H, W]
+  const float* Fin;   // [Cin, R]
+  const float* Fout;  // [Cout, R]
+  const float* FH;    // [Y, R]
+  const float* FW;    // [X, R]
+  float* y;           // [N, Cout, H, W]
+  int N, Cin, Cout, H, W, pad, Y, X, R;
+  int flip;           // 1: tap index t reads factor row (taps-1-t)
+};
+
+enum FwdVariant { FWD_GENERAL = 0, FWD_MFMA = 1, FWD_VARIANT_COUNT = 2 };
+
+bool fwd_general_supported(const FwdArgs&);
+hipError_t fwd_general_launch(const FwdArgs&, hipStream_t);
+bool fwd_mfma_supported(const FwdArgs&);
+hipError_t fwd_mfma_launch(const FwdArgs&, hipStream_t);
+
+// Backward-filter (factor gradients).
+struct BwdFilterArgs {
+  const float *x, *dy, *FK, *FC, *FH, *FW;
+  float *dFK, *dFC, *dFH, *dFW;
+  void* workspace;
+  int N, C, T, H, W, pad, Y, X, R;
+};
+size_t bwd_filter_workspace_bytes(const cp4_shape&);
+hipError_t bwd_filter_launch(const BwdFilterArgs&, hipStream_t);
+hipError_t bwd_filter_full_launch(const cp4_shape&, const float* x,
+                                  const float* dy, float* dK, int accumulate,
+                                  hipStream_t);
+
+// Utilities.
+hipError_t recompose_launch(const cp4_shape&, const float* FK, const float* FC,
+                            const float* FH, const float* FW, float* K,
+                            hipStream_t);
+hipError_t count_exceeding_launch(const float* A, const float* B, size_t n,
+                                  float tol, unsigned long long* d_count,
+                                  hipStream_t);
+hipError_t random_uniform_launch(float* dst, size_t n, unsigned long long seed,
+                                 hipStream_t);
+hipError_t copy_f32_launch(float* dst, const float* src, size_t n, hipStream_t);
+
+}  // namespace cp4
+#endif

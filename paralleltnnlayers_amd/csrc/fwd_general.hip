@@ -1,0 +1,133 @@
+// General forward / backward-data kernel: any rank, channel counts, odd or
+// even filter size and pad; VALU arithmetic, LDS-tiled.
+//
+// One workgroup owns an 8 x 32 output tile of one image and walks the rank in
+// blocks of RB.  Per rank block:
+//   1. A[r][halo pixel] = sum_c Fin[c,r] x[c, pixel]   (global -> registers -> LDS;
+//      32 consecutive lanes read 32 consecutive floats of one NCHW row)
+//   2. B[r][h][halo col] = sum_i FH[i,r] A[r][h+i][col]          (LDS -> LDS)
+//   3. Cc[r] = sum_j FW[j,r] B[r][h][w+j]                        (LDS -> registers)
+//   4. y[k, pixel] (+)= sum_r Fout[k,r] Cc[r]                    (registers -> global)
+// Factor values are wave-uniform and come through scalar loads.  The
+// arithmetic is the reassociated form of Cuda_kernels/cp4Conv2dForward.cu:84-133:
+// the spatial taps are applied to R rank planes instead of C channel planes.
+#include "cp4_internal.h"
+
+namespace cp4 {
+namespace {
+
+constexpr int kTH = 8, kTW = 32, kThreads = kTH * kTW;
+
+template <int RB>
+__global__ __launch_bounds__(kThreads) void fwd_general_kernel(FwdArgs a) {
+  extern __shared__ float lds[];
+  const int HT = kTH + a.Y - 1, WT = kTW + a.X - 1;
+  const int nA = HT * WT, nB = kTH * WT;
+  float* As = lds;            // [RB][HT*WT]
+  float* Bs = lds + RB * nA;  // [RB][kTH*WT]
+  const int n = blockIdx.z, h0 = blockIdx.y * kTH, w0 = blockIdx.x * kTW;
+  const int tid = threadIdx.x;
+  const size_t HW = (size_t)a.H * a.W;
+  const float* xn = a.x + (size_t)n * a.Cin * HW;
+  const int R = a.R;
+
+  for (int r0 = 0; r0 < R; r0 += RB) {
+    // 1. channel -> rank contraction on the halo tile
+    for (int q = tid; q < nA; q += kThreads) {
+      const int hh = q / WT, ww = q - hh * WT;
+      const int gh = h0 + hh - a.pad, gw = w0 + ww - a.pad;
+      float acc[RB];
+#pragma unroll
+      for (int rr = 0; rr < RB; ++rr) acc[rr] = 0.f;
+      if (gh >= 0 && gh < a.H && gw >= 0 && gw < a.W) {
+        const float* xp = xn + (size_t)gh * a.W + gw;
+        for (int c = 0; c < a.Cin; ++c) {
+          const float v = xp[c * HW];
+          const float* f = a.Fin + (size_t)c * R + r0;
+#pragma unroll
+          for (int rr = 0; rr < RB; ++rr)
+            acc[rr] += v * (r0 + rr < R ? f[rr] : 0.f);
+        }
+      }
+#pragma unroll
+      for (int rr = 0; rr < RB; ++rr) As[rr * nA + q] = acc[rr];
+    }
+    __syncthreads();
+    // 2. taps along H
+    for (int q = tid; q < nB; q += kThreads) {
+      const int h = q / WT, ww = q - h * WT;
+#pragma unroll
+      for (int rr = 0; rr < RB; ++rr) {
+        float s = 0.f;
+        if (r0 + rr < R)
+          for (int i = 0; i < a.Y; ++i)
+            s += a.FH[(a.flip ? a.Y - 1 - i : i) * R + r0 + rr] *
+                 As[rr * nA + (h + i) * WT + ww];
+        Bs[rr * nB + q] = s;
+      }
+    }
+    __syncthreads();
+    // 3. taps along W, one output pixel per thread
+    const int h = tid / kTW, w = tid - h * kTW;
+    float cc[RB];
+#pragma unroll
+    for (int rr = 0; rr < RB; ++rr) {
+      float s = 0.f;
+      if (r0 + rr < R)
+        for (int j = 0; j < a.X; ++j)
+          s += a.FW[(a.flip ? a.X - 1 - j : j) * R + r0 + rr] *
+               Bs[rr * nB + h * WT + w + j];
+      cc[rr] = s;
+    }
+    // 4. rank -> output-channel contraction
+    if (h0 + h < a.H && w0 + w < a.W) {
+      float* yp = a.y + (size_t)n * a.Cout * HW + (size_t)(h0 + h) * a.W + w0 + w;
+      for (int k = 0; k < a.Cout; ++k) {
+        const float* f = a.Fout + (size_t)k * R + r0;
+        float s = 0.f;
+#pragma unroll
+        for (int rr = 0; rr < RB; ++rr) s += cc[rr] * (r0 + rr < R ? f[rr] : 0.f);
+        if (r0 > 0) s += yp[k * HW];
+        yp[k * HW] = s;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// LDS floats needed for a rank block of rb.
+size_t lds_floats(const FwdArgs& a, int rb) {
+  const size_t HT = kTH + a.Y - 1, WT = kTW + a.X - 1;
+  return (size_t)rb * (HT * WT + kTH * WT);
+}
+constexpr size_t kLdsBudget = 64 * 1024;
+
+int pick_rank_block(const FwdArgs& a) {
+  int rb = 32;
+  while (rb > 1 && (rb / 2 >= a.R || lds_floats(a, rb) * 4 > kLdsBudget)) rb /= 2;
+  return rb;
+}
+
+}  // namespace
+
+bool fwd_general_supported(const FwdArgs& a) {
+  return lds_floats(a, 1) * 4 <= kLdsBudget && a.N <= 65535 &&
+         (a.H + kTH - 1) / kTH <= 65535;
+}
+
+hipError_t fwd_general_launch(const FwdArgs& a, hipStream_t s) {
+  const int rb = pick_rank_block(a);
+  const dim3 grid((a.W + kTW - 1) / kTW, (a.H + kTH - 1) / kTH, a.N);
+  const size_t smem = lds_floats(a, rb) * sizeof(float);
+  switch (rb) {
+    case 32: fwd_general_kernel<32><<<grid, kThreads, smem, s>>>(a); break;
+    case 16: fwd_general_kernel<16><<<grid, kThreads, smem, s>>>(a); break;
+    case 8: fwd_general_kernel<8><<<grid, kThreads, smem, s>>>(a); break;
+    case 4: fwd_general_kernel<4><<<grid, kThreads, smem, s>>>(a); break;
+    case 2: fwd_general_kernel<2><<<grid, kThreads, smem, s>>>(a); break;
+    default: fwd_general_kernel<1><<<grid, kThreads, smem, s>>>(a); break;
+  }
+  return hipGetLastError();
+}
+
+}  // namespace cp4

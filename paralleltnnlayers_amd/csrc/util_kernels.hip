@@ -1,0 +1,116 @@
+// Test / bench utility kernels: filter recomposition, the reference's
+// relative-error counter, a counter-based uniform generator and a streaming
+// copy used for bandwidth and hardware-counter calibration.
+#include "cp4_internal.h"
+
+namespace cp4 {
+namespace {
+
+// K[t,c,y,x] = sum_r FK[t,r] FC[c,r] FH[y,r] FW[x,r]  (Cuda_kernels/Utils.cu:55-62)
+__global__ __launch_bounds__(256) void recompose_kernel(
+    const float* __restrict__ FK, const float* __restrict__ FC,
+    const float* __restrict__ FH, const float* __restrict__ FW,
+    float* __restrict__ K, int T, int C, int Y, int X, int R) {
+  const size_t total = (size_t)T * C * Y * X;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (size_t)gridDim.x * 256) {
+    const int x = i % X, y = (i / X) % Y, c = (i / ((size_t)X * Y)) % C;
+    const int t = i / ((size_t)X * Y * C);
+    float acc = 0.f;
+    for (int r = 0; r < R; ++r)
+      acc += FK[t * R + r] * FC[c * R + r] * FH[y * R + r] * FW[x * R + r];
+    K[i] = acc;
+  }
+}
+
+// Symmetric relative error, absolute if either value is zero
+// (Cuda_kernels/Utils.cu:143-156); one integer atomic per workgroup.
+__global__ __launch_bounds__(256) void count_exceeding_kernel(
+    const float* __restrict__ A, const float* __restrict__ B, size_t n,
+    float tol, unsigned long long* count) {
+  unsigned bad = 0;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * 256) {
+    const float a = A[i], b = B[i], d = fabsf(a - b);
+    const float err = (a == 0.f || b == 0.f) ? d : fmaxf(d / fabsf(a), d / fabsf(b));
+    // NaN must count as a mismatch
+    bad += !(err <= tol);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) bad += __shfl_down(bad, off, 64);
+  if ((threadIdx.x & 63) == 0 && bad) atomicAdd(count, (unsigned long long)bad);
+}
+
+__device__ __forceinline__ unsigned long long splitmix64(unsigned long long z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+// dst[i] in (0,1]: 24 random bits of hash(seed, i), like cuRAND's uniform
+// range used by random_fill (Cuda_kernels/Utils.cu:22-33).
+__global__ __launch_bounds__(256) void random_uniform_kernel(
+    float* __restrict__ dst, size_t n, unsigned long long seed) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * 256) {
+    const unsigned long long h = splitmix64(splitmix64(seed) ^ i);
+    dst[i] = ((float)(unsigned)(h >> 40) + 1.0f) * (1.0f / 16777216.0f);
+  }
+}
+
+__global__ __launch_bounds__(256) void copy_f32x4_kernel(
+    float4* __restrict__ dst, const float4* __restrict__ src, size_t n4) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4;
+       i += (size_t)gridDim.x * 256)
+    dst[i] = src[i];
+}
+__global__ __launch_bounds__(256) void copy_f32_kernel(
+    float* __restrict__ dst, const float* __restrict__ src, size_t lo, size_t n) {
+  const size_t i = lo + (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
+unsigned grid_for(size_t n, unsigned cap) {
+  const size_t g = (n + 255) / 256;
+  return (unsigned)(g < 1 ? 1 : g > cap ? cap : g);
+}
+
+}  // namespace
+
+hipError_t recompose_launch(const cp4_shape& s, const float* FK, const float* FC,
+                            const float* FH, const float* FW, float* K,
+                            hipStream_t st) {
+  const size_t total = (size_t)s.T * s.C * s.Y * s.X;
+  recompose_kernel<<<grid_for(total, 65536), 256, 0, st>>>(FK, FC, FH, FW, K, s.T, s.C, s.Y, s.X, s.Rank);
+  return hipGetLastError();
+}
+
+hipError_t count_exceeding_launch(const float* A, const float* B, size_t n,
+                                  float tol, unsigned long long* d_count,
+                                  hipStream_t st) {
+  count_exceeding_kernel<<<grid_for(n, 4096), 256, 0, st>>>(A, B, n, tol, d_count);
+  return hipGetLastError();
+}
+
+hipError_t random_uniform_launch(float* dst, size_t n, unsigned long long seed,
+                                 hipStream_t st) {
+  random_uniform_kernel<<<grid_for(n, 65536), 256, 0, st>>>(dst, n, seed);
+  return hipGetLastError();
+}
+
+hipError_t copy_f32_launch(float* dst, const float* src, size_t n, hipStream_t st) {
+  const bool aligned = (((uintptr_t)dst | (uintptr_t)src) & 15) == 0;
+  const size_t n4 = aligned ? n / 4 : 0;
+  if (n4) {
+    // 256 CUs x 8 workgroups, grid-stride
+    copy_f32x4_kernel<<<grid_for(n4, 2048), 256, 0, st>>>(
+        reinterpret_cast<float4*>(dst), reinterpret_cast<const float4*>(src), n4);
+  }
+  const size_t rest = n - n4 * 4;
+  if (rest)
+    copy_f32_kernel<<<(unsigned)((rest + 255) / 256), 256, 0, st>>>(dst, src, n4 * 4, n);
+  return hipGetLastError();
+}
+
+}  // namespace cp4

@@ -1,0 +1,97 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the
+header declares, and rejects bad arguments before touching a device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def L():
+    from paralleltnnlayers_amd import capi
+    return capi.lib()
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "cp4", "capi.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cp4_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_three_passes():
+    names = declared_functions()
+    for n in ("cp4_conv2d_forward", "cp4_conv2d_backward_data",
+              "cp4_conv2d_backward_filter", "cp4_conv2d_backward_filter_full",
+              "cp4_time_forward", "cp4_tune_forward", "cp4_device_malloc"):
+        assert n in names
+    assert len(names) >= 30
+
+
+@pytest.mark.parametrize("name", declared_functions())
+def test_symbol_exported(L, name):
+    assert getattr(L, name) is not None
+
+
+def test_shape_struct_matches_reference_order():
+    from paralleltnnlayers_amd.capi import Shape
+    assert [f for f, _ in Shape._fields_] == ["N", "H", "W", "pad", "T", "C", "Y", "X", "Rank"]
+    assert ctypes.sizeof(Shape) == 36
+
+
+def test_argument_errors_need_no_device(L):
+    from paralleltnnlayers_amd import capi
+    good = capi.Shape(N=1, H=4, W=4, pad=1, T=2, C=2, Y=3, X=3, Rank=2)
+    one = ctypes.c_void_p(16)   # never dereferenced: checks fail first
+    assert L.cp4_conv2d_forward(None, one, one, one, one, one, one, None) == capi.ERR_NULL_POINTER
+    assert L.cp4_conv2d_forward(ctypes.byref(good), None, one, one, one, one, one, None) \
+        == capi.ERR_NULL_POINTER
+    assert b"NULL" in L.cp4_last_error_message()
+    for field in ("H", "W", "T", "C", "Y", "X", "Rank"):
+        bad = capi.Shape(N=1, H=4, W=4, pad=1, T=2, C=2, Y=3, X=3, Rank=2)
+        setattr(bad, field, 0)
+        assert L.cp4_conv2d_forward(ctypes.byref(bad), one, one, one, one, one, one, None) \
+            == capi.ERR_SHAPE, field
+        assert L.cp4_conv2d_backward_data(ctypes.byref(bad), one, one, one, one, one, one, None) \
+            == capi.ERR_SHAPE, field
+    huge = capi.Shape(N=1, H=1 << 16, W=1 << 16, pad=1, T=2, C=2, Y=3, X=3, Rank=2)
+    assert L.cp4_conv2d_forward(ctypes.byref(huge), one, one, one, one, one, one, None) \
+        == capi.ERR_SHAPE
+    # empty batch is a valid no-op and needs no pointers
+    empty = capi.Shape(N=0, H=4, W=4, pad=1, T=2, C=2, Y=3, X=3, Rank=2)
+    assert L.cp4_conv2d_forward(ctypes.byref(empty), None, None, None, None, None, None, None) \
+        == capi.OK
+    assert L.cp4_conv2d_backward_data(ctypes.byref(empty), None, None, None, None, None, None,
+                                      None) == capi.OK
+    # backward-filter: workspace too small is reported before any launch
+    need = L.cp4_conv2d_backward_filter_workspace_bytes(ctypes.byref(good))
+    assert need > 0
+    args = [one] * 10
+    assert L.cp4_conv2d_backward_filter(ctypes.byref(good), *args, one, need - 1, None) \
+        == capi.ERR_WORKSPACE
+    assert L.cp4_conv2d_backward_filter(ctypes.byref(good), *args, None, need, None) \
+        == capi.ERR_WORKSPACE
+    # variant index out of range
+    assert L.cp4_forward_variant_supported(ctypes.byref(good), 99) == capi.ERR_UNSUPPORTED
+    assert L.cp4_forward_variant_supported(ctypes.byref(good), 0) == capi.OK
+    us = ctypes.c_float()
+    assert L.cp4_time_forward(ctypes.byref(good), one, one, one, one, one, one, 0, 0,
+                              ctypes.byref(us), None) == capi.ERR_SHAPE
+
+
+def test_status_strings(L):
+    seen = {L.cp4_status_string(i) for i in range(6)}
+    assert len(seen) == 6 and b"ok" in seen
+
+
+def test_workload_byte_counts():
+    """Algorithmic bytes of the five workloads (reference formula,
+    Cuda_kernels/cp4Conv2d.cu:176-178)."""
+    from paralleltnnlayers_amd.configs import WORKLOADS, algorithmic_bytes, minimal_flops
+    want = {"C1": 132288, "C2": 8397184, "C3": 205587200, "C4": 25707136, "C5": 25955328}
+    for k, v in want.items():
+        assert algorithmic_bytes(WORKLOADS[k]) == v
+    assert minimal_flops(WORKLOADS["C3"]) == 3326869504
+    assert minimal_flops(WORKLOADS["C5"]) == 1673068544

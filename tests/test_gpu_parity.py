@@ -1,0 +1,265 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU
+oracle, the committed golden vectors and size-independent properties.
+
+Tolerances (written out here as the bar for this path):
+  forward / backward-data : |a-b| <= 1e-5 + 1e-4*|b| elementwise, and
+                            max|a-b| <= 1e-4 * max|b| so that small-magnitude
+                            outputs cannot pass vacuously;
+  backward-filter         : |a-b| <= 1e-3*|b| + 1e-4*max|b| elementwise, and
+                            max|a-b| <= 1e-3 * max|b|.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from paralleltnnlayers_amd.configs import WORKLOADS, make_inputs  # noqa: E402
+
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "cp4_golden.npz"))
+GOLD_CASES = sorted({k.split(".")[0] for k in GOLD.files})
+FACTORS = ("FK", "FC", "FH", "FW")
+
+
+@pytest.fixture(scope="module")
+def cp4():
+    import paralleltnnlayers_amd as p
+    p.lib()
+    assert torch.cuda.is_available()
+    return p
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def assert_activation_close(got, want, what=""):
+    scale = float(np.abs(want).max())
+    err = np.abs(got - want)
+    assert np.all(err <= 1e-5 + 1e-4 * np.abs(want)), f"{what}: elementwise, max err {err.max():.3e}"
+    assert err.max() <= 1e-4 * scale, f"{what}: normalised {err.max() / scale:.3e} (scale {scale:.3e})"
+
+
+def assert_gradient_close(got, want, what=""):
+    scale = float(np.abs(want).max())
+    err = np.abs(got - want)
+    assert np.all(err <= 1e-3 * np.abs(want) + 1e-4 * scale), f"{what}: elementwise {err.max():.3e}"
+    assert err.max() <= 1e-3 * scale, f"{what}: normalised {err.max() / scale:.3e}"
+
+
+def gold(name):
+    g = {k: GOLD[f"{name}.{k}"] for k in
+         ("x", "dy", "y", "dx", "dFK", "dFC", "dFH", "dFW") + FACTORS}
+    g["pad"] = int(GOLD[name + ".shape"][3])
+    return g
+
+
+def variants_for(cp4, x_shape, f, pad):
+    s = cp4.capi.shape_for(x_shape, f["FK"], f["FC"], f["FH"], f["FW"], pad)
+    return [v for v, _, ok in cp4.forward_variants(s) if ok]
+
+
+# ---------------------------------------------------------------- golden ----
+@pytest.mark.parametrize("name", GOLD_CASES)
+def test_golden_all_passes(cp4, name):
+    g = gold(name)
+    f = {k: dev(g[k]) for k in FACTORS}
+    x, dy = dev(g["x"]), dev(g["dy"])
+    for v in variants_for(cp4, x.shape, f, g["pad"]):
+        y = host(cp4.conv2d_forward(x, *f.values(), pad=g["pad"], variant=v))
+        assert_activation_close(y, g["y"], f"{name} forward variant {v}")
+    dx = host(cp4.conv2d_backward_data(dy, *f.values(), pad=g["pad"]))
+    assert_activation_close(dx, g["dx"], f"{name} backward-data")
+    grads = cp4.conv2d_backward_filter(x, dy, *f.values(), pad=g["pad"])
+    for got, k in zip(grads, FACTORS):
+        assert_gradient_close(host(got), g["d" + k], f"{name} d{k}")
+
+
+# ------------------------------------------------- the five workloads -------
+@pytest.fixture(scope="module", params=list(WORKLOADS))
+def workload(request):
+    w = WORKLOADS[request.param]
+    return w, make_inputs(w, seed=0)
+
+
+def test_workload_forward(cp4, oracle, workload):
+    w, a = workload
+    want = oracle.forward(a["x"], a["FK"], a["FC"], a["FH"], a["FW"], w.pad)
+    f = {k: dev(a[k]) for k in FACTORS}
+    x = dev(a["x"])
+    vs = variants_for(cp4, x.shape, f, w.pad)
+    assert vs
+    for v in vs + [-1]:
+        y = host(cp4.conv2d_forward(x, *f.values(), pad=w.pad, variant=v))
+        assert_activation_close(y, want, f"{w.name} forward variant {v}")
+
+
+def test_workload_backward_data(cp4, oracle, workload):
+    w, a = workload
+    want = oracle.backward_data(a["dy"], a["FK"], a["FC"], a["FH"], a["FW"], w.pad)
+    f = [dev(a[k]) for k in FACTORS]
+    dx = host(cp4.conv2d_backward_data(dev(a["dy"]), *f, pad=w.pad))
+    assert_activation_close(dx, want, f"{w.name} backward-data")
+
+
+def test_workload_backward_filter(cp4, oracle, workload):
+    w, a = workload
+    want = oracle.backward_filter(a["x"], a["dy"], a["FK"], a["FC"], a["FH"], a["FW"], w.pad)
+    f = [dev(a[k]) for k in FACTORS]
+    got = cp4.conv2d_backward_filter(dev(a["x"]), dev(a["dy"]), *f, pad=w.pad)
+    for g, wnt, k in zip(got, want, FACTORS):
+        assert_gradient_close(host(g), wnt, f"{w.name} d{k}")
+    # bit-reproducible: no floating-point atomics anywhere in the reduction
+    again = cp4.conv2d_backward_filter(dev(a["x"]), dev(a["dy"]), *f, pad=w.pad)
+    for g1, g2 in zip(got, again):
+        assert torch.equal(g1, g2)
+
+
+def test_workload_properties(cp4, workload):
+    """Size-independent properties at full size: linearity in x and the
+    adjoint identity <forward(x), dy> == <x, backward_data(dy)> (2*pad == Y-1
+    for all five workloads)."""
+    w, a = workload
+    f = [dev(a[k]) for k in FACTORS]
+    x, dy = dev(a["x"]), dev(a["dy"])
+    z = torch.roll(x, shifts=(1, 3), dims=(2, 3)) * 0.5
+    y = cp4.conv2d_forward(x, *f, pad=w.pad)
+    yz = cp4.conv2d_forward(z, *f, pad=w.pad)
+    ylin = cp4.conv2d_forward(2.0 * x - 3.0 * z, *f, pad=w.pad)
+    assert_activation_close(host(ylin), host(2.0 * y - 3.0 * yz), f"{w.name} linearity")
+    dx = cp4.conv2d_backward_data(dy, *f, pad=w.pad)
+    lhs = float((y.double() * dy.double()).sum())
+    rhs = float((x.double() * dx.double()).sum())
+    norm = float(y.double().norm() * dy.double().norm())
+    assert abs(lhs - rhs) <= 1e-5 * norm, (lhs, rhs, norm)
+    assert norm > 0 and float(y.abs().max()) > 0
+
+
+# ------------------------------------------------------------ edge cases ----
+EDGE = [
+    # N, C, H, W, pad, T, Y, X, R
+    (1, 48, 55, 55, 5, 256, 11, 11, 16),  # the reference's single-kernel test case
+    (2, 3, 37, 41, 1, 5, 3, 3, 6),        # ragged tile edges, rank not a power of two
+    (1, 1, 1, 1, 0, 1, 1, 1, 1),          # everything equal to one
+    (3, 7, 5, 67, 2, 9, 5, 5, 1),         # rank 1, wide and short
+    (1, 4, 9, 9, 0, 4, 3, 3, 4),          # no padding: output still H x W
+    (1, 4, 9, 9, 3, 4, 3, 3, 4),          # pad larger than the filter radius
+    (2, 5, 8, 8, 1, 3, 2, 2, 3),          # even filter
+    (1, 6, 10, 12, 1, 4, 3, 5, 5),        # rectangular filter (the reference only warns)
+    (1, 2, 20, 20, 8, 2, 17, 17, 2),      # largest filter of the reference's sweeps
+    (4, 40, 16, 16, 1, 72, 3, 3, 48),     # rank above the register block
+    (2, 16, 12, 12, 1, 32, 3, 3, 16),     # MFMA-eligible rank, small image
+]
+
+
+@pytest.mark.parametrize("dims", EDGE, ids=lambda d: "x".join(map(str, d)))
+def test_edge_shapes(cp4, oracle, dims):
+    N, C, H, W, pad, T, Y, X, R = dims
+    rng = np.random.default_rng(sum(dims))
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    dy = rng.standard_normal((N, T, H, W)).astype(np.float32)
+    fac = [rng.standard_normal((d, R)).astype(np.float32) / np.sqrt(R) for d in (T, C, Y, X)]
+    f = [dev(v) for v in fac]
+    fdict = dict(zip(FACTORS, f))
+    want = oracle.forward(x, *fac, pad)
+    for v in variants_for(cp4, x.shape, fdict, pad):
+        y = host(cp4.conv2d_forward(dev(x), *f, pad=pad, variant=v))
+        assert_activation_close(y, want, f"forward variant {v}")
+    dx = host(cp4.conv2d_backward_data(dev(dy), *f, pad=pad))
+    assert_activation_close(dx, oracle.backward_data(dy, *fac, pad), "backward-data")
+    got = cp4.conv2d_backward_filter(dev(x), dev(dy), *f, pad=pad)
+    for g, wnt, k in zip(got, oracle.backward_filter(x, dy, *fac, pad), FACTORS):
+        assert_gradient_close(host(g), wnt, f"d{k}")
+
+
+def test_reference_single_case_against_dense_conv(cp4):
+    """Cuda_kernels/test/test_cp4Conv.cpp.cu:14-44: CP4 forward vs a dense conv
+    of the recomposed kernel, all-positive U(0,1] inputs, compared with the
+    reference's own relative-error counter at 1e-5 ... here 2e-5 because the
+    dense comparator is torch's conv2d in fp32 rather than cuDNN."""
+    n, c, hw, pad, t, f, r = 1, 48, 55, 5, 256, 11, 16
+    x = cp4.random_uniform((n, c, hw, hw), 1234)
+    FK, FC, FH, FW = (cp4.random_uniform((d, r), 1234 + i)
+                      for i, d in enumerate((t, c, f, f)))
+    K = cp4.recompose(FK, FC, FH, FW)
+    y = cp4.conv2d_forward(x, FK, FC, FH, FW, pad=pad)
+    ref = torch.nn.functional.conv2d(x.double(), K.double(), padding=pad).float()
+    assert tuple(y.shape) == (n, t, hw, hw)
+    assert cp4.count_exceeding(y, ref, 2e-5) == 0
+
+
+def test_empty_batch(cp4):
+    f = [torch.ones((d, 2), device="cuda") for d in (3, 4, 3, 3)]
+    x = torch.empty((0, 4, 5, 5), device="cuda")
+    assert cp4.conv2d_forward(x, *f, pad=1).shape == (0, 3, 5, 5)
+    dy = torch.empty((0, 3, 5, 5), device="cuda")
+    assert cp4.conv2d_backward_data(dy, *f, pad=1).shape == (0, 4, 5, 5)
+    for g in cp4.conv2d_backward_filter(x, dy, *f, pad=1):
+        assert float(host(g).max()) == 0.0 and float(host(g).min()) == 0.0
+
+
+def test_dense_filter_gradient(cp4, oracle):
+    g = gold("five5x5")
+    x, dy = dev(g["x"]), dev(g["dy"])
+    want = oracle.backward_filter_full(g["x"], g["dy"], 5, 5, g["pad"])
+    dK = cp4.conv2d_backward_filter_full(x, dy, 5, 5, pad=g["pad"])
+    assert_gradient_close(host(dK), want, "dK")
+    # accumulate flag: the reference adds into the caller's buffer
+    acc = cp4.conv2d_backward_filter_full(x, dy, 5, 5, pad=g["pad"], out=dK.clone())
+    assert_gradient_close(host(acc), 2 * want, "dK accumulate")
+
+
+# -------------------------------------------------------------- utilities ---
+def test_recompose_and_allclose_like_reference(cp4, oracle):
+    """Cuda_kernels/test/test_Utils.cpp.cu:10-51."""
+    K0, K1 = cp4.random_uniform((16, 6), 1), cp4.random_uniform((16, 6), 2)
+    K2, K3 = cp4.random_uniform((3, 6), 3), cp4.random_uniform((3, 6), 4)
+    U = cp4.random_uniform((1, 16, 32, 32), 5)
+    assert float(U.min()) > 0 and float(U.max()) <= 1.0
+    assert torch.equal(U, cp4.random_uniform((1, 16, 32, 32), 5))
+    assert not torch.equal(U, cp4.random_uniform((1, 16, 32, 32), 6))
+    K = cp4.recompose(K0, K1, K2, K3)
+    assert tuple(K.shape) == (16, 16, 3, 3) and K.numel() == 2304
+    want = oracle.recompose(*(host(k) for k in (K0, K1, K2, K3)))
+    np.testing.assert_allclose(host(K), want, rtol=1e-5)
+    V = cp4.conv2d_forward(U, K0, K1, K2, K3, pad=1)
+    V2 = cp4.conv2d_forward(U, K0, K1, K2, K3, pad=1)
+    assert tuple(V.shape) == (1, 16, 32, 32) and bool((V != 0).all())
+    assert cp4.count_exceeding(V, V2, 1e-5) == 0
+    V[0, 0, 0, 0] *= 2
+    assert cp4.count_exceeding(V, V2, 1e-1) == 1
+    a = torch.tensor([0.0, 0.0, 1.0, float("nan")], device="cuda")
+    b = torch.tensor([0.05, 0.0, 1.0, 1.0], device="cuda")
+    assert cp4.count_exceeding(a, b, 1e-1) == 1      # NaN counts, 0.05 abs passes
+    assert cp4.count_exceeding(a, b, 1e-2) == 2
+    assert cp4.count_exceeding(a, b, 1e-2) == oracle.count_exceeding(
+        host(a)[:3], host(b)[:3], 1e-2) + 1
+
+
+def test_timed_launch_and_tuner(cp4):
+    w = WORKLOADS["C2"]
+    a = make_inputs(w)
+    f = [dev(a[k]) for k in FACTORS]
+    x = dev(a["x"])
+    y = torch.empty((w.N, w.T, w.H, w.W), device="cuda")
+    us = cp4.time_forward(x, *f, y, w.pad, warmup=1, profcount=5)
+    assert 0 < us < 1e6
+    best, best_us = cp4.tune_forward(x, *f, y, w.pad, warmup=1, profcount=5)
+    names = dict((v, n) for v, n, _ in cp4.forward_variants())
+    assert best in names and best_us > 0
+    y2 = cp4.conv2d_forward(x, *f, pad=w.pad)          # uses the tuned choice
+    y3 = cp4.conv2d_forward(x, *f, pad=w.pad, variant=best)
+    assert torch.equal(y2, y3)
+    cp4.lib().cp4_tune_clear()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        y4 = cp4.conv2d_forward(x, *f, pad=w.pad, variant=best)   # explicit non-default stream
+    s.synchronize()
+    assert torch.equal(y3, y4)
