@@ -1,0 +1,147 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused CP4 Conv2d hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--no-cpu]
+
+A step is one launch of the workload's pass (default: the forward pass of the
+ResNet-stage workload N=32, C=K=256, 56x56, 3x3, R=32) on synthetic inputs that
+are already resident in HBM.  Prints ONE JSON line:
+
+  value        whole-job throughput = algorithmic bytes * K / wall time of the K
+               steps (host clock, device synchronised on both sides), in GB/s
+  roofline     the same K launches timed with HIP events on the launch stream:
+               achieved GB/s = algorithmic bytes / mean launch duration, against
+               the 8 TB/s HBM peak
+  cpu_baseline the CPU oracle's unfused factor-by-factor computation of the same
+               workload timed on this box's host cores (a reported baseline)
+  passes       mean event-timed microseconds and GB/s of all five workloads
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+FACTORS = ("FK", "FC", "FH", "FW")
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs, scaled by the plain copy kernel's reading (see
+# profiles/): {workload: bytes}.  None until measured for the current kernel.
+MEASURED_TRAFFIC = {}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="C3")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-passes", action="store_true", help="skip the five-workload table")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
+                 "(batch sharding across GPUs is design-only, see DESIGN.md)")
+
+    import torch
+
+    import paralleltnnlayers_amd as cp4
+    from paralleltnnlayers_amd.configs import WORKLOADS, algorithmic_bytes, make_inputs
+
+    cp4.lib()  # fail loudly if the HIP library is missing
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    torch.cuda.set_device(0)
+
+    def device_inputs(w):
+        a = make_inputs(w, seed=0)
+        return a, {k: torch.from_numpy(v).cuda() for k, v in a.items()}
+
+    def timed(w, d, warmup, steps):
+        """(event-timed mean us, wall seconds of the same `steps` launches)."""
+        f = [d[k] for k in FACTORS]
+        if w.pass_ == "forward":
+            out = torch.empty((w.N, w.T, w.H, w.W), device="cuda")
+            run = lambda wu, k: cp4.time_forward(d["x"], *f, out, w.pad, wu, k)
+        elif w.pass_ == "backward_data":
+            out = torch.empty((w.N, w.C, w.H, w.W), device="cuda")
+            run = lambda wu, k: cp4.time_backward_data(d["dy"], *f, out, w.pad, wu, k)
+        else:
+            s = cp4.capi.shape_for(d["x"].shape, *f, w.pad)
+            ws = torch.empty(cp4.backward_filter_workspace_bytes(s) // 4 + 1, device="cuda")
+            run = lambda wu, k: cp4.time_backward_filter(d["x"], d["dy"], *f, w.pad, wu, k,
+                                                         workspace=ws)
+        run(warmup, 1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        us = run(0, steps)          # K launches between one HIP event pair on the stream
+        torch.cuda.synchronize()
+        return us, time.perf_counter() - t0
+
+    w = WORKLOADS[args.workload]
+    host, d = device_inputs(w)
+    nbytes = algorithmic_bytes(w)
+    us, wall = timed(w, d, args.warmup, args.steps)
+    value = nbytes * args.steps / wall / 1e9
+    achieved = nbytes / us / 1e3
+
+    out = {
+        "metric": "CP4 conv2d %s achieved HBM GB/s (algorithmic bytes / time), 1 GPU" % w.pass_,
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall / args.steps * 1e3, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s %s fp32 NCHW N=%d C=%d K=%d H=W=%d %dx%d pad=%d R=%d"
+                               % (w.name, w.pass_, w.N, w.C, w.T, w.H, w.Y, w.X, w.pad, w.R),
+                   "algorithmic_bytes": nbytes, "us_per_launch": round(us, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC.get(w.name)},
+    }
+
+    if not args.no_passes:
+        passes = {}
+        for name, ww in WORKLOADS.items():
+            if name == w.name:
+                t = us
+            else:
+                _, dd = device_inputs(ww)
+                t, _ = timed(ww, dd, 5, 47)     # 47 launches, as the reference's bench drivers
+                del dd
+            b = algorithmic_bytes(ww)
+            passes[name] = {"pass": ww.pass_, "us": round(t, 2),
+                            "GB/s": round(b / t / 1e3, 1),
+                            "hbm_frac": round(b / t / 1e3 / HBM_PEAK_GBS, 4)}
+        out["passes"] = passes
+
+    if not args.no_cpu:
+        from oracle import cp4_oracle
+        fa = [host[k] for k in FACTORS]
+        fn = {"forward": lambda: cp4_oracle.forward(host["x"], *fa, w.pad),
+              "backward_data": lambda: cp4_oracle.backward_data(host["dy"], *fa, w.pad),
+              "backward_filter": lambda: cp4_oracle.backward_filter(host["x"], host["dy"], *fa,
+                                                                    w.pad)}[w.pass_]
+        fn()  # warm-up
+        best, reps, t_start = None, 0, time.perf_counter()
+        while reps < 5 and time.perf_counter() - t_start < 20.0:
+            t0 = time.perf_counter()
+            fn()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+            reps += 1
+        out["cpu_baseline"] = {
+            "value": round(nbytes / best / 1e9, 3), "unit": "GB/s",
+            "cores": cp4_oracle.num_threads(), "kind": "port",
+            "sample": "full %s workload, best of %d runs, %.1f ms each (OpenMP unfused "
+                      "factor-by-factor oracle)" % (w.name, reps, best * 1e3)}
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
