@@ -74,7 +74,8 @@ struct Variant {
 // Order = preference of the untuned heuristic, last to first.
 const Variant kVariants[] = {
     {"general_valu", cp4::fwd_general_supported, cp4::fwd_general_launch},
-    {"mfma_strip", cp4::fwd_mfma_supported, cp4::fwd_mfma_launch},
+    {"mfma_f32_strip", cp4::fwd_mfma_supported, cp4::fwd_mfma_launch},
+    {"mfma_bf16x3_strip", cp4::fwd_split_supported, cp4::fwd_split_launch},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 

@@ -25,12 +25,13 @@ struct FwdArgs {
   int flip;           // 1: tap index t reads factor row (taps-1-t)
 };
 
-enum FwdVariant { FWD_GENERAL = 0, FWD_MFMA = 1, FWD_VARIANT_COUNT = 2 };
 
 bool fwd_general_supported(const FwdArgs&);
 hipError_t fwd_general_launch(const FwdArgs&, hipStream_t);
 bool fwd_mfma_supported(const FwdArgs&);
 hipError_t fwd_mfma_launch(const FwdArgs&, hipStream_t);
+bool fwd_split_supported(const FwdArgs&);
+hipError_t fwd_split_launch(const FwdArgs&, hipStream_t);
 
 // Backward-filter (factor gradients).
 struct BwdFilterArgs {
