@@ -144,6 +144,9 @@ cp4_status cp4_memcpy_h2d(void* dst, const void* src, size_t bytes, cp4_stream);
 cp4_status cp4_memcpy_d2h(void* dst, const void* src, size_t bytes, cp4_stream);
 cp4_status cp4_memcpy_d2d(void* dst, const void* src, size_t bytes, cp4_stream);
 cp4_status cp4_memset_zero(void* dst, size_t bytes, cp4_stream);
+/* *is_device = 1 if ptr is device (HBM) memory, 0 for host memory of any
+ * kind (pinned, pageable, unknown to the runtime). */
+cp4_status cp4_pointer_is_device(const void* ptr, int* is_device);
 cp4_status cp4_stream_synchronize(cp4_stream);
 cp4_status cp4_device_synchronize(void);
 

@@ -89,6 +89,7 @@ def lib():
                                      ctypes.c_void_p]
     L.cp4_memset_zero.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
     L.cp4_stream_synchronize.argtypes = [ctypes.c_void_p]
+    L.cp4_pointer_is_device.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
     L.cp4_set_device.argtypes = [ctypes.c_int]
     _lib = L
     return L

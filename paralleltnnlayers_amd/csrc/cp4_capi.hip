@@ -394,6 +394,19 @@ cp4_status cp4_memset_zero(void* dst, size_t bytes, cp4_stream s) {
   CP4_HIP(hipMemsetAsync(dst, 0, bytes, as_stream(s)));
   return CP4_OK;
 }
+cp4_status cp4_pointer_is_device(const void* ptr, int* is_device) {
+  if (!is_device) return fail(CP4_ERR_NULL_POINTER, "is_device is NULL");
+  *is_device = 0;
+  if (!ptr) return CP4_OK;
+  hipPointerAttribute_t attr;
+  hipError_t e = hipPointerGetAttributes(&attr, ptr);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();  // plain host memory the runtime has never seen
+    return CP4_OK;
+  }
+  *is_device = attr.type == hipMemoryTypeDevice ? 1 : 0;
+  return CP4_OK;
+}
 cp4_status cp4_stream_synchronize(cp4_stream s) {
   CP4_HIP(hipStreamSynchronize(as_stream(s)));
   return CP4_OK;
