@@ -29,7 +29,7 @@ typedef struct cp4_shape {
 typedef enum cp4_status {
   CP4_OK = 0,
   CP4_ERR_NULL_POINTER = 1,
-  CP4_ERR_SHAPE = 2,       /* zero dim, Y != X, sizes beyond 2^31 elements ... */
+  CP4_ERR_SHAPE = 2,       /* zero dim, sizes beyond the documented limits ... */
   CP4_ERR_HIP = 3,         /* a HIP runtime call failed; see cp4_last_error_message */
   CP4_ERR_WORKSPACE = 4,   /* workspace missing or too small */
   CP4_ERR_UNSUPPORTED = 5  /* requested kernel variant cannot run this shape */
@@ -74,6 +74,17 @@ cp4_status cp4_conv2d_backward_filter(const cp4_shape* shape, const float* x,
                                       float* dFH, float* dFW, void* workspace,
                                       size_t workspace_bytes,
                                       cp4_stream stream);
+
+/* Same, with the kernel variant chosen by the caller: -1 library's choice,
+ * 0 general (any shape), 1 matrix-core path (CP4_ERR_UNSUPPORTED if the shape
+ * does not qualify). */
+cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const float* x,
+                                              const float* dy, const float* FK,
+                                              const float* FC, const float* FH,
+                                              const float* FW, float* dFK, float* dFC,
+                                              float* dFH, float* dFW, void* workspace,
+                                              size_t workspace_bytes, int variant,
+                                              cp4_stream stream);
 
 /* Replaces cp4_conv2d_backward_filter_full_gpu
  * (Cuda_kernels/cp4Conv2dBackwardFilter.cuh:7-11, .cu:23-59): dense filter

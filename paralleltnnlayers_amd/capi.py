@@ -64,6 +64,7 @@ def lib():
     L.cp4_conv2d_backward_data.argtypes = fwd + [ctypes.c_void_p]
     bwf = [_S] + [_F] * 10 + [ctypes.c_void_p, ctypes.c_size_t]
     L.cp4_conv2d_backward_filter.argtypes = bwf + [ctypes.c_void_p]
+    L.cp4_conv2d_backward_filter_variant.argtypes = bwf + [ctypes.c_int, ctypes.c_void_p]
     L.cp4_conv2d_backward_filter_full.argtypes = [_S, _F, _F, _F, ctypes.c_int, ctypes.c_void_p]
     timing = [ctypes.c_uint, ctypes.c_uint, ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
     L.cp4_time_forward.argtypes = fwd + timing
@@ -157,15 +158,17 @@ def _workspace(s, device, workspace):
     return workspace, workspace.numel() * 4
 
 
-def conv2d_backward_filter(x, dy, FK, FC, FH, FW, pad=1, workspace=None, stream=None):
+def conv2d_backward_filter(x, dy, FK, FC, FH, FW, pad=1, workspace=None, stream=None,
+                           variant=-1):
     """Returns (dFK, dFC, dFH, dFW)."""
     s = shape_for(x.shape, FK, FC, FH, FW, pad)
     assert tuple(dy.shape) == (s.N, s.T, s.H, s.W) and x.shape[1] == s.C
     outs = [torch.empty_like(f) for f in (FK, FC, FH, FW)]
     ws, ws_bytes = _workspace(s, x.device, workspace)
-    check(lib().cp4_conv2d_backward_filter(
+    check(lib().cp4_conv2d_backward_filter_variant(
         ctypes.byref(s), _ptr(x), _ptr(dy), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
-        *[_ptr(o) for o in outs], ctypes.c_void_p(ws.data_ptr()), ws_bytes, _stream(stream)))
+        *[_ptr(o) for o in outs], ctypes.c_void_p(ws.data_ptr()), ws_bytes, variant,
+        _stream(stream)))
     return tuple(outs)
 
 

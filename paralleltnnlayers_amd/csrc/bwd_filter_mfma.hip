@@ -1,0 +1,386 @@
+// Backward-filter on the fp32 matrix cores (ranks up to 64, even H*W, even
+// channel counts).  Same reassociation of the reference's 8-deep sums
+// (Cuda_kernels/cp4Conv2dBackwardFilter.cu:64-257) as the general path:
+//   A = FC^T x,  B = FH *v A,  Cc = FW *h B,  G3 = FK^T dy,  G2, G1 = adjoint taps
+//   dFK = dy . Cc^T   dFC = x . G1^T   dFW[j] = <G3, shift_j B>   dFH[i] = <G2, shift_i A>
+// in four launches:
+//   1. contract: both channel->rank contractions, one wave per (image, 64-pixel
+//      block, 32-rank tile), x / dy streamed as float2 straight into the MFMA B
+//      operand, the factor from an LDS copy;
+//   2. taps: B, Cc, G2, G1 elementwise from A and G3 (L2-resident);
+//   3. gradient GEMMs: dF[d,r] = sum_{n,p} act[n,d,p] Z[n,r,p], split over
+//      images (and pixel ranges) across workgroups, 32 channel rows per wave,
+//      operands staged through LDS so that global reads stay row-contiguous;
+//      plus the small tap gradients;
+//   4. fixed-order sum of the per-workgroup partials (bit-reproducible).
+#include "cp4_internal.h"
+
+namespace cp4 {
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ f32x16 mfma32(float a, float b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+constexpr int kCT = 256;   // contract / gradient workgroup: 4 waves
+constexpr int kPF = 8;     // channel pairs per prefetch chunk in the contraction
+
+// ---- 1. Z[n,r,p] = sum_c F[c,r] src[n,c,p] ---------------------------------
+struct ContractArgs {
+  const float* src[2];   // x, dy
+  const float* F[2];     // FC, FK
+  float* Z[2];           // A, G3
+  int Cin[2];
+  int N, R, RP, HW, npb, items;   // items per contraction = N * npb * (RP/32)
+};
+
+__global__ __launch_bounds__(kCT) void contract_mfma_kernel(ContractArgs a) {
+  extern __shared__ float Fs[];   // [Cin][RP], zero-padded ranks
+  const int which = blockIdx.y;
+  const int Cin = a.Cin[which], R = a.R, RP = a.RP, HW = a.HW;
+  const float* F = a.F[which];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hi = lane >> 5;
+  for (int i0 = tid; i0 < Cin * RP; i0 += kCT * 4) {
+    float v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u * kCT, c = i / RP, r = i - c * RP;
+      v[u] = (i < Cin * RP && r < R) ? F[(size_t)c * R + r] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i0 + u * kCT < Cin * RP) Fs[i0 + u * kCT] = v[u];
+  }
+  __syncthreads();
+  const int item = blockIdx.x * (kCT / 64) + wave;
+  if (item >= a.items) return;
+  const int nmb = RP >> 5;
+  const int mb = item % nmb, pb = (item / nmb) % a.npb, n = item / (nmb * a.npb);
+  const int p = pb * 64 + 2 * l32;
+  const bool valid = p < HW;
+  const int pc = valid ? p : HW - 2;
+  const float* xp = a.src[which] + ((size_t)n * Cin + hi) * HW + pc;
+  const float* fp = Fs + hi * RP + 32 * mb + l32;
+  f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
+  const int nsteps = Cin >> 1, nchunks = nsteps / kPF;
+  float2 xb0[kPF], xb1[kPF];
+  auto load = [&](float2 (&xb)[kPF], int ch) {
+#pragma unroll
+    for (int s = 0; s < kPF; ++s)
+      xb[s] = *reinterpret_cast<const float2*>(xp + (size_t)(2 * (ch * kPF + s)) * HW);
+  };
+  auto compute = [&](const float2 (&xb)[kPF], int ch) {
+#pragma unroll
+    for (int s = 0; s < kPF; ++s) {
+      const float f = fp[(ch * kPF + s) * 2 * RP];
+      acc0 = mfma32(f, xb[s].x, acc0);
+      acc1 = mfma32(f, xb[s].y, acc1);
+    }
+  };
+  if (nchunks > 0) load(xb0, 0);
+  for (int ch = 0; ch < nchunks; ch += 2) {
+    if (ch + 1 < nchunks) load(xb1, ch + 1);
+    compute(xb0, ch);
+    if (ch + 1 < nchunks) {
+      if (ch + 2 < nchunks) load(xb0, ch + 2);
+      compute(xb1, ch + 1);
+    }
+  }
+  for (int st = nchunks * kPF; st < nsteps; ++st) {
+    const float2 xv = *reinterpret_cast<const float2*>(xp + (size_t)(2 * st) * HW);
+    const float f = fp[st * 2 * RP];
+    acc0 = mfma32(f, xv.x, acc0);
+    acc1 = mfma32(f, xv.y, acc1);
+  }
+  if (valid) {
+    float* zn = a.Z[which] + (size_t)n * R * HW + p;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int r = 32 * mb + 8 * (v >> 2) + 4 * hi + (v & 3);
+      if (r < R) {
+        float2 o;
+        o.x = acc0[v];
+        o.y = acc1[v];
+        *reinterpret_cast<float2*>(zn + (size_t)r * HW) = o;
+      }
+    }
+  }
+}
+
+// ---- 2. taps: B, Cc from A; G2, G1 from G3 ----------------------------------
+__global__ __launch_bounds__(256) void taps_kernel(const float* __restrict__ A,
+                                                   const float* __restrict__ G3,
+                                                   const float* __restrict__ FH,
+                                                   const float* __restrict__ FW,
+                                                   float* __restrict__ B, float* __restrict__ Cc,
+                                                   float* __restrict__ G2, float* __restrict__ G1,
+                                                   size_t total, int R, int H, int W, int Y,
+                                                   int X, int P) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int w = idx % W, h = (idx / W) % H;
+  const size_t plane = idx / ((size_t)W * H);
+  const int r = plane % R;
+  const float* ap = A + plane * (size_t)H * W;
+  const float* gp = G3 + plane * (size_t)H * W;
+  float b = 0.f, cc = 0.f, g2 = 0.f, g1 = 0.f;
+  for (int i = 0; i < Y; ++i) {
+    const float fh = FH[i * R + r];
+    const int hf = h + i - P, hb = h - i + P;     // forward / adjoint row
+    if (hf >= 0 && hf < H) {
+      b += fh * ap[hf * W + w];
+      float s = 0.f;
+      for (int j = 0; j < X; ++j) {
+        const int ww = w + j - P;
+        if (ww >= 0 && ww < W) s += FW[j * R + r] * ap[hf * W + ww];
+      }
+      cc += fh * s;
+    }
+    if (hb >= 0 && hb < H) {
+      float s = 0.f;
+      for (int j = 0; j < X; ++j) {
+        const int ww = w - j + P;
+        if (ww >= 0 && ww < W) s += FW[j * R + r] * gp[hb * W + ww];
+      }
+      g1 += fh * s;
+    }
+  }
+  for (int j = 0; j < X; ++j) {
+    const int ww = w - j + P;
+    if (ww >= 0 && ww < W) g2 += FW[j * R + r] * gp[h * W + ww];
+  }
+  B[idx] = b;
+  Cc[idx] = cc;
+  G2[idx] = g2;
+  G1[idx] = g1;
+}
+
+// ---- 3a. partial[s][d][r] = sum_{p in split s} act[n,d,p] Z[n,r,p] ----------
+struct GradArgs {
+  const float* act[2];   // dy, x
+  const float* Z[2];     // Cc, G1
+  float* part[2];        // [S][D][R]
+  int D[2];
+  int N, R, RP, HW, PS, cps;   // PS pixel splits per image, cps 32-pixel chunks per split
+};
+
+constexpr int kLd = 34;   // LDS row stride of the 32-pixel operand tiles (conflict-free)
+
+template <int RB>
+__global__ __launch_bounds__(kCT) void grad_gemm_kernel(GradArgs a) {
+  __shared__ float Zs[32 * RB * kLd];
+  __shared__ float As[kCT / 64][32 * kLd];
+  const int which = blockIdx.z;
+  const int D = a.D[which], R = a.R, HW = a.HW;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hi = lane >> 5;
+  const int d0 = blockIdx.y * 128 + wave * 32;
+  if ((int)blockIdx.y * 128 >= D) return;
+  const int s = blockIdx.x, n = s / a.PS, ps = s - n * a.PS;
+  const int nch_total = (HW + 31) >> 5;
+  const int ch0 = ps * a.cps, ch1 = min(nch_total, ch0 + a.cps);
+  const float* actn = a.act[which] + (size_t)n * D * HW;
+  const float* zn = a.Z[which] + (size_t)n * R * HW;
+  // tile loads: a lane moves float2; 16 lanes cover one 32-pixel row
+  const int trow = lane >> 4, tcol = 2 * (lane & 15);
+  float2 av[8], zv[RB * 2];
+  auto load_tiles = [&](int ch) {
+    const int p = ch * 32 + tcol;
+    const bool pin = p < HW;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int d = d0 + 4 * j + trow;
+      av[j] = (pin && d < D) ? *reinterpret_cast<const float2*>(actn + (size_t)d * HW + p)
+                             : make_float2(0.f, 0.f);
+    }
+#pragma unroll
+    for (int j = 0; j < RB * 2; ++j) {
+      const int r = 16 * j + 4 * wave + trow;     // 4 waves x 4 rows per j
+      zv[j] = (pin && r < R) ? *reinterpret_cast<const float2*>(zn + (size_t)r * HW + p)
+                             : make_float2(0.f, 0.f);
+    }
+  };
+  auto store_tiles = [&]() {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      *reinterpret_cast<float2*>(&As[wave][(4 * j + trow) * kLd + tcol]) = av[j];
+#pragma unroll
+    for (int j = 0; j < RB * 2; ++j)
+      *reinterpret_cast<float2*>(&Zs[(16 * j + 4 * wave + trow) * kLd + tcol]) = zv[j];
+  };
+  f32x16 acc[RB];
+#pragma unroll
+  for (int mb = 0; mb < RB; ++mb) acc[mb] = (f32x16)(0.f);
+  if (ch0 < ch1) load_tiles(ch0);
+  for (int ch = ch0; ch < ch1; ++ch) {
+    __syncthreads();              // previous chunk's MFMAs are done with the tiles
+    store_tiles();
+    __syncthreads();
+    if (ch + 1 < ch1) load_tiles(ch + 1);   // in flight during the MFMAs
+    const float* ap = &As[wave][l32 * kLd + hi];
+    const float* zp = &Zs[l32 * kLd + hi];
+#pragma unroll
+    for (int st = 0; st < 16; ++st) {
+      const float av1 = ap[2 * st];
+#pragma unroll
+      for (int mb = 0; mb < RB; ++mb) acc[mb] = mfma32(av1, zp[mb * 32 * kLd + 2 * st], acc[mb]);
+    }
+  }
+  float* out = a.part[which] + (size_t)s * D * R;
+#pragma unroll
+  for (int mb = 0; mb < RB; ++mb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int d = d0 + 8 * (v >> 2) + 4 * hi + (v & 3), r = 32 * mb + l32;
+      if (d < D && r < R) out[(size_t)d * R + r] = acc[mb][v];
+    }
+}
+
+// ---- 3b. tap gradients: partial[s][t][r] over images of split s -------------
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return red[0] + red[1] + red[2] + red[3];
+}
+
+__global__ __launch_bounds__(256) void tap_grad_kernel(const float* __restrict__ G2,
+                                                       const float* __restrict__ A,
+                                                       const float* __restrict__ G3,
+                                                       const float* __restrict__ B,
+                                                       float* __restrict__ partH,
+                                                       float* __restrict__ partW, int N, int R,
+                                                       int H, int W, int Y, int X, int P, int S) {
+  __shared__ float red[4];
+  const int t = blockIdx.x, r = blockIdx.y, s = blockIdx.z;   // t < Y: dFH tap, else dFW tap
+  const bool vertical = t < Y;
+  const int tap = vertical ? t : t - Y, o = tap - P, HW = H * W;
+  const float* P0 = vertical ? G2 : G3;
+  const float* P1 = vertical ? A : B;
+  const int n0 = (int)((long)N * s / S), n1 = (int)((long)N * (s + 1) / S);
+  float acc = 0.f;
+  for (int n = n0; n < n1; ++n) {
+    const float* a = P0 + ((size_t)n * R + r) * HW;
+    const float* b = P1 + ((size_t)n * R + r) * HW;
+    for (int p = threadIdx.x; p < HW; p += 256) {
+      const int h = p / W, w = p - h * W;
+      const int hh = vertical ? h + o : h, ww = vertical ? w : w + o;
+      if (hh >= 0 && hh < H && ww >= 0 && ww < W) acc += a[p] * b[hh * W + ww];
+    }
+  }
+  const float tot = block_sum256(acc, red);
+  if (threadIdx.x == 0) {
+    if (vertical) partH[((size_t)s * Y + tap) * R + r] = tot;
+    else partW[((size_t)s * X + tap) * R + r] = tot;
+  }
+}
+
+// ---- 4. out[i] = sum_s partial[s][i], four segments in one launch -----------
+struct ReduceArgs {
+  const float* part[4];
+  float* out[4];
+  int count[4], S[4];
+};
+__global__ __launch_bounds__(256) void reduce4_kernel(ReduceArgs a) {
+  const int seg = blockIdx.y;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= a.count[seg]) return;
+  const float* p = a.part[seg] + i;
+  float s = 0.f;
+  for (int k = 0; k < a.S[seg]; ++k) s += p[(size_t)k * a.count[seg]];
+  a.out[seg][i] = s;
+}
+
+struct Plan {
+  int RP, npb, PS, cps, S, St;
+  size_t plane, part_elems;
+};
+Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R) {
+  Plan p;
+  const int HW = H * W;
+  p.RP = R <= 32 ? 32 : 64;
+  p.npb = (HW + 63) / 64;
+  const int nch = (HW + 31) / 32;
+  const int dgroups = (T + 127) / 128 + (C + 127) / 128;
+  int PS = (512 + N * dgroups - 1) / (N * dgroups);   // aim at >= 512 workgroups
+  if (PS < 1) PS = 1;
+  if (PS > nch) PS = nch;
+  p.cps = (nch + PS - 1) / PS;
+  p.PS = (nch + p.cps - 1) / p.cps;
+  p.S = N * p.PS;
+  p.St = N < 8 ? N : 8;
+  p.plane = (size_t)N * R * HW;
+  p.part_elems = (size_t)p.S * R * ((size_t)T + C) + (size_t)p.St * R * ((size_t)Y + X);
+  return p;
+}
+
+}  // namespace
+
+bool bwd_filter_mfma_supported(const cp4_shape& s) {
+  return s.Rank <= 64 && ((s.H * s.W) & 1) == 0 && (s.C & 1) == 0 && (s.T & 1) == 0 &&
+         (size_t)(s.C > s.T ? s.C : s.T) * (s.Rank <= 32 ? 32 : 64) * 4 <= 160 * 1024 &&
+         s.Y + s.X <= 65535;
+}
+
+size_t bwd_filter_mfma_workspace_bytes(const cp4_shape& s) {
+  const Plan p = make_plan(s.N, s.C, s.T, s.H, s.W, s.Y, s.X, s.Rank);
+  return (6 * p.plane + p.part_elems) * sizeof(float);
+}
+
+hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
+  const int HW = a.H * a.W, R = a.R, N = a.N;
+  const Plan p = make_plan(N, a.C, a.T, a.H, a.W, a.Y, a.X, R);
+  float* ws = static_cast<float*>(a.workspace);
+  float *A = ws, *B = ws + p.plane, *Cc = ws + 2 * p.plane, *G3 = ws + 3 * p.plane,
+        *G2 = ws + 4 * p.plane, *G1 = ws + 5 * p.plane, *part = ws + 6 * p.plane;
+  float* pK = part;
+  float* pC = pK + (size_t)p.S * a.T * R;
+  float* pH = pC + (size_t)p.S * a.C * R;
+  float* pW = pH + (size_t)p.St * a.Y * R;
+
+  ContractArgs c{};
+  c.src[0] = a.x; c.F[0] = a.FC; c.Z[0] = A; c.Cin[0] = a.C;
+  c.src[1] = a.dy; c.F[1] = a.FK; c.Z[1] = G3; c.Cin[1] = a.T;
+  c.N = N; c.R = R; c.RP = p.RP; c.HW = HW; c.npb = p.npb;
+  c.items = N * p.npb * (p.RP / 32);
+  const size_t smem = (size_t)(a.C > a.T ? a.C : a.T) * p.RP * sizeof(float);
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_mfma_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  if (e != hipSuccess) return e;
+  contract_mfma_kernel<<<dim3((c.items + 3) / 4, 2), kCT, smem, st>>>(c);
+
+  taps_kernel<<<(unsigned)((p.plane + 255) / 256), 256, 0, st>>>(A, G3, a.FH, a.FW, B, Cc, G2, G1,
+                                                                  p.plane, R, a.H, a.W, a.Y, a.X,
+                                                                  a.pad);
+
+  GradArgs g{};
+  g.act[0] = a.dy; g.Z[0] = Cc; g.part[0] = pK; g.D[0] = a.T;
+  g.act[1] = a.x; g.Z[1] = G1; g.part[1] = pC; g.D[1] = a.C;
+  g.N = N; g.R = R; g.RP = p.RP; g.HW = HW; g.PS = p.PS; g.cps = p.cps;
+  const int dmax = a.T > a.C ? a.T : a.C;
+  const dim3 ggrid(p.S, (dmax + 127) / 128, 2);
+  if (p.RP == 32) grad_gemm_kernel<1><<<ggrid, kCT, 0, st>>>(g);
+  else grad_gemm_kernel<2><<<ggrid, kCT, 0, st>>>(g);
+  tap_grad_kernel<<<dim3(a.Y + a.X, R, p.St), 256, 0, st>>>(G2, A, G3, B, pH, pW, N, R, a.H, a.W,
+                                                            a.Y, a.X, a.pad, p.St);
+
+  ReduceArgs r{};
+  const float* parts[4] = {pK, pC, pH, pW};
+  float* outs[4] = {a.dFK, a.dFC, a.dFH, a.dFW};
+  const int counts[4] = {a.T * R, a.C * R, a.Y * R, a.X * R};
+  const int Ss[4] = {p.S, p.S, p.St, p.St};
+  int maxc = 0;
+  for (int i = 0; i < 4; ++i) {
+    r.part[i] = parts[i]; r.out[i] = outs[i]; r.count[i] = counts[i]; r.S[i] = Ss[i];
+    if (counts[i] > maxc) maxc = counts[i];
+  }
+  reduce4_kernel<<<dim3((maxc + 255) / 256, 4), 256, 0, st>>>(r);
+  return hipGetLastError();
+}
+
+}  // namespace cp4

@@ -107,6 +107,16 @@ cp4_status run_forward_like(const FwdArgs& a, int variant, hipStream_t st) {
   return CP4_OK;
 }
 
+// One workspace size serves either backward-filter variant.
+size_t filter_workspace(const cp4_shape& s) {
+  size_t b = cp4::bwd_filter_workspace_bytes(s);
+  if (cp4::bwd_filter_mfma_supported(s)) {
+    const size_t m = cp4::bwd_filter_mfma_workspace_bytes(s);
+    if (m > b) b = m;
+  }
+  return b;
+}
+
 cp4_status check_forward_ptrs(const void* x, const void* FK, const void* FC,
                               const void* FH, const void* FW, const void* y) {
   if (!x || !FK || !FC || !FH || !FW || !y)
@@ -195,7 +205,7 @@ cp4_status cp4_conv2d_backward_data(const cp4_shape* shape, const float* dy,
 
 size_t cp4_conv2d_backward_filter_workspace_bytes(const cp4_shape* shape) {
   if (check_shape(shape) != CP4_OK || shape->N == 0) return 0;
-  return cp4::bwd_filter_workspace_bytes(*shape);
+  return filter_workspace(*shape);
 }
 
 cp4_status cp4_conv2d_backward_filter(const cp4_shape* shape, const float* x,
@@ -205,6 +215,17 @@ cp4_status cp4_conv2d_backward_filter(const cp4_shape* shape, const float* x,
                                       float* dFH, float* dFW, void* workspace,
                                       size_t workspace_bytes,
                                       cp4_stream stream) {
+  return cp4_conv2d_backward_filter_variant(shape, x, dy, FK, FC, FH, FW, dFK, dFC, dFH, dFW,
+                                            workspace, workspace_bytes, -1, stream);
+}
+
+cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const float* x,
+                                              const float* dy, const float* FK,
+                                              const float* FC, const float* FH,
+                                              const float* FW, float* dFK, float* dFC,
+                                              float* dFH, float* dFW, void* workspace,
+                                              size_t workspace_bytes, int variant,
+                                              cp4_stream stream) {
   cp4_status rc = check_shape(shape);
   if (rc != CP4_OK) return rc;
   if (!FK || !FC || !FH || !FW || !dFK || !dFC || !dFH || !dFW)
@@ -219,15 +240,21 @@ cp4_status cp4_conv2d_backward_filter(const cp4_shape* shape, const float* x,
     return CP4_OK;
   }
   if (!x || !dy) return fail(CP4_ERR_NULL_POINTER, "x or dy is NULL");
-  if (!workspace || workspace_bytes < cp4::bwd_filter_workspace_bytes(s))
+  if (!workspace || workspace_bytes < filter_workspace(s))
     return fail(CP4_ERR_WORKSPACE,
                 "workspace smaller than cp4_conv2d_backward_filter_workspace_bytes");
+  const bool mfma_ok = cp4::bwd_filter_mfma_supported(s) &&
+                       ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) |
+                         reinterpret_cast<uintptr_t>(workspace)) & 7) == 0;
+  if (variant > 1 || (variant == 1 && !mfma_ok))
+    return fail(CP4_ERR_UNSUPPORTED, "backward-filter variant cannot run this shape");
   cp4::BwdFilterArgs a{};
   a.x = x; a.dy = dy; a.FK = FK; a.FC = FC; a.FH = FH; a.FW = FW;
   a.dFK = dFK; a.dFC = dFC; a.dFH = dFH; a.dFW = dFW; a.workspace = workspace;
   a.N = s.N; a.C = s.C; a.T = s.T; a.H = s.H; a.W = s.W; a.pad = s.pad;
   a.Y = s.Y; a.X = s.X; a.R = s.Rank;
-  CP4_HIP(cp4::bwd_filter_launch(a, st));
+  if (variant == 1 || (variant < 0 && mfma_ok)) CP4_HIP(cp4::bwd_filter_mfma_launch(a, st));
+  else CP4_HIP(cp4::bwd_filter_launch(a, st));
   return CP4_OK;
 }
 

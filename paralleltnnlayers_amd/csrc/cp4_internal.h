@@ -40,8 +40,12 @@ struct BwdFilterArgs {
   void* workspace;
   int N, C, T, H, W, pad, Y, X, R;
 };
+// general (VALU, any shape) and matrix-core variants
 size_t bwd_filter_workspace_bytes(const cp4_shape&);
 hipError_t bwd_filter_launch(const BwdFilterArgs&, hipStream_t);
+bool bwd_filter_mfma_supported(const cp4_shape&);
+size_t bwd_filter_mfma_workspace_bytes(const cp4_shape&);
+hipError_t bwd_filter_mfma_launch(const BwdFilterArgs&, hipStream_t);
 hipError_t bwd_filter_full_launch(const cp4_shape&, const float* x,
                                   const float* dy, float* dK, int accumulate,
                                   hipStream_t);

@@ -66,6 +66,18 @@ def variants_for(cp4, x_shape, f, pad):
     return [v for v, _, ok in cp4.forward_variants(s) if ok]
 
 
+def filter_variants(cp4, x, dy, f, pad):
+    """Backward-filter variants that accept this shape: -1 (library's choice),
+    0 (general) and, where it qualifies, 1 (matrix cores)."""
+    out = [-1, 0]
+    try:
+        cp4.conv2d_backward_filter(x, dy, *f, pad=pad, variant=1)
+        out.append(1)
+    except cp4.Cp4Error as e:
+        assert e.status == cp4.capi.ERR_UNSUPPORTED
+    return out
+
+
 # ---------------------------------------------------------------- golden ----
 @pytest.mark.parametrize("name", GOLD_CASES)
 def test_golden_all_passes(cp4, name):
@@ -77,9 +89,10 @@ def test_golden_all_passes(cp4, name):
         assert_activation_close(y, g["y"], f"{name} forward variant {v}")
     dx = host(cp4.conv2d_backward_data(dy, *f.values(), pad=g["pad"]))
     assert_activation_close(dx, g["dx"], f"{name} backward-data")
-    grads = cp4.conv2d_backward_filter(x, dy, *f.values(), pad=g["pad"])
-    for got, k in zip(grads, FACTORS):
-        assert_gradient_close(host(got), g["d" + k], f"{name} d{k}")
+    for variant in filter_variants(cp4, x, dy, list(f.values()), g["pad"]):
+        grads = cp4.conv2d_backward_filter(x, dy, *f.values(), pad=g["pad"], variant=variant)
+        for got, k in zip(grads, FACTORS):
+            assert_gradient_close(host(got), g["d" + k], f"{name} d{k} variant {variant}")
 
 
 # ------------------------------------------------- the five workloads -------
@@ -113,9 +126,11 @@ def test_workload_backward_filter(cp4, oracle, workload):
     w, a = workload
     want = oracle.backward_filter(a["x"], a["dy"], a["FK"], a["FC"], a["FH"], a["FW"], w.pad)
     f = [dev(a[k]) for k in FACTORS]
-    got = cp4.conv2d_backward_filter(dev(a["x"]), dev(a["dy"]), *f, pad=w.pad)
-    for g, wnt, k in zip(got, want, FACTORS):
-        assert_gradient_close(host(g), wnt, f"{w.name} d{k}")
+    for variant in filter_variants(cp4, dev(a["x"]), dev(a["dy"]), f, w.pad):
+        got = cp4.conv2d_backward_filter(dev(a["x"]), dev(a["dy"]), *f, pad=w.pad,
+                                         variant=variant)
+        for g, wnt, k in zip(got, want, FACTORS):
+            assert_gradient_close(host(g), wnt, f"{w.name} d{k} variant {variant}")
     # bit-reproducible: no floating-point atomics anywhere in the reduction
     again = cp4.conv2d_backward_filter(dev(a["x"]), dev(a["dy"]), *f, pad=w.pad)
     for g1, g2 in zip(got, again):
@@ -174,9 +189,11 @@ def test_edge_shapes(cp4, oracle, dims):
         assert_activation_close(y, want, f"forward variant {v}")
     dx = host(cp4.conv2d_backward_data(dev(dy), *f, pad=pad))
     assert_activation_close(dx, oracle.backward_data(dy, *fac, pad), "backward-data")
-    got = cp4.conv2d_backward_filter(dev(x), dev(dy), *f, pad=pad)
-    for g, wnt, k in zip(got, oracle.backward_filter(x, dy, *fac, pad), FACTORS):
-        assert_gradient_close(host(g), wnt, f"d{k}")
+    want_grads = oracle.backward_filter(x, dy, *fac, pad)
+    for variant in filter_variants(cp4, dev(x), dev(dy), f, pad):
+        got = cp4.conv2d_backward_filter(dev(x), dev(dy), *f, pad=pad, variant=variant)
+        for g, wnt, k in zip(got, want_grads, FACTORS):
+            assert_gradient_close(host(g), wnt, f"d{k} variant {variant}")
 
 
 def test_reference_single_case_against_dense_conv(cp4):
