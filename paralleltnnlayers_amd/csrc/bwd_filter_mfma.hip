@@ -24,7 +24,8 @@ __device__ __forceinline__ f32x16 mfma32(float a, float b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
 
-constexpr int kCT = 256;   // contract / gradient workgroup: 4 waves
+constexpr int kCT = 256;   // gradient-GEMM workgroup: 4 waves
+constexpr int kCW = 256;   // contraction workgroup: 4 waves (one per SIMD) sharing one 32-rank factor tile
 constexpr int kPF = 8;     // channel pairs per prefetch chunk in the contraction
 
 // ---- 1. Z[n,r,p] = sum_c F[c,r] src[n,c,p] ---------------------------------
@@ -33,37 +34,37 @@ struct ContractArgs {
   const float* F[2];     // FC, FK
   float* Z[2];           // A, G3
   int Cin[2];
-  int N, R, RP, HW, npb, items;   // items per contraction = N * npb * (RP/32)
+  int N, R, RP, HW, npb, items;   // items per contraction and rank tile = N * npb
 };
 
-__global__ __launch_bounds__(kCT) void contract_mfma_kernel(ContractArgs a) {
-  extern __shared__ float Fs[];   // [Cin][RP], zero-padded ranks
-  const int which = blockIdx.y;
-  const int Cin = a.Cin[which], R = a.R, RP = a.RP, HW = a.HW;
+__global__ __launch_bounds__(kCW) void contract_mfma_kernel(ContractArgs a) {
+  extern __shared__ float Fs[];   // [Cin][32]: the 32-rank tile mb of F, zero-padded
+  const int which = blockIdx.y, mb = blockIdx.z;
+  const int Cin = a.Cin[which], R = a.R, HW = a.HW;
+  constexpr int RP = 32;
   const float* F = a.F[which];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hi = lane >> 5;
-  for (int i0 = tid; i0 < Cin * RP; i0 += kCT * 4) {
-    float v[4];
+  for (int i0 = tid; i0 < Cin * 32; i0 += kCW * 16) {
+    float v[16];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int i = i0 + u * kCT, c = i / RP, r = i - c * RP;
-      v[u] = (i < Cin * RP && r < R) ? F[(size_t)c * R + r] : 0.f;
+    for (int u = 0; u < 16; ++u) {
+      const int i = i0 + u * kCW, c = i >> 5, r = 32 * mb + (i & 31);
+      v[u] = (i < Cin * 32 && r < R) ? F[(size_t)c * R + r] : 0.f;
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
-      if (i0 + u * kCT < Cin * RP) Fs[i0 + u * kCT] = v[u];
+    for (int u = 0; u < 16; ++u)
+      if (i0 + u * kCW < Cin * 32) Fs[i0 + u * kCW] = v[u];
   }
   __syncthreads();
-  const int item = blockIdx.x * (kCT / 64) + wave;
+  const int item = blockIdx.x * (kCW / 64) + wave;   // (image, 64-pixel block)
   if (item >= a.items) return;
-  const int nmb = RP >> 5;
-  const int mb = item % nmb, pb = (item / nmb) % a.npb, n = item / (nmb * a.npb);
+  const int pb = item % a.npb, n = item / a.npb;
   const int p = pb * 64 + 2 * l32;
   const bool valid = p < HW;
   const int pc = valid ? p : HW - 2;
   const float* xp = a.src[which] + ((size_t)n * Cin + hi) * HW + pc;
-  const float* fp = Fs + hi * RP + 32 * mb + l32;
+  const float* fp = Fs + hi * RP + l32;
   f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
   const int nsteps = Cin >> 1, nchunks = nsteps / kPF;
   float2 xb0[kPF], xb1[kPF];
@@ -158,6 +159,94 @@ __global__ __launch_bounds__(256) void taps_kernel(const float* __restrict__ A,
   G1[idx] = g1;
 }
 
+// Same taps with one workgroup per (image, rank) plane held in LDS, which also
+// yields the plane's tap-gradient partials: partH[n][i][r] = <G2, shift_i A>,
+// partW[n][j][r] = <G3, shift_j B>.  Tap weights are workgroup-uniform.
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return red[0] + red[1] + red[2] + red[3];
+}
+
+__global__ __launch_bounds__(256) void taps_plane_kernel(
+    const float* __restrict__ A, const float* __restrict__ G3, const float* __restrict__ FH,
+    const float* __restrict__ FW, float* __restrict__ B, float* __restrict__ Cc,
+    float* __restrict__ G2, float* __restrict__ G1, float* __restrict__ partH,
+    float* __restrict__ partW, int R, int H, int W, int Y, int X, int P) {
+  extern __shared__ float pl[];
+  const int HW = H * W;
+  float *sA = pl, *sG = pl + HW, *sB = pl + 2 * HW, *sG2 = pl + 3 * HW;
+  const int plane = blockIdx.x, r = plane % R, n = plane / R;
+  const size_t base = (size_t)plane * HW;
+  float* red = pl + 4 * HW;                       // [Y + X][4] wave partials
+  float* fh = red + 4 * (Y + X);                  // this rank's tap weights, read once
+  float* fw = fh + Y;
+  for (int p = threadIdx.x; p < HW; p += 256) {
+    sA[p] = A[base + p];
+    sG[p] = G3[base + p];
+  }
+  if ((int)threadIdx.x < Y) fh[threadIdx.x] = FH[threadIdx.x * R + r];
+  else if ((int)threadIdx.x < Y + X) fw[threadIdx.x - Y] = FW[(threadIdx.x - Y) * R + r];
+  __syncthreads();
+  for (int p = threadIdx.x; p < HW; p += 256) {
+    const int h = p / W, w = p - h * W;
+    float b = 0.f, g2 = 0.f;
+    for (int i = 0; i < Y; ++i) {
+      const int hh = h + i - P;
+      if (hh >= 0 && hh < H) b += fh[i] * sA[hh * W + w];
+    }
+    for (int j = 0; j < X; ++j) {
+      const int ww = w - j + P;
+      if (ww >= 0 && ww < W) g2 += fw[j] * sG[h * W + ww];
+    }
+    sB[p] = b;
+    sG2[p] = g2;
+    B[base + p] = b;
+    G2[base + p] = g2;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < HW; p += 256) {
+    const int h = p / W, w = p - h * W;
+    float cc = 0.f, g1 = 0.f;
+    for (int j = 0; j < X; ++j) {
+      const int ww = w + j - P;
+      if (ww >= 0 && ww < W) cc += fw[j] * sB[h * W + ww];
+    }
+    for (int i = 0; i < Y; ++i) {
+      const int hh = h - i + P;
+      if (hh >= 0 && hh < H) g1 += fh[i] * sG2[hh * W + w];
+    }
+    Cc[base + p] = cc;
+    G1[base + p] = g1;
+  }
+  // tap gradients of this plane: wave sums to LDS, one barrier, then a fixed-order
+  // sum of the four wave partials per tap
+  for (int t = 0; t < Y + X; ++t) {
+    const bool vertical = t < Y;
+    const int o = (vertical ? t : t - Y) - P;
+    float acc = 0.f;
+    for (int p = threadIdx.x; p < HW; p += 256) {
+      const int h = p / W, w = p - h * W;
+      const int hh = vertical ? h + o : h, ww = vertical ? w : w + o;
+      if (hh >= 0 && hh < H && ww >= 0 && ww < W)
+        acc += vertical ? sG2[p] * sA[hh * W + ww] : sG[p] * sB[hh * W + ww];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off, 64);
+    if ((threadIdx.x & 63) == 0) red[t * 4 + (threadIdx.x >> 6)] = acc;
+  }
+  __syncthreads();
+  if ((int)threadIdx.x < Y + X) {
+    const int t = threadIdx.x;
+    const float tot = red[t * 4] + red[t * 4 + 1] + red[t * 4 + 2] + red[t * 4 + 3];
+    if (t < Y) partH[((size_t)n * Y + t) * R + r] = tot;
+    else partW[((size_t)n * X + (t - Y)) * R + r] = tot;
+  }
+}
+
 // ---- 3a. partial[s][d][r] = sum_{p in split s} act[n,d,p] Z[n,r,p] ----------
 struct GradArgs {
   const float* act[2];   // dy, x
@@ -240,14 +329,6 @@ __global__ __launch_bounds__(kCT) void grad_gemm_kernel(GradArgs a) {
 }
 
 // ---- 3b. tap gradients: partial[s][t][r] over images of split s -------------
-__device__ __forceinline__ float block_sum256(float v, float* red) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  return red[0] + red[1] + red[2] + red[3];
-}
 
 __global__ __launch_bounds__(256) void tap_grad_kernel(const float* __restrict__ G2,
                                                        const float* __restrict__ A,
@@ -291,13 +372,24 @@ __global__ __launch_bounds__(256) void reduce4_kernel(ReduceArgs a) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= a.count[seg]) return;
   const float* p = a.part[seg] + i;
+  const size_t stride = a.count[seg];
+  const int S = a.S[seg];
   float s = 0.f;
-  for (int k = 0; k < a.S[seg]; ++k) s += p[(size_t)k * a.count[seg]];
+  int k = 0;
+  for (; k + 8 <= S; k += 8) {   // eight loads in flight, summed in index order
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = p[(size_t)(k + u) * stride];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += v[u];
+  }
+  for (; k < S; ++k) s += p[(size_t)k * stride];
   a.out[seg][i] = s;
 }
 
 struct Plan {
   int RP, npb, PS, cps, S, St;
+  bool plane_taps;
   size_t plane, part_elems;
 };
 Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R) {
@@ -307,15 +399,16 @@ Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R) {
   p.npb = (HW + 63) / 64;
   const int nch = (HW + 31) / 32;
   const int dgroups = (T + 127) / 128 + (C + 127) / 128;
-  int PS = (512 + N * dgroups - 1) / (N * dgroups);   // aim at >= 512 workgroups
+  int PS = (256 + N * dgroups - 1) / (N * dgroups);   // aim at >= 256 workgroups
   if (PS < 1) PS = 1;
   if (PS > nch) PS = nch;
   p.cps = (nch + PS - 1) / PS;
   p.PS = (nch + p.cps - 1) / p.cps;
   p.S = N * p.PS;
-  p.St = N < 8 ? N : 8;
+  p.plane_taps = (size_t)HW * 4 * sizeof(float) <= 64 * 1024 && Y + X <= 256;   // plane fits in LDS
+  p.St = p.plane_taps ? N : (N < 8 ? N : 8);
   p.plane = (size_t)N * R * HW;
-  p.part_elems = (size_t)p.S * R * ((size_t)T + C) + (size_t)p.St * R * ((size_t)Y + X);
+  p.part_elems = (size_t)p.S * R * ((size_t)T + C) + (size_t)N * R * ((size_t)Y + X);
   return p;
 }
 
@@ -347,16 +440,26 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   c.src[0] = a.x; c.F[0] = a.FC; c.Z[0] = A; c.Cin[0] = a.C;
   c.src[1] = a.dy; c.F[1] = a.FK; c.Z[1] = G3; c.Cin[1] = a.T;
   c.N = N; c.R = R; c.RP = p.RP; c.HW = HW; c.npb = p.npb;
-  c.items = N * p.npb * (p.RP / 32);
-  const size_t smem = (size_t)(a.C > a.T ? a.C : a.T) * p.RP * sizeof(float);
+  c.items = N * p.npb;
+  const size_t smem = (size_t)(a.C > a.T ? a.C : a.T) * 32 * sizeof(float);
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_mfma_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (e != hipSuccess) return e;
-  contract_mfma_kernel<<<dim3((c.items + 3) / 4, 2), kCT, smem, st>>>(c);
+  contract_mfma_kernel<<<dim3((c.items + kCW / 64 - 1) / (kCW / 64), 2, p.RP / 32), kCW, smem, st>>>(c);
 
-  taps_kernel<<<(unsigned)((p.plane + 255) / 256), 256, 0, st>>>(A, G3, a.FH, a.FW, B, Cc, G2, G1,
-                                                                  p.plane, R, a.H, a.W, a.Y, a.X,
-                                                                  a.pad);
+  if (p.plane_taps) {
+    const size_t tsm = ((size_t)HW * 4 + 5 * (a.Y + a.X)) * sizeof(float);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(taps_plane_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)tsm);
+    if (e != hipSuccess) return e;
+    taps_plane_kernel<<<N * R, 256, tsm, st>>>(A, G3, a.FH, a.FW, B, Cc, G2, G1, pH, pW, R, a.H,
+                                               a.W, a.Y, a.X, a.pad);
+  } else {
+    taps_kernel<<<(unsigned)((p.plane + 255) / 256), 256, 0, st>>>(
+        A, G3, a.FH, a.FW, B, Cc, G2, G1, p.plane, R, a.H, a.W, a.Y, a.X, a.pad);
+    tap_grad_kernel<<<dim3(a.Y + a.X, R, p.St), 256, 0, st>>>(G2, A, G3, B, pH, pW, N, R, a.H,
+                                                              a.W, a.Y, a.X, a.pad, p.St);
+  }
 
   GradArgs g{};
   g.act[0] = a.dy; g.Z[0] = Cc; g.part[0] = pK; g.D[0] = a.T;
@@ -366,8 +469,6 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   const dim3 ggrid(p.S, (dmax + 127) / 128, 2);
   if (p.RP == 32) grad_gemm_kernel<1><<<ggrid, kCT, 0, st>>>(g);
   else grad_gemm_kernel<2><<<ggrid, kCT, 0, st>>>(g);
-  tap_grad_kernel<<<dim3(a.Y + a.X, R, p.St), 256, 0, st>>>(G2, A, G3, B, pH, pW, N, R, a.H, a.W,
-                                                            a.Y, a.X, a.pad, p.St);
 
   ReduceArgs r{};
   const float* parts[4] = {pK, pC, pH, pW};
