@@ -32,7 +32,7 @@ FACTORS = ("FK", "FC", "FH", "FW")
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs, scaled by the plain copy kernel's reading (see
 # profiles/): {workload: bytes}.  None until measured for the current kernel.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {"C3": 224.6e6}   # fwd_split_kernel<3>: 109.3 MB fetched + 115.4 MB written
 
 
 def main():
@@ -43,6 +43,9 @@ def main():
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-passes", action="store_true", help="skip the five-workload table")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only the plain copy kernel on the workload's input size "
+                         "(hardware-counter and bandwidth calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
@@ -84,6 +87,15 @@ def main():
         return us, time.perf_counter() - t0
 
     w = WORKLOADS[args.workload]
+    if args.calibrate_copy:
+        n = w.N * w.C * w.H * w.W
+        src = torch.randn(n, device="cuda")
+        dst = torch.empty_like(src)
+        us = cp4.time_copy(dst, src, warmup=args.warmup, profcount=args.steps)
+        print(json.dumps({"kernel": "copy_f32x4_kernel", "bytes_read": 4 * n, "bytes_written": 4 * n,
+                          "us_per_launch": round(us, 2),
+                          "GB/s": round(8 * n / us / 1e3, 1)}))
+        return
     host, d = device_inputs(w)
     nbytes = algorithmic_bytes(w)
     us, wall = timed(w, d, args.warmup, args.steps)
