@@ -32,6 +32,8 @@ bool fwd_mfma_supported(const FwdArgs&);
 hipError_t fwd_mfma_launch(const FwdArgs&, hipStream_t);
 bool fwd_split_supported(const FwdArgs&);
 hipError_t fwd_split_launch(const FwdArgs&, hipStream_t);
+bool fwd_pipe_supported(const FwdArgs&);
+hipError_t fwd_pipe_launch(const FwdArgs&, hipStream_t);
 
 // Backward-filter (factor gradients).
 struct BwdFilterArgs {

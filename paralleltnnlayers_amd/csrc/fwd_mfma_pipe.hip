@@ -1,0 +1,495 @@
+// Fused forward / backward-data kernel, producer / consumer form of the
+// split-precision strip kernel (ranks up to 32).
+//
+// Arithmetic and fragments are those of fwd_mfma_split.hip: every fp32 operand
+// is split exactly into three bf16 parts and a product is six bf16 MFMAs
+// accumulated in fp32 (fp32-equivalent accuracy).  What changes is the
+// schedule.  With one strip of TH rows per workgroup the output contraction of
+// a pixel cannot start before the channel contraction of its whole 3x3
+// neighbourhood is done, so a phase-by-phase kernel reads x, then writes y, and
+// HBM never sees both directions at once.  Here the 16 waves take roles:
+//
+//   waves 0-7  producers: the strip (+ halo rows) is swept in rounds of two
+//              32-pixel blocks; in a round wave w works on block (w & 1) of the
+//              pair for channel quarter w >> 1: it streams x (ring of KR
+//              16-channel chunks in flight, refilled across round boundaries),
+//              splits, runs the MFMAs and adds its partial fp32 A[r][q] into
+//              LDS.  The four quarters of a block add in fixed order (an LDS
+//              word per block counts the quarters done), so the sum is
+//              deterministic; the word reaching 4 publishes the block.
+//   waves 8-15 consumers: for each group of 64 output pixels, in sweep order,
+//              wait until the producers have finished every block the group's
+//              taps touch, apply the taps (one wave per rank quad, lane =
+//              pixel), split the result into MFMA B fragments in one of three
+//              rotating LDS tiles and signal an LDS arrival counter; then run
+//              the rank -> output-channel MFMAs for their 32-channel block of
+//              the previous group and store y (float2 per lane).
+//
+// Reads of later blocks therefore overlap the writes of earlier groups.  Odd
+// strips sweep bottom-up, even strips top-down: neighbouring strips then read
+// the halo rows they share at about the same time and the second reader finds
+// them in L2 instead of fetching them from HBM again.
+// All waits are on LDS words written by waves of the same workgroup, which are
+// co-resident by construction: a producer waits only for the lower channel
+// quarters of its own block, consumers wait for producers and for each other's
+// arrivals, nothing waits for a consumer's stores, so every wait is eventually
+// satisfied.  The spins are bounded all the same.
+// Arithmetic follows the reassociated form of
+// Cuda_kernels/cp4Conv2dForward.cu:84-133 (backward-data:
+// cp4Conv2dBackwardData.cu:57-108 through swapped factors and flipped taps).
+#include <cstdlib>
+
+#include "cp4_internal.h"
+
+namespace cp4 {
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 1024;
+constexpr int kProd = 8, kCons = 8;          // producer / consumer waves (4 per SIMD in all)
+constexpr int kRP = 32;
+constexpr int kCcBuf = 24 * 512;             // bytes of one Cc fragment tile (64 pixels)
+constexpr size_t kLdsLimit = 160 * 1024;
+constexpr int kSpinLimit = 1 << 22;
+constexpr int kMaxBlk = 64;                  // per-block progress words in LDS
+
+struct PipePlan {
+  int TH, strips, nWG;
+  int QA;          // LDS row stride of A (floats)
+  int fin_off;     // byte offsets inside LDS
+  int cc_off;
+  int flag_off;
+  size_t lds_bytes;
+#ifdef CP4_DEBUG_PHASES
+  long long* dbg;
+#endif
+};
+
+__device__ __forceinline__ f32x16 mfma16(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                 __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ unsigned pack_hi16(float a, float b) {
+  return __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u);
+}
+__device__ __forceinline__ float trunc_bf16(float v) {
+  return __uint_as_float(__float_as_uint(v) & 0xffff0000u);
+}
+// Exact split of 8 floats into bf16 parts h, m, l (x = h + m + l bit-exactly).
+__device__ __forceinline__ void split8(const float (&v)[8], u32x4& h, u32x4& m, u32x4& l) {
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const float a = v[2 * d], b = v[2 * d + 1];
+    h[d] = pack_hi16(a, b);
+    const float ra = a - trunc_bf16(a), rb = b - trunc_bf16(b);
+    m[d] = pack_hi16(ra, rb);
+    const float sa = ra - trunc_bf16(ra), sb = rb - trunc_bf16(rb);
+    l[d] = pack_hi16(sa, sb);
+  }
+}
+__device__ __forceinline__ f32x16 mfma_split(u32x4 ah, u32x4 am, u32x4 al, u32x4 bh, u32x4 bm,
+                                             u32x4 bl, f32x16 acc) {
+  acc = mfma16(al, bh, acc);
+  acc = mfma16(am, bm, acc);
+  acc = mfma16(ah, bl, acc);
+  acc = mfma16(am, bh, acc);
+  acc = mfma16(ah, bm, acc);
+  acc = mfma16(ah, bh, acc);
+  return acc;
+}
+
+// Wait until *word >= want and return the value seen.  The writer is another
+// wave of this workgroup; the spin is bounded so that a logic error cannot hang
+// the device.
+__device__ __forceinline__ int wait_ge(int* word, int want) {
+  int v = 0;
+  for (int it = 0; it < kSpinLimit; ++it) {
+    v = __hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (v >= want) break;
+    __builtin_amdgcn_s_sleep(1);
+  }
+  return v;
+}
+
+template <int FS, int KR>
+__global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan pl) {
+  extern __shared__ float lds[];
+  float* As = lds;                                                  // [32][QA] fp32
+  unsigned char* ldsb = reinterpret_cast<unsigned char*>(lds);
+  unsigned char* Fb = ldsb + pl.fin_off;     // Fin fragments [chunk][part][hi][r] x 16 B
+  unsigned char* Cb = ldsb + pl.cc_off;      // 3 x Cc fragment tiles
+  // [0..kMaxBlk) quarters done per block (sweep order), then 4 consumer arrival counters
+  int* flags = reinterpret_cast<int*>(ldsb + pl.flag_off);
+
+  const int per = (pl.nWG + 7) >> 3;
+  const int t = (blockIdx.x & 7) * per + (blockIdx.x >> 3);         // XCD-contiguous tile order
+  if (t >= pl.nWG) return;
+  const int n = t / pl.strips, strip = t - n * pl.strips, h0 = strip * pl.TH;
+  const bool rev = strip & 1;                    // odd strips sweep bottom-up
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+#ifdef CP4_DEBUG_PHASES
+#define STAMP(i) if (pl.dbg && lane == 0 && (i) < 32) { pl.dbg[((size_t)t * 16 + wave) * 32 + (i)] = wall_clock64(); }
+#if CP4_DEBUG_PHASES > 1
+#define STAMPX(i) STAMP(i)
+#else
+#define STAMPX(i)
+#endif
+#else
+#define STAMP(i)
+#define STAMPX(i)
+#endif
+  STAMP(0)
+  const int l32 = lane & 31, hi = lane >> 5;
+  const int H = a.H, W = a.W, HW = H * W, R = a.R, Cin = a.Cin, Cout = a.Cout;
+  const int QA = pl.QA;
+  const int rows = min(pl.TH, H - h0);
+  const int nvalid = rows * W;                   // output pixels inside the image
+  const int ngroups = (nvalid + 63) >> 6;
+  const int nkb = (Cout + 31) >> 5;
+  const int qbase = (h0 - a.pad) * W;            // global flat pixel of LDS column 0
+  const int QLEN = (pl.TH + FS - 1) * W;
+  const int nblk = (QLEN + 31) >> 5;             // 32-pixel producer blocks
+  const int nch = Cin >> 4;                      // 16-channel chunks
+
+  // ---- prologue (all waves): flags, Fin -> split -> LDS fragments ----------
+  if (tid < kMaxBlk + 4) flags[tid] = 0;
+  for (int it = tid; it < (Cin >> 3) * 32; it += kThreads) {
+    const int o = it >> 5, r = it & 31;          // channel octet, rank
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = r < R ? a.Fin[(size_t)(8 * o + e) * R + r] : 0.f;
+    u32x4 h, m, l;
+    split8(v, h, m, l);
+    u32x4* dst = reinterpret_cast<u32x4*>(Fb + ((size_t)(o >> 1) * 6 + (o & 1)) * 512 + r * 16);
+    dst[0] = h;          // part stride: 2 planes of 512 B
+    dst[64] = m;
+    dst[128] = l;
+  }
+  __syncthreads();
+  STAMP(1)
+
+  if (wave < kProd) {
+    // =========================== producers ==================================
+    const int bsel = wave & 1, cq = wave >> 1;     // block of the round's pair, channel quarter
+    const int cpq = nch >> 2;                      // 16-channel chunks per quarter
+    const int nrounds = (nblk + 1) >> 1;
+    // lane's channel 16*(cpq*cq + chunk) + 8*hi + e
+    const float* xq = a.x + (size_t)n * Cin * HW + (size_t)(16 * cpq * cq + 8 * hi) * HW;
+    const u32x4* fbase =
+        reinterpret_cast<const u32x4*>(Fb + hi * 512 + l32 * 16) + (size_t)(cq * cpq) * (6 * 32);
+    // Block of round r: sweep index j, LDS column qa of this lane, whether the
+    // lane's pixel exists, and the lane's (clamped, always in-bounds) x pointer.
+    auto geom = [&](int r, int& j, int& qa, bool& valid) -> const float* {
+      j = 2 * r + bsel;
+      const int b = rev ? nblk - 1 - j : j;        // j == nblk happens when nblk is odd
+      qa = 32 * b + l32;
+      const int q = qbase + qa;
+      valid = j < nblk && q >= 0 && q < HW && qa < QLEN;
+      const int qc = q < 0 ? 0 : (q > HW - 1 ? HW - 1 : q);
+      return xq + qc;
+    };
+    auto ld_chunk = [&](float (&dst)[8], const float* xp, int chunk) {   // chunk < cpq
+      const float* base = xp + (size_t)(16 * chunk) * HW;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dst[e] = base[(size_t)e * HW];
+    };
+    float xb[KR][8];
+    int j, qa;
+    bool valid;
+    const float* xp = geom(0, j, qa, valid);
+#pragma unroll
+    for (int u = 0; u < KR; ++u) ld_chunk(xb[u], xp, u);
+    for (int r = 0; r < nrounds; ++r) {
+      int jn, qan;
+      bool validn;
+      const float* xpn = geom(r + 1 < nrounds ? r + 1 : r, jn, qan, validn);
+      f32x16 acc = (f32x16)(0.f);
+      for (int ch = 0; ch < cpq; ch += KR) {
+#pragma unroll
+        for (int u = 0; u < KR; ++u) {
+          const u32x4* fp = fbase + (size_t)(ch + u) * (6 * 32);
+          const u32x4 fh = fp[0], fm = fp[64], fl = fp[128];
+          u32x4 xh, xm, xl;
+          split8(xb[u], xh, xm, xl);
+          acc = mfma_split(fh, fm, fl, xh, xm, xl, acc);
+          // refill this ring slot: same round, or the first chunks of the next
+          const int nxt = ch + u + KR;
+          const bool wrap = nxt >= cpq;
+          ld_chunk(xb[u], wrap ? xpn : xp, wrap ? nxt - cpq : nxt);
+          // keep use-then-refill order per chunk so KR chunks stay in flight
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      if (j < nblk) {
+        // add this quarter's partial sums after the lower quarters
+        int* bf = &flags[j];
+        if (cq > 0) wait_ge(bf, cq);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          float* dst = &As[(8 * (v >> 2) + 4 * hi + (v & 3)) * QA + qa];
+          const float val = valid ? acc[v] : 0.f;
+          *dst = cq == 0 ? val : *dst + val;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        if (lane == 0)
+          __hip_atomic_store(bf, cq + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+      STAMP(2 + r)
+      xp = xpn;
+      j = jn;
+      qa = qan;
+      valid = validn;
+    }
+  } else {
+    // =========================== consumers ==================================
+    const int wc = wave - kProd;                   // 0..7: rank quad in the tap step
+    // Output-factor fragment of this wave's 32-channel block kb = wc (reloaded per
+    // item only when there are more blocks than consumer waves): lane holds row
+    // 32*kb + l32, ranks 16*c + 8*hi + e.
+    u32x4 fkh[2], fkm[2], fkl[2];
+    auto load_fk = [&](int kb) {
+      const int k = 32 * kb + l32;
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int r = 16 * c + 8 * hi + e;
+          v[e] = (k < Cout && r < R) ? a.Fout[(size_t)k * R + r] : 0.f;
+        }
+        split8(v, fkh[c], fkm[c], fkl[c]);
+      }
+    };
+    const bool fk_cached = nkb <= kCons;
+    if (fk_cached && wc < nkb) load_fk(wc);
+    // Tap weights of this wave's 4 ranks (wave-uniform values).
+    float fh[4][FS], fw[4][FS];
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr)
+#pragma unroll
+      for (int j = 0; j < FS; ++j) {
+        const int tap = a.flip ? FS - 1 - j : j, r = 4 * wc + rr;
+        fh[rr][j] = r < R ? a.FH[tap * R + r] : 0.f;
+        fw[rr][j] = r < R ? a.FW[tap * R + r] : 0.f;
+      }
+    float* yn = a.y + (size_t)n * Cout * HW + (size_t)h0 * W;
+    const int reach = (FS - 1) * (W + 1);          // how far past a pixel its taps read in A
+
+    int frontier = 0;                              // blocks [0, frontier) of the sweep are complete
+    int* arrivals = flags + kMaxBlk;               // [4] tap-step arrivals, slot = step & 3
+
+    // Tap step i of the sweep (pixel group g): wait for the producers of every
+    // block the group's taps touch, compute pixel 64*g + lane for ranks 4*wc ..
+    // 4*wc + 3, write the split fragments into fragment tile `cb`, then signal
+    // arrival.
+    auto taps = [&](int i, unsigned char* cb) {
+      const int g = rev ? ngroups - 1 - i : i;
+      {
+        // the taps of pixel p read A columns p - pad .. p + (FS-1)*(W+1) - pad
+        int last = (64 * g + 63 + reach) >> 5;
+        if (last > nblk - 1) last = nblk - 1;
+        const int first = max(64 * g - a.pad, 0) >> 5;
+        const int need = rev ? nblk - 1 - first : last;    // highest sweep index touched
+        while (frontier <= need) {
+          wait_ge(&flags[frontier], 4);
+          ++frontier;
+        }
+      }
+      STAMPX(2 + 4 * i)
+      const int p = 64 * g + lane;
+      const int h = p / W, w = p - h * W;
+      int off[FS];
+      bool in[FS];
+#pragma unroll
+      for (int j = 0; j < FS; ++j) {
+        const int ww = w + j - a.pad;
+        in[j] = ww >= 0 && ww < W;
+        off[j] = ww < 0 ? 0 : (ww >= W ? W - 1 : ww);      // clamped: weight is 0 there
+      }
+      float o[4];
+      const float* ab = As + (size_t)(4 * wc) * QA + h * W;
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        float s = 0.f;
+#pragma unroll
+        for (int ti = 0; ti < FS; ++ti) {
+          float hs = 0.f;
+#pragma unroll
+          for (int j = 0; j < FS; ++j)
+            hs += (in[j] ? fw[rr][j] : 0.f) * ab[rr * QA + ti * W + off[j]];
+          s += fh[rr][ti] * hs;
+        }
+        o[rr] = s;
+        __builtin_amdgcn_sched_barrier(0);       // one rank's LDS reads in flight at a time
+      }
+      // exact split of the four values: two dwords per part
+      u32x2 ph, pm, pl2;
+#pragma unroll
+      for (int d = 0; d < 2; ++d) {
+        const float x0 = o[2 * d], x1 = o[2 * d + 1];
+        ph[d] = pack_hi16(x0, x1);
+        const float r0 = x0 - trunc_bf16(x0), r1 = x1 - trunc_bf16(x1);
+        pm[d] = pack_hi16(r0, r1);
+        pl2[d] = pack_hi16(r0 - trunc_bf16(r0), r1 - trunc_bf16(r1));
+      }
+      // plane ((part*2 + chunk)*2 + hi)*2 + parity, 512 B each; entry lane >> 1;
+      // this quad is the low or high 8 bytes of the 16-byte entry
+      unsigned char* dst = cb + ((((wc >> 2) * 2 + ((wc >> 1) & 1)) * 2 + (lane & 1)) * 512) +
+                           (lane >> 1) * 16 + (wc & 1) * 8;
+      *reinterpret_cast<u32x2*>(dst) = ph;
+      *reinterpret_cast<u32x2*>(dst + 8 * 512) = pm;
+      *reinterpret_cast<u32x2*>(dst + 16 * 512) = pl2;
+      STAMPX(3 + 4 * i)
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      if (lane == 0)
+        __hip_atomic_fetch_add(&arrivals[i & 3], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+
+    // Three fragment tiles in rotation.  Iteration i: once every consumer wave
+    // has arrived for step i (which also means it has finished the contraction
+    // of step i-2, the last reader of the tile written next), do the tap step
+    // i+1, then contract step i.  The arrival of step i was signalled one
+    // contraction earlier, so this wait seldom stalls and the global stores of
+    // consecutive groups follow each other closely.
+    unsigned char* cb_cur = Cb;
+    unsigned char* cb_next = Cb + kCcBuf;
+    unsigned char* cb_free = Cb + 2 * kCcBuf;
+    taps(0, cb_cur);
+    for (int i = 0; i < ngroups; ++i) {
+      const int g = rev ? ngroups - 1 - i : i;
+      wait_ge(&arrivals[i & 3], kCons * ((i >> 2) + 1));
+      STAMPX(4 + 4 * i)
+      if (i + 1 < ngroups) taps(i + 1, cb_next);
+      // ---- rank -> output-channel contraction for this wave's blocks --------
+      const unsigned char* cb = cb_cur;
+      for (int kb = wc; kb < nkb; kb += kCons) {
+        if (!fk_cached) load_fk(kb);
+        f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          const unsigned char* bp = cb + ((c * 2 + hi) * 2) * 512 + l32 * 16;
+          const u32x4 b0h = *reinterpret_cast<const u32x4*>(bp);
+          const u32x4 b1h = *reinterpret_cast<const u32x4*>(bp + 512);
+          const u32x4 b0m = *reinterpret_cast<const u32x4*>(bp + 8 * 512);
+          const u32x4 b1m = *reinterpret_cast<const u32x4*>(bp + 9 * 512);
+          const u32x4 b0l = *reinterpret_cast<const u32x4*>(bp + 16 * 512);
+          const u32x4 b1l = *reinterpret_cast<const u32x4*>(bp + 17 * 512);
+          acc0 = mfma_split(fkh[c], fkm[c], fkl[c], b0h, b0m, b0l, acc0);
+          acc1 = mfma_split(fkh[c], fkm[c], fkl[c], b1h, b1m, b1l, acc1);
+          __builtin_amdgcn_sched_barrier(0);     // one chunk's fragments live at a time
+        }
+        // store rows: uniform row base + one 32-bit lane offset
+        const int p = 64 * g + 2 * l32;
+        if (p < nvalid) {
+          float* rowbase = yn + (size_t)(32 * kb) * HW;
+          const unsigned lofs = (unsigned)(4 * hi * HW + p);
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int kk = 8 * (v >> 2) + (v & 3);             // + 4*hi is in lofs
+            if (32 * kb + kk + 4 * hi < Cout) {
+              float2 o;
+              o.x = acc0[v];
+              o.y = acc1[v];
+              *reinterpret_cast<float2*>(rowbase + (size_t)kk * HW + lofs) = o;
+            }
+          }
+        }
+      }
+      STAMP(5 + 4 * i)
+      unsigned char* tmp = cb_cur;
+      cb_cur = cb_next;
+      cb_next = cb_free;
+      cb_free = tmp;
+    }
+  }
+}
+
+int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+bool layout(const FwdArgs& a, int TH, PipePlan* pl) {
+  const long QLEN = (long)(TH + a.Y - 1) * a.W;
+  // the taps of the last (partly filled) 64-pixel group may read past QLEN
+  const long QA = round_up((int)(round_up(TH * a.W, 64) + (long)(a.Y - 1) * (a.W + 1) + 1), 64) + 8;
+  const size_t a_bytes = (size_t)kRP * QA * sizeof(float);
+  const size_t fin_bytes = (size_t)a.Cin * 192;
+  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 4) * sizeof(int);
+  if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
+  if (bytes > kLdsLimit) return false;
+  pl->TH = TH;
+  pl->strips = (a.H + TH - 1) / TH;
+  pl->nWG = a.N * pl->strips;
+  pl->QA = (int)QA;
+  pl->fin_off = (int)a_bytes;
+  pl->cc_off = (int)(a_bytes + fin_bytes);
+  pl->flag_off = (int)(a_bytes + fin_bytes + 3 * kCcBuf);
+  pl->lds_bytes = bytes;
+  return true;
+}
+
+bool plan(const FwdArgs& a, PipePlan* best) {
+  double best_cost = 0;
+  bool found = false;
+  for (int TH = 1; TH <= a.H; ++TH) {
+    PipePlan pl;
+    if (!layout(a, TH, &pl)) break;
+    const double rounds = (pl.nWG + 255) / 256;
+    const double cost = rounds * ((double)(TH + a.Y - 1) * a.Cin + (double)TH * a.Cout);
+    if (!found || cost < best_cost) {
+      best_cost = cost;
+      *best = pl;
+      found = true;
+    }
+  }
+  return found;
+}
+
+template <int FS, int KR>
+hipError_t launch_as(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
+  const void* fn = reinterpret_cast<const void*>(fwd_pipe_kernel<FS, KR>);
+  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)pl.lds_bytes);
+  if (e != hipSuccess) return e;
+  const unsigned grid = 8u * ((pl.nWG + 7) / 8);
+  fwd_pipe_kernel<FS, KR><<<grid, kThreads, pl.lds_bytes, st>>>(a, pl);
+  return hipGetLastError();
+}
+
+template <int FS>
+hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
+  const int cpq = a.Cin >> 6;                    // 16-channel chunks per channel quarter
+  if (cpq % 4 == 0) return launch_as<FS, 4>(a, pl, st);
+  if (cpq % 2 == 0) return launch_as<FS, 2>(a, pl, st);
+  return launch_as<FS, 1>(a, pl, st);
+}
+
+}  // namespace
+
+bool fwd_pipe_supported(const FwdArgs& a) {
+  if (a.R > kRP || (a.W & 1) || (a.Cin & 63)) return false;
+  if (a.Y != a.X || !(a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7)) return false;
+  if (a.y && (reinterpret_cast<uintptr_t>(a.y) & 7)) return false;
+  PipePlan pl;
+  return plan(a, &pl);
+}
+
+hipError_t fwd_pipe_launch(const FwdArgs& a, hipStream_t st) {
+  PipePlan pl;
+  if (!plan(a, &pl)) return hipErrorInvalidValue;
+#ifdef CP4_DEBUG_PHASES
+  pl.dbg = getenv("CP4_DBG_PTR") ? reinterpret_cast<long long*>(strtoull(getenv("CP4_DBG_PTR"), nullptr, 10)) : nullptr;
+#endif
+  switch (a.Y) {
+    case 1: return launch_fs<1>(a, pl, st);
+    case 3: return launch_fs<3>(a, pl, st);
+    case 5: return launch_fs<5>(a, pl, st);
+    default: return launch_fs<7>(a, pl, st);
+  }
+}
+
+}  // namespace cp4

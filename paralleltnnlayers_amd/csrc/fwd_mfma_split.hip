@@ -39,7 +39,10 @@ typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kThreads = 512, kWaves = kThreads / 64;
 constexpr int kRP = 32;                      // rank padded to one MFMA tile
-constexpr int kRing = 4;                     // 16-channel chunks in flight per lane
+#ifndef CP4_SPLIT_RING
+#define CP4_SPLIT_RING 4
+#endif
+constexpr int kRing = CP4_SPLIT_RING;                     // 16-channel chunks in flight per lane
 constexpr size_t kLdsLimit = 160 * 1024;     // gfx950 LDS per workgroup
 
 struct SplitPlan {
