@@ -2,6 +2,7 @@
 """Benchmark of the fused CP4 Conv2d hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--no-cpu]
+                    [--settle-ms MS]
 
 A step is one launch of the workload's pass (default: the forward pass of the
 ResNet-stage workload N=32, C=K=256, 56x56, 3x3, R=32) on synthetic inputs that
@@ -15,6 +16,12 @@ are already resident in HBM.  Prints ONE JSON line:
   cpu_baseline the CPU oracle's unfused factor-by-factor computation of the same
                workload timed on this box's host cores (a reported baseline)
   passes       mean event-timed microseconds and GB/s of all five workloads
+
+Before the W warm-up launches the headline workload runs untimed for
+--settle-ms milliseconds (default 150): a launch takes ~45 us, and for the first
+~30 ms of back-to-back launches the device's power management is still
+settling (kernel durations rise by 10-20 % and come back down), so a short
+run would time that transient instead of the steady state a training loop sees.
 """
 import argparse
 import json
@@ -41,6 +48,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C3")
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="untimed back-to-back launches of the headline workload for this "
+                         "long before the warm-up, so clocks are at their steady state")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-passes", action="store_true", help="skip the five-workload table")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -65,7 +75,7 @@ def main():
         a = make_inputs(w, seed=0)
         return a, {k: torch.from_numpy(v).cuda() for k, v in a.items()}
 
-    def timed(w, d, warmup, steps):
+    def timed(w, d, warmup, steps, settle_ms=0.0):
         """(event-timed mean us, wall seconds of the same `steps` launches)."""
         f = [d[k] for k in FACTORS]
         if w.pass_ == "forward":
@@ -79,6 +89,9 @@ def main():
             ws = torch.empty(cp4.backward_filter_workspace_bytes(s) // 4 + 1, device="cuda")
             run = lambda wu, k: cp4.time_backward_filter(d["x"], d["dy"], *f, w.pad, wu, k,
                                                          workspace=ws)
+        t_settle = time.perf_counter()
+        while (time.perf_counter() - t_settle) * 1e3 < settle_ms:
+            run(0, 500)
         run(warmup, 1)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -98,7 +111,7 @@ def main():
         return
     host, d = device_inputs(w)
     nbytes = algorithmic_bytes(w)
-    us, wall = timed(w, d, args.warmup, args.steps)
+    us, wall = timed(w, d, args.warmup, args.steps, args.settle_ms)
     value = nbytes * args.steps / wall / 1e9
     achieved = nbytes / us / 1e3
 
@@ -123,7 +136,7 @@ def main():
                 t = us
             else:
                 _, dd = device_inputs(ww)
-                t, _ = timed(ww, dd, 5, 47)     # 47 launches, as the reference's bench drivers
+                t, _ = timed(ww, dd, 5, 47, 30.0)   # 47 launches, as the reference's bench drivers
                 del dd
             b = algorithmic_bytes(ww)
             passes[name] = {"pass": ww.pass_, "us": round(t, 2),

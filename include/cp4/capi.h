@@ -124,7 +124,9 @@ cp4_status cp4_time_backward_filter(const cp4_shape* shape, const float* x,
 /* Replaces the reference's tile heuristic (cp4Conv2dForward.cu:228-233).  The
  * forward / backward-data pass has several kernel variants; variant -1 means
  * "library's choice" (a tuned entry for this shape if cp4_tune_forward has
- * run, else a size heuristic). */
+ * run, else a size heuristic; the environment variable
+ * CP4_FORWARD_VARIANT=<variant name> overrides the heuristic for the shapes
+ * that variant supports). */
 int cp4_forward_variant_count(void);
 const char* cp4_forward_variant_name(int variant);
 /* CP4_OK if `variant` can run `shape`, else CP4_ERR_UNSUPPORTED. */

@@ -94,6 +94,12 @@ int choose_variant(const FwdArgs& a) {
     auto it = g_tuned.find(key_of(a));
     if (it != g_tuned.end()) return it->second;
   }
+  // CP4_FORWARD_VARIANT=<name> overrides the heuristic where that variant can
+  // run the shape (profiling and A/B runs of unmodified callers).
+  if (const char* want = getenv("CP4_FORWARD_VARIANT")) {
+    for (int v = 0; v < kNumVariants; ++v)
+      if (!strcmp(want, kVariants[v].name) && kVariants[v].supported(a)) return v;
+  }
   for (int v = kNumVariants - 1; v >= 0; --v)
     if (kVariants[v].supported(a)) return v;
   return -1;

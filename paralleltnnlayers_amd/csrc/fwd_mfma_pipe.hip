@@ -60,8 +60,7 @@ constexpr int kMaxBlk = 64;                  // per-block progress words in LDS
 struct PipePlan {
   int TH, strips, nWG;
   int QA;          // LDS row stride of A (floats)
-  int fin_off;     // byte offsets inside LDS
-  int cc_off;
+  int cc_off;      // byte offsets inside LDS
   int flag_off;
   size_t lds_bytes;
 #ifdef CP4_DEBUG_PHASES
@@ -115,12 +114,11 @@ __device__ __forceinline__ int wait_ge(int* word, int want) {
   return v;
 }
 
-template <int FS, int KR>
+template <int FS, int CPQ, int KR>
 __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan pl) {
   extern __shared__ float lds[];
   float* As = lds;                                                  // [32][QA] fp32
   unsigned char* ldsb = reinterpret_cast<unsigned char*>(lds);
-  unsigned char* Fb = ldsb + pl.fin_off;     // Fin fragments [chunk][part][hi][r] x 16 B
   unsigned char* Cb = ldsb + pl.cc_off;      // 3 x Cc fragment tiles
   // [0..kMaxBlk) quarters done per block (sweep order), then 4 consumer arrival counters
   int* flags = reinterpret_cast<int*>(ldsb + pl.flag_off);
@@ -145,6 +143,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #define STAMPX(i)
 #endif
   STAMP(0)
+#ifdef CP4_DEBUG_PHASES
+  if (pl.dbg && lane == 0) pl.dbg[((size_t)t * 16 + wave) * 32 + 30] = clock64();
+#endif
   const int l32 = lane & 31, hi = lane >> 5;
   const int H = a.H, W = a.W, HW = H * W, R = a.R, Cin = a.Cin, Cout = a.Cout;
   const int QA = pl.QA;
@@ -157,32 +158,29 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   const int nblk = (QLEN + 31) >> 5;             // 32-pixel producer blocks
   const int nch = Cin >> 4;                      // 16-channel chunks
 
-  // ---- prologue (all waves): flags, Fin -> split -> LDS fragments ----------
+  // ---- prologue: clear the progress words ----------------------------------
   if (tid < kMaxBlk + 4) flags[tid] = 0;
-  for (int it = tid; it < (Cin >> 3) * 32; it += kThreads) {
-    const int o = it >> 5, r = it & 31;          // channel octet, rank
-    float v[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = r < R ? a.Fin[(size_t)(8 * o + e) * R + r] : 0.f;
-    u32x4 h, m, l;
-    split8(v, h, m, l);
-    u32x4* dst = reinterpret_cast<u32x4*>(Fb + ((size_t)(o >> 1) * 6 + (o & 1)) * 512 + r * 16);
-    dst[0] = h;          // part stride: 2 planes of 512 B
-    dst[64] = m;
-    dst[128] = l;
-  }
   __syncthreads();
   STAMP(1)
 
   if (wave < kProd) {
     // =========================== producers ==================================
     const int bsel = wave & 1, cq = wave >> 1;     // block of the round's pair, channel quarter
-    const int cpq = nch >> 2;                      // 16-channel chunks per quarter
+    constexpr int cpq = CPQ;                       // 16-channel chunks per quarter (Cin = 64*CPQ)
     const int nrounds = (nblk + 1) >> 1;
     // lane's channel 16*(cpq*cq + chunk) + 8*hi + e
     const float* xq = a.x + (size_t)n * Cin * HW + (size_t)(16 * cpq * cq + 8 * hi) * HW;
-    const u32x4* fbase =
-        reinterpret_cast<const u32x4*>(Fb + hi * 512 + l32 * 16) + (size_t)(cq * cpq) * (6 * 32);
+    // This wave's slice of the input factor stays in registers for the whole
+    // sweep, already split: lane holds rank l32, channels 16*(cpq*cq+c) + 8*hi + e.
+    u32x4 fh[CPQ], fm[CPQ], fl[CPQ];
+#pragma unroll
+    for (int c = 0; c < CPQ; ++c) {
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        v[e] = l32 < R ? a.Fin[(size_t)(16 * (cpq * cq + c) + 8 * hi + e) * R + l32] : 0.f;
+      split8(v, fh[c], fm[c], fl[c]);
+    }
     // Block of round r: sweep index j, LDS column qa of this lane, whether the
     // lane's pixel exists, and the lane's (clamped, always in-bounds) x pointer.
     auto geom = [&](int r, int& j, int& qa, bool& valid) -> const float* {
@@ -210,18 +208,19 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       bool validn;
       const float* xpn = geom(r + 1 < nrounds ? r + 1 : r, jn, qan, validn);
       f32x16 acc = (f32x16)(0.f);
-      for (int ch = 0; ch < cpq; ch += KR) {
+#pragma unroll
+      for (int ch = 0; ch < CPQ; ch += KR) {
 #pragma unroll
         for (int u = 0; u < KR; ++u) {
-          const u32x4* fp = fbase + (size_t)(ch + u) * (6 * 32);
-          const u32x4 fh = fp[0], fm = fp[64], fl = fp[128];
           u32x4 xh, xm, xl;
           split8(xb[u], xh, xm, xl);
-          acc = mfma_split(fh, fm, fl, xh, xm, xl, acc);
+          acc = mfma_split(fh[ch + u], fm[ch + u], fl[ch + u], xh, xm, xl, acc);
           // refill this ring slot: same round, or the first chunks of the next
           const int nxt = ch + u + KR;
-          const bool wrap = nxt >= cpq;
-          ld_chunk(xb[u], wrap ? xpn : xp, wrap ? nxt - cpq : nxt);
+          if (nxt < CPQ)
+            ld_chunk(xb[u], xp, nxt);
+          else
+            ld_chunk(xb[u], xpn, nxt - CPQ);
           // keep use-then-refill order per chunk so KR chunks stay in flight
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -229,12 +228,25 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       if (j < nblk) {
         // add this quarter's partial sums after the lower quarters
         int* bf = &flags[j];
-        if (cq > 0) wait_ge(bf, cq);
+        float* dst = &As[(4 * hi) * QA + qa];      // row 8*(v>>2) + (v&3) + 4*hi
+        if (cq == 0) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          float* dst = &As[(8 * (v >> 2) + 4 * hi + (v & 3)) * QA + qa];
-          const float val = valid ? acc[v] : 0.f;
-          *dst = cq == 0 ? val : *dst + val;
+          for (int v = 0; v < 16; ++v)
+            dst[(8 * (v >> 2) + (v & 3)) * QA] = valid ? acc[v] : 0.f;
+        } else {
+          wait_ge(bf, cq);
+          // read all, then add, then write all: one LDS round trip per half, not
+          // one per element
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            float old[8];
+#pragma unroll
+            for (int v = 0; v < 8; ++v) old[v] = dst[(8 * ((8 * half + v) >> 2) + (v & 3)) * QA];
+#pragma unroll
+            for (int v = 0; v < 8; ++v)
+              dst[(8 * ((8 * half + v) >> 2) + (v & 3)) * QA] =
+                  old[v] + (valid ? acc[8 * half + v] : 0.f);
+          }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (lane == 0)
@@ -246,9 +258,15 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       qa = qan;
       valid = validn;
     }
+#ifdef CP4_DEBUG_PHASES
+    if (pl.dbg && lane == 0) pl.dbg[((size_t)t * 16 + wave) * 32 + 31] = clock64();
+#endif
   } else {
     // =========================== consumers ==================================
     const int wc = wave - kProd;                   // 0..7: rank quad in the tap step
+#ifdef CP4_PIPE_PRIO
+    __builtin_amdgcn_s_setprio(CP4_PIPE_PRIO);
+#endif
     // Output-factor fragment of this wave's 32-channel block kb = wc (reloaded per
     // item only when there are more blocks than consumer waves): lane holds row
     // 32*kb + l32, ranks 16*c + 8*hi + e.
@@ -284,18 +302,32 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     int frontier = 0;                              // blocks [0, frontier) of the sweep are complete
     int* arrivals = flags + kMaxBlk;               // [4] tap-step arrivals, slot = step & 3
 
-    // Tap step i of the sweep (pixel group g): wait for the producers of every
-    // block the group's taps touch, compute pixel 64*g + lane for ranks 4*wc ..
-    // 4*wc + 3, write the split fragments into fragment tile `cb`, then signal
-    // arrival.
+    // Tap step i of the sweep (pixel group g), `taps` below: wait for the
+    // producers of every block the group's taps touch, compute pixel 64*g + lane
+    // for ranks 4*wc .. 4*wc + 3, write the split fragments into fragment tile
+    // `cb`, then signal arrival.
+    // Highest sweep index among the blocks the taps of step i touch: the taps of
+    // pixel p read A columns p - pad .. p + (FS-1)*(W+1) - pad.
+    auto need_of = [&](int i) {
+      const int g = rev ? ngroups - 1 - i : i;
+      int last = (64 * g + 63 + reach) >> 5;
+      if (last > nblk - 1) last = nblk - 1;
+      const int first = max(64 * g - a.pad, 0) >> 5;
+      return rev ? nblk - 1 - first : last;
+    };
+    // Non-blocking: advance the frontier over finished blocks, say whether step
+    // i could run its taps now.
+    auto ready = [&](int i) {
+      const int need = need_of(i);
+      while (frontier <= need &&
+             __hip_atomic_load(&flags[frontier], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) >= 4)
+        ++frontier;
+      return frontier > need;
+    };
     auto taps = [&](int i, unsigned char* cb) {
       const int g = rev ? ngroups - 1 - i : i;
       {
-        // the taps of pixel p read A columns p - pad .. p + (FS-1)*(W+1) - pad
-        int last = (64 * g + 63 + reach) >> 5;
-        if (last > nblk - 1) last = nblk - 1;
-        const int first = max(64 * g - a.pad, 0) >> 5;
-        const int need = rev ? nblk - 1 - first : last;    // highest sweep index touched
+        const int need = need_of(i);
         while (frontier <= need) {
           wait_ge(&flags[frontier], 4);
           ++frontier;
@@ -354,9 +386,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // Three fragment tiles in rotation.  Iteration i: once every consumer wave
     // has arrived for step i (which also means it has finished the contraction
     // of step i-2, the last reader of the tile written next), do the tap step
-    // i+1, then contract step i.  The arrival of step i was signalled one
-    // contraction earlier, so this wait seldom stalls and the global stores of
-    // consecutive groups follow each other closely.
+    // i+1 and contract step i, in either order.  The arrival of step i was
+    // signalled about one contraction earlier, so this wait seldom stalls.
     unsigned char* cb_cur = Cb;
     unsigned char* cb_next = Cb + kCcBuf;
     unsigned char* cb_free = Cb + 2 * kCcBuf;
@@ -365,7 +396,10 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       const int g = rev ? ngroups - 1 - i : i;
       wait_ge(&arrivals[i & 3], kCons * ((i >> 2) + 1));
       STAMPX(4 + 4 * i)
-      if (i + 1 < ngroups) taps(i + 1, cb_next);
+      // tap step i+1 goes first when its blocks are there (keeps the stores of
+      // consecutive groups close), else after this group's contraction
+      const bool early = i + 1 < ngroups && ready(i + 1);
+      if (early) taps(i + 1, cb_next);
       // ---- rank -> output-channel contraction for this wave's blocks --------
       const unsigned char* cb = cb_cur;
       for (int kb = wc; kb < nkb; kb += kCons) {
@@ -389,19 +423,30 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         if (p < nvalid) {
           float* rowbase = yn + (size_t)(32 * kb) * HW;
           const unsigned lofs = (unsigned)(4 * hi * HW + p);
+          if (32 * kb + 32 <= Cout) {
 #pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int kk = 8 * (v >> 2) + (v & 3);             // + 4*hi is in lofs
-            if (32 * kb + kk + 4 * hi < Cout) {
+            for (int v = 0; v < 16; ++v) {
               float2 o;
               o.x = acc0[v];
               o.y = acc1[v];
-              *reinterpret_cast<float2*>(rowbase + (size_t)kk * HW + lofs) = o;
+              *reinterpret_cast<float2*>(rowbase + (size_t)(8 * (v >> 2) + (v & 3)) * HW + lofs) = o;
+            }
+          } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const int kk = 8 * (v >> 2) + (v & 3);           // + 4*hi is in lofs
+              if (32 * kb + kk + 4 * hi < Cout) {
+                float2 o;
+                o.x = acc0[v];
+                o.y = acc1[v];
+                *reinterpret_cast<float2*>(rowbase + (size_t)kk * HW + lofs) = o;
+              }
             }
           }
         }
       }
       STAMP(5 + 4 * i)
+      if (i + 1 < ngroups && !early) taps(i + 1, cb_next);
       unsigned char* tmp = cb_cur;
       cb_cur = cb_next;
       cb_next = cb_free;
@@ -417,17 +462,15 @@ bool layout(const FwdArgs& a, int TH, PipePlan* pl) {
   // the taps of the last (partly filled) 64-pixel group may read past QLEN
   const long QA = round_up((int)(round_up(TH * a.W, 64) + (long)(a.Y - 1) * (a.W + 1) + 1), 64) + 8;
   const size_t a_bytes = (size_t)kRP * QA * sizeof(float);
-  const size_t fin_bytes = (size_t)a.Cin * 192;
-  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 4) * sizeof(int);
+  const size_t bytes = a_bytes + 3 * kCcBuf + (kMaxBlk + 4) * sizeof(int);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
   pl->strips = (a.H + TH - 1) / TH;
   pl->nWG = a.N * pl->strips;
   pl->QA = (int)QA;
-  pl->fin_off = (int)a_bytes;
-  pl->cc_off = (int)(a_bytes + fin_bytes);
-  pl->flag_off = (int)(a_bytes + fin_bytes + 3 * kCcBuf);
+  pl->cc_off = (int)a_bytes;
+  pl->flag_off = (int)(a_bytes + 3 * kCcBuf);
   pl->lds_bytes = bytes;
   return true;
 }
@@ -449,29 +492,32 @@ bool plan(const FwdArgs& a, PipePlan* best) {
   return found;
 }
 
-template <int FS, int KR>
+template <int FS, int CPQ, int KR>
 hipError_t launch_as(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
-  const void* fn = reinterpret_cast<const void*>(fwd_pipe_kernel<FS, KR>);
+  const void* fn = reinterpret_cast<const void*>(fwd_pipe_kernel<FS, CPQ, KR>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)pl.lds_bytes);
   if (e != hipSuccess) return e;
   const unsigned grid = 8u * ((pl.nWG + 7) / 8);
-  fwd_pipe_kernel<FS, KR><<<grid, kThreads, pl.lds_bytes, st>>>(a, pl);
+  fwd_pipe_kernel<FS, CPQ, KR><<<grid, kThreads, pl.lds_bytes, st>>>(a, pl);
   return hipGetLastError();
 }
 
 template <int FS>
 hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
-  const int cpq = a.Cin >> 6;                    // 16-channel chunks per channel quarter
-  if (cpq % 4 == 0) return launch_as<FS, 4>(a, pl, st);
-  if (cpq % 2 == 0) return launch_as<FS, 2>(a, pl, st);
-  return launch_as<FS, 1>(a, pl, st);
+  switch (a.Cin >> 6) {                          // 16-channel chunks per channel quarter
+    case 1: return launch_as<FS, 1, 1>(a, pl, st);
+    case 2: return launch_as<FS, 2, 2>(a, pl, st);
+    case 3: return launch_as<FS, 3, 1>(a, pl, st);
+    case 4: return launch_as<FS, 4, 2>(a, pl, st);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 }  // namespace
 
 bool fwd_pipe_supported(const FwdArgs& a) {
-  if (a.R > kRP || (a.W & 1) || (a.Cin & 63)) return false;
+  if (a.R > kRP || (a.W & 1) || (a.Cin & 63) || a.Cin > 256) return false;
   if (a.Y != a.X || !(a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7)) return false;
   if (a.y && (reinterpret_cast<uintptr_t>(a.y) & 7)) return false;
   PipePlan pl;
