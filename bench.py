@@ -39,13 +39,13 @@ FACTORS = ("FK", "FC", "FH", "FW")
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs, scaled by the plain copy kernel's reading (see
 # profiles/): {workload: bytes}.  None until measured for the current kernel.
-MEASURED_TRAFFIC = {"C3": 224.6e6}   # fwd_split_kernel<3>: 109.3 MB fetched + 115.4 MB written
+MEASURED_TRAFFIC = {"C3": 224.7e6}   # fwd_pipe_kernel<3,4,2>: 109.8 MB fetched + 114.9 MB written
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--settle-ms", type=float, default=150.0,

@@ -156,7 +156,6 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   const int qbase = (h0 - a.pad) * W;            // global flat pixel of LDS column 0
   const int QLEN = (pl.TH + FS - 1) * W;
   const int nblk = (QLEN + 31) >> 5;             // 32-pixel producer blocks
-  const int nch = Cin >> 4;                      // 16-channel chunks
 
   // ---- prologue: clear the progress words ----------------------------------
   if (tid < kMaxBlk + 4) flags[tid] = 0;

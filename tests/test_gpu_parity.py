@@ -171,6 +171,13 @@ EDGE = [
     (1, 2, 20, 20, 8, 2, 17, 17, 2),      # largest filter of the reference's sweeps
     (4, 40, 16, 16, 1, 72, 3, 3, 48),     # rank above the register block
     (2, 16, 12, 12, 1, 32, 3, 3, 16),     # MFMA-eligible rank, small image
+    # shapes the producer/consumer strip kernels accept (channels a multiple of
+    # 64, even width), sized so that an image needs several strips
+    (2, 64, 40, 50, 1, 40, 3, 3, 7),      # ragged last strip, partial output-channel block
+    (1, 128, 33, 38, 2, 128, 5, 5, 32),   # 5x5, both passes eligible, odd strip count
+    (1, 192, 30, 26, 3, 64, 7, 7, 16),    # 7x7, three chunks per channel quarter
+    (2, 256, 57, 18, 0, 32, 3, 3, 20),    # no padding, tall image
+    (3, 64, 9, 120, 1, 64, 1, 1, 9),      # 1x1 filter, wide rows
 ]
 
 
