@@ -10,7 +10,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB = os.path.join(_HERE, "csrc", "libcp4conv.so")
+# CP4_LIBRARY points at another build of the same library (A/B timing of kernels).
+_LIB = os.environ.get("CP4_LIBRARY") or os.path.join(_HERE, "csrc", "libcp4conv.so")
 
 
 class Cp4Error(RuntimeError):

@@ -343,21 +343,32 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         in[j] = ww >= 0 && ww < W;
         off[j] = ww < 0 ? 0 : (ww >= W ? W - 1 : ww);      // clamped: weight is 0 there
       }
-      float o[4];
+      // the LDS reads of RBT ranks go out together, then their arithmetic
+      constexpr int RBT = FS <= 3 ? 4 : (FS == 5 ? 2 : 1);
       const float* ab = As + (size_t)(4 * wc) * QA + h * W;
+      float o[4];
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        float s = 0.f;
+      for (int r0 = 0; r0 < 4; r0 += RBT) {
+        float av[RBT][FS][FS];
 #pragma unroll
-        for (int ti = 0; ti < FS; ++ti) {
-          float hs = 0.f;
+        for (int rr = 0; rr < RBT; ++rr)
 #pragma unroll
-          for (int j = 0; j < FS; ++j)
-            hs += (in[j] ? fw[rr][j] : 0.f) * ab[rr * QA + ti * W + off[j]];
-          s += fh[rr][ti] * hs;
+          for (int ti = 0; ti < FS; ++ti)
+#pragma unroll
+            for (int j = 0; j < FS; ++j) av[rr][ti][j] = ab[(r0 + rr) * QA + ti * W + off[j]];
+#pragma unroll
+        for (int rr = 0; rr < RBT; ++rr) {
+          float s = 0.f;
+#pragma unroll
+          for (int ti = 0; ti < FS; ++ti) {
+            float hs = 0.f;
+#pragma unroll
+            for (int j = 0; j < FS; ++j) hs += (in[j] ? fw[r0 + rr][j] : 0.f) * av[rr][ti][j];
+            s += fh[r0 + rr][ti] * hs;
+          }
+          o[r0 + rr] = s;
         }
-        o[rr] = s;
-        __builtin_amdgcn_sched_barrier(0);       // one rank's LDS reads in flight at a time
+        if (RBT < 4) __builtin_amdgcn_sched_barrier(0);
       }
       // exact split of the four values: two dwords per part
       u32x2 ph, pm, pl2;
