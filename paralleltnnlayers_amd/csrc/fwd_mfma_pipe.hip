@@ -151,7 +151,11 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   const int QA = pl.QA;
   const int rows = min(pl.TH, H - h0);
   const int nvalid = rows * W;                   // output pixels inside the image
-  const int ngroups = (nvalid + 63) >> 6;
+  // 64-pixel output groups start `gshift` pixels before the strip so that their
+  // boundaries fall on 128-byte lines of y (pixel h0*W + 64*g - gshift is a
+  // multiple of 32); pixels before the strip are computed and not stored.
+  const int gshift = (h0 * W) & 31;
+  const int ngroups = (nvalid + gshift + 63) >> 6;
   const int nkb = (Cout + 31) >> 5;
   const int qbase = (h0 - a.pad) * W;            // global flat pixel of LDS column 0
   const int QLEN = (pl.TH + FS - 1) * W;
@@ -309,9 +313,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // pixel p read A columns p - pad .. p + (FS-1)*(W+1) - pad.
     auto need_of = [&](int i) {
       const int g = rev ? ngroups - 1 - i : i;
-      int last = (64 * g + 63 + reach) >> 5;
+      int last = max(64 * g - gshift + 63 + reach, 0) >> 5;
       if (last > nblk - 1) last = nblk - 1;
-      const int first = max(64 * g - a.pad, 0) >> 5;
+      const int first = max(64 * g - gshift - a.pad, 0) >> 5;
       return rev ? nblk - 1 - first : last;
     };
     // Non-blocking: advance the frontier over finished blocks, say whether step
@@ -333,7 +337,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         }
       }
       STAMPX(2 + 4 * i)
-      const int p = 64 * g + lane;
+      const int p = max(64 * g - gshift + lane, 0);      // lanes before the strip: any valid column
       const int h = p / W, w = p - h * W;
       int off[FS];
       bool in[FS];
@@ -429,8 +433,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           __builtin_amdgcn_sched_barrier(0);     // one chunk's fragments live at a time
         }
         // store rows: uniform row base + one 32-bit lane offset
-        const int p = 64 * g + 2 * l32;
-        if (p < nvalid) {
+        const int p = 64 * g - gshift + 2 * l32;       // even: W is even
+        if (p >= 0 && p < nvalid) {
           float* rowbase = yn + (size_t)(32 * kb) * HW;
           const unsigned lofs = (unsigned)(4 * hi * HW + p);
           if (32 * kb + 32 <= Cout) {
@@ -469,8 +473,10 @@ int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
 bool layout(const FwdArgs& a, int TH, PipePlan* pl) {
   const long QLEN = (long)(TH + a.Y - 1) * a.W;
-  // the taps of the last (partly filled) 64-pixel group may read past QLEN
-  const long QA = round_up((int)(round_up(TH * a.W, 64) + (long)(a.Y - 1) * (a.W + 1) + 1), 64) + 8;
+  // the taps of the last (partly filled) 64-pixel group may read past QLEN; the
+  // groups start up to 31 pixels before the strip, so they end up to 31 + 63 past it
+  const long QA =
+      round_up((int)(round_up(TH * a.W + 31, 64) + (long)(a.Y - 1) * (a.W + 1) + 1), 64) + 8;
   const size_t a_bytes = (size_t)kRP * QA * sizeof(float);
   const size_t bytes = a_bytes + 3 * kCcBuf + (kMaxBlk + 4) * sizeof(int);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
