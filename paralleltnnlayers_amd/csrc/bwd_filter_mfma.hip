@@ -247,6 +247,126 @@ __global__ __launch_bounds__(256) void taps_plane_kernel(
   }
 }
 
+// ---- 2'. the same for small planes: one WAVE per (image, rank) plane -------
+// A plane of at most 256 pixels fits one wave with PP pixels per lane; its four
+// intermediate planes live in a wave-private LDS slice, so there is no
+// workgroup barrier, no idle thread and 4 planes per workgroup.  B and G2 stay
+// on chip: only Cc, G1 and the tap-gradient partials leave the CU.
+template <int FS, int PP>
+__global__ __launch_bounds__(256) void taps_wave_kernel(
+    const float* __restrict__ A, const float* __restrict__ G3, const float* __restrict__ FH,
+    const float* __restrict__ FW, float* __restrict__ Cc, float* __restrict__ G1,
+    float* __restrict__ partH, float* __restrict__ partW, int R, int H, int W, int P,
+    int nplanes) {
+  extern __shared__ float pl[];
+  const int HW = H * W;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int plane = blockIdx.x * 4 + wave;
+  if (plane >= nplanes) return;                   // whole wave; no workgroup barrier below
+  const int r = plane % R, n = plane / R;
+  float* sA = pl + (size_t)wave * 4 * HW;
+  float *sG = sA + HW, *sB = sA + 2 * HW, *sG2 = sA + 3 * HW;
+  const size_t base = (size_t)plane * HW;
+  float fh[FS], fw[FS];
+#pragma unroll
+  for (int i = 0; i < FS; ++i) {
+    fh[i] = FH[i * R + r];
+    fw[i] = FW[i * R + r];
+  }
+  int ph[PP], pw[PP];
+  float g[PP], g2[PP];
+#pragma unroll
+  for (int k = 0; k < PP; ++k) {
+    const int p = lane + 64 * k;
+    ph[k] = p / W;
+    pw[k] = p - ph[k] * W;
+    g[k] = 0.f;
+    if (p < HW) {
+      sA[p] = A[base + p];
+      g[k] = G3[base + p];
+      sG[p] = g[k];
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int k = 0; k < PP; ++k) {
+    const int p = lane + 64 * k, h = ph[k], w = pw[k];
+    float b = 0.f, v = 0.f;
+    if (p < HW) {
+#pragma unroll
+      for (int i = 0; i < FS; ++i) {
+        const int hh = h + i - P, ww = w - i + P;
+        if (hh >= 0 && hh < H) b += fh[i] * sA[hh * W + w];
+        if (ww >= 0 && ww < W) v += fw[i] * sG[h * W + ww];
+      }
+      sB[p] = b;
+      sG2[p] = v;
+    }
+    g2[k] = v;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  float accH[FS], accW[FS];
+#pragma unroll
+  for (int i = 0; i < FS; ++i) accH[i] = accW[i] = 0.f;
+#pragma unroll
+  for (int k = 0; k < PP; ++k) {
+    const int p = lane + 64 * k, h = ph[k], w = pw[k];
+    if (p < HW) {
+      float cc = 0.f, g1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < FS; ++i) {
+        const int ww = w + i - P, hh = h - i + P;
+        if (ww >= 0 && ww < W) cc += fw[i] * sB[h * W + ww];
+        if (hh >= 0 && hh < H) g1 += fh[i] * sG2[hh * W + w];
+        // tap gradients: dFH[i] += G2[p] A[p shifted down by i-P], dFW[i] += G3[p] B[...]
+        const int hv = h + i - P;
+        if (hv >= 0 && hv < H) accH[i] += g2[k] * sA[hv * W + w];
+        if (ww >= 0 && ww < W) accW[i] += g[k] * sB[h * W + ww];
+      }
+      Cc[base + p] = cc;
+      G1[base + p] = g1;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < FS; ++i) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      accH[i] += __shfl_down(accH[i], off, 64);
+      accW[i] += __shfl_down(accW[i], off, 64);
+    }
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int i = 0; i < FS; ++i) {
+      partH[((size_t)n * FS + i) * R + r] = accH[i];
+      partW[((size_t)n * FS + i) * R + r] = accW[i];
+    }
+  }
+}
+
+template <int FS>
+hipError_t launch_taps_wave(const float* A, const float* G3, const BwdFilterArgs& a, float* Cc,
+                            float* G1, float* pH, float* pW, hipStream_t st) {
+  const int HW = a.H * a.W, nplanes = a.N * a.R;
+  const size_t smem = (size_t)4 * 4 * HW * sizeof(float);
+  const unsigned grid = (unsigned)((nplanes + 3) / 4);
+  const int PP = (HW + 63) / 64;
+#define CP4_TW(pp)                                                                            \
+  taps_wave_kernel<FS, pp><<<grid, 256, smem, st>>>(A, G3, a.FH, a.FW, Cc, G1, pH, pW, a.R,  \
+                                                    a.H, a.W, a.pad, nplanes)
+  switch (PP) {
+    case 1: CP4_TW(1); break;
+    case 2: CP4_TW(2); break;
+    case 3: CP4_TW(3); break;
+    default: CP4_TW(4); break;
+  }
+#undef CP4_TW
+  return hipGetLastError();
+}
+
 // ---- 3a. partial[s][d][r] = sum_{p in split s} act[n,d,p] Z[n,r,p] ----------
 struct GradArgs {
   const float* act[2];   // dy, x
@@ -447,7 +567,17 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   if (e != hipSuccess) return e;
   contract_mfma_kernel<<<dim3((c.items + kCW / 64 - 1) / (kCW / 64), 2, p.RP / 32), kCW, smem, st>>>(c);
 
-  if (p.plane_taps) {
+  const bool wave_taps = p.plane_taps && HW <= 256 && a.Y == a.X &&
+                         (a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7);
+  if (wave_taps) {
+    switch (a.Y) {
+      case 1: e = launch_taps_wave<1>(A, G3, a, Cc, G1, pH, pW, st); break;
+      case 3: e = launch_taps_wave<3>(A, G3, a, Cc, G1, pH, pW, st); break;
+      case 5: e = launch_taps_wave<5>(A, G3, a, Cc, G1, pH, pW, st); break;
+      default: e = launch_taps_wave<7>(A, G3, a, Cc, G1, pH, pW, st); break;
+    }
+    if (e != hipSuccess) return e;
+  } else if (p.plane_taps) {
     const size_t tsm = ((size_t)HW * 4 + 5 * (a.Y + a.X)) * sizeof(float);
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(taps_plane_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)tsm);
