@@ -1,15 +1,17 @@
 // cp4_bench_time tensor_file [results_file] [device]
 // The reference's BenchBothTime driver (Cuda_kernels/bench/BenchBothTime.cu):
 // for every unique shape of the list, mean microseconds over 47 forward
-// launches for ranks 1, 2, 4, 8, 16, as CSV.  The reference's first data
-// column is cuDNN's dense convolution; no dense comparator is built here, so
-// that column prints "nan".
+// launches for ranks 1, 2, 4, 8, 16, as CSV.  The first data column is the
+// vendor library's dense convolution (cuDNN in the reference,
+// BenchBothTime.cu:90; MIOpen here through namespace NV); shapes it cannot
+// take (2*pad != Y-1) print "nan".
 #include <cstdlib>
 #include <iomanip>
 
 #include "bench_common.h"
 #include "cp4/capi.h"
 #include "cp4/cp4conv2d.h"
+#include "cp4/nvconv2d.h"
 
 int main(int argc, char** argv) {
   std::ofstream of;
@@ -34,7 +36,11 @@ int main(int argc, char** argv) {
   }
   for (auto& p : shapes) {
     results << p.N << " " << p.C << " " << p.H << " " << p.W << " " << p.pad << " " << p.T << " "
-            << p.Y << " " << p.X << ", nan";
+            << p.Y << " " << p.X << ", ";
+    if (2 * p.pad + 1 == p.Y && p.Y == p.X)
+      results << NV::run_convolution(p, 47).first;
+    else
+      results << "nan";
     for (unsigned r = 1; r <= 16; r *= 2) {
       p.Rank = r;
       results << ", " << CP::run_convolution(p, 47).first;

@@ -15,8 +15,8 @@ def L():
     return capi.lib()
 
 
-def declared_functions():
-    text = open(os.path.join(ROOT, "include", "cp4", "capi.h")).read()
+def declared_functions(header="capi.h"):
+    text = open(os.path.join(ROOT, "include", "cp4", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(cp4_[a-z0-9_]+)\s*\(", text)))
 
@@ -33,6 +33,24 @@ def test_header_declares_the_three_passes():
 @pytest.mark.parametrize("name", declared_functions())
 def test_symbol_exported(L, name):
     assert getattr(L, name) is not None
+
+
+@pytest.mark.parametrize("name", declared_functions("dense.h"))
+def test_dense_symbol_exported(name):
+    """libcp4dense.so (MIOpen comparator) loads without a GPU and exports what
+    include/cp4/dense.h declares."""
+    from paralleltnnlayers_amd import dense
+    assert getattr(dense.lib(), name) is not None
+
+
+def test_dense_argument_errors_need_no_device():
+    from paralleltnnlayers_amd import capi, dense
+    D = dense.lib()
+    one = ctypes.c_void_p(16)   # never dereferenced: checks fail first
+    assert D.cp4_dense_conv2d_forward(None, one, one, one, None) == capi.ERR_NULL_POINTER
+    valid = capi.Shape(N=1, H=4, W=4, pad=0, T=2, C=2, Y=3, X=3, Rank=0)
+    assert D.cp4_dense_conv2d_forward(ctypes.byref(valid), one, one, one, None) == capi.ERR_SHAPE
+    assert b"2*pad" in D.cp4_dense_last_error_message()
 
 
 def test_shape_struct_matches_reference_order():
