@@ -1,0 +1,81 @@
+"""PyTorch autograd binding of the fused CP4 Conv2d C ABI.
+
+Stands where the reference registers its TensorFlow custom op
+(Kernels/cp4_conv_nchw.cc:6-108, ``Cp4Conv2dNchw``: input + four factor
+tensors -> output, NCHW): a ``torch.autograd.Function`` whose forward, input
+gradient and factor gradients are the three passes of ``libcp4conv.so``.
+PyTorch only owns the tensors and the stream; all arithmetic is in the HIP
+library, and there is no eager fallback.
+
+Factor layout is the C ABI's: FK [T,R], FC [C,R], FH [Y,R], FW [X,R].
+Gradients are exact for "same" padding (2*pad = Y-1 = X-1), the only case in
+which the reference's backward-data formula (flipped taps at offset +y-pad,
+Cuda_kernels/cp4Conv2dBackwardData.cu:79-87) is the adjoint of its forward;
+other paddings are refused for autograd use.
+"""
+import torch
+
+from . import capi
+
+
+class CP4Conv2dFunction(torch.autograd.Function):
+    """y = cp4conv2d(x, FK, FC, FH, FW, pad)."""
+
+    @staticmethod
+    def forward(ctx, x, FK, FC, FH, FW, pad):
+        if 2 * pad + 1 != FH.shape[0] or 2 * pad + 1 != FW.shape[0]:
+            raise ValueError("autograd binding needs 2*pad = Y-1 = X-1 (the reference's "
+                             "backward-data pass is the adjoint only then)")
+        x, FK, FC, FH, FW = (t.contiguous().float() for t in (x, FK, FC, FH, FW))
+        ctx.pad = pad
+        ctx.save_for_backward(x, FK, FC, FH, FW)
+        return capi.conv2d_forward(x, FK, FC, FH, FW, pad=pad)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, FK, FC, FH, FW = ctx.saved_tensors
+        dy = dy.contiguous().float()
+        dx = None
+        if ctx.needs_input_grad[0]:
+            dx = capi.conv2d_backward_data(dy, FK, FC, FH, FW, pad=ctx.pad)
+        grads = (None, None, None, None)
+        if any(ctx.needs_input_grad[1:5]):
+            grads = capi.conv2d_backward_filter(x, dy, FK, FC, FH, FW, pad=ctx.pad)
+            grads = tuple(g if need else None
+                          for g, need in zip(grads, ctx.needs_input_grad[1:5]))
+        return (dx,) + grads + (None,)
+
+
+def cp4_conv2d(x, FK, FC, FH, FW, pad):
+    """Functional form: differentiable fused CP4 convolution (NCHW, stride 1)."""
+    return CP4Conv2dFunction.apply(x, FK, FC, FH, FW, pad)
+
+
+class CP4Conv2d(torch.nn.Module):
+    """A rank-R CP4-decomposed convolution layer, "same" padding, stride 1.
+
+    Equivalent dense filter: K[t,c,y,x] = sum_r FK[t,r] FC[c,r] FH[y,r] FW[x,r]
+    (Cuda_kernels/Utils.cu:55-62).  Factors start as normal(0, s) with s chosen
+    so that the recomposed filter has the variance of a Kaiming-normal dense
+    filter of the same shape.
+    """
+
+    def __init__(self, in_channels, out_channels, kernel_size, rank, device="cuda"):
+        super().__init__()
+        if kernel_size % 2 != 1:
+            raise ValueError("kernel_size must be odd (same padding)")
+        self.pad = kernel_size // 2
+        fan_in = in_channels * kernel_size * kernel_size
+        # Var[K] = R * s^8 for four independent N(0, s^2) factors; target 2 / fan_in
+        s = (2.0 / (fan_in * rank)) ** 0.125
+        mk = lambda d: torch.nn.Parameter(torch.randn(d, rank, device=device) * s)
+        self.FK, self.FC = mk(out_channels), mk(in_channels)
+        self.FH, self.FW = mk(kernel_size), mk(kernel_size)
+
+    def forward(self, x):
+        return cp4_conv2d(x, self.FK, self.FC, self.FH, self.FW, self.pad)
+
+    def dense_filter(self):
+        """The recomposed [T,C,Y,X] filter (on the device, through cp4_recompose)."""
+        return capi.recompose(self.FK.detach(), self.FC.detach(), self.FH.detach(),
+                              self.FW.detach())

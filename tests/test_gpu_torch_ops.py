@@ -1,0 +1,88 @@
+"""The autograd binding (replacement of the reference's TF custom-op boundary,
+Kernels/cp4_conv_nchw.cc:6-108) against PyTorch's own dense convolution on the
+recomposed filter: forward values and all five gradients."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    import paralleltnnlayers_amd as p
+    p.lib()
+    from paralleltnnlayers_amd import torch_ops
+    return torch_ops
+
+
+def recomposed(FK, FC, FH, FW):
+    return torch.einsum("tr,cr,yr,xr->tcyx", FK, FC, FH, FW)
+
+
+@pytest.mark.parametrize("dims", [(2, 16, 12, 14, 24, 3, 8), (1, 64, 20, 20, 64, 5, 16),
+                                  (3, 5, 9, 9, 7, 1, 3)],
+                         ids=lambda d: "x".join(map(str, d)))
+def test_gradients_match_dense_autograd(ops, dims):
+    N, C, H, W, T, Y, R = dims
+    g = torch.Generator(device="cuda").manual_seed(sum(dims))
+    mk = lambda *s: torch.randn(*s, device="cuda", generator=g)
+    x = mk(N, C, H, W).requires_grad_()
+    fac = [(mk(d, R) / R ** 0.25).requires_grad_() for d in (T, C, Y, Y)]
+    dy = mk(N, T, H, W)
+    y = ops.cp4_conv2d(x, *fac, Y // 2)
+    y.backward(dy)
+    got = [x.grad.clone()] + [f.grad.clone() for f in fac]
+
+    # float64 dense reference through PyTorch autograd on the recomposed filter
+    xd = x.detach().double().requires_grad_()
+    fd = [f.detach().double().requires_grad_() for f in fac]
+    yd = torch.nn.functional.conv2d(xd, recomposed(*fd), padding=Y // 2)
+    yd.backward(dy.double())
+    want = [xd.grad] + [f.grad for f in fd]
+    assert (y.detach().double() - yd.detach()).abs().max() <= 1e-4 * yd.detach().abs().max()
+    for name, a, b in zip(("dx", "dFK", "dFC", "dFH", "dFW"), got, want):
+        tol = 1e-4 if name == "dx" else 1e-3
+        assert (a.double() - b).abs().max() <= tol * b.abs().max(), name
+
+
+def test_only_requested_gradients(ops):
+    x = torch.randn(1, 8, 6, 6, device="cuda")
+    fac = [torch.randn(d, 4, device="cuda") for d in (8, 8, 3, 3)]
+    fac[0].requires_grad_()
+    ops.cp4_conv2d(x, *fac, 1).sum().backward()
+    assert fac[0].grad is not None and all(f.grad is None for f in fac[1:]) and x.grad is None
+
+
+def test_non_same_padding_is_refused(ops):
+    x = torch.randn(1, 8, 6, 6, device="cuda")
+    fac = [torch.randn(d, 4, device="cuda") for d in (8, 8, 3, 3)]
+    with pytest.raises(ValueError):
+        ops.cp4_conv2d(x, *fac, 0)
+
+
+def test_layer_trains(ops):
+    """A few SGD steps on a CP4Conv2d layer lower a regression loss: forward,
+    both backward passes and the optimizer see consistent tensors."""
+    torch.manual_seed(0)
+    layer = ops.CP4Conv2d(16, 16, 3, rank=8)
+    target = ops.CP4Conv2d(16, 16, 3, rank=8)
+    x = torch.randn(4, 16, 10, 10, device="cuda")
+    with torch.no_grad():
+        want = target(x)
+    opt = torch.optim.SGD(layer.parameters(), lr=0.05)
+    losses = []
+    for _ in range(30):
+        opt.zero_grad()
+        loss = ((layer(x) - want) ** 2).mean()
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+    assert losses[-1] < 0.7 * losses[0]
+    K = layer.dense_filter()
+    assert K.shape == (16, 16, 3, 3)
+    dense = torch.nn.functional.conv2d(x, K, padding=1)
+    assert (layer(x).detach() - dense).abs().max() <= 1e-4 * dense.abs().max()
