@@ -14,11 +14,12 @@
 //      plus the small tap gradients;
 //   4. fixed-order sum of the per-workgroup partials (bit-reproducible).
 #include "cp4_internal.h"
+#include "split_bf16.h"
 
 namespace cp4 {
 namespace {
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
+using split::f32x16;
 
 __device__ __forceinline__ f32x16 mfma32(float a, float b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
@@ -107,6 +108,118 @@ __global__ __launch_bounds__(kCW) void contract_mfma_kernel(ContractArgs a) {
         o.y = acc1[v];
         *reinterpret_cast<float2*>(zn + (size_t)r * HW) = o;
       }
+    }
+  }
+}
+
+// ---- 1'. the same contraction as exact fp32 products on the bf16 matrix cores
+// (channel counts that are multiples of 16).  A workgroup of 8 waves shares the
+// 32-rank factor tile as pre-split MFMA A fragments in LDS
+// ([16-channel chunk][part][half][rank] x 16 B); a wave owns one (image,
+// 32-pixel block): it streams x / dy through a register ring as the B operand,
+// splits each 16-channel chunk and issues six bf16 MFMAs for it - 2.7x less
+// matrix time than the fp32 MFMA and twice as many waves to hide latency with.
+constexpr int kSplitRing = 4;
+constexpr int kSW = 512;    // 8 waves share one factor tile: one fill per 8 items
+__global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
+  using namespace split;
+  extern __shared__ float Fs[];
+  unsigned char* Fb = reinterpret_cast<unsigned char*>(Fs);
+  const int which = blockIdx.y, mb = blockIdx.z;
+  const int Cin = a.Cin[which], R = a.R, HW = a.HW;
+  const float* F = a.F[which];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hi = lane >> 5;
+  // This wave's item; waves past the end keep a valid (clamped) item for their
+  // loads and skip the store, so that every wave reaches the barrier.
+  const int item_raw = blockIdx.x * (kSW / 64) + wave;    // (image, 32-pixel block)
+  const bool has_item = item_raw < a.items;
+  const int item = has_item ? item_raw : a.items - 1;
+  const int pb = item % a.npb, n = item / a.npb;
+  const int p = pb * 32 + l32;
+  const bool valid = has_item && p < HW;
+  const int pc = p < HW ? p : HW - 1;
+  // lane's channel 16*chunk + 8*hi + e
+  const float* xp = a.src[which] + ((size_t)n * Cin + 8 * hi) * HW + pc;
+  const int nch = Cin >> 4;
+  float xb[kSplitRing][8];
+  auto ld_chunk = [&](float (&dst)[8], int ch) {
+    ch = ch < nch ? ch : nch - 1;                     // clamped, not branched
+    const float* base = xp + (size_t)(16 * ch) * HW;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dst[e] = base[(size_t)e * HW];
+  };
+  // the first activation chunks are requested before the factor tile is built,
+  // so their HBM latency runs under the fill
+#pragma unroll
+  for (int u = 0; u < kSplitRing; ++u) ld_chunk(xb[u], u);
+  for (int it = tid; it < (Cin >> 3) * 32; it += kSW) {
+    const int o = it >> 5, r = 32 * mb + (it & 31);   // channel octet, rank
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = r < R ? F[(size_t)(8 * o + e) * R + r] : 0.f;
+    u32x4 h, m, l;
+    split8(v, h, m, l);
+    u32x4* dst =
+        reinterpret_cast<u32x4*>(Fb + ((size_t)(o >> 1) * 6 + (o & 1)) * 512 + (it & 31) * 16);
+    dst[0] = h;          // part stride: 2 planes of 512 B
+    dst[64] = m;
+    dst[128] = l;
+  }
+  __syncthreads();
+  const u32x4* fbase = reinterpret_cast<const u32x4*>(Fb + hi * 512 + l32 * 16);
+  // Software pipeline: while the six MFMAs of chunk c run (two accumulators, so
+  // they do not wait for each other), the vector ALU splits chunk c+1.
+  f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
+  u32x4 xh, xm, xl;
+  split8(xb[0], xh, xm, xl);
+  ld_chunk(xb[0], kSplitRing);
+  for (int ch = 0; ch < nch; ch += kSplitRing) {
+#pragma unroll
+    for (int u = 0; u < kSplitRing; ++u) {
+      const int c = ch + u;                           // chunk whose parts are in xh/xm/xl
+      u32x4 nh = xh, nm = xm, nl = xl;
+      if (c < nch) {
+        const u32x4* fp = fbase + (size_t)c * (6 * 32);
+        const u32x4 fh = fp[0], fm = fp[64], fl = fp[128];
+        // one MFMA, then a quarter of the next chunk's split, pinned in this order
+        float (&nx)[8] = xb[(u + 1) % kSplitRing];
+        auto piece = [&](int d) {
+          const float x0 = nx[2 * d], x1 = nx[2 * d + 1];
+          nh[d] = pack_hi16(x0, x1);
+          const float r0 = x0 - trunc_bf16(x0), r1 = x1 - trunc_bf16(x1);
+          nm[d] = pack_hi16(r0, r1);
+          nl[d] = pack_hi16(r0 - trunc_bf16(r0), r1 - trunc_bf16(r1));
+        };
+        acc0 = mfma16(fl, xh, acc0);
+        piece(0);
+        __builtin_amdgcn_sched_barrier(0);
+        acc1 = mfma16(fm, xm, acc1);
+        piece(1);
+        __builtin_amdgcn_sched_barrier(0);
+        acc0 = mfma16(fh, xl, acc0);
+        piece(2);
+        __builtin_amdgcn_sched_barrier(0);
+        acc1 = mfma16(fm, xh, acc1);
+        piece(3);
+        __builtin_amdgcn_sched_barrier(0);
+        acc0 = mfma16(fh, xm, acc0);
+        acc1 = mfma16(fh, xh, acc1);
+        ld_chunk(nx, c + 1 + kSplitRing);             // refill the slot just split
+      }
+      xh = nh;
+      xm = nm;
+      xl = nl;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  f32x16 acc = acc0 + acc1;
+  if (valid) {
+    float* zn = a.Z[which] + (size_t)n * R * HW + p;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int r = 32 * mb + 8 * (v >> 2) + 4 * hi + (v & 3);
+      if (r < R) zn[(size_t)r * HW] = acc[v];
     }
   }
 }
@@ -561,11 +674,26 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   c.src[1] = a.dy; c.F[1] = a.FK; c.Z[1] = G3; c.Cin[1] = a.T;
   c.N = N; c.R = R; c.RP = p.RP; c.HW = HW; c.npb = p.npb;
   c.items = N * p.npb;
-  const size_t smem = (size_t)(a.C > a.T ? a.C : a.T) * 32 * sizeof(float);
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_mfma_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-  if (e != hipSuccess) return e;
-  contract_mfma_kernel<<<dim3((c.items + kCW / 64 - 1) / (kCW / 64), 2, p.RP / 32), kCW, smem, st>>>(c);
+  const int cmax = a.C > a.T ? a.C : a.T;
+  hipError_t e;
+  if ((a.C & 15) == 0 && (a.T & 15) == 0 && (size_t)cmax * 192 <= 160 * 1024) {
+    // exact split products: 32-pixel blocks, fragments of 6 bytes per factor entry
+    c.npb = (HW + 31) / 32;
+    c.items = N * c.npb;
+    const size_t smem = (size_t)cmax * 192;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_split_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    contract_split_kernel<<<dim3((c.items + kSW / 64 - 1) / (kSW / 64), 2, p.RP / 32), kSW, smem,
+                            st>>>(c);
+  } else {
+    const size_t smem = (size_t)cmax * 32 * sizeof(float);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_mfma_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    contract_mfma_kernel<<<dim3((c.items + kCW / 64 - 1) / (kCW / 64), 2, p.RP / 32), kCW, smem,
+                           st>>>(c);
+  }
 
   const bool wave_taps = p.plane_taps && HW <= 256 && a.Y == a.X &&
                          (a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7);
