@@ -265,6 +265,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         fw[rr][j] = r < R ? a.FW[tap * R + r] : 0.f;
       }
     float* yn = a.y + (size_t)n * Cout * HW + (size_t)h0 * W;
+    const bool pair_stores =
+        ((W | HW) & 1) == 0 && (reinterpret_cast<uintptr_t>(a.y) & 7) == 0;   // float2 stores legal
     const int reach = (FS - 1) * (W + 1);          // how far past a pixel its taps read in A
 
     int frontier = 0;                              // blocks [0, frontier) of the sweep are complete
@@ -398,28 +400,44 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           __builtin_amdgcn_sched_barrier(0);     // one chunk's fragments live at a time
         }
         // store rows: uniform row base + one 32-bit lane offset
-        const int p = 64 * g - gshift + 2 * l32;       // even: W is even
-        if (p >= 0 && p < nvalid) {
-          float* rowbase = yn + (size_t)(32 * kb) * HW;
-          const unsigned lofs = (unsigned)(4 * hi * HW + p);
-          if (32 * kb + 32 <= Cout) {
+        const int p = 64 * g - gshift + 2 * l32;       // lane's pixel pair p, p + 1
+        float* rowbase = yn + (size_t)(32 * kb) * HW;
+        if (pair_stores) {
+          // W and H*W even, y 8-byte aligned: p is even and the pair is one store
+          if (p >= 0 && p < nvalid) {
+            const unsigned lofs = (unsigned)(4 * hi * HW + p);
+            if (32 * kb + 32 <= Cout) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-              float2 o;
-              o.x = acc0[v];
-              o.y = acc1[v];
-              *reinterpret_cast<float2*>(rowbase + (size_t)(8 * (v >> 2) + (v & 3)) * HW + lofs) = o;
-            }
-          } else {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-              const int kk = 8 * (v >> 2) + (v & 3);           // + 4*hi is in lofs
-              if (32 * kb + kk + 4 * hi < Cout) {
+              for (int v = 0; v < 16; ++v) {
                 float2 o;
                 o.x = acc0[v];
                 o.y = acc1[v];
-                *reinterpret_cast<float2*>(rowbase + (size_t)kk * HW + lofs) = o;
+                *reinterpret_cast<float2*>(rowbase + (size_t)(8 * (v >> 2) + (v & 3)) * HW + lofs) = o;
               }
+            } else {
+#pragma unroll
+              for (int v = 0; v < 16; ++v) {
+                const int kk = 8 * (v >> 2) + (v & 3);         // + 4*hi is in lofs
+                if (32 * kb + kk + 4 * hi < Cout) {
+                  float2 o;
+                  o.x = acc0[v];
+                  o.y = acc1[v];
+                  *reinterpret_cast<float2*>(rowbase + (size_t)kk * HW + lofs) = o;
+                }
+              }
+            }
+          }
+        } else {
+          // odd widths or planes: the two pixels are stored and bounded one by one
+          const bool in0 = p >= 0 && p < nvalid, in1 = p + 1 >= 0 && p + 1 < nvalid;
+          const long lofs = (long)(4 * hi) * HW + p;
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int kk = 8 * (v >> 2) + (v & 3);
+            if (32 * kb + kk + 4 * hi < Cout) {
+              float* rp = rowbase + (size_t)kk * HW + lofs;
+              if (in0) rp[0] = acc0[v];
+              if (in1) rp[1] = acc1[v];
             }
           }
         }
@@ -498,9 +516,8 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 }  // namespace
 
 bool fwd_pipe_supported(const FwdArgs& a) {
-  if (a.R > kRP || (a.W & 1) || (a.Cin & 63) || a.Cin > 256) return false;
+  if (a.R > kRP || (a.Cin & 63) || a.Cin > 256) return false;
   if (a.Y != a.X || !(a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7)) return false;
-  if (a.y && (reinterpret_cast<uintptr_t>(a.y) & 7)) return false;
   PipePlan pl;
   return plan(a, &pl);
 }

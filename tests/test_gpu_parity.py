@@ -178,6 +178,11 @@ EDGE = [
     (1, 192, 30, 26, 3, 64, 7, 7, 16),    # 7x7, three chunks per channel quarter
     (2, 256, 57, 18, 0, 32, 3, 3, 20),    # no padding, tall image
     (3, 64, 9, 120, 1, 64, 1, 1, 9),      # 1x1 filter, wide rows
+    # odd widths on the matrix-core path (the reference's AlexNet layers 3-5,
+    # Cuda_kernels/bench/tensors_alexnet.txt): per-pixel stores, 12 output blocks
+    (1, 192, 13, 13, 1, 384, 3, 3, 16),
+    (1, 256, 27, 27, 1, 384, 3, 3, 8),
+    (2, 64, 9, 11, 2, 40, 5, 5, 5),
 ]
 
 
