@@ -33,7 +33,7 @@ FilterGradients Conv2dBackwardFilter(Tensor const& dLdO, Tensor const& In, Tenso
                                      unsigned pad = 1);
 
 // Cuda_kernels/cp4Conv2d.cu:158-190: device buffers of the given shape
-// (contents unspecified), PROFCOUNT timed forward launches; returns
+// (contents unspecified), one untimed then PROFCOUNT timed forward launches; returns
 // {mean microseconds, algorithmic bytes 4*(N*T*H*W + N*C*H*W + Rank*(T+C+X+Y))}.
 std::pair<float, unsigned> run_convolution(tensor_shape, unsigned PROFCOUNT = 1);
 

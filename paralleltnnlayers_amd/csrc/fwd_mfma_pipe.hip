@@ -79,7 +79,7 @@ __device__ __forceinline__ int wait_ge(int* word, int want) {
   return v;
 }
 
-template <int FS, int CPQ, int KR>
+template <int FS, int CPQ, int KR, bool PAD>
 __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan pl) {
   extern __shared__ float lds[];
   float* As = lds;                                                  // [32][QA] fp32
@@ -134,10 +134,12 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   if (wave < kProd) {
     // =========================== producers ==================================
     const int bsel = wave & 1, cq = wave >> 1;     // block of the round's pair, channel quarter
-    constexpr int cpq = CPQ;                       // 16-channel chunks per quarter (Cin = 64*CPQ)
+    constexpr int cpq = CPQ;                       // 16-channel chunks per quarter (Cin <= 64*CPQ)
     const int nrounds = (nblk + 1) >> 1;
     // lane's channel 16*(cpq*cq + chunk) + 8*hi + e
-    const float* xq = a.x + (size_t)n * Cin * HW + (size_t)(16 * cpq * cq + 8 * hi) * HW;
+    // (PAD: Cin is not a multiple of 64; channel groups past Cin read group 0 and count as zero)
+    const int cg0 = 16 * cpq * cq + 8 * hi;        // lane's first channel of chunk 0
+    const float* xq = a.x + (size_t)n * Cin * HW + (size_t)cg0 * HW;
     // This wave's slice of the input factor stays in registers for the whole
     // sweep, already split: lane holds rank l32, channels 16*(cpq*cq+c) + 8*hi + e.
     u32x4 fh[CPQ], fm[CPQ], fl[CPQ];
@@ -146,7 +148,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       float v[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e)
-        v[e] = l32 < R ? a.Fin[(size_t)(16 * (cpq * cq + c) + 8 * hi + e) * R + l32] : 0.f;
+        v[e] = (l32 < R && (!PAD || cg0 + 16 * c < Cin))
+                   ? a.Fin[(size_t)(cg0 + 16 * c + e) * R + l32]
+                   : 0.f;
       split8(v, fh[c], fm[c], fl[c]);
     }
     // Block of round r: sweep index j, LDS column qa of this lane, whether the
@@ -161,9 +165,13 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       return xq + qc;
     };
     auto ld_chunk = [&](float (&dst)[8], const float* xp, int chunk) {   // chunk < cpq
-      const float* base = xp + (size_t)(16 * chunk) * HW;
+      const bool ok = !PAD || cg0 + 16 * chunk < Cin;
+      const float* base = ok ? xp + (size_t)(16 * chunk) * HW : xp - (size_t)cg0 * HW;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) dst[e] = base[(size_t)e * HW];
+      for (int e = 0; e < 8; ++e) {
+        const float v = base[(size_t)e * HW];
+        dst[e] = ok ? v : 0.f;
+      }
     };
     float xb[KR][8];
     int j, qa;
@@ -491,32 +499,37 @@ bool plan(const FwdArgs& a, PipePlan* best) {
   return found;
 }
 
-template <int FS, int CPQ, int KR>
+template <int FS, int CPQ, int KR, bool PAD>
 hipError_t launch_as(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
-  const void* fn = reinterpret_cast<const void*>(fwd_pipe_kernel<FS, CPQ, KR>);
+  const void* fn = reinterpret_cast<const void*>(fwd_pipe_kernel<FS, CPQ, KR, PAD>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)pl.lds_bytes);
   if (e != hipSuccess) return e;
   const unsigned grid = 8u * ((pl.nWG + 7) / 8);
-  fwd_pipe_kernel<FS, CPQ, KR><<<grid, kThreads, pl.lds_bytes, st>>>(a, pl);
+  fwd_pipe_kernel<FS, CPQ, KR, PAD><<<grid, kThreads, pl.lds_bytes, st>>>(a, pl);
   return hipGetLastError();
+}
+
+template <int FS, bool PAD>
+hipError_t launch_cpq(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
+  switch ((a.Cin + 63) >> 6) {                   // 16-channel chunks per channel quarter
+    case 1: return launch_as<FS, 1, 1, PAD>(a, pl, st);
+    case 2: return launch_as<FS, 2, 2, PAD>(a, pl, st);
+    case 3: return launch_as<FS, 3, 1, PAD>(a, pl, st);
+    case 4: return launch_as<FS, 4, 2, PAD>(a, pl, st);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 template <int FS>
 hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
-  switch (a.Cin >> 6) {                          // 16-channel chunks per channel quarter
-    case 1: return launch_as<FS, 1, 1>(a, pl, st);
-    case 2: return launch_as<FS, 2, 2>(a, pl, st);
-    case 3: return launch_as<FS, 3, 1>(a, pl, st);
-    case 4: return launch_as<FS, 4, 2>(a, pl, st);
-    default: return hipErrorInvalidValue;
-  }
+  return (a.Cin & 63) ? launch_cpq<FS, true>(a, pl, st) : launch_cpq<FS, false>(a, pl, st);
 }
 
 }  // namespace
 
 bool fwd_pipe_supported(const FwdArgs& a) {
-  if (a.R > kRP || (a.Cin & 63) || a.Cin > 256) return false;
+  if (a.R > kRP || (a.Cin & 7) || a.Cin > 256) return false;
   if (a.Y != a.X || !(a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7)) return false;
   PipePlan pl;
   return plan(a, &pl);

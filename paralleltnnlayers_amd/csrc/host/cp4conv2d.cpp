@@ -265,6 +265,10 @@ std::pair<float, unsigned> run_convolution(tensor_shape p, unsigned PROFCOUNT) {
   const unsigned mem = (unsigned)(sizeof(float) * ((size_t)p.N * p.T * p.H * p.W +
                                                    (size_t)p.N * p.C * p.H * p.W +
                                                    (size_t)p.Rank * (p.T + p.C + p.X + p.Y)));
+  // one untimed launch first: the first use of a kernel loads its code object
+  // (about a millisecond), which is not launch time
+  (void)cp4_conv2d_forward_gpu(p, (float*)buf[0], (float*)buf[1], (float*)buf[2], (float*)buf[3],
+                               (float*)buf[4], (float*)buf[5], 1);
   const float us =
       cp4_conv2d_forward_gpu(p, (float*)buf[0], (float*)buf[1], (float*)buf[2], (float*)buf[3],
                              (float*)buf[4], (float*)buf[5], PROFCOUNT);

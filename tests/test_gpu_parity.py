@@ -183,6 +183,10 @@ EDGE = [
     (1, 192, 13, 13, 1, 384, 3, 3, 16),
     (1, 256, 27, 27, 1, 384, 3, 3, 8),
     (2, 64, 9, 11, 2, 40, 5, 5, 5),
+    # channel counts that are multiples of 8 but not of 64 (padded channel quarters)
+    (1, 48, 55, 55, 2, 256, 5, 5, 16),    # AlexNet layer 2
+    (2, 24, 10, 12, 1, 16, 3, 3, 4),
+    (1, 200, 9, 9, 1, 32, 3, 3, 7),
 ]
 
 
