@@ -480,6 +480,140 @@ hipError_t launch_taps_wave(const float* A, const float* G3, const BwdFilterArgs
   return hipGetLastError();
 }
 
+// ---- 2''. taps for planes up to 64 pixels wide: one wave per (image, rank)
+// plane, lane = column, walking down the rows.  The last FS rows of A, G3 and
+// G2 live in registers; the horizontal taps read the neighbouring columns'
+// registers through wave shuffles; nothing goes through LDS and there is no
+// barrier.  Row t of A and G3 is requested kRowsAhead steps before it is used.
+// Step t completes B and Cc on row t-(FS-1-P), G2 on row t, G1 on row t-P and
+// the tap-gradient terms of row t-(FS-1-P).  Needs P <= FS-1.
+constexpr int kRowsAhead = 4;
+template <int FS>
+__global__ __launch_bounds__(256) void taps_column_kernel(
+    const float* __restrict__ A, const float* __restrict__ G3, const float* __restrict__ FH,
+    const float* __restrict__ FW, float* __restrict__ Cc, float* __restrict__ G1,
+    float* __restrict__ partH, float* __restrict__ partW, int R, int H, int W, int P,
+    int nplanes) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int plane = blockIdx.x * 4 + wave;
+  if (plane >= nplanes) return;
+  const int r = plane % R, n = plane / R;
+  const size_t base = (size_t)plane * H * W;
+  const bool col = lane < W;
+  const int wc = col ? lane : W - 1;             // clamped column for addresses
+  float fh[FS], fw[FS];
+#pragma unroll
+  for (int i = 0; i < FS; ++i) {
+    fh[i] = FH[i * R + r];
+    fw[i] = FW[i * R + r];
+  }
+  // source lanes of the horizontal taps; a tap that falls outside the row reads
+  // lane 0 and is masked
+  int srcf[FS], srcb[FS];
+  bool okf[FS], okb[FS];
+#pragma unroll
+  for (int j = 0; j < FS; ++j) {
+    const int wf = lane + j - P, wb = lane - j + P;   // forward / adjoint neighbour
+    okf[j] = col && wf >= 0 && wf < W;
+    okb[j] = col && wb >= 0 && wb < W;
+    srcf[j] = okf[j] ? wf : 0;
+    srcb[j] = okb[j] ? wb : 0;
+  }
+  float aw[FS], gw[FS], g2w[FS];                   // rows t-FS+1 .. t of A, G3, G2
+#pragma unroll
+  for (int i = 0; i < FS; ++i) aw[i] = gw[i] = g2w[i] = 0.f;
+  float accH[FS], accW[FS];
+#pragma unroll
+  for (int i = 0; i < FS; ++i) accH[i] = accW[i] = 0.f;
+  float ar[kRowsAhead], gr[kRowsAhead];
+  auto request = [&](int slot, int row) {          // rows past the plane count as zero
+    const int rc = row < H ? row : H - 1;
+    ar[slot] = A[base + (size_t)rc * W + wc];
+    gr[slot] = G3[base + (size_t)rc * W + wc];
+  };
+#pragma unroll
+  for (int u = 0; u < kRowsAhead; ++u) request(u, u);
+  const int tail = (FS - 1 - P) > P ? (FS - 1 - P) : P;
+  for (int t0 = 0; t0 < H + tail; t0 += kRowsAhead) {
+#pragma unroll
+    for (int u = 0; u < kRowsAhead; ++u) {
+      const int t = t0 + u;
+      if (t < H + tail) {
+        const bool live = col && t < H;
+        const float a_t = live ? ar[u] : 0.f, g_t = live ? gr[u] : 0.f;
+        request(u, t + kRowsAhead);
+        // G2 row t: horizontal adjoint taps of G3 row t
+        float g2_t = 0.f;
+#pragma unroll
+        for (int j = 0; j < FS; ++j) {
+          const float v = __shfl(g_t, srcb[j], 64);
+          g2_t += okb[j] ? fw[j] * v : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i + 1 < FS; ++i) {
+          aw[i] = aw[i + 1];
+          gw[i] = gw[i + 1];
+          g2w[i] = g2w[i + 1];
+        }
+        aw[FS - 1] = a_t;
+        gw[FS - 1] = g_t;
+        g2w[FS - 1] = g2_t;
+        // B, Cc and the tap-gradient terms of row hb
+        const int hb = t - (FS - 1 - P);
+        if (hb >= 0 && hb < H) {
+          float b = 0.f;
+#pragma unroll
+          for (int i = 0; i < FS; ++i) b += fh[i] * aw[i];
+          float cc = 0.f;
+#pragma unroll
+          for (int j = 0; j < FS; ++j) {
+            const float v = __shfl(b, srcf[j], 64);
+            const float bj = okf[j] ? v : 0.f;
+            cc += fw[j] * bj;
+            accW[j] += gw[P] * bj;                  // G3[hb][w] * B[hb][w+j-P]
+          }
+#pragma unroll
+          for (int i = 0; i < FS; ++i) accH[i] += g2w[P] * aw[i];   // G2[hb][w] * A[hb+i-P][w]
+          if (col) Cc[base + (size_t)hb * W + lane] = cc;
+        }
+        // G1 row hg: vertical adjoint taps of the G2 window
+        const int hg = t - P;
+        if (hg >= 0 && hg < H) {
+          float g1 = 0.f;
+#pragma unroll
+          for (int i = 0; i < FS; ++i) g1 += fh[i] * g2w[FS - 1 - i];
+          if (col) G1[base + (size_t)hg * W + lane] = g1;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < FS; ++i) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      accH[i] += __shfl_down(accH[i], off, 64);
+      accW[i] += __shfl_down(accW[i], off, 64);
+    }
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int i = 0; i < FS; ++i) {
+      partH[((size_t)n * FS + i) * R + r] = accH[i];
+      partW[((size_t)n * FS + i) * R + r] = accW[i];
+    }
+  }
+}
+
+template <int FS>
+hipError_t launch_taps_column(const float* A, const float* G3, const BwdFilterArgs& a, float* Cc,
+                              float* G1, float* pH, float* pW, hipStream_t st) {
+  const int nplanes = a.N * a.R;
+  taps_column_kernel<FS><<<(unsigned)((nplanes + 3) / 4), 256, 0, st>>>(
+      A, G3, a.FH, a.FW, Cc, G1, pH, pW, a.R, a.H, a.W, a.pad, nplanes);
+  return hipGetLastError();
+}
+
 // ---- 3a. partial[s][d][r] = sum_{p in split s} act[n,d,p] Z[n,r,p] ----------
 struct GradArgs {
   const float* act[2];   // dy, x
@@ -622,10 +756,10 @@ __global__ __launch_bounds__(256) void reduce4_kernel(ReduceArgs a) {
 
 struct Plan {
   int RP, npb, PS, cps, S, St;
-  bool plane_taps;
+  bool plane_taps, wave_taps, column_taps;
   size_t plane, part_elems;
 };
-Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R) {
+Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R, int pad) {
   Plan p;
   const int HW = H * W;
   p.RP = R <= 32 ? 32 : 64;
@@ -639,7 +773,10 @@ Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R) {
   p.PS = (nch + p.cps - 1) / p.cps;
   p.S = N * p.PS;
   p.plane_taps = (size_t)HW * 4 * sizeof(float) <= 64 * 1024 && Y + X <= 256;   // plane fits in LDS
-  p.St = p.plane_taps ? N : (N < 8 ? N : 8);
+  const bool odd_square = Y == X && (Y == 1 || Y == 3 || Y == 5 || Y == 7);
+  p.wave_taps = p.plane_taps && HW <= 256 && odd_square;              // one wave per plane, in LDS
+  p.column_taps = !p.wave_taps && W <= 64 && odd_square && pad <= Y - 1;   // one wave per plane, in registers
+  p.St = (p.plane_taps || p.column_taps) ? N : (N < 8 ? N : 8);
   p.plane = (size_t)N * R * HW;
   p.part_elems = (size_t)p.S * R * ((size_t)T + C) + (size_t)N * R * ((size_t)Y + X);
   return p;
@@ -654,13 +791,13 @@ bool bwd_filter_mfma_supported(const cp4_shape& s) {
 }
 
 size_t bwd_filter_mfma_workspace_bytes(const cp4_shape& s) {
-  const Plan p = make_plan(s.N, s.C, s.T, s.H, s.W, s.Y, s.X, s.Rank);
+  const Plan p = make_plan(s.N, s.C, s.T, s.H, s.W, s.Y, s.X, s.Rank, s.pad);
   return (6 * p.plane + p.part_elems) * sizeof(float);
 }
 
 hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   const int HW = a.H * a.W, R = a.R, N = a.N;
-  const Plan p = make_plan(N, a.C, a.T, a.H, a.W, a.Y, a.X, R);
+  const Plan p = make_plan(N, a.C, a.T, a.H, a.W, a.Y, a.X, R, a.pad);
   float* ws = static_cast<float*>(a.workspace);
   float *A = ws, *B = ws + p.plane, *Cc = ws + 2 * p.plane, *G3 = ws + 3 * p.plane,
         *G2 = ws + 4 * p.plane, *G1 = ws + 5 * p.plane, *part = ws + 6 * p.plane;
@@ -695,9 +832,16 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
                            st>>>(c);
   }
 
-  const bool wave_taps = p.plane_taps && HW <= 256 && a.Y == a.X &&
-                         (a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7);
-  if (wave_taps) {
+  const bool wave_taps = p.wave_taps, column_taps = p.column_taps;
+  if (column_taps) {
+    switch (a.Y) {
+      case 1: e = launch_taps_column<1>(A, G3, a, Cc, G1, pH, pW, st); break;
+      case 3: e = launch_taps_column<3>(A, G3, a, Cc, G1, pH, pW, st); break;
+      case 5: e = launch_taps_column<5>(A, G3, a, Cc, G1, pH, pW, st); break;
+      default: e = launch_taps_column<7>(A, G3, a, Cc, G1, pH, pW, st); break;
+    }
+    if (e != hipSuccess) return e;
+  } else if (wave_taps) {
     switch (a.Y) {
       case 1: e = launch_taps_wave<1>(A, G3, a, Cc, G1, pH, pW, st); break;
       case 3: e = launch_taps_wave<3>(A, G3, a, Cc, G1, pH, pW, st); break;
