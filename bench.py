@@ -136,7 +136,7 @@ def main():
                 t = us
             else:
                 _, dd = device_inputs(ww)
-                t, _ = timed(ww, dd, 5, 47, 30.0)   # 47 launches, as the reference's bench drivers
+                t, _ = timed(ww, dd, 5, 200, args.settle_ms)
                 del dd
             b = algorithmic_bytes(ww)
             passes[name] = {"pass": ww.pass_, "us": round(t, 2),

@@ -766,9 +766,12 @@ Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R, int pad) 
   p.npb = (HW + 63) / 64;
   const int nch = (HW + 31) / 32;
   const int dgroups = (T + 127) / 128 + (C + 127) / 128;
-  int PS = (256 + N * dgroups - 1) / (N * dgroups);   // aim at >= 256 workgroups
+  // Pixel splits per image: aim at 1024 workgroups (4 waves per SIMD hide the
+  // load -> LDS -> MFMA latency of a chunk), but keep at least 6 chunks per split
+  // so that the partials to write and sum stay small next to the operands.
+  int PS = (1024 + N * dgroups - 1) / (N * dgroups);
+  if (PS > nch / 6) PS = nch / 6;
   if (PS < 1) PS = 1;
-  if (PS > nch) PS = nch;
   p.cps = (nch + PS - 1) / PS;
   p.PS = (nch + p.cps - 1) / p.cps;
   p.S = N * p.PS;
