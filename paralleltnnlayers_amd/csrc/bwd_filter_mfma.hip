@@ -487,7 +487,7 @@ hipError_t launch_taps_wave(const float* A, const float* G3, const BwdFilterArgs
 // barrier.  Row t of A and G3 is requested kRowsAhead steps before it is used.
 // Step t completes B and Cc on row t-(FS-1-P), G2 on row t, G1 on row t-P and
 // the tap-gradient terms of row t-(FS-1-P).  Needs P <= FS-1.
-constexpr int kRowsAhead = 4;
+constexpr int kRowsAhead = 8;
 template <int FS>
 __global__ __launch_bounds__(256) void taps_column_kernel(
     const float* __restrict__ A, const float* __restrict__ G3, const float* __restrict__ FH,
