@@ -13,6 +13,8 @@
 //      operands staged through LDS so that global reads stay row-contiguous;
 //      plus the small tap gradients;
 //   4. fixed-order sum of the per-workgroup partials (bit-reproducible).
+#include <cstdint>
+
 #include "cp4_internal.h"
 #include "split_bf16.h"
 
@@ -695,6 +697,101 @@ __global__ __launch_bounds__(kCT) void grad_gemm_kernel(GradArgs a) {
     }
 }
 
+// ---- 3a'. the same gradient GEMMs as exact split-bf16 products (H*W a
+// multiple of 4 so that rows can be moved as float4).  Per 32-pixel chunk the
+// workgroup splits the Z tile once, cooperatively, straight from global memory
+// into MFMA B fragments in LDS ([rank block][16-pixel step][part][half][rank] x
+// 16 B, double-buffered: one barrier per chunk); every wave stages its own 32
+// activation rows through a wave-private LDS tile (row-contiguous global reads)
+// and splits them as the A operand.
+constexpr int kLdS = 36;   // LDS row stride (floats) of the activation tile: 16-byte aligned rows
+
+template <int RB>
+__global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
+  using namespace split;
+  __shared__ __attribute__((aligned(16))) float As[kCT / 64][32 * kLdS];
+  __shared__ u32x4 Zf[2][RB * 2 * 3 * 2 * 32];
+  const int which = blockIdx.z;
+  const int D = a.D[which], R = a.R, HW = a.HW;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hi = lane >> 5;
+  const int d0 = blockIdx.y * 128 + wave * 32;
+  if ((int)blockIdx.y * 128 >= D) return;
+  const int s = blockIdx.x, n = s / a.PS, ps = s - n * a.PS;
+  const int nch_total = (HW + 31) >> 5;
+  const int ch0 = ps * a.cps, ch1 = min(nch_total, ch0 + a.cps);
+  const float* actn = a.act[which] + (size_t)n * D * HW;
+  const float* zn = a.Z[which] + (size_t)n * R * HW;
+  // activation tile: lane moves float4; 8 lanes cover one 32-pixel row, 8 rows per load
+  const int arow = lane >> 3, acol = 4 * (lane & 7);
+  // Z tile: thread t splits the 8 pixels (octet zo) of rank row zr
+  const int zr = tid >> 2, zo = tid & 3;             // 64 rows x 4 octets = 256 threads
+  const bool zmine = zr < 32 * RB;
+  float4 av[4], zv[2];
+  auto load_tiles = [&](int ch) {
+    const int p = ch * 32 + acol;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int d = d0 + 8 * j + arow;
+      av[j] = (p < HW && d < D) ? *reinterpret_cast<const float4*>(actn + (size_t)d * HW + p)
+                                : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    const int pz = ch * 32 + 8 * zo;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      zv[j] = (zmine && zr < R && pz + 4 * j < HW)
+                  ? *reinterpret_cast<const float4*>(zn + (size_t)zr * HW + pz + 4 * j)
+                  : make_float4(0.f, 0.f, 0.f, 0.f);
+  };
+  auto store_tiles = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      *reinterpret_cast<float4*>(&As[wave][(8 * j + arow) * kLdS + acol]) = av[j];
+    if (zmine) {
+      const float v[8] = {zv[0].x, zv[0].y, zv[0].z, zv[0].w, zv[1].x, zv[1].y, zv[1].z, zv[1].w};
+      u32x4 h, m, l;
+      split8(v, h, m, l);
+      // fragment (rank block zr/32, step zo/2, part, half zo&1, rank zr%32)
+      u32x4* dst = &Zf[buf][(((zr >> 5) * 2 + (zo >> 1)) * 3 * 2 + (zo & 1)) * 32 + (zr & 31)];
+      dst[0] = h;
+      dst[64] = m;          // part stride: 2 halves x 32 ranks
+      dst[128] = l;
+    }
+  };
+  f32x16 acc[RB];
+#pragma unroll
+  for (int mb = 0; mb < RB; ++mb) acc[mb] = (f32x16)(0.f);
+  if (ch0 < ch1) load_tiles(ch0);
+  for (int ch = ch0; ch < ch1; ++ch) {
+    const int buf = (ch - ch0) & 1;
+    store_tiles(buf);
+    __syncthreads();        // Z fragments of this chunk are complete; the other buffer is free
+    if (ch + 1 < ch1) load_tiles(ch + 1);   // in flight during the MFMAs
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const float* ap = &As[wave][l32 * kLdS + 16 * st + 8 * hi];
+      const float4 a0 = *reinterpret_cast<const float4*>(ap);
+      const float4 a1 = *reinterpret_cast<const float4*>(ap + 4);
+      const float v[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+      u32x4 ah, am, al;
+      split8(v, ah, am, al);
+#pragma unroll
+      for (int mb = 0; mb < RB; ++mb) {
+        const u32x4* zp = &Zf[buf][((mb * 2 + st) * 3 * 2 + hi) * 32 + l32];
+        acc[mb] = mfma_split(ah, am, al, zp[0], zp[64], zp[128], acc[mb]);
+      }
+    }
+  }
+  float* out = a.part[which] + (size_t)s * D * R;
+#pragma unroll
+  for (int mb = 0; mb < RB; ++mb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int d = d0 + 8 * (v >> 2) + 4 * hi + (v & 3), r = 32 * mb + l32;
+      if (d < D && r < R) out[(size_t)d * R + r] = acc[mb][v];
+    }
+}
+
 // ---- 3b. tap gradients: partial[s][t][r] over images of split s -------------
 
 __global__ __launch_bounds__(256) void tap_grad_kernel(const float* __restrict__ G2,
@@ -734,24 +831,35 @@ struct ReduceArgs {
   float* out[4];
   int count[4], S[4];
 };
+// A workgroup owns 64 consecutive outputs; its four waves each sum a quarter of
+// the S partials in index order (eight loads in flight), then the four quarter
+// sums are added in wave order: the result does not depend on timing.
 __global__ __launch_bounds__(256) void reduce4_kernel(ReduceArgs a) {
+  __shared__ float quarter[4][64];
   const int seg = blockIdx.y;
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= a.count[seg]) return;
-  const float* p = a.part[seg] + i;
-  const size_t stride = a.count[seg];
-  const int S = a.S[seg];
+  const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
+  const int i = blockIdx.x * 64 + lane;
+  const int count = a.count[seg], S = a.S[seg];
+  if ((int)blockIdx.x * 64 >= count) return;               // whole workgroup
+  const int k0 = (int)((long)S * q / 4), k1 = (int)((long)S * (q + 1) / 4);
   float s = 0.f;
-  int k = 0;
-  for (; k + 8 <= S; k += 8) {   // eight loads in flight, summed in index order
-    float v[8];
+  if (i < count) {
+    const float* p = a.part[seg] + i;
+    const size_t stride = count;
+    int k = k0;
+    for (; k + 8 <= k1; k += 8) {
+      float v[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = p[(size_t)(k + u) * stride];
+      for (int u = 0; u < 8; ++u) v[u] = p[(size_t)(k + u) * stride];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) s += v[u];
+      for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    for (; k < k1; ++k) s += p[(size_t)k * stride];
   }
-  for (; k < S; ++k) s += p[(size_t)k * stride];
-  a.out[seg][i] = s;
+  quarter[q][lane] = s;
+  __syncthreads();
+  if (q == 0 && i < count)
+    a.out[seg][i] = ((quarter[0][lane] + quarter[1][lane]) + quarter[2][lane]) + quarter[3][lane];
 }
 
 struct Plan {
@@ -872,8 +980,16 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   g.N = N; g.R = R; g.RP = p.RP; g.HW = HW; g.PS = p.PS; g.cps = p.cps;
   const int dmax = a.T > a.C ? a.T : a.C;
   const dim3 ggrid(p.S, (dmax + 127) / 128, 2);
-  if (p.RP == 32) grad_gemm_kernel<1><<<ggrid, kCT, 0, st>>>(g);
-  else grad_gemm_kernel<2><<<ggrid, kCT, 0, st>>>(g);
+  const bool grad_split = (HW & 3) == 0 &&
+                          ((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.dy) |
+                            reinterpret_cast<uintptr_t>(ws)) & 15) == 0;
+  if (grad_split) {
+    if (p.RP == 32) grad_split_kernel<1><<<ggrid, kCT, 0, st>>>(g);
+    else grad_split_kernel<2><<<ggrid, kCT, 0, st>>>(g);
+  } else {
+    if (p.RP == 32) grad_gemm_kernel<1><<<ggrid, kCT, 0, st>>>(g);
+    else grad_gemm_kernel<2><<<ggrid, kCT, 0, st>>>(g);
+  }
 
   ReduceArgs r{};
   const float* parts[4] = {pK, pC, pH, pW};
@@ -885,7 +1001,7 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
     r.part[i] = parts[i]; r.out[i] = outs[i]; r.count[i] = counts[i]; r.S[i] = Ss[i];
     if (counts[i] > maxc) maxc = counts[i];
   }
-  reduce4_kernel<<<dim3((maxc + 255) / 256, 4), 256, 0, st>>>(r);
+  reduce4_kernel<<<dim3((maxc + 63) / 64, 4), 256, 0, st>>>(r);
   return hipGetLastError();
 }
 
