@@ -187,6 +187,10 @@ EDGE = [
     (1, 48, 55, 55, 2, 256, 5, 5, 16),    # AlexNet layer 2
     (2, 24, 10, 12, 1, 16, 3, 3, 4),
     (1, 200, 9, 9, 1, 32, 3, 3, 7),
+    # many small planes (wave-per-plane tap kernel, one partial per image)
+    (64, 32, 8, 8, 1, 48, 3, 3, 20),
+    (70, 16, 6, 10, 2, 16, 5, 5, 40),     # two rank tiles, the second partly filled
+    (64, 16, 14, 14, 0, 32, 1, 1, 8),     # 1x1 filter, no padding
 ]
 
 
