@@ -137,9 +137,15 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     constexpr int cpq = CPQ;                       // 16-channel chunks per quarter (Cin <= 64*CPQ)
     const int nrounds = (nblk + 1) >> 1;
     // lane's channel 16*(cpq*cq + chunk) + 8*hi + e
-    // (PAD: Cin is not a multiple of 64; channel groups past Cin read group 0 and count as zero)
+    // (PAD: Cin is not a multiple of 64; channel groups past Cin count as zero)
     const int cg0 = 16 * cpq * cq + 8 * hi;        // lane's first channel of chunk 0
-    const float* xq = a.x + (size_t)n * Cin * HW + (size_t)cg0 * HW;
+    // x is read through a buffer descriptor over this image: the address is
+    // (descriptor base) + (32-bit lane offset) + (scalar offset), so the walk
+    // over channels runs on the scalar unit and no 64-bit vector adds sit between
+    // the MFMAs; reads past the last channel (padded channel groups) return 0.
+    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(a.x + (size_t)n * Cin * HW), 0, Cin * HW * 4, 0x00020000);
+    const unsigned sbase = (unsigned)(16 * cpq * cq) * (unsigned)HW * 4u;   // uniform byte offset
     // This wave's slice of the input factor stays in registers for the whole
     // sweep, already split: lane holds rank l32, channels 16*(cpq*cq+c) + 8*hi + e.
     u32x4 fh[CPQ], fm[CPQ], fl[CPQ];
@@ -154,35 +160,33 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       split8(v, fh[c], fm[c], fl[c]);
     }
     // Block of round r: sweep index j, LDS column qa of this lane, whether the
-    // lane's pixel exists, and the lane's (clamped, always in-bounds) x pointer.
-    auto geom = [&](int r, int& j, int& qa, bool& valid) -> const float* {
+    // lane's pixel exists, and the lane's byte offset (clamped pixel, channel 8*hi).
+    auto geom = [&](int r, int& j, int& qa, bool& valid) -> unsigned {
       j = 2 * r + bsel;
       const int b = rev ? nblk - 1 - j : j;        // j == nblk happens when nblk is odd
       qa = 32 * b + l32;
       const int q = qbase + qa;
       valid = j < nblk && q >= 0 && q < HW && qa < QLEN;
       const int qc = q < 0 ? 0 : (q > HW - 1 ? HW - 1 : q);
-      return xq + qc;
+      return (unsigned)(8 * hi * HW + qc) * 4u;
     };
-    auto ld_chunk = [&](float (&dst)[8], const float* xp, int chunk) {   // chunk < cpq
-      const bool ok = !PAD || cg0 + 16 * chunk < Cin;
-      const float* base = ok ? xp + (size_t)(16 * chunk) * HW : xp - (size_t)cg0 * HW;
+    auto ld_chunk = [&](float (&dst)[8], unsigned voff, int chunk) {   // chunk < cpq
+      const unsigned soff = sbase + (unsigned)(16 * chunk) * (unsigned)HW * 4u;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float v = base[(size_t)e * HW];
-        dst[e] = ok ? v : 0.f;
-      }
+      for (int e = 0; e < 8; ++e)
+        dst[e] = __builtin_bit_cast(
+            float, __builtin_amdgcn_raw_buffer_load_b32(xrs, voff, soff + (unsigned)e * HW * 4u, 0));
     };
     float xb[KR][8];
     int j, qa;
     bool valid;
-    const float* xp = geom(0, j, qa, valid);
+    unsigned xp = geom(0, j, qa, valid);
 #pragma unroll
     for (int u = 0; u < KR; ++u) ld_chunk(xb[u], xp, u);
     for (int r = 0; r < nrounds; ++r) {
       int jn, qan;
       bool validn;
-      const float* xpn = geom(r + 1 < nrounds ? r + 1 : r, jn, qan, validn);
+      const unsigned xpn = geom(r + 1 < nrounds ? r + 1 : r, jn, qan, validn);
       f32x16 acc = (f32x16)(0.f);
 #pragma unroll
       for (int ch = 0; ch < CPQ; ch += KR) {
@@ -530,6 +534,7 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 
 bool fwd_pipe_supported(const FwdArgs& a) {
   if (a.R > kRP || (a.Cin & 7) || a.Cin > 256) return false;
+  if ((size_t)a.Cin * a.H * a.W * sizeof(float) >= (1ull << 31)) return false;   // buffer offsets
   if (a.Y != a.X || !(a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7)) return false;
   PipePlan pl;
   return plan(a, &pl);
