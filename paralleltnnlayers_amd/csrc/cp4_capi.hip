@@ -100,9 +100,18 @@ int choose_variant(const FwdArgs& a) {
     for (int v = 0; v < kNumVariants; ++v)
       if (!strcmp(want, kVariants[v].name) && kVariants[v].supported(a)) return v;
   }
-  for (int v = kNumVariants - 1; v >= 0; --v)
-    if (kVariants[v].supported(a)) return v;
-  return -1;
+  int pick = -1;
+  for (int v = kNumVariants - 1; v >= 0 && pick < 0; --v)
+    if (kVariants[v].supported(a)) pick = v;
+  // Above 256 input channels the producer/consumer kernel keeps its factor in
+  // LDS and its strips get short; on large problems the phase-by-phase split
+  // kernel, where it applies (even widths), is then the faster one.
+  if (pick >= 0 && !strcmp(kVariants[pick].name, "mfma_bf16x3_pipe") && a.Cin > 256 &&
+      (long)a.N * a.H * a.W > 8192) {
+    for (int v = 0; v < kNumVariants; ++v)
+      if (!strcmp(kVariants[v].name, "mfma_bf16x3_strip") && kVariants[v].supported(a)) pick = v;
+  }
+  return pick;
 }
 
 cp4_status run_forward_like(const FwdArgs& a, int variant, hipStream_t st) {

@@ -11,7 +11,9 @@
 //
 //   waves 0-7  producers: the strip (+ halo rows) is swept in rounds of two
 //              32-pixel blocks; in a round wave w works on block (w & 1) of the
-//              pair for channel quarter w >> 1: it streams x (ring of KR
+//              pair for channel quarter w >> 1 (its slice of the input factor,
+//              pre-split, sits in registers up to 256 input channels and in
+//              LDS above): it streams x (ring of KR
 //              16-channel chunks in flight, refilled across round boundaries),
 //              splits, runs the MFMAs and adds its partial fp32 A[r][q] into
 //              LDS.  The four quarters of a block add in fixed order (an LDS
@@ -58,7 +60,8 @@ constexpr int kMaxBlk = 64;                  // per-block progress words in LDS
 struct PipePlan {
   int TH, strips, nWG;
   int QA;          // LDS row stride of A (floats)
-  int cc_off;      // byte offsets inside LDS
+  int fin_off;     // byte offsets inside LDS; factor fragments only above 256 input channels
+  int cc_off;
   int flag_off;
   size_t lds_bytes;
 #ifdef CP4_DEBUG_PHASES
@@ -84,6 +87,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   extern __shared__ float lds[];
   float* As = lds;                                                  // [32][QA] fp32
   unsigned char* ldsb = reinterpret_cast<unsigned char*>(lds);
+  unsigned char* Fb = ldsb + pl.fin_off;     // Fin fragments [chunk][part][hi][r] x 16 B (CPQ == 0)
   unsigned char* Cb = ldsb + pl.cc_off;      // 3 x Cc fragment tiles
   // [0..kMaxBlk) quarters done per block (sweep order), then 4 consumer arrival counters
   int* flags = reinterpret_cast<int*>(ldsb + pl.flag_off);
@@ -126,15 +130,32 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   const int QLEN = (pl.TH + FS - 1) * W;
   const int nblk = (QLEN + 31) >> 5;             // 32-pixel producer blocks
 
-  // ---- prologue: clear the progress words ----------------------------------
+  // ---- prologue: clear the progress words; above 256 input channels the input
+  // factor does not fit the producers' registers and goes to LDS, pre-split ----
+  constexpr bool FLDS = CPQ == 0;
+  const int cpq = FLDS ? (Cin + 63) >> 6 : CPQ;    // 16-channel chunks per channel quarter
   if (tid < kMaxBlk + 4) flags[tid] = 0;
+  if (FLDS) {
+    for (int it = tid; it < 8 * cpq * 32; it += kThreads) {
+      const int o = it >> 5, r = it & 31;          // channel octet (of the padded count), rank
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        v[e] = (r < R && 8 * o + e < Cin) ? a.Fin[(size_t)(8 * o + e) * R + r] : 0.f;
+      u32x4 h, m, l;
+      split8(v, h, m, l);
+      u32x4* dst = reinterpret_cast<u32x4*>(Fb + ((size_t)(o >> 1) * 6 + (o & 1)) * 512 + r * 16);
+      dst[0] = h;          // part stride: 2 planes of 512 B
+      dst[64] = m;
+      dst[128] = l;
+    }
+  }
   __syncthreads();
   STAMP(1)
 
   if (wave < kProd) {
     // =========================== producers ==================================
     const int bsel = wave & 1, cq = wave >> 1;     // block of the round's pair, channel quarter
-    constexpr int cpq = CPQ;                       // 16-channel chunks per quarter (Cin <= 64*CPQ)
     const int nrounds = (nblk + 1) >> 1;
     // lane's channel 16*(cpq*cq + chunk) + 8*hi + e
     // (PAD: Cin is not a multiple of 64; channel groups past Cin count as zero)
@@ -148,17 +169,22 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     const unsigned sbase = (unsigned)(16 * cpq * cq) * (unsigned)HW * 4u;   // uniform byte offset
     // This wave's slice of the input factor stays in registers for the whole
     // sweep, already split: lane holds rank l32, channels 16*(cpq*cq+c) + 8*hi + e.
-    u32x4 fh[CPQ], fm[CPQ], fl[CPQ];
+    constexpr int NF = FLDS ? 1 : CPQ;
+    u32x4 fh[NF], fm[NF], fl[NF];
+    if (!FLDS) {
 #pragma unroll
-    for (int c = 0; c < CPQ; ++c) {
-      float v[8];
+      for (int c = 0; c < NF; ++c) {
+        float v[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        v[e] = (l32 < R && (!PAD || cg0 + 16 * c < Cin))
-                   ? a.Fin[(size_t)(cg0 + 16 * c + e) * R + l32]
-                   : 0.f;
-      split8(v, fh[c], fm[c], fl[c]);
+        for (int e = 0; e < 8; ++e)
+          v[e] = (l32 < R && (!PAD || cg0 + 16 * c < Cin))
+                     ? a.Fin[(size_t)(cg0 + 16 * c + e) * R + l32]
+                     : 0.f;
+        split8(v, fh[c], fm[c], fl[c]);
+      }
     }
+    const u32x4* fbase =
+        reinterpret_cast<const u32x4*>(Fb + hi * 512 + l32 * 16) + (size_t)(cq * cpq) * (6 * 32);
     // Block of round r: sweep index j, LDS column qa of this lane, whether the
     // lane's pixel exists, and the lane's byte offset (clamped pixel, channel 8*hi).
     auto geom = [&](int r, int& j, int& qa, bool& valid) -> unsigned {
@@ -188,21 +214,35 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       bool validn;
       const unsigned xpn = geom(r + 1 < nrounds ? r + 1 : r, jn, qan, validn);
       f32x16 acc = (f32x16)(0.f);
+      auto step = [&](int ch, int u) {
+        u32x4 xh, xm, xl;
+        split8(xb[u], xh, xm, xl);
+        if (FLDS) {
+          const u32x4* fp = fbase + (size_t)(ch + u) * (6 * 32);
+          acc = mfma_split(fp[0], fp[64], fp[128], xh, xm, xl, acc);
+        } else {
+          acc = mfma_split(fh[FLDS ? 0 : ch + u], fm[FLDS ? 0 : ch + u], fl[FLDS ? 0 : ch + u], xh,
+                           xm, xl, acc);
+        }
+        // refill this ring slot: same round, or the first chunks of the next
+        const int nxt = ch + u + KR;
+        if (nxt < cpq)
+          ld_chunk(xb[u], xp, nxt);
+        else
+          ld_chunk(xb[u], xpn, nxt - cpq);
+        // keep use-then-refill order per chunk so KR chunks stay in flight
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      if (FLDS) {
+        for (int ch = 0; ch < cpq; ch += KR) {
 #pragma unroll
-      for (int ch = 0; ch < CPQ; ch += KR) {
+          for (int u = 0; u < KR; ++u) step(ch, u);
+        }
+      } else {
 #pragma unroll
-        for (int u = 0; u < KR; ++u) {
-          u32x4 xh, xm, xl;
-          split8(xb[u], xh, xm, xl);
-          acc = mfma_split(fh[ch + u], fm[ch + u], fl[ch + u], xh, xm, xl, acc);
-          // refill this ring slot: same round, or the first chunks of the next
-          const int nxt = ch + u + KR;
-          if (nxt < CPQ)
-            ld_chunk(xb[u], xp, nxt);
-          else
-            ld_chunk(xb[u], xpn, nxt - CPQ);
-          // keep use-then-refill order per chunk so KR chunks stay in flight
-          __builtin_amdgcn_sched_barrier(0);
+        for (int ch = 0; ch < NF; ch += KR) {
+#pragma unroll
+          for (int u = 0; u < KR; ++u) step(ch, u);
         }
       }
       if (j < nblk) {
@@ -473,15 +513,18 @@ bool layout(const FwdArgs& a, int TH, PipePlan* pl) {
   const long QA =
       round_up((int)(round_up(TH * a.W + 31, 64) + (long)(a.Y - 1) * (a.W + 1) + 1), 64) + 8;
   const size_t a_bytes = (size_t)kRP * QA * sizeof(float);
-  const size_t bytes = a_bytes + 3 * kCcBuf + (kMaxBlk + 4) * sizeof(int);
+  // above 256 input channels: pre-split factor fragments, 192 B per (padded) channel
+  const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
+  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 4) * sizeof(int);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
   pl->strips = (a.H + TH - 1) / TH;
   pl->nWG = a.N * pl->strips;
   pl->QA = (int)QA;
-  pl->cc_off = (int)a_bytes;
-  pl->flag_off = (int)(a_bytes + 3 * kCcBuf);
+  pl->fin_off = (int)a_bytes;
+  pl->cc_off = (int)(a_bytes + fin_bytes);
+  pl->flag_off = (int)(a_bytes + fin_bytes + 3 * kCcBuf);
   pl->lds_bytes = bytes;
   return true;
 }
@@ -516,12 +559,14 @@ hipError_t launch_as(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 
 template <int FS, bool PAD>
 hipError_t launch_cpq(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
-  switch ((a.Cin + 63) >> 6) {                   // 16-channel chunks per channel quarter
+  const int cpq = (a.Cin + 63) >> 6;             // 16-channel chunks per channel quarter
+  switch (cpq) {
     case 1: return launch_as<FS, 1, 1, PAD>(a, pl, st);
     case 2: return launch_as<FS, 2, 2, PAD>(a, pl, st);
     case 3: return launch_as<FS, 3, 1, PAD>(a, pl, st);
     case 4: return launch_as<FS, 4, 2, PAD>(a, pl, st);
-    default: return hipErrorInvalidValue;
+    default:                                      // factor fragments in LDS
+      return (cpq & 1) ? launch_as<FS, 0, 1, PAD>(a, pl, st) : launch_as<FS, 0, 2, PAD>(a, pl, st);
   }
 }
 
@@ -533,7 +578,7 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 }  // namespace
 
 bool fwd_pipe_supported(const FwdArgs& a) {
-  if (a.R > kRP || (a.Cin & 7) || a.Cin > 256) return false;
+  if (a.R > kRP || (a.Cin & 7) || a.Cin > 768) return false;
   if ((size_t)a.Cin * a.H * a.W * sizeof(float) >= (1ull << 31)) return false;   // buffer offsets
   if (a.Y != a.X || !(a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7)) return false;
   PipePlan pl;

@@ -187,6 +187,10 @@ EDGE = [
     (1, 48, 55, 55, 2, 256, 5, 5, 16),    # AlexNet layer 2
     (2, 24, 10, 12, 1, 16, 3, 3, 4),
     (1, 200, 9, 9, 1, 32, 3, 3, 7),
+    # more than 256 input channels: factor fragments in LDS; odd width, odd chunk count
+    (2, 512, 7, 7, 1, 64, 3, 3, 32),
+    (1, 320, 14, 14, 1, 96, 3, 3, 16),
+    (1, 384, 13, 13, 2, 384, 5, 5, 16),   # both passes above 256 channels
     # many small planes (wave-per-plane tap kernel, one partial per image)
     (64, 32, 8, 8, 1, 48, 3, 3, 20),
     (70, 16, 6, 10, 2, 16, 5, 5, 40),     # two rank tiles, the second partly filled
