@@ -706,7 +706,7 @@ __global__ __launch_bounds__(kCT) void grad_gemm_kernel(GradArgs a) {
 // and splits them as the A operand.
 constexpr int kLdS = 36;   // LDS row stride (floats) of the activation tile: 16-byte aligned rows
 
-template <int RB>
+template <int RB, bool VEC>
 __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
   using namespace split;
   __shared__ __attribute__((aligned(16))) float As[kCT / 64][32 * kLdS];
@@ -728,20 +728,32 @@ __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
   const int zr = tid >> 2, zo = tid & 3;             // 64 rows x 4 octets = 256 threads
   const bool zmine = zr < 32 * RB;
   float4 av[4], zv[2];
+  // VEC: H*W is a multiple of 4 and the operands are 16-byte aligned, rows move
+  // as float4; otherwise element by element with per-pixel bounds.
+  auto load4 = [&](const float* row, int p) {
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (VEC) {
+      if (p < HW) v = *reinterpret_cast<const float4*>(row + p);
+    } else {
+      if (p < HW) v.x = row[p];
+      if (p + 1 < HW) v.y = row[p + 1];
+      if (p + 2 < HW) v.z = row[p + 2];
+      if (p + 3 < HW) v.w = row[p + 3];
+    }
+    return v;
+  };
   auto load_tiles = [&](int ch) {
     const int p = ch * 32 + acol;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int d = d0 + 8 * j + arow;
-      av[j] = (p < HW && d < D) ? *reinterpret_cast<const float4*>(actn + (size_t)d * HW + p)
-                                : make_float4(0.f, 0.f, 0.f, 0.f);
+      av[j] = d < D ? load4(actn + (size_t)d * HW, p) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     const int pz = ch * 32 + 8 * zo;
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-      zv[j] = (zmine && zr < R && pz + 4 * j < HW)
-                  ? *reinterpret_cast<const float4*>(zn + (size_t)zr * HW + pz + 4 * j)
-                  : make_float4(0.f, 0.f, 0.f, 0.f);
+      zv[j] = (zmine && zr < R) ? load4(zn + (size_t)zr * HW, pz + 4 * j)
+                                : make_float4(0.f, 0.f, 0.f, 0.f);
   };
   auto store_tiles = [&](int buf) {
 #pragma unroll
@@ -896,7 +908,11 @@ Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R, int pad) 
 }  // namespace
 
 bool bwd_filter_mfma_supported(const cp4_shape& s) {
-  return s.Rank <= 64 && ((s.H * s.W) & 1) == 0 && (s.C & 1) == 0 && (s.T & 1) == 0 &&
+  // odd planes need the split contraction (scalar loads): channel counts multiples of 16
+  const bool odd_plane_ok = (s.C & 15) == 0 && (s.T & 15) == 0 &&
+                            (size_t)(s.C > s.T ? s.C : s.T) * 192 <= 160 * 1024;
+  return s.Rank <= 64 && (((s.H * s.W) & 1) == 0 || odd_plane_ok) && (s.C & 1) == 0 &&
+         (s.T & 1) == 0 &&
          (size_t)(s.C > s.T ? s.C : s.T) * (s.Rank <= 32 ? 32 : 64) * 4 <= 160 * 1024 &&
          s.Y + s.X <= 65535;
 }
@@ -984,8 +1000,12 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
                           ((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.dy) |
                             reinterpret_cast<uintptr_t>(ws)) & 15) == 0;
   if (grad_split) {
-    if (p.RP == 32) grad_split_kernel<1><<<ggrid, kCT, 0, st>>>(g);
-    else grad_split_kernel<2><<<ggrid, kCT, 0, st>>>(g);
+    if (p.RP == 32) grad_split_kernel<1, true><<<ggrid, kCT, 0, st>>>(g);
+    else grad_split_kernel<2, true><<<ggrid, kCT, 0, st>>>(g);
+  } else if (HW & 1) {
+    // odd planes: the float2 staging of the fp32 kernel does not apply
+    if (p.RP == 32) grad_split_kernel<1, false><<<ggrid, kCT, 0, st>>>(g);
+    else grad_split_kernel<2, false><<<ggrid, kCT, 0, st>>>(g);
   } else {
     if (p.RP == 32) grad_gemm_kernel<1><<<ggrid, kCT, 0, st>>>(g);
     else grad_gemm_kernel<2><<<ggrid, kCT, 0, st>>>(g);

@@ -191,6 +191,10 @@ EDGE = [
     (2, 512, 7, 7, 1, 64, 3, 3, 32),
     (1, 320, 14, 14, 1, 96, 3, 3, 16),
     (1, 384, 13, 13, 2, 384, 5, 5, 16),   # both passes above 256 channels
+    # odd planes (7x7, 13x13, 27x27) on the matrix-core backward-filter path
+    (4, 32, 7, 7, 1, 48, 3, 3, 8),
+    (3, 64, 13, 13, 1, 32, 3, 3, 16),
+    (2, 16, 27, 27, 2, 16, 5, 5, 4),
     # many small planes (wave-per-plane tap kernel, one partial per image)
     (64, 32, 8, 8, 1, 48, 3, 3, 20),
     (70, 16, 6, 10, 2, 16, 5, 5, 40),     # two rank tiles, the second partly filled
