@@ -249,10 +249,10 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
   const cp4_shape& s = *shape;
   hipStream_t st = as_stream(stream);
   if (s.N == 0) {  // empty batch: the gradients are zero
-    CP4_HIP(hipMemsetAsync(dFK, 0, sizeof(float) * s.T * s.Rank, st));
-    CP4_HIP(hipMemsetAsync(dFC, 0, sizeof(float) * s.C * s.Rank, st));
-    CP4_HIP(hipMemsetAsync(dFH, 0, sizeof(float) * s.Y * s.Rank, st));
-    CP4_HIP(hipMemsetAsync(dFW, 0, sizeof(float) * s.X * s.Rank, st));
+    CP4_HIP(cp4::zero_f32_launch(dFK, (size_t)s.T * s.Rank, st));
+    CP4_HIP(cp4::zero_f32_launch(dFC, (size_t)s.C * s.Rank, st));
+    CP4_HIP(cp4::zero_f32_launch(dFH, (size_t)s.Y * s.Rank, st));
+    CP4_HIP(cp4::zero_f32_launch(dFW, (size_t)s.X * s.Rank, st));
     return CP4_OK;
   }
   if (!x || !dy) return fail(CP4_ERR_NULL_POINTER, "x or dy is NULL");
@@ -288,7 +288,7 @@ cp4_status cp4_conv2d_backward_filter_full(const cp4_shape* shape,
   hipStream_t st = as_stream(stream);
   if (s.N == 0) {
     if (!accumulate)
-      CP4_HIP(hipMemsetAsync(dK, 0, sizeof(float) * s.T * s.C * s.Y * s.X, st));
+      CP4_HIP(cp4::zero_f32_launch(dK, (size_t)s.T * s.C * s.Y * s.X, st));
     return CP4_OK;
   }
   if (!x || !dy) return fail(CP4_ERR_NULL_POINTER, "x or dy is NULL");

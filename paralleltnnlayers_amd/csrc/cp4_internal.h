@@ -62,6 +62,9 @@ hipError_t count_exceeding_launch(const float* A, const float* B, size_t n,
 hipError_t random_uniform_launch(float* dst, size_t n, unsigned long long seed,
                                  hipStream_t);
 hipError_t copy_f32_launch(float* dst, const float* src, size_t n, hipStream_t);
+// Fill kernel rather than a memset node, so that callers may capture the
+// empty-batch paths into a graph like every other launch.
+hipError_t zero_f32_launch(float* dst, size_t n, hipStream_t);
 
 }  // namespace cp4
 #endif

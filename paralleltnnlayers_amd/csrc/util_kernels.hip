@@ -71,6 +71,12 @@ __global__ __launch_bounds__(256) void copy_f32_kernel(
   if (i < n) dst[i] = src[i];
 }
 
+__global__ __launch_bounds__(256) void zero_f32_kernel(float* __restrict__ dst, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * 256)
+    dst[i] = 0.f;
+}
+
 unsigned grid_for(size_t n, unsigned cap) {
   const size_t g = (n + 255) / 256;
   return (unsigned)(g < 1 ? 1 : g > cap ? cap : g);
@@ -96,6 +102,12 @@ hipError_t count_exceeding_launch(const float* A, const float* B, size_t n,
 hipError_t random_uniform_launch(float* dst, size_t n, unsigned long long seed,
                                  hipStream_t st) {
   random_uniform_kernel<<<grid_for(n, 65536), 256, 0, st>>>(dst, n, seed);
+  return hipGetLastError();
+}
+
+hipError_t zero_f32_launch(float* dst, size_t n, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  zero_f32_kernel<<<grid_for(n, 2048), 256, 0, st>>>(dst, n);
   return hipGetLastError();
 }
 
