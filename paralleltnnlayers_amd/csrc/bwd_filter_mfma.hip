@@ -911,7 +911,8 @@ bool bwd_filter_mfma_supported(const cp4_shape& s) {
   // odd planes need the split contraction (scalar loads): channel counts multiples of 16
   const bool odd_plane_ok = (s.C & 15) == 0 && (s.T & 15) == 0 &&
                             (size_t)(s.C > s.T ? s.C : s.T) * 192 <= 160 * 1024;
-  return s.Rank <= 64 && (((s.H * s.W) & 1) == 0 || odd_plane_ok) && (s.C & 1) == 0 &&
+  return s.Rank <= 64 && fits_int_indexing((int)s.N, (int)s.H, (int)s.W) &&
+         (((s.H * s.W) & 1) == 0 || odd_plane_ok) && (s.C & 1) == 0 &&
          (s.T & 1) == 0 &&
          (size_t)(s.C > s.T ? s.C : s.T) * (s.Rank <= 32 ? 32 : 64) * 4 <= 160 * 1024 &&
          s.Y + s.X <= 65535;

@@ -26,6 +26,15 @@ struct FwdArgs {
 };
 
 
+// The matrix-core kernels index pixels, strips and work items with 32-bit
+// integers: planes up to 2^24 pixels and batch x plane products that keep every
+// such count below 2^31.  Larger problems run on the general kernels, whose
+// indices are 64-bit throughout.
+inline bool fits_int_indexing(int N, int H, int W) {
+  const size_t HW = (size_t)H * W;
+  return HW <= (1u << 24) && (size_t)N * HW < (1ull << 35) && (size_t)N * H < (1ull << 30);
+}
+
 bool fwd_general_supported(const FwdArgs&);
 hipError_t fwd_general_launch(const FwdArgs&, hipStream_t);
 bool fwd_mfma_supported(const FwdArgs&);

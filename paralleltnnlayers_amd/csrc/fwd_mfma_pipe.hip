@@ -579,6 +579,7 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 
 bool fwd_pipe_supported(const FwdArgs& a) {
   if (a.R > kRP || (a.Cin & 7) || a.Cin > 768) return false;
+  if (!fits_int_indexing(a.N, a.H, a.W)) return false;
   if ((size_t)a.Cin * a.H * a.W * sizeof(float) >= (1ull << 31)) return false;   // buffer offsets
   if (a.Y != a.X || !(a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7)) return false;
   PipePlan pl;
