@@ -51,6 +51,18 @@ cp4_status cp4_conv2d_forward(const cp4_shape* shape, const float* x,
                               const float* FH, const float* FW, float* y,
                               cp4_stream stream);
 
+/* Forward with the layer's epilogue fused into the stores:
+ * y[n,t,h,w] = act(conv[n,t,h,w] + bias[t]).  The reference adds the bias as a
+ * separate framework op after the convolution (test/layers.py:282, use_bias) and
+ * applies the activation in another; here neither re-reads y.  bias is [T] in
+ * device memory or NULL; activation is a cp4_activation. */
+typedef enum cp4_activation { CP4_ACT_NONE = 0, CP4_ACT_RELU = 1 } cp4_activation;
+cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
+                                       const float* FK, const float* FC,
+                                       const float* FH, const float* FW,
+                                       const float* bias, int activation, float* y,
+                                       cp4_stream stream);
+
 /* Replaces cp4_conv2d_backward_data_gpu
  * (Cuda_kernels/cp4Conv2dBackwardData.cuh:7-14, .cu:112-282):
  * dy[N,T,H,W] -> dx[N,C,H,W] with the reference's flipped taps. */

@@ -63,6 +63,8 @@ def lib():
     L.cp4_conv2d_forward.argtypes = fwd + [ctypes.c_void_p]
     L.cp4_conv2d_forward_variant.argtypes = fwd + [ctypes.c_int, ctypes.c_void_p]
     L.cp4_conv2d_backward_data.argtypes = fwd + [ctypes.c_void_p]
+    L.cp4_conv2d_forward_bias_act.argtypes = [_S, _F, _F, _F, _F, _F, _F, ctypes.c_int, _F,
+                                              ctypes.c_void_p]
     bwf = [_S] + [_F] * 10 + [ctypes.c_void_p, ctypes.c_size_t]
     L.cp4_conv2d_backward_filter.argtypes = bwf + [ctypes.c_void_p]
     L.cp4_conv2d_backward_filter_variant.argtypes = bwf + [ctypes.c_int, ctypes.c_void_p]
@@ -135,6 +137,24 @@ def conv2d_forward(x, FK, FC, FH, FW, pad=1, out=None, variant=-1, stream=None):
     check(lib().cp4_conv2d_forward_variant(ctypes.byref(s), _ptr(x), _ptr(FK), _ptr(FC),
                                            _ptr(FH), _ptr(FW), _ptr(y), variant,
                                            _stream(stream)))
+    return y
+
+
+ACTIVATIONS = {None: 0, "none": 0, "relu": 1}
+
+
+def conv2d_forward_bias_act(x, FK, FC, FH, FW, bias=None, activation=None, pad=1, out=None,
+                            stream=None):
+    """y = act(conv(x) + bias[t]) with the epilogue fused into the stores."""
+    s = shape_for(x.shape, FK, FC, FH, FW, pad)
+    assert x.shape[1] == s.C and FC.shape[1] == s.Rank
+    assert bias is None or tuple(bias.shape) == (s.T,)
+    y = out if out is not None else torch.empty((s.N, s.T, s.H, s.W), device=x.device,
+                                                dtype=torch.float32)
+    check(lib().cp4_conv2d_forward_bias_act(
+        ctypes.byref(s), _ptr(x), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
+        _ptr(bias) if bias is not None else None, ACTIVATIONS[activation], _ptr(y),
+        _stream(stream)))
     return y
 
 

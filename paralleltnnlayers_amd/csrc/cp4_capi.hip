@@ -206,6 +206,39 @@ cp4_status cp4_conv2d_forward(const cp4_shape* shape, const float* x,
   return cp4_conv2d_forward_variant(shape, x, FK, FC, FH, FW, y, -1, stream);
 }
 
+cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
+                                       const float* FK, const float* FC,
+                                       const float* FH, const float* FW,
+                                       const float* bias, int activation, float* y,
+                                       cp4_stream stream) {
+  if (activation != CP4_ACT_NONE && activation != CP4_ACT_RELU)
+    return fail(CP4_ERR_UNSUPPORTED, "activation must be CP4_ACT_NONE or CP4_ACT_RELU");
+  if (!bias && activation == CP4_ACT_NONE)
+    return cp4_conv2d_forward(shape, x, FK, FC, FH, FW, y, stream);
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return CP4_OK;
+  rc = check_forward_ptrs(x, FK, FC, FH, FW, y);
+  if (rc != CP4_OK) return rc;
+  FwdArgs a = forward_args(*shape, x, FK, FC, FH, FW, y);
+  a.bias = bias;
+  a.act = activation;
+  hipStream_t st = as_stream(stream);
+  // The kernel the plain forward would pick decides: when that is the producer /
+  // consumer kernel its epilogue build runs, otherwise the chosen variant is
+  // followed by the in-place bias / activation kernel.
+  const int v = choose_variant(a);
+  if (v < 0) return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape");
+  if (!strcmp(kVariants[v].name, "mfma_bf16x3_pipe") && cp4::fwd_pipe_epi_supported(a)) {
+    CP4_HIP(cp4::fwd_pipe_epi_launch(a, st));
+    return CP4_OK;
+  }
+  CP4_HIP(kVariants[v].launch(a, st));
+  CP4_HIP(cp4::bias_act_launch(y, bias, activation, shape->N, shape->T,
+                               (size_t)shape->H * shape->W, st));
+  return CP4_OK;
+}
+
 cp4_status cp4_conv2d_backward_data(const cp4_shape* shape, const float* dy,
                                     const float* FK, const float* FC,
                                     const float* FH, const float* FW,

@@ -23,6 +23,10 @@ struct FwdArgs {
   float* y;           // [N, Cout, H, W]
   int N, Cin, Cout, H, W, pad, Y, X, R;
   int flip;           // 1: tap index t reads factor row (taps-1-t)
+  // Output epilogue y = act(conv + bias[k]); only kernels that say so apply it
+  // (the caller runs bias_act_launch after the others).
+  const float* bias;  // [Cout] or null
+  int act;            // 0: none, 1: max(., 0)
 };
 
 
@@ -43,6 +47,12 @@ bool fwd_split_supported(const FwdArgs&);
 hipError_t fwd_split_launch(const FwdArgs&, hipStream_t);
 bool fwd_pipe_supported(const FwdArgs&);
 hipError_t fwd_pipe_launch(const FwdArgs&, hipStream_t);
+// The same kernel compiled with the bias / activation epilogue in its stores.
+bool fwd_pipe_epi_supported(const FwdArgs&);
+hipError_t fwd_pipe_epi_launch(const FwdArgs&, hipStream_t);
+// In-place y[n,k,:] = act(y[n,k,:] + bias[k]) for variants without the epilogue.
+hipError_t bias_act_launch(float* y, const float* bias, int act, size_t N, size_t K, size_t HW,
+                           hipStream_t);
 
 // Backward-filter (factor gradients).
 struct BwdFilterArgs {

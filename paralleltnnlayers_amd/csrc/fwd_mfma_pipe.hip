@@ -39,6 +39,11 @@
 // Arithmetic follows the reassociated form of
 // Cuda_kernels/cp4Conv2dForward.cu:84-133 (backward-data:
 // cp4Conv2dBackwardData.cu:57-108 through swapped factors and flipped taps).
+//
+// This file is compiled twice: as is, and with CP4_PIPE_EPILOGUE defined, which
+// adds y = act(conv + bias[k]) to the stores (the bias of the lane's sixteen
+// output rows rides in registers next to the output-factor fragment) and exports
+// the entry points under the names fwd_pipe_epi_*.
 #include <cstdlib>
 
 #include "cp4_internal.h"
@@ -291,8 +296,19 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // item only when there are more blocks than consumer waves): lane holds row
     // 32*kb + l32, ranks 16*c + 8*hi + e.
     u32x4 fkh[2], fkm[2], fkl[2];
+#ifdef CP4_PIPE_EPILOGUE
+    float bs[16];                                  // bias of accumulator row v
+    const bool relu = a.act != 0;
+#endif
     auto load_fk = [&](int kb) {
       const int k = 32 * kb + l32;
+#ifdef CP4_PIPE_EPILOGUE
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int kk = 32 * kb + 8 * (v >> 2) + 4 * hi + (v & 3);
+        bs[v] = (a.bias && kk < Cout) ? a.bias[kk] : 0.f;
+      }
+#endif
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         float v[8];
@@ -451,6 +467,18 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           acc1 = mfma_split(fkh[c], fkm[c], fkl[c], b1h, b1m, b1l, acc1);
           __builtin_amdgcn_sched_barrier(0);     // one chunk's fragments live at a time
         }
+#ifdef CP4_PIPE_EPILOGUE
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          float o0 = acc0[v] + bs[v], o1 = acc1[v] + bs[v];
+          if (relu) {
+            o0 = o0 < 0.f ? 0.f : o0;
+            o1 = o1 < 0.f ? 0.f : o1;
+          }
+          acc0[v] = o0;
+          acc1[v] = o1;
+        }
+#endif
         // store rows: uniform row base + one 32-bit lane offset
         const int p = 64 * g - gshift + 2 * l32;       // lane's pixel pair p, p + 1
         float* rowbase = yn + (size_t)(32 * kb) * HW;
@@ -576,6 +604,11 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 }
 
 }  // namespace
+
+#ifdef CP4_PIPE_EPILOGUE
+#define fwd_pipe_supported fwd_pipe_epi_supported
+#define fwd_pipe_launch fwd_pipe_epi_launch
+#endif
 
 bool fwd_pipe_supported(const FwdArgs& a) {
   if (a.R > kRP || (a.Cin & 7) || a.Cin > 768) return false;

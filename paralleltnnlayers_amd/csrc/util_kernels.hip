@@ -77,6 +77,22 @@ __global__ __launch_bounds__(256) void zero_f32_kernel(float* __restrict__ dst, 
     dst[i] = 0.f;
 }
 
+// one workgroup per (image, channel) plane segment: the bias is a scalar
+__global__ __launch_bounds__(256) void bias_act_kernel(float* __restrict__ y,
+                                                       const float* __restrict__ bias, int act,
+                                                       size_t planes, size_t K, size_t HW) {
+  for (size_t plane = blockIdx.x; plane < planes; plane += gridDim.x) {   // n * K + k
+    const float b = bias ? bias[plane % K] : 0.f;
+    float* row = y + plane * HW;
+    for (size_t i = (size_t)blockIdx.y * 256 + threadIdx.x; i < HW;
+         i += (size_t)gridDim.y * 256) {
+      float v = row[i] + b;
+      if (act) v = v < 0.f ? 0.f : v;
+      row[i] = v;
+    }
+  }
+}
+
 unsigned grid_for(size_t n, unsigned cap) {
   const size_t g = (n + 255) / 256;
   return (unsigned)(g < 1 ? 1 : g > cap ? cap : g);
@@ -102,6 +118,16 @@ hipError_t count_exceeding_launch(const float* A, const float* B, size_t n,
 hipError_t random_uniform_launch(float* dst, size_t n, unsigned long long seed,
                                  hipStream_t st) {
   random_uniform_kernel<<<grid_for(n, 65536), 256, 0, st>>>(dst, n, seed);
+  return hipGetLastError();
+}
+
+hipError_t bias_act_launch(float* y, const float* bias, int act, size_t N, size_t K, size_t HW,
+                           hipStream_t st) {
+  if (N * K == 0 || HW == 0 || (!bias && !act)) return hipSuccess;
+  const unsigned segs = (unsigned)((HW + 4095) / 4096 > 64 ? 64 : (HW + 4095) / 4096);
+  const size_t planes = N * K;
+  const unsigned gx = (unsigned)(planes > (1u << 20) ? (1u << 20) : planes);
+  bias_act_kernel<<<dim3(gx, segs), 256, 0, st>>>(y, bias, act, planes, K, HW);
   return hipGetLastError();
 }
 

@@ -19,22 +19,29 @@ from . import capi
 
 
 class CP4Conv2dFunction(torch.autograd.Function):
-    """y = cp4conv2d(x, FK, FC, FH, FW, pad)."""
+    """y = act(cp4conv2d(x, FK, FC, FH, FW, pad) + bias)."""
 
     @staticmethod
-    def forward(ctx, x, FK, FC, FH, FW, pad):
+    def forward(ctx, x, FK, FC, FH, FW, pad, bias=None, activation=None):
         if 2 * pad + 1 != FH.shape[0] or 2 * pad + 1 != FW.shape[0]:
             raise ValueError("autograd binding needs 2*pad = Y-1 = X-1 (the reference's "
                              "backward-data pass is the adjoint only then)")
         x, FK, FC, FH, FW = (t.contiguous().float() for t in (x, FK, FC, FH, FW))
+        if bias is not None:
+            bias = bias.contiguous().float()
         ctx.pad = pad
-        ctx.save_for_backward(x, FK, FC, FH, FW)
-        return capi.conv2d_forward(x, FK, FC, FH, FW, pad=pad)
+        y = capi.conv2d_forward_bias_act(x, FK, FC, FH, FW, bias, activation, pad=pad)
+        ctx.relu = capi.ACTIVATIONS[activation] == 1
+        ctx.save_for_backward(x, FK, FC, FH, FW, y if ctx.relu else None)
+        return y
 
     @staticmethod
     def backward(ctx, dy):
-        x, FK, FC, FH, FW = ctx.saved_tensors
+        x, FK, FC, FH, FW, y = ctx.saved_tensors
         dy = dy.contiguous().float()
+        if ctx.relu:
+            dy = dy * (y > 0)
+        dbias = dy.sum(dim=(0, 2, 3)) if ctx.needs_input_grad[6] else None
         dx = None
         if ctx.needs_input_grad[0]:
             dx = capi.conv2d_backward_data(dy, FK, FC, FH, FW, pad=ctx.pad)
@@ -43,12 +50,13 @@ class CP4Conv2dFunction(torch.autograd.Function):
             grads = capi.conv2d_backward_filter(x, dy, FK, FC, FH, FW, pad=ctx.pad)
             grads = tuple(g if need else None
                           for g, need in zip(grads, ctx.needs_input_grad[1:5]))
-        return (dx,) + grads + (None,)
+        return (dx,) + grads + (None, dbias, None)
 
 
-def cp4_conv2d(x, FK, FC, FH, FW, pad):
-    """Functional form: differentiable fused CP4 convolution (NCHW, stride 1)."""
-    return CP4Conv2dFunction.apply(x, FK, FC, FH, FW, pad)
+def cp4_conv2d(x, FK, FC, FH, FW, pad, bias=None, activation=None):
+    """Functional form: differentiable fused CP4 convolution (NCHW, stride 1), with
+    the optional bias [T] and activation ("relu") fused into the forward stores."""
+    return CP4Conv2dFunction.apply(x, FK, FC, FH, FW, pad, bias, activation)
 
 
 class CP4Conv2d(torch.nn.Module):
@@ -60,7 +68,8 @@ class CP4Conv2d(torch.nn.Module):
     filter of the same shape.
     """
 
-    def __init__(self, in_channels, out_channels, kernel_size, rank, device="cuda"):
+    def __init__(self, in_channels, out_channels, kernel_size, rank, device="cuda", bias=False,
+                 activation=None):
         super().__init__()
         if kernel_size % 2 != 1:
             raise ValueError("kernel_size must be odd (same padding)")
@@ -71,9 +80,12 @@ class CP4Conv2d(torch.nn.Module):
         mk = lambda d: torch.nn.Parameter(torch.randn(d, rank, device=device) * s)
         self.FK, self.FC = mk(out_channels), mk(in_channels)
         self.FH, self.FW = mk(kernel_size), mk(kernel_size)
+        self.bias = torch.nn.Parameter(torch.zeros(out_channels, device=device)) if bias else None
+        self.activation = activation
 
     def forward(self, x):
-        return cp4_conv2d(x, self.FK, self.FC, self.FH, self.FW, self.pad)
+        return cp4_conv2d(x, self.FK, self.FC, self.FH, self.FW, self.pad, self.bias,
+                          self.activation)
 
     def dense_filter(self):
         """The recomposed [T,C,Y,X] filter (on the device, through cp4_recompose)."""
