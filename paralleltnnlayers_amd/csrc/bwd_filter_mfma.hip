@@ -38,6 +38,7 @@ struct ContractArgs {
   float* Z[2];           // A, G3
   int Cin[2];
   int N, R, RP, HW, npb, items;   // items per contraction and rank tile = N * npb
+  int ks;   // split kernel: waves per item, each contracting 1/ks of the channels (1, 2 or 4)
 };
 
 __global__ __launch_bounds__(kCW) void contract_mfma_kernel(ContractArgs a) {
@@ -121,8 +122,13 @@ __global__ __launch_bounds__(kCW) void contract_mfma_kernel(ContractArgs a) {
 // 32-pixel block): it streams x / dy through a register ring as the B operand,
 // splits each 16-channel chunk and issues six bf16 MFMAs for it - 2.7x less
 // matrix time than the fp32 MFMA and twice as many waves to hide latency with.
+// When there are few items (small planes, small batches) ks = 2 or 4 adjacent
+// waves share an item, each contracting 1/ks of the channels - shorter dependent
+// load chains and ks times the waves - and add their partial sums through LDS
+// in fixed order.
 constexpr int kSplitRing = 4;
-constexpr int kSW = 512;    // 8 waves share one factor tile: one fill per 8 items
+constexpr long kKsWaves = 1024;   // channel splits only while the grid stays below this many waves
+constexpr int kSW = 512;    // 8 waves share one factor tile: one fill per workgroup
 __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
   using namespace split;
   extern __shared__ float Fs[];
@@ -134,7 +140,9 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
   const int l32 = lane & 31, hi = lane >> 5;
   // This wave's item; waves past the end keep a valid (clamped) item for their
   // loads and skip the store, so that every wave reaches the barrier.
-  const int item_raw = blockIdx.x * (kSW / 64) + wave;    // (image, 32-pixel block)
+  const int ks = a.ks;
+  const int slot = blockIdx.x * (kSW / 64) + wave;        // (item, channel split)
+  const int item_raw = slot / ks, part = slot - item_raw * ks;   // item = (image, 32-pixel block)
   const bool has_item = item_raw < a.items;
   const int item = has_item ? item_raw : a.items - 1;
   const int pb = item % a.npb, n = item / a.npb;
@@ -142,8 +150,8 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
   const bool valid = has_item && p < HW;
   const int pc = p < HW ? p : HW - 1;
   // lane's channel 16*chunk + 8*hi + e
-  const float* xp = a.src[which] + ((size_t)n * Cin + 8 * hi) * HW + pc;
-  const int nch = Cin >> 4;
+  const int nch = (Cin >> 4) / ks, c0 = part * nch;     // this wave's chunks c0 .. c0 + nch - 1
+  const float* xp = a.src[which] + ((size_t)n * Cin + 16 * c0 + 8 * hi) * HW + pc;
   float xb[kSplitRing][8];
   auto ld_chunk = [&](float (&dst)[8], int ch) {
     ch = ch < nch ? ch : nch - 1;                     // clamped, not branched
@@ -155,18 +163,29 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
   // so their HBM latency runs under the fill
 #pragma unroll
   for (int u = 0; u < kSplitRing; ++u) ld_chunk(xb[u], u);
-  for (int it = tid; it < (Cin >> 3) * 32; it += kSW) {
-    const int o = it >> 5, r = 32 * mb + (it & 31);   // channel octet, rank
-    float v[8];
+  // two (channel octet, rank) entries per thread and round, their sixteen factor
+  // loads issued together
+  const int nfill = (Cin >> 3) * 32, fr = 32 * mb + (tid & 31);
+  for (int it = tid; it < nfill; it += 2 * kSW) {
+    float v[2][8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = r < R ? F[(size_t)(8 * o + e) * R + r] : 0.f;
-    u32x4 h, m, l;
-    split8(v, h, m, l);
-    u32x4* dst =
-        reinterpret_cast<u32x4*>(Fb + ((size_t)(o >> 1) * 6 + (o & 1)) * 512 + (it & 31) * 16);
-    dst[0] = h;          // part stride: 2 planes of 512 B
-    dst[64] = m;
-    dst[128] = l;
+    for (int t = 0; t < 2; ++t) {
+      const int o = min(it + t * kSW, nfill - 1) >> 5;       // channel octet (clamped)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[t][e] = fr < R ? F[(size_t)(8 * o + e) * R + fr] : 0.f;
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      if (it + t * kSW >= nfill) break;
+      const int o = (it + t * kSW) >> 5;
+      u32x4 h, m, l;
+      split8(v[t], h, m, l);
+      u32x4* dst =
+          reinterpret_cast<u32x4*>(Fb + ((size_t)(o >> 1) * 6 + (o & 1)) * 512 + (tid & 31) * 16);
+      dst[0] = h;          // part stride: 2 planes of 512 B
+      dst[64] = m;
+      dst[128] = l;
+    }
   }
   __syncthreads();
   const u32x4* fbase = reinterpret_cast<const u32x4*>(Fb + hi * 512 + l32 * 16);
@@ -182,7 +201,7 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
       const int c = ch + u;                           // chunk whose parts are in xh/xm/xl
       u32x4 nh = xh, nm = xm, nl = xl;
       if (c < nch) {
-        const u32x4* fp = fbase + (size_t)c * (6 * 32);
+        const u32x4* fp = fbase + (size_t)(c0 + c) * (6 * 32);
         const u32x4 fh = fp[0], fm = fp[64], fl = fp[128];
         // one MFMA, then a quarter of the next chunk's split, pinned in this order
         float (&nx)[8] = xb[(u + 1) % kSplitRing];
@@ -216,13 +235,33 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
     }
   }
   f32x16 acc = acc0 + acc1;
-  if (valid) {
-    float* zn = a.Z[which] + (size_t)n * R * HW + p;
+  float* zn = a.Z[which] + (size_t)n * R * HW + p;
+  if (ks == 1) {
+    if (valid) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int r = 32 * mb + 8 * (v >> 2) + 4 * hi + (v & 3);
-      if (r < R) zn[(size_t)r * HW] = acc[v];
+      for (int v = 0; v < 16; ++v) {
+        const int r = 32 * mb + 8 * (v >> 2) + 4 * hi + (v & 3);
+        if (r < R) zn[(size_t)r * HW] = acc[v];
+      }
     }
+    return;
+  }
+  // ks waves hold partial sums of one item: exchange through LDS (over the
+  // factor tile, which nobody reads any more) and let wave `part` add and store
+  // rows v = part, part + ks, ... in the fixed order of the splits.
+  __syncthreads();
+  float* red = Fs;                                   // [wave][v][lane]
+#pragma unroll
+  for (int v = 0; v < 16; ++v) red[(wave * 16 + v) * 64 + lane] = acc[v];
+  __syncthreads();
+  const int w0 = wave - part;                        // first wave of this item
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    if ((v & (ks - 1)) != part) continue;            // wave-uniform
+    float sum = 0.f;
+    for (int q = 0; q < ks; ++q) sum += red[((w0 + q) * 16 + v) * 64 + lane];
+    const int r = 32 * mb + 8 * (v >> 2) + 4 * hi + (v & 3);
+    if (valid && r < R) zn[(size_t)r * HW] = sum;
   }
 }
 
@@ -945,12 +984,23 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
     // exact split products: 32-pixel blocks, fragments of 6 bytes per factor entry
     c.npb = (HW + 31) / 32;
     c.items = N * c.npb;
-    const size_t smem = (size_t)cmax * 192;
+    // few items: 2 or 4 waves per item, each on a slice of the channels, until
+    // there are about 1024 waves (every workgroup builds the whole factor tile,
+    // so more splits than that cost more than they hide; a slice keeps >= 2 chunks)
+    c.ks = 1;
+    const int nch_min = (a.C < a.T ? a.C : a.T) >> 4;
+    while (c.ks < 4 && (long)c.items * 2 * (p.RP / 32) * c.ks < kKsWaves &&
+           ((a.C >> 4) % (2 * c.ks)) == 0 && ((a.T >> 4) % (2 * c.ks)) == 0 &&
+           nch_min / (2 * c.ks) >= 2)
+      c.ks *= 2;
+    size_t smem = (size_t)cmax * 192;
+    if (c.ks > 1 && smem < (size_t)kSW * 16 * sizeof(float)) smem = (size_t)kSW * 16 * sizeof(float);
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_split_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
-    contract_split_kernel<<<dim3((c.items + kSW / 64 - 1) / (kSW / 64), 2, p.RP / 32), kSW, smem,
-                            st>>>(c);
+    const long slots = (long)c.items * c.ks;
+    contract_split_kernel<<<dim3((unsigned)((slots + kSW / 64 - 1) / (kSW / 64)), 2, p.RP / 32),
+                            kSW, smem, st>>>(c);
   } else {
     const size_t smem = (size_t)cmax * 32 * sizeof(float);
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_mfma_kernel),
