@@ -401,64 +401,103 @@ __global__ __launch_bounds__(256) void taps_plane_kernel(
   }
 }
 
+// Sum of v over the 64 lanes, valid in lane 63: a shift-and-add scan inside each
+// row of 16 lanes, then the row totals passed on to the following rows, all as
+// data-parallel-primitive moves (no LDS traffic).  Lanes a move does not reach
+// read 0.
+template <int CTRL, int ROW_MASK, bool BOUND>
+__device__ __forceinline__ float dpp_move(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL,
+                                                               ROW_MASK, 0xf, BOUND));
+}
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+  v += dpp_move<0x111, 0xf, true>(v);    // row_shr:1
+  v += dpp_move<0x112, 0xf, true>(v);    // row_shr:2
+  v += dpp_move<0x114, 0xf, true>(v);    // row_shr:4
+  v += dpp_move<0x118, 0xf, true>(v);    // row_shr:8: lane 15 of a row holds the row's sum
+  v += dpp_move<0x142, 0xa, false>(v);   // row_bcast:15 into rows 1 and 3
+  v += dpp_move<0x143, 0xc, false>(v);   // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // ---- 2'. the same for small planes: one WAVE per (image, rank) plane -------
 // A plane of at most 256 pixels fits one wave with PP pixels per lane; its four
 // intermediate planes live in a wave-private LDS slice, so there is no
 // workgroup barrier, no idle thread and 4 planes per workgroup.  B and G2 stay
 // on chip: only Cc, G1 and the tap-gradient partials leave the CU.
+// The LDS planes carry a zero border of Q = max(P, FS-1-P) cells on every side,
+// so that every tap is an unconditional read at a fixed offset from the pixel's
+// cell: no bounds arithmetic in the tap loops.
 template <int FS, int PP>
 __global__ __launch_bounds__(256) void taps_wave_kernel(
     const float* __restrict__ A, const float* __restrict__ G3, const float* __restrict__ FH,
     const float* __restrict__ FW, float* __restrict__ Cc, float* __restrict__ G1,
-    float* __restrict__ partH, float* __restrict__ partW, int R, int H, int W, int P,
-    int nplanes) {
-  extern __shared__ float pl[];
-  const int HW = H * W;
+    float* __restrict__ partH, float* __restrict__ partW, int R, int H, int W, int P, int Q,
+    unsigned wmagic, int nplanes) {
+  extern __shared__ __attribute__((aligned(16))) float pl[];
+  const int HW = H * W, Wp = W + 2 * Q, cells = (H + 2 * Q) * Wp;   // cells: multiple of 4 (host)
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int plane = blockIdx.x * 4 + wave;
   if (plane >= nplanes) return;                   // whole wave; no workgroup barrier below
   const int r = plane % R, n = plane / R;
-  float* sA = pl + (size_t)wave * 4 * HW;
-  float *sG = sA + HW, *sB = sA + 2 * HW, *sG2 = sA + 3 * HW;
+  float* sA = pl + (size_t)wave * 4 * cells;
+  float *sG = sA + cells, *sB = sA + 2 * cells, *sG2 = sA + 3 * cells;
   const size_t base = (size_t)plane * HW;
+  // the plane's values are requested first, the LDS clear runs under their latency
+  float a[PP], g[PP];
+#pragma unroll
+  for (int k = 0; k < PP; ++k) {
+    const int p = min(lane + 64 * k, HW - 1);     // only the last k can pass the end
+    a[k] = A[base + p];
+    g[k] = G3[base + p];
+  }
   float fh[FS], fw[FS];
 #pragma unroll
   for (int i = 0; i < FS; ++i) {
     fh[i] = FH[i * R + r];
     fw[i] = FW[i * R + r];
   }
-  int ph[PP], pw[PP];
-  float g[PP], g2[PP];
+  for (int q = lane; q < cells; q += 64)          // 4 planes x cells floats = cells float4
+    reinterpret_cast<float4*>(sA)[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+  // cell of pixel k in a padded plane; lanes past the plane's end take pixel 0's
+  // cell: they recompute and rewrite that pixel's values and add nothing to the sums
+  int c[PP];
+  bool ok[PP];
 #pragma unroll
   for (int k = 0; k < PP; ++k) {
     const int p = lane + 64 * k;
-    ph[k] = p / W;
-    pw[k] = p - ph[k] * W;
-    g[k] = 0.f;
-    if (p < HW) {
-      sA[p] = A[base + p];
-      g[k] = G3[base + p];
-      sG[p] = g[k];
-    }
+    ok[k] = k < PP - 1 || p < HW;
+    const int pc = ok[k] ? p : 0;
+    const int h = (int)__umulhi((unsigned)pc, wmagic), w = pc - h * W;
+    c[k] = (h + Q) * Wp + w + Q;
+    if (!ok[k]) g[k] = 0.f;
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
 #pragma unroll
-  for (int k = 0; k < PP; ++k) {
-    const int p = lane + 64 * k, h = ph[k], w = pw[k];
-    float b = 0.f, v = 0.f;
-    if (p < HW) {
-#pragma unroll
-      for (int i = 0; i < FS; ++i) {
-        const int hh = h + i - P, ww = w - i + P;
-        if (hh >= 0 && hh < H) b += fh[i] * sA[hh * W + w];
-        if (ww >= 0 && ww < W) v += fw[i] * sG[h * W + ww];
-      }
-      sB[p] = b;
-      sG2[p] = v;
+  for (int k = 0; k < PP; ++k)
+    if (ok[k]) {
+      sA[c[k]] = a[k];
+      sG[c[k]] = g[k];
     }
-    g2[k] = v;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  float av[PP][FS], g2[PP];
+#pragma unroll
+  for (int k = 0; k < PP; ++k) {
+    float b = 0.f, v = 0.f;
+#pragma unroll
+    for (int i = 0; i < FS; ++i) {
+      av[k][i] = sA[c[k] + (i - P) * Wp];         // A one row per tap below / above
+      b += fh[i] * av[k][i];
+      v += fw[i] * sG[c[k] + (P - i)];
+    }
+    if (ok[k]) {
+      sB[c[k]] = b;
+      sG2[c[k]] = v;
+    }
+    g2[k] = ok[k] ? v : 0.f;
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
@@ -467,32 +506,27 @@ __global__ __launch_bounds__(256) void taps_wave_kernel(
   for (int i = 0; i < FS; ++i) accH[i] = accW[i] = 0.f;
 #pragma unroll
   for (int k = 0; k < PP; ++k) {
-    const int p = lane + 64 * k, h = ph[k], w = pw[k];
-    if (p < HW) {
-      float cc = 0.f, g1 = 0.f;
+    float cc = 0.f, g1 = 0.f;
 #pragma unroll
-      for (int i = 0; i < FS; ++i) {
-        const int ww = w + i - P, hh = h - i + P;
-        if (ww >= 0 && ww < W) cc += fw[i] * sB[h * W + ww];
-        if (hh >= 0 && hh < H) g1 += fh[i] * sG2[hh * W + w];
-        // tap gradients: dFH[i] += G2[p] A[p shifted down by i-P], dFW[i] += G3[p] B[...]
-        const int hv = h + i - P;
-        if (hv >= 0 && hv < H) accH[i] += g2[k] * sA[hv * W + w];
-        if (ww >= 0 && ww < W) accW[i] += g[k] * sB[h * W + ww];
-      }
-      Cc[base + p] = cc;
-      G1[base + p] = g1;
+    for (int i = 0; i < FS; ++i) {
+      const float bv = sB[c[k] + (i - P)];
+      cc += fw[i] * bv;
+      g1 += fh[i] * sG2[c[k] + (P - i) * Wp];
+      // tap gradients: dFH[i] += G2[p] A[p shifted down by i-P], dFW[i] += G3[p] B[p shifted right]
+      accH[i] += g2[k] * av[k][i];
+      accW[i] += g[k] * bv;
+    }
+    if (ok[k]) {
+      Cc[base + lane + 64 * k] = cc;
+      G1[base + lane + 64 * k] = g1;
     }
   }
 #pragma unroll
   for (int i = 0; i < FS; ++i) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      accH[i] += __shfl_down(accH[i], off, 64);
-      accW[i] += __shfl_down(accW[i], off, 64);
-    }
+    accH[i] = wave_sum_to_lane63(accH[i]);
+    accW[i] = wave_sum_to_lane63(accW[i]);
   }
-  if (lane == 0) {
+  if (lane == 63) {
 #pragma unroll
     for (int i = 0; i < FS; ++i) {
       partH[((size_t)n * FS + i) * R + r] = accH[i];
@@ -501,16 +535,31 @@ __global__ __launch_bounds__(256) void taps_wave_kernel(
   }
 }
 
+// Border and size of the padded LDS planes of taps_wave_kernel.
+struct WaveTapLayout {
+  int Q, cells;
+  size_t smem;
+};
+WaveTapLayout wave_tap_layout(int H, int W, int FS, int P) {
+  WaveTapLayout l;
+  l.Q = P > FS - 1 - P ? P : FS - 1 - P;
+  const int raw = (H + 2 * l.Q) * (W + 2 * l.Q);
+  l.cells = (raw + 3) & ~3;
+  l.smem = (size_t)4 * 4 * l.cells * sizeof(float);
+  return l;
+}
+
 template <int FS>
 hipError_t launch_taps_wave(const float* A, const float* G3, const BwdFilterArgs& a, float* Cc,
                             float* G1, float* pH, float* pW, hipStream_t st) {
   const int HW = a.H * a.W, nplanes = a.N * a.R;
-  const size_t smem = (size_t)4 * 4 * HW * sizeof(float);
+  const WaveTapLayout l = wave_tap_layout(a.H, a.W, FS, a.pad);
   const unsigned grid = (unsigned)((nplanes + 3) / 4);
+  const unsigned wmagic = (unsigned)(0x100000000ull / (unsigned)a.W) + 1u;   // p / W for p < 65536
   const int PP = (HW + 63) / 64;
-#define CP4_TW(pp)                                                                            \
-  taps_wave_kernel<FS, pp><<<grid, 256, smem, st>>>(A, G3, a.FH, a.FW, Cc, G1, pH, pW, a.R,  \
-                                                    a.H, a.W, a.pad, nplanes)
+#define CP4_TW(pp)                                                                             \
+  taps_wave_kernel<FS, pp><<<grid, 256, l.smem, st>>>(A, G3, a.FH, a.FW, Cc, G1, pH, pW, a.R, \
+                                                      a.H, a.W, a.pad, l.Q, wmagic, nplanes)
   switch (PP) {
     case 1: CP4_TW(1); break;
     case 2: CP4_TW(2); break;
@@ -936,7 +985,8 @@ Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R, int pad) 
   p.S = N * p.PS;
   p.plane_taps = (size_t)HW * 4 * sizeof(float) <= 64 * 1024 && Y + X <= 256;   // plane fits in LDS
   const bool odd_square = Y == X && (Y == 1 || Y == 3 || Y == 5 || Y == 7);
-  p.wave_taps = p.plane_taps && HW <= 256 && odd_square;              // one wave per plane, in LDS
+  p.wave_taps = p.plane_taps && HW <= 256 && W >= 2 && odd_square &&  // one wave per plane, in LDS
+                wave_tap_layout(H, W, Y, pad).smem <= 64 * 1024;
   p.column_taps = !p.wave_taps && W <= 64 && odd_square && pad <= Y - 1;   // one wave per plane, in registers
   p.St = (p.plane_taps || p.column_taps) ? N : (N < 8 ? N : 8);
   p.plane = (size_t)N * R * HW;
