@@ -14,6 +14,7 @@
 //      plus the small tap gradients;
 //   4. fixed-order sum of the per-workgroup partials (bit-reproducible).
 #include <cstdint>
+#include <cstdlib>
 
 #include "cp4_internal.h"
 #include "split_bf16.h"
@@ -27,6 +28,14 @@ __device__ __forceinline__ f32x16 mfma32(float a, float b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
 
+#ifdef CP4_DEBUG_PHASES
+// Debug builds: wall-clock stamps per (kernel slot, workgroup, wave) into a caller's buffer.
+#define BSTAMP(dbg, slot, wg, nw, i)                                                          \
+  if ((dbg) && (threadIdx.x & 63) == 0)                                                       \
+    (dbg)[(((size_t)(slot) * 4096 + (wg)) * (nw) + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64();
+#else
+#define BSTAMP(dbg, slot, wg, nw, i)
+#endif
 constexpr int kCT = 256;   // gradient-GEMM workgroup: 4 waves
 constexpr int kCW = 256;   // contraction workgroup: 4 waves (one per SIMD) sharing one 32-rank factor tile
 constexpr int kPF = 8;     // channel pairs per prefetch chunk in the contraction
@@ -39,6 +48,7 @@ struct ContractArgs {
   int Cin[2];
   int N, R, RP, HW, npb, items;   // items per contraction and rank tile = N * npb
   int ks;   // split kernel: waves per item, each contracting 1/ks of the channels (1, 2 or 4)
+  long long* dbg;
 };
 
 __global__ __launch_bounds__(kCW) void contract_mfma_kernel(ContractArgs a) {
@@ -141,6 +151,8 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
   // This wave's item; waves past the end keep a valid (clamped) item for their
   // loads and skip the store, so that every wave reaches the barrier.
   const int ks = a.ks;
+  [[maybe_unused]] const int dwg = (blockIdx.z * 2 + blockIdx.y) * gridDim.x + blockIdx.x;
+  BSTAMP(a.dbg, 0, dwg, 8, 0)
   const int slot = blockIdx.x * (kSW / 64) + wave;        // (item, channel split)
   const int item_raw = slot / ks, part = slot - item_raw * ks;   // item = (image, 32-pixel block)
   const bool has_item = item_raw < a.items;
@@ -187,13 +199,16 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
       dst[128] = l;
     }
   }
+  BSTAMP(a.dbg, 0, dwg, 8, 1)
   __syncthreads();
+  BSTAMP(a.dbg, 0, dwg, 8, 2)
   const u32x4* fbase = reinterpret_cast<const u32x4*>(Fb + hi * 512 + l32 * 16);
   // Software pipeline: while the six MFMAs of chunk c run (two accumulators, so
   // they do not wait for each other), the vector ALU splits chunk c+1.
   f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
   u32x4 xh, xm, xl;
   split8(xb[0], xh, xm, xl);
+  BSTAMP(a.dbg, 0, dwg, 8, 5)
   ld_chunk(xb[0], kSplitRing);
   for (int ch = 0; ch < nch; ch += kSplitRing) {
 #pragma unroll
@@ -235,6 +250,7 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
     }
   }
   f32x16 acc = acc0 + acc1;
+  BSTAMP(a.dbg, 0, dwg, 8, 3)
   float* zn = a.Z[which] + (size_t)n * R * HW + p;
   if (ks == 1) {
     if (valid) {
@@ -244,6 +260,7 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
         if (r < R) zn[(size_t)r * HW] = acc[v];
       }
     }
+    BSTAMP(a.dbg, 0, dwg, 8, 4)
     return;
   }
   // ks waves hold partial sums of one item: exchange through LDS (over the
@@ -711,6 +728,7 @@ struct GradArgs {
   float* part[2];        // [S][D][R]
   int D[2];
   int N, R, RP, HW, PS, cps;   // PS pixel splits per image, cps 32-pixel chunks per split
+  long long* dbg;
 };
 
 constexpr int kLd = 34;   // LDS row stride of the 32-pixel operand tiles (conflict-free)
@@ -806,6 +824,8 @@ __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
   const int d0 = blockIdx.y * 128 + wave * 32;
   if ((int)blockIdx.y * 128 >= D) return;
   const int s = blockIdx.x, n = s / a.PS, ps = s - n * a.PS;
+  [[maybe_unused]] const int dwg = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+  BSTAMP(a.dbg, 1, dwg, 4, 0)
   const int nch_total = (HW + 31) >> 5;
   const int ch0 = ps * a.cps, ch1 = min(nch_total, ch0 + a.cps);
   const float* actn = a.act[which] + (size_t)n * D * HW;
@@ -865,6 +885,7 @@ __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
   for (int ch = ch0; ch < ch1; ++ch) {
     const int buf = (ch - ch0) & 1;
     store_tiles(buf);
+    if (ch - ch0 < 3) { BSTAMP(a.dbg, 1, dwg, 4, 1 + (ch - ch0)) }
     __syncthreads();        // Z fragments of this chunk are complete; the other buffer is free
     if (ch + 1 < ch1) load_tiles(ch + 1);   // in flight during the MFMAs
 #pragma unroll
@@ -882,6 +903,7 @@ __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
       }
     }
   }
+  BSTAMP(a.dbg, 1, dwg, 4, 4)
   float* out = a.part[which] + (size_t)s * D * R;
 #pragma unroll
   for (int mb = 0; mb < RB; ++mb)
@@ -890,6 +912,7 @@ __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
       const int d = d0 + 8 * (v >> 2) + 4 * hi + (v & 3), r = 32 * mb + l32;
       if (d < D && r < R) out[(size_t)d * R + r] = acc[mb][v];
     }
+  BSTAMP(a.dbg, 1, dwg, 4, 5)
 }
 
 // ---- 3b. tap gradients: partial[s][t][r] over images of split s -------------
@@ -1028,6 +1051,9 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   c.src[1] = a.dy; c.F[1] = a.FK; c.Z[1] = G3; c.Cin[1] = a.T;
   c.N = N; c.R = R; c.RP = p.RP; c.HW = HW; c.npb = p.npb;
   c.items = N * p.npb;
+#ifdef CP4_DEBUG_PHASES
+  c.dbg = getenv("CP4_DBG_PTR") ? reinterpret_cast<long long*>(strtoull(getenv("CP4_DBG_PTR"), nullptr, 10)) : nullptr;
+#endif
   const int cmax = a.C > a.T ? a.C : a.T;
   hipError_t e;
   if ((a.C & 15) == 0 && (a.T & 15) == 0 && (size_t)cmax * 192 <= 160 * 1024) {
@@ -1095,6 +1121,9 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   g.act[0] = a.dy; g.Z[0] = Cc; g.part[0] = pK; g.D[0] = a.T;
   g.act[1] = a.x; g.Z[1] = G1; g.part[1] = pC; g.D[1] = a.C;
   g.N = N; g.R = R; g.RP = p.RP; g.HW = HW; g.PS = p.PS; g.cps = p.cps;
+#ifdef CP4_DEBUG_PHASES
+  g.dbg = getenv("CP4_DBG_PTR") ? reinterpret_cast<long long*>(strtoull(getenv("CP4_DBG_PTR"), nullptr, 10)) : nullptr;
+#endif
   const int dmax = a.T > a.C ? a.T : a.C;
   const dim3 ggrid(p.S, (dmax + 127) / 128, 2);
   const bool grad_split = (HW & 3) == 0 &&
