@@ -63,6 +63,27 @@ cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
                                        const float* bias, int activation, float* y,
                                        cp4_stream stream);
 
+/* Forward and backward-data with bfloat16 activations in memory: x / dy and
+ * y / dx are NCHW arrays of 16-bit bfloat16, the four factors and the bias stay
+ * fp32 and so does all arithmetic (exact products of the bf16 inputs with the
+ * fp32 factors, fp32 accumulation, one rounding to nearest-even at the store).
+ * Half the HBM bytes of the fp32 entry points.  The reference has fp32 only; this
+ * is the layer's mixed-precision form.  Runs on the producer / consumer kernel
+ * alone: CP4_ERR_UNSUPPORTED for shapes it does not take (Rank > 32, C not a
+ * multiple of 8 or above 768, filters other than square 1/3/5/7);
+ * cp4_bf16_supported answers beforehand (backward_data != 0: the shape is read
+ * as that pass's, channels swapped). */
+int cp4_bf16_supported(const cp4_shape* shape, int backward_data);
+cp4_status cp4_conv2d_forward_bf16(const cp4_shape* shape, const void* x_bf16,
+                                   const float* FK, const float* FC,
+                                   const float* FH, const float* FW,
+                                   const float* bias, int activation,
+                                   void* y_bf16, cp4_stream stream);
+cp4_status cp4_conv2d_backward_data_bf16(const cp4_shape* shape, const void* dy_bf16,
+                                         const float* FK, const float* FC,
+                                         const float* FH, const float* FW,
+                                         void* dx_bf16, cp4_stream stream);
+
 /* Replaces cp4_conv2d_backward_data_gpu
  * (Cuda_kernels/cp4Conv2dBackwardData.cuh:7-14, .cu:112-282):
  * dy[N,T,H,W] -> dx[N,C,H,W] with the reference's flipped taps. */

@@ -65,6 +65,11 @@ def lib():
     L.cp4_conv2d_backward_data.argtypes = fwd + [ctypes.c_void_p]
     L.cp4_conv2d_forward_bias_act.argtypes = [_S, _F, _F, _F, _F, _F, _F, ctypes.c_int, _F,
                                               ctypes.c_void_p]
+    L.cp4_bf16_supported.argtypes = [_S, ctypes.c_int]
+    L.cp4_conv2d_forward_bf16.argtypes = [_S, ctypes.c_void_p, _F, _F, _F, _F, _F, ctypes.c_int,
+                                          ctypes.c_void_p, ctypes.c_void_p]
+    L.cp4_conv2d_backward_data_bf16.argtypes = [_S, ctypes.c_void_p, _F, _F, _F, _F,
+                                                ctypes.c_void_p, ctypes.c_void_p]
     bwf = [_S] + [_F] * 10 + [ctypes.c_void_p, ctypes.c_size_t]
     L.cp4_conv2d_backward_filter.argtypes = bwf + [ctypes.c_void_p]
     L.cp4_conv2d_backward_filter_variant.argtypes = bwf + [ctypes.c_int, ctypes.c_void_p]
@@ -156,6 +161,41 @@ def conv2d_forward_bias_act(x, FK, FC, FH, FW, bias=None, activation=None, pad=1
         _ptr(bias) if bias is not None else None, ACTIVATIONS[activation], _ptr(y),
         _stream(stream)))
     return y
+
+
+def _ptr16(t):
+    assert t.is_cuda and t.is_contiguous() and t.dtype == torch.bfloat16
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def bf16_supported(s, backward_data=False):
+    return bool(lib().cp4_bf16_supported(ctypes.byref(s), int(backward_data)))
+
+
+def conv2d_forward_bf16(x, FK, FC, FH, FW, bias=None, activation=None, pad=1, out=None,
+                        stream=None):
+    """bfloat16 x -> bfloat16 y = act(conv(x) + bias); fp32 factors, bias and arithmetic."""
+    s = shape_for(x.shape, FK, FC, FH, FW, pad)
+    assert x.shape[1] == s.C and FC.shape[1] == s.Rank
+    assert bias is None or tuple(bias.shape) == (s.T,)
+    y = out if out is not None else torch.empty((s.N, s.T, s.H, s.W), device=x.device,
+                                                dtype=torch.bfloat16)
+    check(lib().cp4_conv2d_forward_bf16(
+        ctypes.byref(s), _ptr16(x), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
+        _ptr(bias) if bias is not None else None, ACTIVATIONS[activation], _ptr16(y),
+        _stream(stream)))
+    return y
+
+
+def conv2d_backward_data_bf16(dy, FK, FC, FH, FW, pad=1, out=None, stream=None):
+    """bfloat16 dy -> bfloat16 dx; fp32 factors and arithmetic."""
+    s = shape_for(dy.shape, FK, FC, FH, FW, pad)
+    assert dy.shape[1] == s.T
+    dx = out if out is not None else torch.empty((s.N, s.C, s.H, s.W), device=dy.device,
+                                                 dtype=torch.bfloat16)
+    check(lib().cp4_conv2d_backward_data_bf16(ctypes.byref(s), _ptr16(dy), _ptr(FK), _ptr(FC),
+                                              _ptr(FH), _ptr(FW), _ptr16(dx), _stream(stream)))
+    return dx
 
 
 def conv2d_backward_data(dy, FK, FC, FH, FW, pad=1, out=None, stream=None):

@@ -257,6 +257,54 @@ size_t cp4_conv2d_backward_filter_workspace_bytes(const cp4_shape* shape) {
   return filter_workspace(*shape);
 }
 
+int cp4_bf16_supported(const cp4_shape* shape, int backward_data) {
+  if (check_shape(shape) != CP4_OK) return 0;
+  const FwdArgs a = backward_data
+                        ? backward_data_args(*shape, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr)
+                        : forward_args(*shape, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr);
+  return cp4::fwd_pipe_io16_supported(a) ? 1 : 0;
+}
+
+cp4_status cp4_conv2d_forward_bf16(const cp4_shape* shape, const void* x_bf16,
+                                   const float* FK, const float* FC,
+                                   const float* FH, const float* FW,
+                                   const float* bias, int activation,
+                                   void* y_bf16, cp4_stream stream) {
+  if (activation != CP4_ACT_NONE && activation != CP4_ACT_RELU)
+    return fail(CP4_ERR_UNSUPPORTED, "activation must be CP4_ACT_NONE or CP4_ACT_RELU");
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return CP4_OK;
+  rc = check_forward_ptrs(x_bf16, FK, FC, FH, FW, y_bf16);
+  if (rc != CP4_OK) return rc;
+  // the kernel reads FwdArgs::x / y as 16-bit elements
+  FwdArgs a = forward_args(*shape, static_cast<const float*>(x_bf16), FK, FC, FH, FW,
+                           static_cast<float*>(y_bf16));
+  a.bias = bias;
+  a.act = activation;
+  if (!cp4::fwd_pipe_io16_supported(a))
+    return fail(CP4_ERR_UNSUPPORTED, "bfloat16 I/O: shape not taken by the producer/consumer kernel");
+  CP4_HIP(cp4::fwd_pipe_io16_launch(a, as_stream(stream)));
+  return CP4_OK;
+}
+
+cp4_status cp4_conv2d_backward_data_bf16(const cp4_shape* shape, const void* dy_bf16,
+                                         const float* FK, const float* FC,
+                                         const float* FH, const float* FW,
+                                         void* dx_bf16, cp4_stream stream) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return CP4_OK;
+  rc = check_forward_ptrs(dy_bf16, FK, FC, FH, FW, dx_bf16);
+  if (rc != CP4_OK) return rc;
+  const FwdArgs a = backward_data_args(*shape, static_cast<const float*>(dy_bf16), FK, FC, FH, FW,
+                                       static_cast<float*>(dx_bf16));
+  if (!cp4::fwd_pipe_io16_supported(a))
+    return fail(CP4_ERR_UNSUPPORTED, "bfloat16 I/O: shape not taken by the producer/consumer kernel");
+  CP4_HIP(cp4::fwd_pipe_io16_launch(a, as_stream(stream)));
+  return CP4_OK;
+}
+
 cp4_status cp4_conv2d_backward_filter(const cp4_shape* shape, const float* x,
                                       const float* dy, const float* FK,
                                       const float* FC, const float* FH,

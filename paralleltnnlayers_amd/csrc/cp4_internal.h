@@ -50,6 +50,10 @@ hipError_t fwd_pipe_launch(const FwdArgs&, hipStream_t);
 // The same kernel compiled with the bias / activation epilogue in its stores.
 bool fwd_pipe_epi_supported(const FwdArgs&);
 hipError_t fwd_pipe_epi_launch(const FwdArgs&, hipStream_t);
+// The same kernel with bfloat16 x and y in memory (FwdArgs::x / y point at
+// 16-bit elements; factors and bias stay fp32), epilogue included.
+bool fwd_pipe_io16_supported(const FwdArgs&);
+hipError_t fwd_pipe_io16_launch(const FwdArgs&, hipStream_t);
 // In-place y[n,k,:] = act(y[n,k,:] + bias[k]) for variants without the epilogue.
 hipError_t bias_act_launch(float* y, const float* bias, int act, size_t N, size_t K, size_t HW,
                            hipStream_t);

@@ -40,17 +40,35 @@
 // Cuda_kernels/cp4Conv2dForward.cu:84-133 (backward-data:
 // cp4Conv2dBackwardData.cu:57-108 through swapped factors and flipped taps).
 //
-// This file is compiled twice: as is, and with CP4_PIPE_EPILOGUE defined, which
+// This file is compiled three times: as is; with CP4_PIPE_EPILOGUE defined, which
 // adds y = act(conv + bias[k]) to the stores (the bias of the lane's sixteen
 // output rows rides in registers next to the output-factor fragment) and exports
-// the entry points under the names fwd_pipe_epi_*.
+// the entry points under the names fwd_pipe_epi_*; and with CP4_PIPE_IO16, where
+// x and y are bfloat16 in memory (factors, bias and all arithmetic stay fp32):
+// a bf16 activation is its own high part, so the channel contraction needs
+// neither the split nor the three MFMAs of the lower parts, and y is rounded to
+// nearest-even as pixel pairs (entry points fwd_pipe_io16_*, epilogue included).
 #include <cstdlib>
 
 #include "cp4_internal.h"
 #include "split_bf16.h"
 
+#ifdef CP4_PIPE_IO16
+#define CP4_PIPE_EPILOGUE 1
+#endif
+
 namespace cp4 {
 namespace {
+
+#ifdef CP4_PIPE_IO16
+using io_t = unsigned short;     // bfloat16 bits
+__device__ __forceinline__ unsigned short to_io(float v) {
+  return __builtin_bit_cast(unsigned short, static_cast<__bf16>(v));   // round to nearest even
+}
+#else
+using io_t = float;
+#endif
+constexpr int kIoBytes = (int)sizeof(io_t);
 
 using namespace split;
 
@@ -170,8 +188,10 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // over channels runs on the scalar unit and no 64-bit vector adds sit between
     // the MFMAs; reads past the last channel (padded channel groups) return 0.
     const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float*>(a.x + (size_t)n * Cin * HW), 0, Cin * HW * 4, 0x00020000);
-    const unsigned sbase = (unsigned)(16 * cpq * cq) * (unsigned)HW * 4u;   // uniform byte offset
+        const_cast<io_t*>(reinterpret_cast<const io_t*>(a.x) + (size_t)n * Cin * HW), 0,
+        Cin * HW * kIoBytes, 0x00020000);
+    const unsigned sbase =
+        (unsigned)(16 * cpq * cq) * (unsigned)HW * (unsigned)kIoBytes;   // uniform byte offset
     // This wave's slice of the input factor stays in registers for the whole
     // sweep, already split: lane holds rank l32, channels 16*(cpq*cq+c) + 8*hi + e.
     constexpr int NF = FLDS ? 1 : CPQ;
@@ -199,16 +219,29 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       const int q = qbase + qa;
       valid = j < nblk && q >= 0 && q < HW && qa < QLEN;
       const int qc = q < 0 ? 0 : (q > HW - 1 ? HW - 1 : q);
-      return (unsigned)(8 * hi * HW + qc) * 4u;
+      return (unsigned)(8 * hi * HW + qc) * (unsigned)kIoBytes;
     };
-    auto ld_chunk = [&](float (&dst)[8], unsigned voff, int chunk) {   // chunk < cpq
+#ifdef CP4_PIPE_IO16
+    // ring entries hold the raw bfloat16 bits, zero-extended
+    using ring_t = unsigned;
+    auto ld_chunk = [&](ring_t (&dst)[8], unsigned voff, int chunk) {   // chunk < cpq
+      const unsigned soff = sbase + (unsigned)(16 * chunk) * (unsigned)HW * 2u;
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        dst[e] = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(
+            xrs, voff, soff + (unsigned)e * HW * 2u, 0);
+    };
+#else
+    using ring_t = float;
+    auto ld_chunk = [&](ring_t (&dst)[8], unsigned voff, int chunk) {   // chunk < cpq
       const unsigned soff = sbase + (unsigned)(16 * chunk) * (unsigned)HW * 4u;
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         dst[e] = __builtin_bit_cast(
             float, __builtin_amdgcn_raw_buffer_load_b32(xrs, voff, soff + (unsigned)e * HW * 4u, 0));
     };
-    float xb[KR][8];
+#endif
+    ring_t xb[KR][8];
     int j, qa;
     bool valid;
     unsigned xp = geom(0, j, qa, valid);
@@ -220,6 +253,23 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       const unsigned xpn = geom(r + 1 < nrounds ? r + 1 : r, jn, qan, validn);
       f32x16 acc = (f32x16)(0.f);
       auto step = [&](int ch, int u) {
+#ifdef CP4_PIPE_IO16
+        // the activations are bfloat16 already: pack pairs, multiply by the three
+        // factor parts (smallest first)
+        u32x4 xh;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) xh[d] = xb[u][2 * d] | (xb[u][2 * d + 1] << 16);
+        if (FLDS) {
+          const u32x4* fp = fbase + (size_t)(ch + u) * (6 * 32);
+          acc = mfma16(fp[128], xh, acc);
+          acc = mfma16(fp[64], xh, acc);
+          acc = mfma16(fp[0], xh, acc);
+        } else {
+          acc = mfma16(fl[FLDS ? 0 : ch + u], xh, acc);
+          acc = mfma16(fm[FLDS ? 0 : ch + u], xh, acc);
+          acc = mfma16(fh[FLDS ? 0 : ch + u], xh, acc);
+        }
+#else
         u32x4 xh, xm, xl;
         split8(xb[u], xh, xm, xl);
         if (FLDS) {
@@ -229,6 +279,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           acc = mfma_split(fh[FLDS ? 0 : ch + u], fm[FLDS ? 0 : ch + u], fl[FLDS ? 0 : ch + u], xh,
                            xm, xl, acc);
         }
+#endif
         // refill this ring slot: same round, or the first chunks of the next
         const int nxt = ch + u + KR;
         if (nxt < cpq)
@@ -332,9 +383,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         fh[rr][j] = r < R ? a.FH[tap * R + r] : 0.f;
         fw[rr][j] = r < R ? a.FW[tap * R + r] : 0.f;
       }
-    float* yn = a.y + (size_t)n * Cout * HW + (size_t)h0 * W;
-    const bool pair_stores =
-        ((W | HW) & 1) == 0 && (reinterpret_cast<uintptr_t>(a.y) & 7) == 0;   // float2 stores legal
+    io_t* yn = reinterpret_cast<io_t*>(a.y) + (size_t)n * Cout * HW + (size_t)h0 * W;
+    const bool pair_stores =                       // one store per pixel pair is legal
+        ((W | HW) & 1) == 0 && (reinterpret_cast<uintptr_t>(a.y) & (2 * kIoBytes - 1)) == 0;
     const int reach = (FS - 1) * (W + 1);          // how far past a pixel its taps read in A
 
     int frontier = 0;                              // blocks [0, frontier) of the sweep are complete
@@ -481,29 +532,39 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #endif
         // store rows: uniform row base + one 32-bit lane offset
         const int p = 64 * g - gshift + 2 * l32;       // lane's pixel pair p, p + 1
-        float* rowbase = yn + (size_t)(32 * kb) * HW;
+        io_t* rowbase = yn + (size_t)(32 * kb) * HW;
+        // the lane's pixel pair as one store: float2, or two bfloat16 in a dword
+        auto store_pair = [&](io_t* dst, float v0, float v1) {
+#ifdef CP4_PIPE_IO16
+          *reinterpret_cast<unsigned*>(dst) = (unsigned)to_io(v0) | ((unsigned)to_io(v1) << 16);
+#else
+          float2 o;
+          o.x = v0;
+          o.y = v1;
+          *reinterpret_cast<float2*>(dst) = o;
+#endif
+        };
+        auto store_one = [&](io_t* dst, float v) {
+#ifdef CP4_PIPE_IO16
+          *dst = to_io(v);
+#else
+          *dst = v;
+#endif
+        };
         if (pair_stores) {
-          // W and H*W even, y 8-byte aligned: p is even and the pair is one store
+          // W and H*W even, y aligned to a pair: p is even and the pair is one store
           if (p >= 0 && p < nvalid) {
             const unsigned lofs = (unsigned)(4 * hi * HW + p);
             if (32 * kb + 32 <= Cout) {
 #pragma unroll
-              for (int v = 0; v < 16; ++v) {
-                float2 o;
-                o.x = acc0[v];
-                o.y = acc1[v];
-                *reinterpret_cast<float2*>(rowbase + (size_t)(8 * (v >> 2) + (v & 3)) * HW + lofs) = o;
-              }
+              for (int v = 0; v < 16; ++v)
+                store_pair(rowbase + (size_t)(8 * (v >> 2) + (v & 3)) * HW + lofs, acc0[v], acc1[v]);
             } else {
 #pragma unroll
               for (int v = 0; v < 16; ++v) {
                 const int kk = 8 * (v >> 2) + (v & 3);         // + 4*hi is in lofs
-                if (32 * kb + kk + 4 * hi < Cout) {
-                  float2 o;
-                  o.x = acc0[v];
-                  o.y = acc1[v];
-                  *reinterpret_cast<float2*>(rowbase + (size_t)kk * HW + lofs) = o;
-                }
+                if (32 * kb + kk + 4 * hi < Cout)
+                  store_pair(rowbase + (size_t)kk * HW + lofs, acc0[v], acc1[v]);
               }
             }
           }
@@ -515,9 +576,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           for (int v = 0; v < 16; ++v) {
             const int kk = 8 * (v >> 2) + (v & 3);
             if (32 * kb + kk + 4 * hi < Cout) {
-              float* rp = rowbase + (size_t)kk * HW + lofs;
-              if (in0) rp[0] = acc0[v];
-              if (in1) rp[1] = acc1[v];
+              io_t* rp = rowbase + (size_t)kk * HW + lofs;
+              if (in0) store_one(rp, acc0[v]);
+              if (in1) store_one(rp + 1, acc1[v]);
             }
           }
         }
@@ -605,7 +666,10 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 
 }  // namespace
 
-#ifdef CP4_PIPE_EPILOGUE
+#if defined(CP4_PIPE_IO16)
+#define fwd_pipe_supported fwd_pipe_io16_supported
+#define fwd_pipe_launch fwd_pipe_io16_launch
+#elif defined(CP4_PIPE_EPILOGUE)
 #define fwd_pipe_supported fwd_pipe_epi_supported
 #define fwd_pipe_launch fwd_pipe_epi_launch
 #endif
@@ -613,7 +677,7 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 bool fwd_pipe_supported(const FwdArgs& a) {
   if (a.R > kRP || (a.Cin & 7) || a.Cin > 768) return false;
   if (!fits_int_indexing(a.N, a.H, a.W)) return false;
-  if ((size_t)a.Cin * a.H * a.W * sizeof(float) >= (1ull << 31)) return false;   // buffer offsets
+  if ((size_t)a.Cin * a.H * a.W * sizeof(io_t) >= (1ull << 31)) return false;   // buffer offsets
   if (a.Y != a.X || !(a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7)) return false;
   PipePlan pl;
   return plan(a, &pl);
