@@ -49,6 +49,7 @@
 // neither the split nor the three MFMAs of the lower parts, and y is rounded to
 // nearest-even as pixel pairs (entry points fwd_pipe_io16_*, epilogue included).
 #include <cstdlib>
+#include <type_traits>
 
 #include "cp4_internal.h"
 #include "split_bf16.h"
@@ -112,7 +113,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   unsigned char* ldsb = reinterpret_cast<unsigned char*>(lds);
   unsigned char* Fb = ldsb + pl.fin_off;     // Fin fragments [chunk][part][hi][r] x 16 B (CPQ == 0)
   unsigned char* Cb = ldsb + pl.cc_off;      // 3 x Cc fragment tiles
-  // [0..kMaxBlk) quarters done per block (sweep order), then 4 consumer arrival counters
+  // [0..kMaxBlk) quarters done per block (sweep order), then 4 consumer arrival
+  // counters, then the contraction counter of the split-role schedule
   int* flags = reinterpret_cast<int*>(ldsb + pl.flag_off);
 
   const int per = (pl.nWG + 7) >> 3;
@@ -157,7 +159,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   // factor does not fit the producers' registers and goes to LDS, pre-split ----
   constexpr bool FLDS = CPQ == 0;
   const int cpq = FLDS ? (Cin + 63) >> 6 : CPQ;    // 16-channel chunks per channel quarter
-  if (tid < kMaxBlk + 4) flags[tid] = 0;
+  if (tid < kMaxBlk + 8) flags[tid] = 0;
   if (FLDS) {
     for (int it = tid; it < 8 * cpq * 32; it += kThreads) {
       const int o = it >> 5, r = it & 31;          // channel octet (of the padded count), rank
@@ -373,13 +375,20 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     };
     const bool fk_cached = nkb <= kCons;
     if (fk_cached && wc < nkb) load_fk(wc);
+    // With at most 16 ranks and at most 4 channel blocks only four waves have
+    // ranks in the tap step and only four have a block to contract: the roles
+    // are then split - waves 4-7 run the taps (rank quad wc - 4), waves 0-3 the
+    // contractions - so that the tap step of one group overlaps the contraction
+    // of the previous one, and the contraction skips the empty upper rank chunk.
+    const bool split_roles = FS <= 5 && R <= 16 && nkb <= 4;   // (7x7: no registers to spare)
+    const int wq = split_roles ? (wc >= 4 ? wc - 4 : 0) : wc;     // rank quad in the tap step
     // Tap weights of this wave's 4 ranks (wave-uniform values).
     float fh[4][FS], fw[4][FS];
 #pragma unroll
     for (int rr = 0; rr < 4; ++rr)
 #pragma unroll
       for (int j = 0; j < FS; ++j) {
-        const int tap = a.flip ? FS - 1 - j : j, r = 4 * wc + rr;
+        const int tap = a.flip ? FS - 1 - j : j, r = 4 * wq + rr;
         fh[rr][j] = r < R ? a.FH[tap * R + r] : 0.f;
         fw[rr][j] = r < R ? a.FW[tap * R + r] : 0.f;
       }
@@ -390,6 +399,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 
     int frontier = 0;                              // blocks [0, frontier) of the sweep are complete
     int* arrivals = flags + kMaxBlk;               // [4] tap-step arrivals, slot = step & 3
+    int* cdone = flags + kMaxBlk + 4;              // split roles: contractions finished, all steps
 
     // Tap step i of the sweep (pixel group g), `taps` below: wait for the
     // producers of every block the group's taps touch, compute pixel 64*g + lane
@@ -435,7 +445,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       }
       // the LDS reads of RBT ranks go out together, then their arithmetic
       constexpr int RBT = FS <= 3 ? 4 : (FS == 5 ? 2 : 1);
-      const float* ab = As + (size_t)(4 * wc) * QA + h * W;
+      const float* ab = As + (size_t)(4 * wq) * QA + h * W;
       float o[4];
 #pragma unroll
       for (int r0 = 0; r0 < 4; r0 += RBT) {
@@ -472,8 +482,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       }
       // plane ((part*2 + chunk)*2 + hi)*2 + parity, 512 B each; entry lane >> 1;
       // this quad is the low or high 8 bytes of the 16-byte entry
-      unsigned char* dst = cb + ((((wc >> 2) * 2 + ((wc >> 1) & 1)) * 2 + (lane & 1)) * 512) +
-                           (lane >> 1) * 16 + (wc & 1) * 8;
+      unsigned char* dst = cb + ((((wq >> 2) * 2 + ((wq >> 1) & 1)) * 2 + (lane & 1)) * 512) +
+                           (lane >> 1) * 16 + (wq & 1) * 8;
       *reinterpret_cast<u32x2*>(dst) = ph;
       *reinterpret_cast<u32x2*>(dst + 8 * 512) = pm;
       *reinterpret_cast<u32x2*>(dst + 16 * 512) = pl2;
@@ -483,6 +493,112 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         __hip_atomic_fetch_add(&arrivals[i & 3], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     };
 
+    // Contraction ranks -> the 32 output channels of block kb for pixel group g
+    // from fragment tile cb (nch rank chunks of 16), epilogue, stores.
+    auto contract_block = [&](const unsigned char* cb, int g, int kb, auto nch, bool signal) {
+      f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
+#pragma unroll
+      for (int c = 0; c < decltype(nch)::value; ++c) {
+        const unsigned char* bp = cb + ((c * 2 + hi) * 2) * 512 + l32 * 16;
+        const u32x4 b0h = *reinterpret_cast<const u32x4*>(bp);
+        const u32x4 b1h = *reinterpret_cast<const u32x4*>(bp + 512);
+        const u32x4 b0m = *reinterpret_cast<const u32x4*>(bp + 8 * 512);
+        const u32x4 b1m = *reinterpret_cast<const u32x4*>(bp + 9 * 512);
+        const u32x4 b0l = *reinterpret_cast<const u32x4*>(bp + 16 * 512);
+        const u32x4 b1l = *reinterpret_cast<const u32x4*>(bp + 17 * 512);
+        acc0 = mfma_split(fkh[c], fkm[c], fkl[c], b0h, b0m, b0l, acc0);
+        acc1 = mfma_split(fkh[c], fkm[c], fkl[c], b1h, b1m, b1l, acc1);
+        __builtin_amdgcn_sched_barrier(0);     // one chunk's fragments live at a time
+      }
+      if (signal) {
+        // the tile has been read: the tap waves may write it again three steps on
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        if (lane == 0)
+          __hip_atomic_fetch_add(cdone, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+#ifdef CP4_PIPE_EPILOGUE
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        float o0 = acc0[v] + bs[v], o1 = acc1[v] + bs[v];
+        if (relu) {
+          o0 = o0 < 0.f ? 0.f : o0;
+          o1 = o1 < 0.f ? 0.f : o1;
+        }
+        acc0[v] = o0;
+        acc1[v] = o1;
+      }
+#endif
+      // store rows: uniform row base + one 32-bit lane offset
+      const int p = 64 * g - gshift + 2 * l32;       // lane's pixel pair p, p + 1
+      io_t* rowbase = yn + (size_t)(32 * kb) * HW;
+      // the lane's pixel pair as one store: float2, or two bfloat16 in a dword
+      auto store_pair = [&](io_t* dst, float v0, float v1) {
+#ifdef CP4_PIPE_IO16
+        *reinterpret_cast<unsigned*>(dst) = (unsigned)to_io(v0) | ((unsigned)to_io(v1) << 16);
+#else
+        float2 o;
+        o.x = v0;
+        o.y = v1;
+        *reinterpret_cast<float2*>(dst) = o;
+#endif
+      };
+      auto store_one = [&](io_t* dst, float v) {
+#ifdef CP4_PIPE_IO16
+        *dst = to_io(v);
+#else
+        *dst = v;
+#endif
+      };
+      if (pair_stores) {
+        // W and H*W even, y aligned to a pair: p is even and the pair is one store
+        if (p >= 0 && p < nvalid) {
+          const unsigned lofs = (unsigned)(4 * hi * HW + p);
+          if (32 * kb + 32 <= Cout) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+              store_pair(rowbase + (size_t)(8 * (v >> 2) + (v & 3)) * HW + lofs, acc0[v], acc1[v]);
+          } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const int kk = 8 * (v >> 2) + (v & 3);         // + 4*hi is in lofs
+              if (32 * kb + kk + 4 * hi < Cout)
+                store_pair(rowbase + (size_t)kk * HW + lofs, acc0[v], acc1[v]);
+            }
+          }
+        }
+      } else {
+        // odd widths or planes: the two pixels are stored and bounded one by one
+        const bool in0 = p >= 0 && p < nvalid, in1 = p + 1 >= 0 && p + 1 < nvalid;
+        const long lofs = (long)(4 * hi) * HW + p;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int kk = 8 * (v >> 2) + (v & 3);
+          if (32 * kb + kk + 4 * hi < Cout) {
+            io_t* rp = rowbase + (size_t)kk * HW + lofs;
+            if (in0) store_one(rp, acc0[v]);
+            if (in1) store_one(rp + 1, acc1[v]);
+          }
+        }
+      }
+    };
+
+    if (split_roles) {
+      // tile of step i is i % 3; it is written by the tap waves after the
+      // contractions of step i - 3 have read it (cdone counts nkb per step)
+      if (wc >= 4) {
+        for (int i = 0; i < ngroups; ++i) {
+          if (i >= 3) wait_ge(cdone, nkb * (i - 2));
+          taps(i, Cb + (i % 3) * kCcBuf);
+        }
+      } else if (wc < nkb) {
+        for (int i = 0; i < ngroups; ++i) {
+          const int g = rev ? ngroups - 1 - i : i;
+          wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1));
+          contract_block(Cb + (i % 3) * kCcBuf, g, wc, std::integral_constant<int, 1>{}, true);
+        }
+      }
+      return;
+    }
     // Three fragment tiles in rotation.  Iteration i: once every consumer wave
     // has arrived for step i (which also means it has finished the contraction
     // of step i-2, the last reader of the tile written next), do the tap step
@@ -504,84 +620,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       const unsigned char* cb = cb_cur;
       for (int kb = wc; kb < nkb; kb += kCons) {
         if (!fk_cached) load_fk(kb);
-        f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-          const unsigned char* bp = cb + ((c * 2 + hi) * 2) * 512 + l32 * 16;
-          const u32x4 b0h = *reinterpret_cast<const u32x4*>(bp);
-          const u32x4 b1h = *reinterpret_cast<const u32x4*>(bp + 512);
-          const u32x4 b0m = *reinterpret_cast<const u32x4*>(bp + 8 * 512);
-          const u32x4 b1m = *reinterpret_cast<const u32x4*>(bp + 9 * 512);
-          const u32x4 b0l = *reinterpret_cast<const u32x4*>(bp + 16 * 512);
-          const u32x4 b1l = *reinterpret_cast<const u32x4*>(bp + 17 * 512);
-          acc0 = mfma_split(fkh[c], fkm[c], fkl[c], b0h, b0m, b0l, acc0);
-          acc1 = mfma_split(fkh[c], fkm[c], fkl[c], b1h, b1m, b1l, acc1);
-          __builtin_amdgcn_sched_barrier(0);     // one chunk's fragments live at a time
-        }
-#ifdef CP4_PIPE_EPILOGUE
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          float o0 = acc0[v] + bs[v], o1 = acc1[v] + bs[v];
-          if (relu) {
-            o0 = o0 < 0.f ? 0.f : o0;
-            o1 = o1 < 0.f ? 0.f : o1;
-          }
-          acc0[v] = o0;
-          acc1[v] = o1;
-        }
-#endif
-        // store rows: uniform row base + one 32-bit lane offset
-        const int p = 64 * g - gshift + 2 * l32;       // lane's pixel pair p, p + 1
-        io_t* rowbase = yn + (size_t)(32 * kb) * HW;
-        // the lane's pixel pair as one store: float2, or two bfloat16 in a dword
-        auto store_pair = [&](io_t* dst, float v0, float v1) {
-#ifdef CP4_PIPE_IO16
-          *reinterpret_cast<unsigned*>(dst) = (unsigned)to_io(v0) | ((unsigned)to_io(v1) << 16);
-#else
-          float2 o;
-          o.x = v0;
-          o.y = v1;
-          *reinterpret_cast<float2*>(dst) = o;
-#endif
-        };
-        auto store_one = [&](io_t* dst, float v) {
-#ifdef CP4_PIPE_IO16
-          *dst = to_io(v);
-#else
-          *dst = v;
-#endif
-        };
-        if (pair_stores) {
-          // W and H*W even, y aligned to a pair: p is even and the pair is one store
-          if (p >= 0 && p < nvalid) {
-            const unsigned lofs = (unsigned)(4 * hi * HW + p);
-            if (32 * kb + 32 <= Cout) {
-#pragma unroll
-              for (int v = 0; v < 16; ++v)
-                store_pair(rowbase + (size_t)(8 * (v >> 2) + (v & 3)) * HW + lofs, acc0[v], acc1[v]);
-            } else {
-#pragma unroll
-              for (int v = 0; v < 16; ++v) {
-                const int kk = 8 * (v >> 2) + (v & 3);         // + 4*hi is in lofs
-                if (32 * kb + kk + 4 * hi < Cout)
-                  store_pair(rowbase + (size_t)kk * HW + lofs, acc0[v], acc1[v]);
-              }
-            }
-          }
-        } else {
-          // odd widths or planes: the two pixels are stored and bounded one by one
-          const bool in0 = p >= 0 && p < nvalid, in1 = p + 1 >= 0 && p + 1 < nvalid;
-          const long lofs = (long)(4 * hi) * HW + p;
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int kk = 8 * (v >> 2) + (v & 3);
-            if (32 * kb + kk + 4 * hi < Cout) {
-              io_t* rp = rowbase + (size_t)kk * HW + lofs;
-              if (in0) store_one(rp, acc0[v]);
-              if (in1) store_one(rp + 1, acc1[v]);
-            }
-          }
-        }
+        contract_block(cb, g, kb, std::integral_constant<int, 2>{}, false);
       }
       STAMP(5 + 4 * i)
       if (i + 1 < ngroups && !early) taps(i + 1, cb_next);
@@ -604,7 +643,7 @@ bool layout(const FwdArgs& a, int TH, PipePlan* pl) {
   const size_t a_bytes = (size_t)kRP * QA * sizeof(float);
   // above 256 input channels: pre-split factor fragments, 192 B per (padded) channel
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
-  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 4) * sizeof(int);
+  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 8) * sizeof(int);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
