@@ -195,6 +195,10 @@ EDGE = [
     (4, 32, 7, 7, 1, 48, 3, 3, 8),
     (3, 64, 13, 13, 1, 32, 3, 3, 16),
     (2, 16, 27, 27, 2, 16, 5, 5, 4),
+    # at most 16 ranks and 4 output-channel blocks: consumer waves in split roles
+    (2, 64, 20, 22, 1, 80, 3, 3, 12),     # three channel blocks, the last partly filled
+    (1, 32, 40, 40, 0, 128, 1, 1, 16),    # 1x1, four blocks
+    (3, 16, 30, 34, 2, 96, 5, 5, 9),      # 5x5, several groups per strip
     # many small planes (wave-per-plane tap kernel, one partial per image)
     (64, 32, 8, 8, 1, 48, 3, 3, 20),
     (70, 16, 6, 10, 2, 16, 5, 5, 40),     # two rank tiles, the second partly filled
