@@ -114,7 +114,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   unsigned char* Fb = ldsb + pl.fin_off;     // Fin fragments [chunk][part][hi][r] x 16 B (CPQ == 0)
   unsigned char* Cb = ldsb + pl.cc_off;      // 3 x Cc fragment tiles
   // [0..kMaxBlk) quarters done per block (sweep order), then 4 consumer arrival
-  // counters, then the contraction counter of the split-role schedule
+  // counters, then the 4 contraction counters of the split-role schedule
   int* flags = reinterpret_cast<int*>(ldsb + pl.flag_off);
 
   const int per = (pl.nWG + 7) >> 3;
@@ -399,7 +399,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 
     int frontier = 0;                              // blocks [0, frontier) of the sweep are complete
     int* arrivals = flags + kMaxBlk;               // [4] tap-step arrivals, slot = step & 3
-    int* cdone = flags + kMaxBlk + 4;              // split roles: contractions finished, all steps
+    int* cdone = flags + kMaxBlk + 4;              // [4] split roles: contractions done, slot = step & 3
 
     // Tap step i of the sweep (pixel group g), `taps` below: wait for the
     // producers of every block the group's taps touch, compute pixel 64*g + lane
@@ -495,7 +495,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 
     // Contraction ranks -> the 32 output channels of block kb for pixel group g
     // from fragment tile cb (nch rank chunks of 16), epilogue, stores.
-    auto contract_block = [&](const unsigned char* cb, int g, int kb, auto nch, bool signal) {
+    auto contract_block = [&](const unsigned char* cb, int g, int kb, auto nch, bool signal,
+                              int step) {
       f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
 #pragma unroll
       for (int c = 0; c < decltype(nch)::value; ++c) {
@@ -514,7 +515,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         // the tile has been read: the tap waves may write it again three steps on
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (lane == 0)
-          __hip_atomic_fetch_add(cdone, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+          __hip_atomic_fetch_add(&cdone[step & 3], 1, __ATOMIC_RELEASE,
+                                 __HIP_MEMORY_SCOPE_WORKGROUP);
       }
 #ifdef CP4_PIPE_EPILOGUE
 #pragma unroll
@@ -583,18 +585,21 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     };
 
     if (split_roles) {
-      // tile of step i is i % 3; it is written by the tap waves after the
-      // contractions of step i - 3 have read it (cdone counts nkb per step)
+      // The tile of step i is i % 3; the tap waves write it after every
+      // contraction wave has read it for step i - 3.  cdone[s] counts one per
+      // contraction wave for the steps = s mod 4 (a single running total would
+      // not do: a fast wave's later steps could stand in for a slow wave's
+      // missing one); like the arrivals, a slot cannot run a whole cycle ahead.
       if (wc >= 4) {
         for (int i = 0; i < ngroups; ++i) {
-          if (i >= 3) wait_ge(cdone, nkb * (i - 2));
+          if (i >= 3) wait_ge(&cdone[(i - 3) & 3], nkb * (((i - 3) >> 2) + 1));
           taps(i, Cb + (i % 3) * kCcBuf);
         }
       } else if (wc < nkb) {
         for (int i = 0; i < ngroups; ++i) {
           const int g = rev ? ngroups - 1 - i : i;
           wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1));
-          contract_block(Cb + (i % 3) * kCcBuf, g, wc, std::integral_constant<int, 1>{}, true);
+          contract_block(Cb + (i % 3) * kCcBuf, g, wc, std::integral_constant<int, 1>{}, true, i);
         }
       }
       return;
@@ -620,7 +625,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       const unsigned char* cb = cb_cur;
       for (int kb = wc; kb < nkb; kb += kCons) {
         if (!fk_cached) load_fk(kb);
-        contract_block(cb, g, kb, std::integral_constant<int, 2>{}, false);
+        contract_block(cb, g, kb, std::integral_constant<int, 2>{}, false, i);
       }
       STAMP(5 + 4 * i)
       if (i + 1 < ngroups && !early) taps(i + 1, cb_next);

@@ -199,6 +199,8 @@ EDGE = [
     (2, 64, 20, 22, 1, 80, 3, 3, 12),     # three channel blocks, the last partly filled
     (1, 32, 40, 40, 0, 128, 1, 1, 16),    # 1x1, four blocks
     (3, 16, 30, 34, 2, 96, 5, 5, 9),      # 5x5, several groups per strip
+    (2, 64, 6, 288, 1, 128, 3, 3, 16),    # long rows: five groups per strip, fragment tiles reused
+    (1, 32, 3, 576, 0, 64, 1, 1, 8),      # ten groups per strip
     # many small planes (wave-per-plane tap kernel, one partial per image)
     (64, 32, 8, 8, 1, 48, 3, 3, 20),
     (70, 16, 6, 10, 2, 16, 5, 5, 40),     # two rank tiles, the second partly filled
