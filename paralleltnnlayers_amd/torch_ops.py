@@ -53,14 +53,23 @@ class CP4Conv2dFunction(torch.autograd.Function):
         return (dx,) + grads + (None, dbias, None)
 
 
-def cp4_conv2d(x, FK, FC, FH, FW, pad, bias=None, activation=None):
-    """Functional form: differentiable fused CP4 convolution (NCHW, stride 1), with
-    the optional bias [T] and activation ("relu") fused into the forward stores."""
-    return CP4Conv2dFunction.apply(x, FK, FC, FH, FW, pad, bias, activation)
+def cp4_conv2d(x, FK, FC, FH, FW, pad, bias=None, activation=None, stride=1):
+    """Functional form: differentiable fused CP4 convolution (NCHW), with the
+    optional bias [T] and activation ("relu") fused into the forward stores.
+
+    The kernels are stride 1 (as the reference's, whose tensor_shape has no stride
+    field).  ``stride`` > 1 keeps every stride-th row and column of that result -
+    for "same" padding exactly the strided convolution the reference's Python
+    layers build with ``strides`` (test/layers.py:264-277) - at the cost of
+    computing the skipped outputs; autograd scatters the upstream gradient back
+    into the full-resolution one.
+    """
+    y = CP4Conv2dFunction.apply(x, FK, FC, FH, FW, pad, bias, activation)
+    return y if stride == 1 else y[:, :, ::stride, ::stride]
 
 
 class CP4Conv2d(torch.nn.Module):
-    """A rank-R CP4-decomposed convolution layer, "same" padding, stride 1.
+    """A rank-R CP4-decomposed convolution layer, "same" padding.
 
     Equivalent dense filter: K[t,c,y,x] = sum_r FK[t,r] FC[c,r] FH[y,r] FW[x,r]
     (Cuda_kernels/Utils.cu:55-62).  Factors start as normal(0, s) with s chosen
@@ -69,7 +78,7 @@ class CP4Conv2d(torch.nn.Module):
     """
 
     def __init__(self, in_channels, out_channels, kernel_size, rank, device="cuda", bias=False,
-                 activation=None):
+                 activation=None, stride=1):
         super().__init__()
         if kernel_size % 2 != 1:
             raise ValueError("kernel_size must be odd (same padding)")
@@ -82,10 +91,11 @@ class CP4Conv2d(torch.nn.Module):
         self.FH, self.FW = mk(kernel_size), mk(kernel_size)
         self.bias = torch.nn.Parameter(torch.zeros(out_channels, device=device)) if bias else None
         self.activation = activation
+        self.stride = stride
 
     def forward(self, x):
         return cp4_conv2d(x, self.FK, self.FC, self.FH, self.FW, self.pad, self.bias,
-                          self.activation)
+                          self.activation, self.stride)
 
     def dense_filter(self):
         """The recomposed [T,C,Y,X] filter (on the device, through cp4_recompose)."""

@@ -86,3 +86,27 @@ def test_layer_trains(ops):
     assert K.shape == (16, 16, 3, 3)
     dense = torch.nn.functional.conv2d(x, K, padding=1)
     assert (layer(x).detach() - dense).abs().max() <= 1e-4 * dense.abs().max()
+
+
+def test_strided_layer_matches_dense_strided_conv(ops):
+    """stride 2 = every second row and column of the stride-1 result, which for
+    "same" padding is PyTorch's strided convolution with the recomposed filter;
+    the gradients flow through the subsampling."""
+    g = torch.Generator(device="cuda").manual_seed(11)
+    mk = lambda *s: torch.randn(*s, device="cuda", generator=g)
+    N, C, H, W, T, Y, R = 2, 16, 13, 16, 24, 3, 8
+    x = mk(N, C, H, W).requires_grad_()
+    fac = [(mk(d, R) / R ** 0.25).requires_grad_() for d in (T, C, Y, Y)]
+    y = ops.cp4_conv2d(x, *fac, 1, stride=2)
+    dy = mk(*y.shape)
+    y.backward(dy)
+    xd = x.detach().double().requires_grad_()
+    fd = [f.detach().double().requires_grad_() for f in fac]
+    yd = torch.nn.functional.conv2d(xd, recomposed(*fd), padding=1, stride=2)
+    assert yd.shape == y.shape
+    yd.backward(dy.double())
+    assert (y.detach().double() - yd.detach()).abs().max() <= 1e-4 * yd.detach().abs().max()
+    for name, a, b in zip(("dx", "dFK", "dFC", "dFH", "dFW"), [x.grad] + [f.grad for f in fac],
+                          [xd.grad] + [f.grad for f in fd]):
+        tol = 1e-4 if name == "dx" else 1e-3
+        assert (a.double() - b).abs().max() <= tol * b.abs().max(), name
