@@ -83,6 +83,17 @@ cp4_status cp4_conv2d_backward_data_bf16(const cp4_shape* shape, const void* dy_
                                          const float* FK, const float* FC,
                                          const float* FH, const float* FW,
                                          void* dx_bf16, cp4_stream stream);
+/* Backward-filter with bfloat16 x and dy in memory; factors, gradients, the
+ * workspace (cp4_conv2d_backward_filter_workspace_bytes) and all arithmetic stay
+ * fp32.  Matrix-core path only: Rank <= 64, C and T multiples of 16
+ * (cp4_bf16_backward_filter_supported); CP4_ERR_UNSUPPORTED otherwise. */
+int cp4_bf16_backward_filter_supported(const cp4_shape* shape);
+cp4_status cp4_conv2d_backward_filter_bf16(const cp4_shape* shape, const void* x_bf16,
+                                           const void* dy_bf16, const float* FK,
+                                           const float* FC, const float* FH,
+                                           const float* FW, float* dFK, float* dFC,
+                                           float* dFH, float* dFW, void* workspace,
+                                           size_t workspace_bytes, cp4_stream stream);
 
 /* Replaces cp4_conv2d_backward_data_gpu
  * (Cuda_kernels/cp4Conv2dBackwardData.cuh:7-14, .cu:112-282):

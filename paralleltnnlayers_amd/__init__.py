@@ -7,7 +7,7 @@ layer under ``csrc/host``.  There is no CPU or PyTorch fallback: importing
 ``paralleltnnlayers_amd.capi`` without the built library raises.
 """
 from .capi import (Shape, Cp4Error, lib, library_path, conv2d_forward, conv2d_forward_bias_act, conv2d_forward_bf16,
-                   conv2d_backward_data_bf16, bf16_supported,
+                   conv2d_backward_data_bf16, conv2d_backward_filter_bf16, bf16_supported,
                    conv2d_backward_data, conv2d_backward_filter,
                    conv2d_backward_filter_full, backward_filter_workspace_bytes,
                    time_forward, time_backward_data, time_backward_filter,

@@ -19,12 +19,34 @@
 #include "cp4_internal.h"
 #include "split_bf16.h"
 
+// Compiled a second time with CP4_BWF_IO16: x and dy are then bfloat16 in memory
+// (factors, intermediates and gradients stay fp32).  Only the split-bf16 kernels
+// exist in that build (contract_split_kernel, grad_split_kernel): a bf16
+// activation is its own high part, so neither splits its activations and both
+// run three MFMAs per product instead of six; the entry points are exported as
+// bwd_filter_mfma_io16_*.
+#ifdef CP4_BWF_IO16
+#define bwd_filter_mfma_supported bwd_filter_mfma_io16_supported
+#define bwd_filter_mfma_workspace_bytes bwd_filter_mfma_io16_workspace_bytes
+#define bwd_filter_mfma_launch bwd_filter_mfma_io16_launch
+#endif
+
 namespace cp4 {
 namespace {
 
+#ifdef CP4_BWF_IO16
+using act_t = unsigned short;      // bfloat16 bits
+[[maybe_unused]] __device__ __forceinline__ float act_to_f32(act_t v) {
+  return __uint_as_float((unsigned)v << 16);
+}
+#else
+using act_t = float;
+[[maybe_unused]] __device__ __forceinline__ float act_to_f32(act_t v) { return v; }
+#endif
+
 using split::f32x16;
 
-__device__ __forceinline__ f32x16 mfma32(float a, float b, f32x16 c) {
+[[maybe_unused]] __device__ __forceinline__ f32x16 mfma32(float a, float b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
 
@@ -37,12 +59,12 @@ __device__ __forceinline__ f32x16 mfma32(float a, float b, f32x16 c) {
 #define BSTAMP(dbg, slot, wg, nw, i)
 #endif
 constexpr int kCT = 256;   // gradient-GEMM workgroup: 4 waves
-constexpr int kCW = 256;   // contraction workgroup: 4 waves (one per SIMD) sharing one 32-rank factor tile
-constexpr int kPF = 8;     // channel pairs per prefetch chunk in the contraction
+[[maybe_unused]] constexpr int kCW = 256;   // contraction workgroup: 4 waves (one per SIMD) sharing one 32-rank factor tile
+[[maybe_unused]] constexpr int kPF = 8;     // channel pairs per prefetch chunk in the contraction
 
 // ---- 1. Z[n,r,p] = sum_c F[c,r] src[n,c,p] ---------------------------------
 struct ContractArgs {
-  const float* src[2];   // x, dy
+  const act_t* src[2];   // x, dy
   const float* F[2];     // FC, FK
   float* Z[2];           // A, G3
   int Cin[2];
@@ -51,6 +73,7 @@ struct ContractArgs {
   long long* dbg;
 };
 
+#ifndef CP4_BWF_IO16
 __global__ __launch_bounds__(kCW) void contract_mfma_kernel(ContractArgs a) {
   extern __shared__ float Fs[];   // [Cin][32]: the 32-rank tile mb of F, zero-padded
   const int which = blockIdx.y, mb = blockIdx.z;
@@ -125,6 +148,8 @@ __global__ __launch_bounds__(kCW) void contract_mfma_kernel(ContractArgs a) {
   }
 }
 
+#endif  // !CP4_BWF_IO16
+
 // ---- 1'. the same contraction as exact fp32 products on the bf16 matrix cores
 // (channel counts that are multiples of 16).  A workgroup of 8 waves shares the
 // 32-rank factor tile as pre-split MFMA A fragments in LDS
@@ -163,11 +188,16 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
   const int pc = p < HW ? p : HW - 1;
   // lane's channel 16*chunk + 8*hi + e
   const int nch = (Cin >> 4) / ks, c0 = part * nch;     // this wave's chunks c0 .. c0 + nch - 1
-  const float* xp = a.src[which] + ((size_t)n * Cin + 16 * c0 + 8 * hi) * HW + pc;
-  float xb[kSplitRing][8];
-  auto ld_chunk = [&](float (&dst)[8], int ch) {
+  const act_t* xp = a.src[which] + ((size_t)n * Cin + 16 * c0 + 8 * hi) * HW + pc;
+#ifdef CP4_BWF_IO16
+  using ring_t = unsigned;     // raw bfloat16 bits, zero-extended
+#else
+  using ring_t = float;
+#endif
+  ring_t xb[kSplitRing][8];
+  auto ld_chunk = [&](ring_t (&dst)[8], int ch) {
     ch = ch < nch ? ch : nch - 1;                     // clamped, not branched
-    const float* base = xp + (size_t)(16 * ch) * HW;
+    const act_t* base = xp + (size_t)(16 * ch) * HW;
 #pragma unroll
     for (int e = 0; e < 8; ++e) dst[e] = base[(size_t)e * HW];
   };
@@ -207,7 +237,17 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
   // they do not wait for each other), the vector ALU splits chunk c+1.
   f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
   u32x4 xh, xm, xl;
+#ifdef CP4_BWF_IO16
+  // bfloat16 activations: the chunk's B operand is the packed bits themselves
+  auto pack8 = [](const ring_t (&v)[8], u32x4& h) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) h[d] = v[2 * d] | (v[2 * d + 1] << 16);
+  };
+  pack8(xb[0], xh);
+  xm = xl = xh;                 // unused
+#else
   split8(xb[0], xh, xm, xl);
+#endif
   BSTAMP(a.dbg, 0, dwg, 8, 5)
   ld_chunk(xb[0], kSplitRing);
   for (int ch = 0; ch < nch; ch += kSplitRing) {
@@ -219,7 +259,14 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
         const u32x4* fp = fbase + (size_t)(c0 + c) * (6 * 32);
         const u32x4 fh = fp[0], fm = fp[64], fl = fp[128];
         // one MFMA, then a quarter of the next chunk's split, pinned in this order
-        float (&nx)[8] = xb[(u + 1) % kSplitRing];
+        ring_t (&nx)[8] = xb[(u + 1) % kSplitRing];
+#ifdef CP4_BWF_IO16
+        acc0 = mfma16(fl, xh, acc0);
+        acc1 = mfma16(fm, xh, acc1);
+        acc0 = mfma16(fh, xh, acc0);
+        pack8(nx, nh);
+        ld_chunk(nx, c + 1 + kSplitRing);             // refill the slot just packed
+#else
         auto piece = [&](int d) {
           const float x0 = nx[2 * d], x1 = nx[2 * d + 1];
           nh[d] = pack_hi16(x0, x1);
@@ -242,6 +289,7 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
         acc0 = mfma16(fh, xm, acc0);
         acc1 = mfma16(fh, xh, acc1);
         ld_chunk(nx, c + 1 + kSplitRing);             // refill the slot just split
+#endif
       }
       xh = nh;
       xm = nm;
@@ -723,7 +771,7 @@ hipError_t launch_taps_column(const float* A, const float* G3, const BwdFilterAr
 
 // ---- 3a. partial[s][d][r] = sum_{p in split s} act[n,d,p] Z[n,r,p] ----------
 struct GradArgs {
-  const float* act[2];   // dy, x
+  const act_t* act[2];   // dy, x
   const float* Z[2];     // Cc, G1
   float* part[2];        // [S][D][R]
   int D[2];
@@ -731,8 +779,9 @@ struct GradArgs {
   long long* dbg;
 };
 
-constexpr int kLd = 34;   // LDS row stride of the 32-pixel operand tiles (conflict-free)
+[[maybe_unused]] constexpr int kLd = 34;   // LDS row stride of the 32-pixel operand tiles (conflict-free)
 
+#ifndef CP4_BWF_IO16
 template <int RB>
 __global__ __launch_bounds__(kCT) void grad_gemm_kernel(GradArgs a) {
   __shared__ float Zs[32 * RB * kLd];
@@ -803,6 +852,8 @@ __global__ __launch_bounds__(kCT) void grad_gemm_kernel(GradArgs a) {
     }
 }
 
+#endif  // !CP4_BWF_IO16
+
 // ---- 3a'. the same gradient GEMMs as exact split-bf16 products (H*W a
 // multiple of 4 so that rows can be moved as float4).  Per 32-pixel chunk the
 // workgroup splits the Z tile once, cooperatively, straight from global memory
@@ -828,7 +879,7 @@ __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
   BSTAMP(a.dbg, 1, dwg, 4, 0)
   const int nch_total = (HW + 31) >> 5;
   const int ch0 = ps * a.cps, ch1 = min(nch_total, ch0 + a.cps);
-  const float* actn = a.act[which] + (size_t)n * D * HW;
+  const act_t* actn = a.act[which] + (size_t)n * D * HW;
   const float* zn = a.Z[which] + (size_t)n * R * HW;
   // activation tile: lane moves float4; 8 lanes cover one 32-pixel row, 8 rows per load
   const int arow = lane >> 3, acol = 4 * (lane & 7);
@@ -836,6 +887,27 @@ __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
   const int zr = tid >> 2, zo = tid & 3;             // 64 rows x 4 octets = 256 threads
   const bool zmine = zr < 32 * RB;
   float4 av[4], zv[2];
+#ifdef CP4_BWF_IO16
+  // four bfloat16 activations (one 8-byte load when VEC) widened to fp32
+  auto load4_act = [&](const act_t* row, int p) {
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (VEC) {
+      if (p < HW) {
+        const uint2 b = *reinterpret_cast<const uint2*>(row + p);
+        v.x = __uint_as_float(b.x << 16);
+        v.y = __uint_as_float(b.x & 0xffff0000u);
+        v.z = __uint_as_float(b.y << 16);
+        v.w = __uint_as_float(b.y & 0xffff0000u);
+      }
+    } else {
+      if (p < HW) v.x = act_to_f32(row[p]);
+      if (p + 1 < HW) v.y = act_to_f32(row[p + 1]);
+      if (p + 2 < HW) v.z = act_to_f32(row[p + 2]);
+      if (p + 3 < HW) v.w = act_to_f32(row[p + 3]);
+    }
+    return v;
+  };
+#endif
   // VEC: H*W is a multiple of 4 and the operands are 16-byte aligned, rows move
   // as float4; otherwise element by element with per-pixel bounds.
   auto load4 = [&](const float* row, int p) {
@@ -855,7 +927,11 @@ __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int d = d0 + 8 * j + arow;
+#ifdef CP4_BWF_IO16
+      av[j] = d < D ? load4_act(actn + (size_t)d * HW, p) : make_float4(0.f, 0.f, 0.f, 0.f);
+#else
       av[j] = d < D ? load4(actn + (size_t)d * HW, p) : make_float4(0.f, 0.f, 0.f, 0.f);
+#endif
     }
     const int pz = ch * 32 + 8 * zo;
 #pragma unroll
@@ -894,6 +970,19 @@ __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
       const float4 a0 = *reinterpret_cast<const float4*>(ap);
       const float4 a1 = *reinterpret_cast<const float4*>(ap + 4);
       const float v[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#ifdef CP4_BWF_IO16
+      // the activations are bfloat16 values: their high part is all of them
+      u32x4 ah;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) ah[d] = pack_hi16(v[2 * d], v[2 * d + 1]);
+#pragma unroll
+      for (int mb = 0; mb < RB; ++mb) {
+        const u32x4* zp = &Zf[buf][((mb * 2 + st) * 3 * 2 + hi) * 32 + l32];
+        acc[mb] = mfma16(ah, zp[128], acc[mb]);
+        acc[mb] = mfma16(ah, zp[64], acc[mb]);
+        acc[mb] = mfma16(ah, zp[0], acc[mb]);
+      }
+#else
       u32x4 ah, am, al;
       split8(v, ah, am, al);
 #pragma unroll
@@ -901,6 +990,7 @@ __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
         const u32x4* zp = &Zf[buf][((mb * 2 + st) * 3 * 2 + hi) * 32 + l32];
         acc[mb] = mfma_split(ah, am, al, zp[0], zp[64], zp[128], acc[mb]);
       }
+#endif
     }
   }
   BSTAMP(a.dbg, 1, dwg, 4, 4)
@@ -1023,6 +1113,9 @@ bool bwd_filter_mfma_supported(const cp4_shape& s) {
   // odd planes need the split contraction (scalar loads): channel counts multiples of 16
   const bool odd_plane_ok = (s.C & 15) == 0 && (s.T & 15) == 0 &&
                             (size_t)(s.C > s.T ? s.C : s.T) * 192 <= 160 * 1024;
+#ifdef CP4_BWF_IO16
+  if (!odd_plane_ok) return false;      // the bfloat16 build has the split kernels only
+#endif
   return s.Rank <= 64 && fits_int_indexing((int)s.N, (int)s.H, (int)s.W) &&
          (((s.H * s.W) & 1) == 0 || odd_plane_ok) && (s.C & 1) == 0 &&
          (s.T & 1) == 0 &&
@@ -1047,8 +1140,11 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   float* pW = pH + (size_t)p.St * a.Y * R;
 
   ContractArgs c{};
-  c.src[0] = a.x; c.F[0] = a.FC; c.Z[0] = A; c.Cin[0] = a.C;
-  c.src[1] = a.dy; c.F[1] = a.FK; c.Z[1] = G3; c.Cin[1] = a.T;
+  // (bfloat16 build: BwdFilterArgs::x / dy point at 16-bit elements)
+  const act_t* ax = reinterpret_cast<const act_t*>(a.x);
+  const act_t* ady = reinterpret_cast<const act_t*>(a.dy);
+  c.src[0] = ax; c.F[0] = a.FC; c.Z[0] = A; c.Cin[0] = a.C;
+  c.src[1] = ady; c.F[1] = a.FK; c.Z[1] = G3; c.Cin[1] = a.T;
   c.N = N; c.R = R; c.RP = p.RP; c.HW = HW; c.npb = p.npb;
   c.items = N * p.npb;
 #ifdef CP4_DEBUG_PHASES
@@ -1078,12 +1174,16 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
     contract_split_kernel<<<dim3((unsigned)((slots + kSW / 64 - 1) / (kSW / 64)), 2, p.RP / 32),
                             kSW, smem, st>>>(c);
   } else {
+#ifdef CP4_BWF_IO16
+    return hipErrorInvalidValue;      // excluded by bwd_filter_mfma_io16_supported
+#else
     const size_t smem = (size_t)cmax * 32 * sizeof(float);
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_mfma_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
     contract_mfma_kernel<<<dim3((c.items + kCW / 64 - 1) / (kCW / 64), 2, p.RP / 32), kCW, smem,
                            st>>>(c);
+#endif
   }
 
   const bool wave_taps = p.wave_taps, column_taps = p.column_taps;
@@ -1118,20 +1218,29 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   }
 
   GradArgs g{};
-  g.act[0] = a.dy; g.Z[0] = Cc; g.part[0] = pK; g.D[0] = a.T;
-  g.act[1] = a.x; g.Z[1] = G1; g.part[1] = pC; g.D[1] = a.C;
+  g.act[0] = ady; g.Z[0] = Cc; g.part[0] = pK; g.D[0] = a.T;
+  g.act[1] = ax; g.Z[1] = G1; g.part[1] = pC; g.D[1] = a.C;
   g.N = N; g.R = R; g.RP = p.RP; g.HW = HW; g.PS = p.PS; g.cps = p.cps;
 #ifdef CP4_DEBUG_PHASES
   g.dbg = getenv("CP4_DBG_PTR") ? reinterpret_cast<long long*>(strtoull(getenv("CP4_DBG_PTR"), nullptr, 10)) : nullptr;
 #endif
   const int dmax = a.T > a.C ? a.T : a.C;
   const dim3 ggrid(p.S, (dmax + 127) / 128, 2);
-  const bool grad_split = (HW & 3) == 0 &&
-                          ((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.dy) |
-                            reinterpret_cast<uintptr_t>(ws)) & 15) == 0;
+  // rows of four pixels as one load: 16 bytes of fp32, 8 bytes of bfloat16
+  const bool grad_split =
+      (HW & 3) == 0 && (reinterpret_cast<uintptr_t>(ws) & 15) == 0 &&
+      ((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.dy)) &
+       (4 * sizeof(act_t) - 1)) == 0;
   if (grad_split) {
     if (p.RP == 32) grad_split_kernel<1, true><<<ggrid, kCT, 0, st>>>(g);
     else grad_split_kernel<2, true><<<ggrid, kCT, 0, st>>>(g);
+#ifdef CP4_BWF_IO16
+  } else {
+    // the element-wise staging takes any plane size and alignment
+    if (p.RP == 32) grad_split_kernel<1, false><<<ggrid, kCT, 0, st>>>(g);
+    else grad_split_kernel<2, false><<<ggrid, kCT, 0, st>>>(g);
+  }
+#else
   } else if (HW & 1) {
     // odd planes: the float2 staging of the fp32 kernel does not apply
     if (p.RP == 32) grad_split_kernel<1, false><<<ggrid, kCT, 0, st>>>(g);
@@ -1140,6 +1249,7 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
     if (p.RP == 32) grad_gemm_kernel<1><<<ggrid, kCT, 0, st>>>(g);
     else grad_gemm_kernel<2><<<ggrid, kCT, 0, st>>>(g);
   }
+#endif
 
   ReduceArgs r{};
   const float* parts[4] = {pK, pC, pH, pW};

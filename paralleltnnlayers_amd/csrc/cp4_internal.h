@@ -71,6 +71,11 @@ hipError_t bwd_filter_launch(const BwdFilterArgs&, hipStream_t);
 bool bwd_filter_mfma_supported(const cp4_shape&);
 size_t bwd_filter_mfma_workspace_bytes(const cp4_shape&);
 hipError_t bwd_filter_mfma_launch(const BwdFilterArgs&, hipStream_t);
+// The same with bfloat16 x and dy in memory (BwdFilterArgs::x / dy point at 16-bit
+// elements); split-bf16 kernels only: C and T multiples of 16.
+bool bwd_filter_mfma_io16_supported(const cp4_shape&);
+size_t bwd_filter_mfma_io16_workspace_bytes(const cp4_shape&);
+hipError_t bwd_filter_mfma_io16_launch(const BwdFilterArgs&, hipStream_t);
 hipError_t bwd_filter_full_launch(const cp4_shape&, const float* x,
                                   const float* dy, float* dK, int accumulate,
                                   hipStream_t);

@@ -99,3 +99,54 @@ def test_bf16_unsupported_shapes_are_refused(cp4):
     with pytest.raises(cp4.Cp4Error) as e:
         cp4.conv2d_forward_bf16(x, *fac, pad=1)
     assert e.value.status == cp4.capi.ERR_UNSUPPORTED
+
+
+def assert_gradient_close(got, want, what):
+    scale = float(np.abs(want).max())
+    err = np.abs(got - want)
+    assert np.all(err <= 1e-3 * np.abs(want) + 1e-4 * scale), f"{what}: elementwise {err.max():.3e}"
+    assert err.max() <= 1e-3 * scale, f"{what}: normalised {err.max() / scale:.3e}"
+
+
+# (N, C, H, W, pad, T, Y, R): channel counts multiples of 16
+FILTER_SHAPES = [
+    (2, 64, 28, 28, 1, 64, 3, 16),
+    (1, 256, 56, 56, 1, 256, 3, 32),
+    (1, 320, 14, 14, 1, 304, 3, 32),
+    (2, 16, 32, 32, 0, 16, 1, 8),
+    (4, 32, 7, 7, 1, 48, 3, 8),          # odd plane: element-wise staging
+    (8, 256, 14, 14, 1, 256, 3, 64),     # two rank tiles, the backward-filter workload's shape
+    (3, 48, 9, 10, 2, 80, 5, 20),        # plane not a multiple of 4 pixels
+]
+
+
+@pytest.mark.parametrize("dims", FILTER_SHAPES, ids=lambda d: "x".join(map(str, d)))
+def test_backward_filter_bf16(cp4, oracle, dims):
+    """x and dy bfloat16 in memory, gradients fp32: the same bar as the fp32 pass
+    (the arithmetic is the same exact-product, fp32-accumulate one)."""
+    N, C, H, W, pad, T, Y, R = dims
+    rng = np.random.default_rng(sum(dims) + 1)
+    x = bf16_values(rng, (N, C, H, W))
+    dy = bf16_values(rng, (N, T, H, W))
+    fac = [(rng.standard_normal((d, R)) / np.sqrt(R)).astype(np.float32) for d in (T, C, Y, Y)]
+    f = [torch.from_numpy(v).cuda() for v in fac]
+    got = cp4.conv2d_backward_filter_bf16(x.cuda(), dy.cuda(), *f, pad=pad)
+    want = oracle.backward_filter(x.float().numpy(), dy.float().numpy(), *fac, pad)
+    for g, wnt, name in zip(got, want, ("dFK", "dFC", "dFH", "dFW")):
+        assert g.dtype == torch.float32
+        assert_gradient_close(g.cpu().numpy(), wnt, name)
+    # bit-identical to the fp32 entry point on the widened inputs? not required: the
+    # fp32 path splits its activations into three parts whose lower two are zero here,
+    # so the sums agree to rounding order
+    ref = cp4.conv2d_backward_filter(x.float().cuda(), dy.float().cuda(), *f, pad=pad)
+    for g, r in zip(got, ref):
+        assert (g - r).abs().max().item() <= 1e-5 * r.abs().max().item()
+
+
+def test_backward_filter_bf16_unsupported(cp4):
+    x = torch.randn(1, 24, 6, 6, device="cuda").to(torch.bfloat16)      # 24 channels: not a multiple of 16
+    dy = torch.randn(1, 16, 6, 6, device="cuda").to(torch.bfloat16)
+    fac = [torch.randn(d, 4, device="cuda") for d in (16, 24, 3, 3)]
+    with pytest.raises(cp4.Cp4Error) as e:
+        cp4.conv2d_backward_filter_bf16(x, dy, *fac, pad=1)
+    assert e.value.status == cp4.capi.ERR_UNSUPPORTED
