@@ -176,6 +176,10 @@ def bf16_supported(s, backward_data=False):
     return bool(lib().cp4_bf16_supported(ctypes.byref(s), int(backward_data)))
 
 
+def bf16_backward_filter_supported(s):
+    return bool(lib().cp4_bf16_backward_filter_supported(ctypes.byref(s)))
+
+
 def conv2d_forward_bf16(x, FK, FC, FH, FW, bias=None, activation=None, pad=1, out=None,
                         stream=None):
     """bfloat16 x -> bfloat16 y = act(conv(x) + bias); fp32 factors, bias and arithmetic."""

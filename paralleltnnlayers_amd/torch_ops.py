@@ -19,35 +19,61 @@ from . import capi
 
 
 class CP4Conv2dFunction(torch.autograd.Function):
-    """y = act(cp4conv2d(x, FK, FC, FH, FW, pad) + bias)."""
+    """y = act(cp4conv2d(x, FK, FC, FH, FW, pad) + bias).
+
+    A bfloat16 ``x`` selects the library's bfloat16-activation entry points
+    (y and the input gradient are bfloat16 then; factors, bias and their
+    gradients stay float32); shapes those do not take are widened to float32.
+    """
 
     @staticmethod
     def forward(ctx, x, FK, FC, FH, FW, pad, bias=None, activation=None):
         if 2 * pad + 1 != FH.shape[0] or 2 * pad + 1 != FW.shape[0]:
             raise ValueError("autograd binding needs 2*pad = Y-1 = X-1 (the reference's "
                              "backward-data pass is the adjoint only then)")
-        x, FK, FC, FH, FW = (t.contiguous().float() for t in (x, FK, FC, FH, FW))
+        FK, FC, FH, FW = (t.contiguous().float() for t in (FK, FC, FH, FW))
         if bias is not None:
             bias = bias.contiguous().float()
+        s = capi.shape_for(x.shape, FK, FC, FH, FW, pad)
+        ctx.bf16 = x.dtype == torch.bfloat16
+        ctx.fwd16 = ctx.bf16 and capi.bf16_supported(s)
+        x = x.contiguous() if ctx.bf16 else x.contiguous().float()
         ctx.pad = pad
-        y = capi.conv2d_forward_bias_act(x, FK, FC, FH, FW, bias, activation, pad=pad)
+        if ctx.fwd16:
+            y = capi.conv2d_forward_bf16(x, FK, FC, FH, FW, bias, activation, pad=pad)
+        else:
+            y = capi.conv2d_forward_bias_act(x.float(), FK, FC, FH, FW, bias, activation, pad=pad)
+            if ctx.bf16:
+                y = y.to(torch.bfloat16)
         ctx.relu = capi.ACTIVATIONS[activation] == 1
+        ctx.shape = s
         ctx.save_for_backward(x, FK, FC, FH, FW, y if ctx.relu else None)
         return y
 
     @staticmethod
     def backward(ctx, dy):
         x, FK, FC, FH, FW, y = ctx.saved_tensors
-        dy = dy.contiguous().float()
+        s = ctx.shape
+        dy = dy.contiguous()
         if ctx.relu:
             dy = dy * (y > 0)
-        dbias = dy.sum(dim=(0, 2, 3)) if ctx.needs_input_grad[6] else None
+        dbias = dy.float().sum(dim=(0, 2, 3)) if ctx.needs_input_grad[6] else None
+        dy16 = ctx.bf16 and dy.dtype == torch.bfloat16
         dx = None
         if ctx.needs_input_grad[0]:
-            dx = capi.conv2d_backward_data(dy, FK, FC, FH, FW, pad=ctx.pad)
+            if dy16 and capi.bf16_supported(s, backward_data=True):
+                dx = capi.conv2d_backward_data_bf16(dy, FK, FC, FH, FW, pad=ctx.pad)
+            else:
+                dx = capi.conv2d_backward_data(dy.float(), FK, FC, FH, FW, pad=ctx.pad)
+                if ctx.bf16:
+                    dx = dx.to(torch.bfloat16)
         grads = (None, None, None, None)
         if any(ctx.needs_input_grad[1:5]):
-            grads = capi.conv2d_backward_filter(x, dy, FK, FC, FH, FW, pad=ctx.pad)
+            if dy16 and capi.bf16_backward_filter_supported(s):
+                grads = capi.conv2d_backward_filter_bf16(x, dy, FK, FC, FH, FW, pad=ctx.pad)
+            else:
+                grads = capi.conv2d_backward_filter(x.float(), dy.float(), FK, FC, FH, FW,
+                                                    pad=ctx.pad)
             grads = tuple(g if need else None
                           for g, need in zip(grads, ctx.needs_input_grad[1:5]))
         return (dx,) + grads + (None, dbias, None)

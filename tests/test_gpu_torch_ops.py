@@ -110,3 +110,27 @@ def test_strided_layer_matches_dense_strided_conv(ops):
                           [xd.grad] + [f.grad for f in fd]):
         tol = 1e-4 if name == "dx" else 1e-3
         assert (a.double() - b).abs().max() <= tol * b.abs().max(), name
+
+
+def test_bfloat16_activations_through_autograd(ops):
+    """bfloat16 x: forward, input gradient and factor gradients run the library's
+    bfloat16-activation entry points; compared with float64 autograd on the same
+    (bfloat16-representable) inputs within the bfloat16 rounding of y, dx and dy."""
+    g = torch.Generator(device="cuda").manual_seed(21)
+    mk = lambda *s: torch.randn(*s, device="cuda", generator=g)
+    N, C, H, W, T, Y, R = 2, 32, 12, 16, 48, 3, 8
+    x = mk(N, C, H, W).to(torch.bfloat16).requires_grad_()
+    fac = [(mk(d, R) / R ** 0.25).requires_grad_() for d in (T, C, Y, Y)]
+    y = ops.cp4_conv2d(x, *fac, 1)
+    assert y.dtype == torch.bfloat16
+    dy = mk(N, T, H, W).to(torch.bfloat16)
+    y.backward(dy)
+    assert x.grad.dtype == torch.bfloat16 and fac[0].grad.dtype == torch.float32
+    xd = x.detach().double().requires_grad_()
+    fd = [f.detach().double().requires_grad_() for f in fac]
+    yd = torch.nn.functional.conv2d(xd, recomposed(*fd), padding=1)
+    yd.backward(dy.double())
+    assert (y.detach().double() - yd.detach()).abs().max() <= 2.0 ** -7 * yd.detach().abs().max()
+    assert (x.grad.double() - xd.grad).abs().max() <= 2.0 ** -7 * xd.grad.abs().max()
+    for name, a, b in zip(("dFK", "dFC", "dFH", "dFW"), [f.grad for f in fac], [f.grad for f in fd]):
+        assert (a.double() - b).abs().max() <= 1e-3 * b.abs().max(), name
