@@ -230,6 +230,21 @@ def test_edge_shapes(cp4, oracle, dims):
             assert_gradient_close(host(g), wnt, f"d{k} variant {variant}")
 
 
+def test_split_role_schedule_at_scale(cp4, oracle):
+    """Twice as many workgroups as compute units, five 64-pixel groups per strip,
+    at most 16 ranks and 4 channel blocks: tap waves and contraction waves of a
+    workgroup run several groups apart and the fragment tiles are reused."""
+    N, C, H, W, pad, T, Y, R = 64, 64, 8, 288, 1, 128, 3, 16
+    rng = np.random.default_rng(99)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    fac = [(rng.standard_normal((d, R)) / np.sqrt(R)).astype(np.float32) for d in (T, C, Y, Y)]
+    f = [dev(v) for v in fac]
+    want = oracle.forward(x, *fac, pad)
+    xd = dev(x)
+    for _ in range(3):      # a race would not show on every launch
+        assert_activation_close(host(cp4.conv2d_forward(xd, *f, pad=pad)), want, "forward")
+
+
 def test_reference_single_case_against_dense_conv(cp4):
     """Cuda_kernels/test/test_cp4Conv.cpp.cu:14-44: CP4 forward vs a dense conv
     of the recomposed kernel, all-positive U(0,1] inputs, compared with the
