@@ -71,12 +71,37 @@ struct Variant {
   bool (*supported)(const FwdArgs&);
   hipError_t (*launch)(const FwdArgs&, hipStream_t);
 };
+// Ranks 33 to 64 on the producer / consumer kernel (which holds 32): the sum over
+// ranks splits, so the kernel runs on ranks [0, 32) and then on the rest with
+// y += - the factor pointers moved 32 columns in, the row stride unchanged.
+FwdArgs rank_pass(const FwdArgs& a, int pass) {
+  FwdArgs b = a;
+  b.ldf = a.R;
+  if (pass == 0) {
+    b.R = 32;
+  } else {
+    b.R = a.R - 32;
+    b.Fin += 32; b.Fout += 32; b.FH += 32; b.FW += 32;
+    b.accumulate = 1;
+  }
+  return b;
+}
+bool fwd_pipe2_supported(const FwdArgs& a) {
+  return a.R > 32 && a.R <= 64 && !a.ldf && !a.accumulate && !a.bias && !a.act &&
+         cp4::fwd_pipe_supported(rank_pass(a, 0)) && cp4::fwd_pipe_supported(rank_pass(a, 1));
+}
+hipError_t fwd_pipe2_launch(const FwdArgs& a, hipStream_t st) {
+  const hipError_t e = cp4::fwd_pipe_launch(rank_pass(a, 0), st);
+  return e != hipSuccess ? e : cp4::fwd_pipe_launch(rank_pass(a, 1), st);
+}
+
 // Order = preference of the untuned heuristic, last to first.
 const Variant kVariants[] = {
     {"general_valu", cp4::fwd_general_supported, cp4::fwd_general_launch},
     {"mfma_f32_strip", cp4::fwd_mfma_supported, cp4::fwd_mfma_launch},
     {"mfma_bf16x3_strip", cp4::fwd_split_supported, cp4::fwd_split_launch},
     {"mfma_bf16x3_pipe", cp4::fwd_pipe_supported, cp4::fwd_pipe_launch},
+    {"mfma_bf16x3_pipe_2pass", fwd_pipe2_supported, fwd_pipe2_launch},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -110,6 +135,13 @@ int choose_variant(const FwdArgs& a) {
       (long)a.N * a.H * a.W > 8192) {
     for (int v = 0; v < kNumVariants; ++v)
       if (!strcmp(kVariants[v].name, "mfma_bf16x3_strip") && kVariants[v].supported(a)) pick = v;
+  }
+  // Two rank passes read x twice and y once more: on small problems the fp32
+  // matrix-core strip kernel, where it applies, is the faster one for ranks 33-64.
+  if (pick >= 0 && !strcmp(kVariants[pick].name, "mfma_bf16x3_pipe_2pass") &&
+      (long)a.N * a.H * a.W * (a.Cin + a.Cout) < (16l << 20)) {
+    for (int v = 0; v < kNumVariants; ++v)
+      if (!strcmp(kVariants[v].name, "mfma_f32_strip") && kVariants[v].supported(a)) pick = v;
   }
   return pick;
 }
@@ -227,13 +259,16 @@ cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
   // The kernel the plain forward would pick decides: when that is the producer /
   // consumer kernel its epilogue build runs, otherwise the chosen variant is
   // followed by the in-place bias / activation kernel.
-  const int v = choose_variant(a);
+  FwdArgs plain = a;
+  plain.bias = nullptr;
+  plain.act = 0;
+  const int v = choose_variant(plain);
   if (v < 0) return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape");
   if (!strcmp(kVariants[v].name, "mfma_bf16x3_pipe") && cp4::fwd_pipe_epi_supported(a)) {
     CP4_HIP(cp4::fwd_pipe_epi_launch(a, st));
     return CP4_OK;
   }
-  CP4_HIP(kVariants[v].launch(a, st));
+  CP4_HIP(kVariants[v].launch(plain, st));
   CP4_HIP(cp4::bias_act_launch(y, bias, activation, shape->N, shape->T,
                                (size_t)shape->H * shape->W, st));
   return CP4_OK;

@@ -27,6 +27,11 @@ struct FwdArgs {
   // (the caller runs bias_act_launch after the others).
   const float* bias;  // [Cout] or null
   int act;            // 0: none, 1: max(., 0)
+  // Rank passes (producer / consumer kernel only): the factor pointers may address
+  // a column block of wider matrices - ldf is their row stride in floats (0: R) -
+  // and accumulate != 0 adds to y instead of overwriting it.
+  int ldf;
+  int accumulate;
 };
 
 

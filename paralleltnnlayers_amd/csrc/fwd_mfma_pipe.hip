@@ -143,6 +143,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   const int l32 = lane & 31, hi = lane >> 5;
   const int H = a.H, W = a.W, HW = H * W, R = a.R, Cin = a.Cin, Cout = a.Cout;
   const int QA = pl.QA;
+  const int ldf = a.ldf ? a.ldf : R;             // row stride of the factor matrices
   const int rows = min(pl.TH, H - h0);
   const int nvalid = rows * W;                   // output pixels inside the image
   // 64-pixel output groups start `gshift` pixels before the strip so that their
@@ -166,7 +167,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       float v[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e)
-        v[e] = (r < R && 8 * o + e < Cin) ? a.Fin[(size_t)(8 * o + e) * R + r] : 0.f;
+        v[e] = (r < R && 8 * o + e < Cin) ? a.Fin[(size_t)(8 * o + e) * ldf + r] : 0.f;
       u32x4 h, m, l;
       split8(v, h, m, l);
       u32x4* dst = reinterpret_cast<u32x4*>(Fb + ((size_t)(o >> 1) * 6 + (o & 1)) * 512 + r * 16);
@@ -205,7 +206,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #pragma unroll
         for (int e = 0; e < 8; ++e)
           v[e] = (l32 < R && (!PAD || cg0 + 16 * c < Cin))
-                     ? a.Fin[(size_t)(cg0 + 16 * c + e) * R + l32]
+                     ? a.Fin[(size_t)(cg0 + 16 * c + e) * ldf + l32]
                      : 0.f;
         split8(v, fh[c], fm[c], fl[c]);
       }
@@ -368,7 +369,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int r = 16 * c + 8 * hi + e;
-          v[e] = (k < Cout && r < R) ? a.Fout[(size_t)k * R + r] : 0.f;
+          v[e] = (k < Cout && r < R) ? a.Fout[(size_t)k * ldf + r] : 0.f;
         }
         split8(v, fkh[c], fkm[c], fkl[c]);
       }
@@ -389,10 +390,11 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #pragma unroll
       for (int j = 0; j < FS; ++j) {
         const int tap = a.flip ? FS - 1 - j : j, r = 4 * wq + rr;
-        fh[rr][j] = r < R ? a.FH[tap * R + r] : 0.f;
-        fw[rr][j] = r < R ? a.FW[tap * R + r] : 0.f;
+        fh[rr][j] = r < R ? a.FH[tap * ldf + r] : 0.f;
+        fw[rr][j] = r < R ? a.FW[tap * ldf + r] : 0.f;
       }
     io_t* yn = reinterpret_cast<io_t*>(a.y) + (size_t)n * Cout * HW + (size_t)h0 * W;
+    [[maybe_unused]] const bool accumulate = a.accumulate != 0;
     const bool pair_stores =                       // one store per pixel pair is legal
         ((W | HW) & 1) == 0 && (reinterpret_cast<uintptr_t>(a.y) & (2 * kIoBytes - 1)) == 0;
     const int reach = (FS - 1) * (W + 1);          // how far past a pixel its taps read in A
@@ -541,6 +543,11 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         float2 o;
         o.x = v0;
         o.y = v1;
+        if (accumulate) {                        // second rank pass: y += (wave-uniform)
+          const float2 old = *reinterpret_cast<const float2*>(dst);
+          o.x += old.x;
+          o.y += old.y;
+        }
         *reinterpret_cast<float2*>(dst) = o;
 #endif
       };
@@ -548,7 +555,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #ifdef CP4_PIPE_IO16
         *dst = to_io(v);
 #else
-        *dst = v;
+        *dst = accumulate ? *dst + v : v;
 #endif
       };
       if (pair_stores) {
@@ -720,6 +727,9 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 
 bool fwd_pipe_supported(const FwdArgs& a) {
   if (a.R > kRP || (a.Cin & 7) || a.Cin > 768) return false;
+#ifdef CP4_PIPE_EPILOGUE
+  if (a.accumulate) return false;                // the epilogue builds write y once
+#endif
   if (!fits_int_indexing(a.N, a.H, a.W)) return false;
   if ((size_t)a.Cin * a.H * a.W * sizeof(io_t) >= (1ull << 31)) return false;   // buffer offsets
   if (a.Y != a.X || !(a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7)) return false;
