@@ -88,11 +88,12 @@ FwdArgs rank_pass(const FwdArgs& a, int pass) {
 }
 bool fwd_pipe2_supported(const FwdArgs& a) {
   return a.R > 32 && a.R <= 64 && !a.ldf && !a.accumulate && !a.bias && !a.act &&
-         cp4::fwd_pipe_supported(rank_pass(a, 0)) && cp4::fwd_pipe_supported(rank_pass(a, 1));
+         cp4::fwd_pipe_rankpass_supported(rank_pass(a, 0)) &&
+         cp4::fwd_pipe_rankpass_supported(rank_pass(a, 1));
 }
 hipError_t fwd_pipe2_launch(const FwdArgs& a, hipStream_t st) {
-  const hipError_t e = cp4::fwd_pipe_launch(rank_pass(a, 0), st);
-  return e != hipSuccess ? e : cp4::fwd_pipe_launch(rank_pass(a, 1), st);
+  const hipError_t e = cp4::fwd_pipe_rankpass_launch(rank_pass(a, 0), st);
+  return e != hipSuccess ? e : cp4::fwd_pipe_rankpass_launch(rank_pass(a, 1), st);
 }
 
 // Order = preference of the untuned heuristic, last to first.

@@ -27,7 +27,7 @@ struct FwdArgs {
   // (the caller runs bias_act_launch after the others).
   const float* bias;  // [Cout] or null
   int act;            // 0: none, 1: max(., 0)
-  // Rank passes (producer / consumer kernel only): the factor pointers may address
+  // Rank passes (rank-pass build of the producer / consumer kernel only): the factor pointers may address
   // a column block of wider matrices - ldf is their row stride in floats (0: R) -
   // and accumulate != 0 adds to y instead of overwriting it.
   int ldf;
@@ -59,6 +59,9 @@ hipError_t fwd_pipe_epi_launch(const FwdArgs&, hipStream_t);
 // 16-bit elements; factors and bias stay fp32), epilogue included.
 bool fwd_pipe_io16_supported(const FwdArgs&);
 hipError_t fwd_pipe_io16_launch(const FwdArgs&, hipStream_t);
+// The same kernel honouring FwdArgs::ldf and FwdArgs::accumulate (rank passes).
+bool fwd_pipe_rankpass_supported(const FwdArgs&);
+hipError_t fwd_pipe_rankpass_launch(const FwdArgs&, hipStream_t);
 // In-place y[n,k,:] = act(y[n,k,:] + bias[k]) for variants without the epilogue.
 hipError_t bias_act_launch(float* y, const float* bias, int act, size_t N, size_t K, size_t HW,
                            hipStream_t);

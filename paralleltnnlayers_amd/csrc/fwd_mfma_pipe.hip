@@ -40,14 +40,17 @@
 // Cuda_kernels/cp4Conv2dForward.cu:84-133 (backward-data:
 // cp4Conv2dBackwardData.cu:57-108 through swapped factors and flipped taps).
 //
-// This file is compiled three times: as is; with CP4_PIPE_EPILOGUE defined, which
+// This file is compiled four times: as is; with CP4_PIPE_EPILOGUE defined, which
 // adds y = act(conv + bias[k]) to the stores (the bias of the lane's sixteen
 // output rows rides in registers next to the output-factor fragment) and exports
 // the entry points under the names fwd_pipe_epi_*; and with CP4_PIPE_IO16, where
 // x and y are bfloat16 in memory (factors, bias and all arithmetic stay fp32):
 // a bf16 activation is its own high part, so the channel contraction needs
 // neither the split nor the three MFMAs of the lower parts, and y is rounded to
-// nearest-even as pixel pairs (entry points fwd_pipe_io16_*, epilogue included).
+// nearest-even as pixel pairs (entry points fwd_pipe_io16_*, epilogue included);
+// and with CP4_PIPE_RANKPASS, the build behind the two-pass variant for ranks
+// 33-64: factor matrices with a row stride of their own (FwdArgs::ldf) and stores
+// that add to y (FwdArgs::accumulate), entry points fwd_pipe_rankpass_*.
 #include <cstdlib>
 #include <type_traits>
 
@@ -143,7 +146,11 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   const int l32 = lane & 31, hi = lane >> 5;
   const int H = a.H, W = a.W, HW = H * W, R = a.R, Cin = a.Cin, Cout = a.Cout;
   const int QA = pl.QA;
+#ifdef CP4_PIPE_RANKPASS
   const int ldf = a.ldf ? a.ldf : R;             // row stride of the factor matrices
+#else
+  const int ldf = R;
+#endif
   const int rows = min(pl.TH, H - h0);
   const int nvalid = rows * W;                   // output pixels inside the image
   // 64-pixel output groups start `gshift` pixels before the strip so that their
@@ -543,11 +550,13 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         float2 o;
         o.x = v0;
         o.y = v1;
+#ifdef CP4_PIPE_RANKPASS
         if (accumulate) {                        // second rank pass: y += (wave-uniform)
           const float2 old = *reinterpret_cast<const float2*>(dst);
           o.x += old.x;
           o.y += old.y;
         }
+#endif
         *reinterpret_cast<float2*>(dst) = o;
 #endif
       };
@@ -555,7 +564,11 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #ifdef CP4_PIPE_IO16
         *dst = to_io(v);
 #else
+#ifdef CP4_PIPE_RANKPASS
         *dst = accumulate ? *dst + v : v;
+#else
+        *dst = v;
+#endif
 #endif
       };
       if (pair_stores) {
@@ -717,7 +730,10 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 
 }  // namespace
 
-#if defined(CP4_PIPE_IO16)
+#if defined(CP4_PIPE_RANKPASS)
+#define fwd_pipe_supported fwd_pipe_rankpass_supported
+#define fwd_pipe_launch fwd_pipe_rankpass_launch
+#elif defined(CP4_PIPE_IO16)
 #define fwd_pipe_supported fwd_pipe_io16_supported
 #define fwd_pipe_launch fwd_pipe_io16_launch
 #elif defined(CP4_PIPE_EPILOGUE)
@@ -727,8 +743,8 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 
 bool fwd_pipe_supported(const FwdArgs& a) {
   if (a.R > kRP || (a.Cin & 7) || a.Cin > 768) return false;
-#ifdef CP4_PIPE_EPILOGUE
-  if (a.accumulate) return false;                // the epilogue builds write y once
+#ifndef CP4_PIPE_RANKPASS
+  if (a.accumulate || a.ldf) return false;       // only the rank-pass build has these
 #endif
   if (!fits_int_indexing(a.N, a.H, a.W)) return false;
   if ((size_t)a.Cin * a.H * a.W * sizeof(io_t) >= (1ull << 31)) return false;   // buffer offsets
