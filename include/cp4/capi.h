@@ -69,8 +69,9 @@ cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
  * fp32 factors, fp32 accumulation, one rounding to nearest-even at the store).
  * Half the HBM bytes of the fp32 entry points.  The reference has fp32 only; this
  * is the layer's mixed-precision form.  Runs on the producer / consumer kernel
- * alone: CP4_ERR_UNSUPPORTED for shapes it does not take (Rank > 32, C not a
- * multiple of 8 or above 768, filters other than square 1/3/5/7);
+ * alone: CP4_ERR_UNSUPPORTED for shapes it does not take (Rank > 32, more than
+ * 768 input channels, filters other than square 1/3/5/7, rows too long for its
+ * whole-row strips);
  * cp4_bf16_supported answers beforehand (backward_data != 0: the shape is read
  * as that pass's, channels swapped). */
 int cp4_bf16_supported(const cp4_shape* shape, int backward_data);

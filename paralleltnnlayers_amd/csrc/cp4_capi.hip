@@ -101,6 +101,7 @@ const Variant kVariants[] = {
     {"general_valu", cp4::fwd_general_supported, cp4::fwd_general_launch},
     {"mfma_f32_strip", cp4::fwd_mfma_supported, cp4::fwd_mfma_launch},
     {"mfma_bf16x3_strip", cp4::fwd_split_supported, cp4::fwd_split_launch},
+    {"mfma_bf16x3_pipe_tiled", cp4::fwd_pipe_tiled_supported, cp4::fwd_pipe_tiled_launch},
     {"mfma_bf16x3_pipe", cp4::fwd_pipe_supported, cp4::fwd_pipe_launch},
     {"mfma_bf16x3_pipe_2pass", fwd_pipe2_supported, fwd_pipe2_launch},
 };
@@ -136,6 +137,21 @@ int choose_variant(const FwdArgs& a) {
       (long)a.N * a.H * a.W > 8192) {
     for (int v = 0; v < kNumVariants; ++v)
       if (!strcmp(kVariants[v].name, "mfma_bf16x3_strip") && kVariants[v].supported(a)) pick = v;
+  }
+  // A handful of channels on either side (3 -> 1, say) leaves the 32 x 32 matrix
+  // tiles almost empty: the general kernel, whose cost follows the real channel
+  // counts, is then as fast or faster.
+  if (pick >= 0 && !strncmp(kVariants[pick].name, "mfma_bf16x3_pipe", 16) &&
+      a.Cin + a.Cout < 24) {
+    for (int v = 0; v < kNumVariants; ++v)
+      if (!strcmp(kVariants[v].name, "general_valu") && kVariants[v].supported(a)) pick = v;
+  }
+  // Planes wider than 128 pixels: whole-row strips get short (2 rows at W = 224)
+  // and pay for it in halo rows; tiles of TH x Wt do better there.
+  if (pick >= 0 && !strcmp(kVariants[pick].name, "mfma_bf16x3_pipe") && a.W > 128) {
+    for (int v = 0; v < kNumVariants; ++v)
+      if (!strcmp(kVariants[v].name, "mfma_bf16x3_pipe_tiled") && kVariants[v].supported(a))
+        pick = v;
   }
   // Two rank passes read x twice and y once more: on small problems the fp32
   // matrix-core strip kernel, where it applies, is the faster one for ranks 33-64.

@@ -62,6 +62,9 @@ hipError_t fwd_pipe_io16_launch(const FwdArgs&, hipStream_t);
 // The same kernel honouring FwdArgs::ldf and FwdArgs::accumulate (rank passes).
 bool fwd_pipe_rankpass_supported(const FwdArgs&);
 hipError_t fwd_pipe_rankpass_launch(const FwdArgs&, hipStream_t);
+// The same kernel on tiles of TH rows x Wt columns (wide planes).
+bool fwd_pipe_tiled_supported(const FwdArgs&);
+hipError_t fwd_pipe_tiled_launch(const FwdArgs&, hipStream_t);
 // In-place y[n,k,:] = act(y[n,k,:] + bias[k]) for variants without the epilogue.
 hipError_t bias_act_launch(float* y, const float* bias, int act, size_t N, size_t K, size_t HW,
                            hipStream_t);

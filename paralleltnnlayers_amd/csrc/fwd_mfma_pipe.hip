@@ -40,7 +40,7 @@
 // Cuda_kernels/cp4Conv2dForward.cu:84-133 (backward-data:
 // cp4Conv2dBackwardData.cu:57-108 through swapped factors and flipped taps).
 //
-// This file is compiled four times: as is; with CP4_PIPE_EPILOGUE defined, which
+// This file is compiled five times: as is; with CP4_PIPE_EPILOGUE defined, which
 // adds y = act(conv + bias[k]) to the stores (the bias of the lane's sixteen
 // output rows rides in registers next to the output-factor fragment) and exports
 // the entry points under the names fwd_pipe_epi_*; and with CP4_PIPE_IO16, where
@@ -50,7 +50,12 @@
 // nearest-even as pixel pairs (entry points fwd_pipe_io16_*, epilogue included);
 // and with CP4_PIPE_RANKPASS, the build behind the two-pass variant for ranks
 // 33-64: factor matrices with a row stride of their own (FwdArgs::ldf) and stores
-// that add to y (FwdArgs::accumulate), entry points fwd_pipe_rankpass_*.
+// that add to y (FwdArgs::accumulate), entry points fwd_pipe_rankpass_*;
+// and with CP4_PIPE_TILED, for wide planes: a workgroup's tile is TH rows by Wt
+// columns (Wt a power of two, at least 64) instead of TH whole rows; the LDS
+// plane holds the tile plus its halo in rows of Wt + FS - 1 cells, so the taps
+// need no border masks (cells outside the image are stored as zeros) and every
+// 64-pixel output group is one row segment; entry points fwd_pipe_tiled_*.
 #include <cstdlib>
 #include <type_traits>
 
@@ -91,6 +96,8 @@ struct PipePlan {
   int cc_off;
   int flag_off;
   size_t lds_bytes;
+  int Wt, lgWt, cols;       // tiled build: tile width, its log2, column tiles per row strip
+  unsigned wl_magic;        // tiled build: 2^32 / (Wt + FS - 1) + 1, for the division by the row length
 #ifdef CP4_DEBUG_PHASES
   long long* dbg;
 #endif
@@ -123,8 +130,15 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   const int per = (pl.nWG + 7) >> 3;
   const int t = (blockIdx.x & 7) * per + (blockIdx.x >> 3);         // XCD-contiguous tile order
   if (t >= pl.nWG) return;
+#ifdef CP4_PIPE_TILED
+  const int per_img = pl.strips * pl.cols;
+  const int n = t / per_img, trem = t - n * per_img;
+  const int strip = trem / pl.cols, h0 = strip * pl.TH, w0 = (trem - strip * pl.cols) * pl.Wt;
+  const bool rev = false;
+#else
   const int n = t / pl.strips, strip = t - n * pl.strips, h0 = strip * pl.TH;
   const bool rev = strip & 1;                    // odd strips sweep bottom-up
+#endif
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -152,15 +166,27 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   const int ldf = R;
 #endif
   const int rows = min(pl.TH, H - h0);
+#ifdef CP4_PIPE_TILED
+  const int Wt = pl.Wt, lgWt = pl.lgWt, WL = Wt + FS - 1;   // tile width, LDS row length
+  const int wcols = min(Wt, W - w0);             // tile columns inside the image
+  const int nvalid = rows * Wt;                  // output cells of the tile (a multiple of 64)
+  const int gshift = 0;
+  const int ngroups = nvalid >> 6;
+#else
   const int nvalid = rows * W;                   // output pixels inside the image
   // 64-pixel output groups start `gshift` pixels before the strip so that their
   // boundaries fall on 128-byte lines of y (pixel h0*W + 64*g - gshift is a
   // multiple of 32); pixels before the strip are computed and not stored.
   const int gshift = (h0 * W) & 31;
   const int ngroups = (nvalid + gshift + 63) >> 6;
+#endif
   const int nkb = (Cout + 31) >> 5;
+#ifdef CP4_PIPE_TILED
+  const int QLEN = (pl.TH + FS - 1) * WL;
+#else
   const int qbase = (h0 - a.pad) * W;            // global flat pixel of LDS column 0
   const int QLEN = (pl.TH + FS - 1) * W;
+#endif
   const int nblk = (QLEN + 31) >> 5;             // 32-pixel producer blocks
 
   // ---- prologue: clear the progress words; above 256 input channels the input
@@ -212,7 +238,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         float v[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          v[e] = (l32 < R && (!PAD || cg0 + 16 * c < Cin))
+          v[e] = (l32 < R && (!PAD || cg0 + 16 * c + e < Cin))
                      ? a.Fin[(size_t)(cg0 + 16 * c + e) * ldf + l32]
                      : 0.f;
         split8(v, fh[c], fm[c], fl[c]);
@@ -226,9 +252,17 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       j = 2 * r + bsel;
       const int b = rev ? nblk - 1 - j : j;        // j == nblk happens when nblk is odd
       qa = 32 * b + l32;
+#ifdef CP4_PIPE_TILED
+      // cell qa of the tile plane: row lr, column lc -> image pixel (grow, gcol)
+      const int lr = (int)__umulhi((unsigned)qa, pl.wl_magic), lc = qa - lr * WL;
+      const int grow = h0 - a.pad + lr, gcol = w0 - a.pad + lc;
+      valid = j < nblk && qa < QLEN && grow >= 0 && grow < H && gcol >= 0 && gcol < W;
+      const int qc = valid ? grow * W + gcol : 0;
+#else
       const int q = qbase + qa;
       valid = j < nblk && q >= 0 && q < HW && qa < QLEN;
       const int qc = q < 0 ? 0 : (q > HW - 1 ? HW - 1 : q);
+#endif
       return (unsigned)(8 * hi * HW + qc) * (unsigned)kIoBytes;
     };
 #ifdef CP4_PIPE_IO16
@@ -400,11 +434,17 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         fh[rr][j] = r < R ? a.FH[tap * ldf + r] : 0.f;
         fw[rr][j] = r < R ? a.FW[tap * ldf + r] : 0.f;
       }
+#ifdef CP4_PIPE_TILED
+    io_t* yn = reinterpret_cast<io_t*>(a.y) + (size_t)n * Cout * HW + (size_t)h0 * W + w0;
+#else
     io_t* yn = reinterpret_cast<io_t*>(a.y) + (size_t)n * Cout * HW + (size_t)h0 * W;
+#endif
     [[maybe_unused]] const bool accumulate = a.accumulate != 0;
     const bool pair_stores =                       // one store per pixel pair is legal
         ((W | HW) & 1) == 0 && (reinterpret_cast<uintptr_t>(a.y) & (2 * kIoBytes - 1)) == 0;
+#ifndef CP4_PIPE_TILED
     const int reach = (FS - 1) * (W + 1);          // how far past a pixel its taps read in A
+#endif
 
     int frontier = 0;                              // blocks [0, frontier) of the sweep are complete
     int* arrivals = flags + kMaxBlk;               // [4] tap-step arrivals, slot = step & 3
@@ -417,11 +457,19 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // Highest sweep index among the blocks the taps of step i touch: the taps of
     // pixel p read A columns p - pad .. p + (FS-1)*(W+1) - pad.
     auto need_of = [&](int i) {
+#ifdef CP4_PIPE_TILED
+      // group i is the row segment (h, w .. w + 63): its taps read plane rows
+      // h .. h + FS - 1, columns w .. w + 62 + FS
+      const int h = (64 * i) >> lgWt, w = (64 * i) & (Wt - 1);
+      const int last = ((h + FS - 1) * WL + w + 63 + FS - 1) >> 5;
+      return last > nblk - 1 ? nblk - 1 : last;
+#else
       const int g = rev ? ngroups - 1 - i : i;
       int last = max(64 * g - gshift + 63 + reach, 0) >> 5;
       if (last > nblk - 1) last = nblk - 1;
       const int first = max(64 * g - gshift - a.pad, 0) >> 5;
       return rev ? nblk - 1 - first : last;
+#endif
     };
     // Non-blocking: advance the frontier over finished blocks, say whether step
     // i could run its taps now.
@@ -442,6 +490,21 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         }
       }
       STAMPX(2 + 4 * i)
+#ifdef CP4_PIPE_TILED
+      // the plane carries the halo columns: tap (ti, j) of cell (h, w) is plane
+      // cell (h + ti, w + j), no border cases
+      const int p = 64 * g + lane;
+      const int h = p >> lgWt, w = p & (Wt - 1);
+      const int RL = WL;                           // row length of the plane
+      int off[FS];
+      bool in[FS];
+#pragma unroll
+      for (int j = 0; j < FS; ++j) {
+        in[j] = true;
+        off[j] = w + j;
+      }
+#else
+      const int RL = W;
       const int p = max(64 * g - gshift + lane, 0);      // lanes before the strip: any valid column
       const int h = p / W, w = p - h * W;
       int off[FS];
@@ -452,9 +515,10 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         in[j] = ww >= 0 && ww < W;
         off[j] = ww < 0 ? 0 : (ww >= W ? W - 1 : ww);      // clamped: weight is 0 there
       }
+#endif
       // the LDS reads of RBT ranks go out together, then their arithmetic
       constexpr int RBT = FS <= 3 ? 4 : (FS == 5 ? 2 : 1);
-      const float* ab = As + (size_t)(4 * wq) * QA + h * W;
+      const float* ab = As + (size_t)(4 * wq) * QA + h * RL;
       float o[4];
 #pragma unroll
       for (int r0 = 0; r0 < 4; r0 += RBT) {
@@ -464,7 +528,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #pragma unroll
           for (int ti = 0; ti < FS; ++ti)
 #pragma unroll
-            for (int j = 0; j < FS; ++j) av[rr][ti][j] = ab[(r0 + rr) * QA + ti * W + off[j]];
+            for (int j = 0; j < FS; ++j) av[rr][ti][j] = ab[(r0 + rr) * QA + ti * RL + off[j]];
 #pragma unroll
         for (int rr = 0; rr < RBT; ++rr) {
           float s = 0.f;
@@ -541,6 +605,15 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #endif
       // store rows: uniform row base + one 32-bit lane offset
       const int p = 64 * g - gshift + 2 * l32;       // lane's pixel pair p, p + 1
+#ifdef CP4_PIPE_TILED
+      // tile cell p = (row, column) -> offset in the image plane from the tile's corner
+      const int pcol = p & (Wt - 1);
+      const int pofs = (p >> lgWt) * W + pcol;
+      const bool pin0 = pcol < wcols, pin1 = pcol + 1 < wcols;
+#else
+      const int pofs = p;
+      const bool pin0 = p >= 0 && p < nvalid, pin1 = p + 1 >= 0 && p + 1 < nvalid;
+#endif
       io_t* rowbase = yn + (size_t)(32 * kb) * HW;
       // the lane's pixel pair as one store: float2, or two bfloat16 in a dword
       auto store_pair = [&](io_t* dst, float v0, float v1) {
@@ -573,8 +646,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       };
       if (pair_stores) {
         // W and H*W even, y aligned to a pair: p is even and the pair is one store
-        if (p >= 0 && p < nvalid) {
-          const unsigned lofs = (unsigned)(4 * hi * HW + p);
+        if (pin0) {
+          const unsigned lofs = (unsigned)(4 * hi * HW + pofs);
           if (32 * kb + 32 <= Cout) {
 #pragma unroll
             for (int v = 0; v < 16; ++v)
@@ -590,8 +663,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         }
       } else {
         // odd widths or planes: the two pixels are stored and bounded one by one
-        const bool in0 = p >= 0 && p < nvalid, in1 = p + 1 >= 0 && p + 1 < nvalid;
-        const long lofs = (long)(4 * hi) * HW + p;
+        const bool in0 = pin0, in1 = pin1;
+        const long lofs = (long)(4 * hi) * HW + pofs;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int kk = 8 * (v >> 2) + (v & 3);
@@ -659,7 +732,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 
 int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
-bool layout(const FwdArgs& a, int TH, PipePlan* pl) {
+[[maybe_unused]] bool layout(const FwdArgs& a, int TH, PipePlan* pl) {
   const long QLEN = (long)(TH + a.Y - 1) * a.W;
   // the taps of the last (partly filled) 64-pixel group may read past QLEN; the
   // groups start up to 31 pixels before the strip, so they end up to 31 + 63 past it
@@ -682,6 +755,52 @@ bool layout(const FwdArgs& a, int TH, PipePlan* pl) {
   return true;
 }
 
+#ifdef CP4_PIPE_TILED
+// Tile of TH rows x Wt columns: plane of (TH + Y - 1) rows of Wt + Y - 1 cells.
+bool layout_tiled(const FwdArgs& a, int TH, int lgWt, PipePlan* pl) {
+  const int Wt = 1 << lgWt, WL = Wt + a.Y - 1;
+  const long QLEN = (long)(TH + a.Y - 1) * WL;
+  const long QA = round_up((int)QLEN, 64) + 8;
+  const size_t a_bytes = (size_t)kRP * QA * sizeof(float);
+  const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
+  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 8) * sizeof(int);
+  if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
+  if (bytes > kLdsLimit) return false;
+  pl->TH = TH;
+  pl->strips = (a.H + TH - 1) / TH;
+  pl->Wt = Wt;
+  pl->lgWt = lgWt;
+  pl->cols = (a.W + Wt - 1) / Wt;
+  pl->wl_magic = (unsigned)(0x100000000ull / (unsigned)WL) + 1u;   // exact quotients below 2^16
+  pl->nWG = a.N * pl->strips * pl->cols;
+  pl->QA = (int)QA;
+  pl->fin_off = (int)a_bytes;
+  pl->cc_off = (int)(a_bytes + fin_bytes);
+  pl->flag_off = (int)(a_bytes + fin_bytes + 3 * kCcBuf);
+  pl->lds_bytes = bytes;
+  return true;
+}
+bool plan(const FwdArgs& a, PipePlan* best) {
+  double best_cost = 0;
+  bool found = false;
+  for (int lgWt = 6; lgWt <= 8; ++lgWt)
+    for (int TH = 1; TH <= a.H; ++TH) {
+      PipePlan pl;
+      if (!layout_tiled(a, TH, lgWt, &pl)) break;
+      const double rounds = (pl.nWG + 255) / 256;
+      // cells read per channel and cells written per channel, with the tiles of the
+      // last column counted whole
+      const double cost = rounds * ((double)(TH + a.Y - 1) * (pl.Wt + a.Y - 1) * a.Cin +
+                                    (double)TH * pl.Wt * a.Cout);
+      if (!found || cost < best_cost) {
+        best_cost = cost;
+        *best = pl;
+        found = true;
+      }
+    }
+  return found;
+}
+#else
 bool plan(const FwdArgs& a, PipePlan* best) {
   double best_cost = 0;
   bool found = false;
@@ -698,6 +817,7 @@ bool plan(const FwdArgs& a, PipePlan* best) {
   }
   return found;
 }
+#endif
 
 template <int FS, int CPQ, int KR, bool PAD>
 hipError_t launch_as(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
@@ -730,7 +850,10 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 
 }  // namespace
 
-#if defined(CP4_PIPE_RANKPASS)
+#if defined(CP4_PIPE_TILED)
+#define fwd_pipe_supported fwd_pipe_tiled_supported
+#define fwd_pipe_launch fwd_pipe_tiled_launch
+#elif defined(CP4_PIPE_RANKPASS)
 #define fwd_pipe_supported fwd_pipe_rankpass_supported
 #define fwd_pipe_launch fwd_pipe_rankpass_launch
 #elif defined(CP4_PIPE_IO16)
@@ -742,7 +865,7 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 #endif
 
 bool fwd_pipe_supported(const FwdArgs& a) {
-  if (a.R > kRP || (a.Cin & 7) || a.Cin > 768) return false;
+  if (a.R > kRP || a.Cin > 768) return false;
 #ifndef CP4_PIPE_RANKPASS
   if (a.accumulate || a.ldf) return false;       // only the rank-pass build has these
 #endif
