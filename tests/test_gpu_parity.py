@@ -201,6 +201,12 @@ EDGE = [
     (3, 16, 30, 34, 2, 96, 5, 5, 9),      # 5x5, several groups per strip
     (2, 64, 6, 288, 1, 128, 3, 3, 16),    # long rows: five groups per strip, fragment tiles reused
     (1, 32, 3, 576, 0, 64, 1, 1, 8),      # ten groups per strip
+    # wide planes: tiles of TH rows x Wt columns (producer/consumer kernel, tiled build)
+    (1, 16, 9, 200, 1, 32, 3, 3, 8),      # four column tiles, the last one 8 columns wide
+    (2, 24, 5, 131, 2, 16, 5, 5, 12),     # odd width across three tiles, 5x5
+    (1, 64, 20, 300, 0, 64, 3, 3, 32),    # no padding, 32 ranks, ragged last row strip
+    (1, 8, 3, 1000, 3, 8, 7, 7, 4),       # 7x7, very wide and short
+    (2, 3, 40, 224, 1, 64, 3, 3, 16),     # three input channels, first-layer shape
     # many small planes (wave-per-plane tap kernel, one partial per image)
     (64, 32, 8, 8, 1, 48, 3, 3, 20),
     (70, 16, 6, 10, 2, 16, 5, 5, 40),     # two rank tiles, the second partly filled
