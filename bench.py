@@ -48,6 +48,9 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C3")
+    ap.add_argument("--shape", default=None, metavar="PASS,N,C,H,W,pad,T,Y,R",
+                    help="time an ad-hoc shape instead of a named workload, e.g. "
+                         "forward,8,64,224,224,1,64,3,16 (uniform inputs; no CPU leg, no table)")
     ap.add_argument("--settle-ms", type=float, default=150.0,
                     help="untimed back-to-back launches of the headline workload for this "
                          "long before the warm-up, so clocks are at their steady state")
@@ -100,6 +103,12 @@ def main():
         return us, time.perf_counter() - t0
 
     w = WORKLOADS[args.workload]
+    if args.shape:
+        from paralleltnnlayers_amd.configs import Workload
+        f = args.shape.split(",")
+        N, C, H, W_, pad, T, Y, R = (int(v) for v in f[1:])
+        w = Workload("adhoc", f[0], N, C, H, W_, pad, T, Y, Y, R, "uniform")
+        args.no_cpu = args.no_passes = True
     if args.calibrate_copy:
         n = w.N * w.C * w.H * w.W
         src = torch.randn(n, device="cuda")
