@@ -635,8 +635,12 @@ hipError_t launch_taps_wave(const float* A, const float* G3, const BwdFilterArgs
   return hipGetLastError();
 }
 
-// ---- 2''. taps for planes up to 64 pixels wide: one wave per (image, rank)
-// plane, lane = column, walking down the rows.  The last FS rows of A, G3 and
+// ---- 2''. taps with lane = column: one wave per (image, rank) plane up to 64
+// pixels wide; wider planes are cut into column segments of 64 - 2Q output
+// columns (Q = max(P, FS-1-P), the reach of the horizontal taps), one wave per
+// segment, whose 64 lanes also carry the Q halo columns on either side - read
+// from memory like the others, so the shuffles below stay inside the wave - and
+// which stores and sums only its own columns.  The wave walks down the rows.  The last FS rows of A, G3 and
 // G2 live in registers; the horizontal taps read the neighbouring columns'
 // registers through wave shuffles; nothing goes through LDS and there is no
 // barrier.  Row t of A and G3 is requested kRowsAhead steps before it is used.
@@ -648,15 +652,20 @@ __global__ __launch_bounds__(256) void taps_column_kernel(
     const float* __restrict__ A, const float* __restrict__ G3, const float* __restrict__ FH,
     const float* __restrict__ FW, float* __restrict__ Cc, float* __restrict__ G1,
     float* __restrict__ partH, float* __restrict__ partW, int R, int H, int W, int P,
-    int nplanes) {
+    int nplanes, int segs, int Q) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int plane = blockIdx.x * 4 + wave;
-  if (plane >= nplanes) return;
+  const int unit = blockIdx.x * 4 + wave;        // (plane, column segment)
+  if (unit >= nplanes * segs) return;
+  const int plane = unit / segs, seg = unit - plane * segs;
   const int r = plane % R, n = plane / R;
   const size_t base = (size_t)plane * H * W;
-  const bool col = lane < W;
-  const int wc = col ? lane : W - 1;             // clamped column for addresses
+  // lane's image column; one segment: lane = column, no halo
+  const int gc = segs == 1 ? lane : seg * (64 - 2 * Q) - Q + lane;
+  const bool col = gc >= 0 && gc < W;
+  // columns this wave stores and sums (the halo lanes belong to the neighbours)
+  const bool mine = col && (segs == 1 || (lane >= Q && lane < 64 - Q));
+  const int wc = gc < 0 ? 0 : (gc < W ? gc : W - 1);   // clamped column for addresses
   float fh[FS], fw[FS];
 #pragma unroll
   for (int i = 0; i < FS; ++i) {
@@ -669,9 +678,9 @@ __global__ __launch_bounds__(256) void taps_column_kernel(
   bool okf[FS], okb[FS];
 #pragma unroll
   for (int j = 0; j < FS; ++j) {
-    const int wf = lane + j - P, wb = lane - j + P;   // forward / adjoint neighbour
-    okf[j] = col && wf >= 0 && wf < W;
-    okb[j] = col && wb >= 0 && wb < W;
+    const int wf = lane + j - P, wb = lane - j + P;   // forward / adjoint neighbour lane
+    okf[j] = col && wf >= 0 && wf < 64 && gc + j - P >= 0 && gc + j - P < W;
+    okb[j] = col && wb >= 0 && wb < 64 && gc - j + P >= 0 && gc - j + P < W;
     srcf[j] = okf[j] ? wf : 0;
     srcb[j] = okb[j] ? wb : 0;
   }
@@ -726,11 +735,12 @@ __global__ __launch_bounds__(256) void taps_column_kernel(
             const float v = __shfl(b, srcf[j], 64);
             const float bj = okf[j] ? v : 0.f;
             cc += fw[j] * bj;
-            accW[j] += gw[P] * bj;                  // G3[hb][w] * B[hb][w+j-P]
+            accW[j] += mine ? gw[P] * bj : 0.f;     // G3[hb][w] * B[hb][w+j-P]
           }
 #pragma unroll
-          for (int i = 0; i < FS; ++i) accH[i] += g2w[P] * aw[i];   // G2[hb][w] * A[hb+i-P][w]
-          if (col) Cc[base + (size_t)hb * W + lane] = cc;
+          for (int i = 0; i < FS; ++i)
+            accH[i] += mine ? g2w[P] * aw[i] : 0.f;   // G2[hb][w] * A[hb+i-P][w]
+          if (mine) Cc[base + (size_t)hb * W + gc] = cc;
         }
         // G1 row hg: vertical adjoint taps of the G2 window
         const int hg = t - P;
@@ -738,7 +748,7 @@ __global__ __launch_bounds__(256) void taps_column_kernel(
           float g1 = 0.f;
 #pragma unroll
           for (int i = 0; i < FS; ++i) g1 += fh[i] * g2w[FS - 1 - i];
-          if (col) G1[base + (size_t)hg * W + lane] = g1;
+          if (mine) G1[base + (size_t)hg * W + gc] = g1;
         }
       }
     }
@@ -754,18 +764,26 @@ __global__ __launch_bounds__(256) void taps_column_kernel(
   if (lane == 0) {
 #pragma unroll
     for (int i = 0; i < FS; ++i) {
-      partH[((size_t)n * FS + i) * R + r] = accH[i];
-      partW[((size_t)n * FS + i) * R + r] = accW[i];
+      partH[(((size_t)n * segs + seg) * FS + i) * R + r] = accH[i];
+      partW[(((size_t)n * segs + seg) * FS + i) * R + r] = accW[i];
     }
   }
+}
+
+// Column segments of taps_column_kernel for a plane W wide.
+int column_segments(int W, int FS, int P) {
+  const int Q = P > FS - 1 - P ? P : FS - 1 - P;
+  return W <= 64 ? 1 : (W + (64 - 2 * Q) - 1) / (64 - 2 * Q);
 }
 
 template <int FS>
 hipError_t launch_taps_column(const float* A, const float* G3, const BwdFilterArgs& a, float* Cc,
                               float* G1, float* pH, float* pW, hipStream_t st) {
-  const int nplanes = a.N * a.R;
-  taps_column_kernel<FS><<<(unsigned)((nplanes + 3) / 4), 256, 0, st>>>(
-      A, G3, a.FH, a.FW, Cc, G1, pH, pW, a.R, a.H, a.W, a.pad, nplanes);
+  const int nplanes = a.N * a.R, segs = column_segments(a.W, FS, a.pad);
+  const int Q = a.pad > FS - 1 - a.pad ? a.pad : FS - 1 - a.pad;
+  const long units = (long)nplanes * segs;
+  taps_column_kernel<FS><<<(unsigned)((units + 3) / 4), 256, 0, st>>>(
+      A, G3, a.FH, a.FW, Cc, G1, pH, pW, a.R, a.H, a.W, a.pad, nplanes, segs, Q);
   return hipGetLastError();
 }
 
@@ -1100,10 +1118,12 @@ Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R, int pad) 
   const bool odd_square = Y == X && (Y == 1 || Y == 3 || Y == 5 || Y == 7);
   p.wave_taps = p.plane_taps && HW <= 256 && W >= 2 && odd_square &&  // one wave per plane, in LDS
                 wave_tap_layout(H, W, Y, pad).smem <= 64 * 1024;
-  p.column_taps = !p.wave_taps && W <= 64 && odd_square && pad <= Y - 1;   // one wave per plane, in registers
-  p.St = (p.plane_taps || p.column_taps) ? N : (N < 8 ? N : 8);
+  // one wave per plane (or per column segment of a wide plane), in registers
+  p.column_taps = !p.wave_taps && odd_square && pad <= Y - 1;
+  p.St = p.column_taps ? N * column_segments(W, Y, pad)
+                       : (p.plane_taps ? N : (N < 8 ? N : 8));
   p.plane = (size_t)N * R * HW;
-  p.part_elems = (size_t)p.S * R * ((size_t)T + C) + (size_t)N * R * ((size_t)Y + X);
+  p.part_elems = (size_t)p.S * R * ((size_t)T + C) + (size_t)p.St * R * ((size_t)Y + X);
   return p;
 }
 
