@@ -208,6 +208,33 @@ cp4_status cp4_pointer_is_device(const void* ptr, int* is_device);
 cp4_status cp4_stream_synchronize(cp4_stream);
 cp4_status cp4_device_synchronize(void);
 
+/* ---- 3-factor CP sibling op ------------------------------------------------
+ * Stands where the reference registers its TensorFlow op Conv2dCpFusedNchw
+ * (Kernels/cp_fused_nchw.cc:6-30, launcher Conv2dCpFusedNchwKernelLauncher :33):
+ *   y[n,t,h,w] = sum_r K2[r,t] sum_{i,j} K1[i,j,r] sum_c K0[c,r] x[n,c,h+i-pad,w+j-pad]
+ * with K0 [C,Rank], K1 [Y,X,Rank], K2 [Rank,T] (the reference's op is a generated
+ * kernel for the single shape N1 C16 32x32 3x3 Rank 6 T16; any shape here).
+ * The op runs on the CP4 kernels: cp3_expand_factors writes the equivalent CP4
+ * factors of rank Y*Rank (FK [T,Y*Rank], FC [C,Y*Rank], FH [Y,Y*Rank] - unit
+ * columns -, FW [X,Y*Rank]); the products with those ones and zeros are exact for
+ * finite inputs.  For training, run cp4_conv2d_backward_data / _backward_filter
+ * on the expanded factors (shape.Rank = Y*Rank) and cp3_fold_gradients on the
+ * result: dK0 [C,Rank], dK1 [Y,X,Rank], dK2 [Rank,T], fixed summation order.
+ * In every cp3_* call shape->Rank is the CP rank. */
+cp4_status cp3_expand_factors(const cp4_shape* shape, const float* K0,
+                              const float* K1, const float* K2, float* FK,
+                              float* FC, float* FH, float* FW, cp4_stream stream);
+cp4_status cp3_fold_gradients(const cp4_shape* shape, const float* dFK,
+                              const float* dFC, const float* dFW, float* dK0,
+                              float* dK1, float* dK2, cp4_stream stream);
+/* Forward in one call; `workspace` (device memory, at least
+ * cp3_conv2d_forward_workspace_bytes(shape) bytes) receives the expanded factors. */
+size_t cp3_conv2d_forward_workspace_bytes(const cp4_shape* shape);
+cp4_status cp3_conv2d_forward(const cp4_shape* shape, const float* x,
+                              const float* K0, const float* K1, const float* K2,
+                              float* y, void* workspace, size_t workspace_bytes,
+                              cp4_stream stream);
+
 /* ---- test / bench utilities (Cuda_kernels/Utils.cuh:9-13) ---------------- */
 
 /* Replaces cp_recompose (Utils.cu:36-98): K[T,C,Y,X] = sum_r FK FC FH FW. */

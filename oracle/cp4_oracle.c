@@ -13,6 +13,8 @@
  *        filter grads   Cuda_kernels/cp4Conv2dBackwardFilter.cu:23-257
  *        recomposition  Cuda_kernels/Utils.cu:55-62
  *        comparator     Cuda_kernels/Utils.cu:143-156
+ *        3-factor CP    test/layers.py:265-282 (forward only; its gradients are
+ *                       checked against float64 autograd in the GPU tests)
  *
  *  (2) "unfused" functions: the factor-by-factor sequence
  *        1x1 conv by FC -> depthwise 1-D conv by FH -> depthwise 1-D conv by
@@ -103,6 +105,51 @@ void cp4o_forward_direct(const cp4o_shape* s, const float* In, const float* FK,
           }
           Out[((n * T + t) * H + h) * W + w] = (float)acc;
         }
+}
+
+/* 3-factor CP sibling op, as the reference's Python layer defines it
+ * (test/layers.py:265-282: 1x1 conv by K0 [C,R], depthwise conv by K1 [Y,X,R],
+ * 1x1 conv by K2 [R,T]; Kernels/cp_fused_nchw.cc:20-24 for the layouts), same
+ * H x W output and zero reads outside the image as everywhere in this file:
+ *   Out[n,t,h,w] = sum_r K2[r,t] sum_{y,x} K1[y,x,r] sum_c K0[c,r]
+ *                  In[n,c,h+y-pad,w+x-pad]
+ * Pinned in tests/test_oracle.py against torch's dense conv2d on the kernel
+ * einsum('cr,ijr,rt->tcij') of test/test_conv2d_cp.py:20. */
+void cp3o_forward_direct(const cp4o_shape* s, const float* In, const float* K0,
+                         const float* K1, const float* K2, float* Out) {
+  const long N = s->N, H = s->H, W = s->W, P = s->pad, T = s->T, C = s->C,
+             Y = s->Y, X = s->X, R = s->Rank;
+  double* u0 = (double*)malloc(sizeof(double) * (size_t)(R * H * W));
+  double* u1 = (double*)malloc(sizeof(double) * (size_t)(R * H * W));
+  for (long n = 0; n < N; ++n) {
+    for (long r = 0; r < R; ++r)
+      for (long q = 0; q < H * W; ++q) {
+        double acc = 0.0;
+        for (long c = 0; c < C; ++c)
+          acc += (double)In[(n * C + c) * H * W + q] * (double)K0[c * R + r];
+        u0[r * H * W + q] = acc;
+      }
+    for (long r = 0; r < R; ++r)
+      for (long h = 0; h < H; ++h)
+        for (long w = 0; w < W; ++w) {
+          double acc = 0.0;
+          for (long y = 0; y < Y; ++y)
+            for (long x = 0; x < X; ++x) {
+              const long hh = h + y - P, ww = w + x - P;
+              if (hh >= 0 && hh < H && ww >= 0 && ww < W)
+                acc += u0[(r * H + hh) * W + ww] * (double)K1[(y * X + x) * R + r];
+            }
+          u1[(r * H + h) * W + w] = acc;
+        }
+    for (long t = 0; t < T; ++t)
+      for (long q = 0; q < H * W; ++q) {
+        double acc = 0.0;
+        for (long r = 0; r < R; ++r) acc += u1[r * H * W + q] * (double)K2[r * T + t];
+        Out[(n * T + t) * H * W + q] = (float)acc;
+      }
+  }
+  free(u0);
+  free(u1);
 }
 
 /* dx[n,c,h,w] = sum_r FC[c,r] sum_t FK[t,r] sum_{y,x} FH[Y-1-y,r] FW[X-1-x,r]

@@ -80,6 +80,18 @@ def forward(x, FK, FC, FH, FW, pad, direct=False):
     return y
 
 
+def cp3_forward(x, K0, K1, K2, pad):
+    """3-factor CP forward (pointwise K0 [C,R], depthwise K1 [Y,X,R], pointwise K2 [R,T])."""
+    x, K0, K1, K2 = map(_f32, (x, K0, K1, K2))
+    N, C, H, W = x.shape
+    s = Shape(N=N, H=H, W=W, pad=pad, T=K2.shape[1], C=C, Y=K1.shape[0], X=K1.shape[1],
+              Rank=K0.shape[1])
+    assert K0.shape == (C, s.Rank) and K1.shape[2] == s.Rank and K2.shape[0] == s.Rank
+    y = np.empty((N, s.T, H, W), np.float32)
+    lib().cp3o_forward_direct(ctypes.byref(s), _fp(x), _fp(K0), _fp(K1), _fp(K2), _fp(y))
+    return y
+
+
 def backward_data(dy, FK, FC, FH, FW, pad, direct=False):
     dy, FK, FC, FH, FW = map(_f32, (dy, FK, FC, FH, FW))
     N, T, H, W = dy.shape

@@ -88,6 +88,12 @@ def lib():
                                          ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
     L.cp4_tune_clear.restype = None
     L.cp4_recompose.argtypes = [_S, _F, _F, _F, _F, _F, ctypes.c_void_p]
+    L.cp3_expand_factors.argtypes = [_S] + [_F] * 7 + [ctypes.c_void_p]
+    L.cp3_fold_gradients.argtypes = [_S] + [_F] * 6 + [ctypes.c_void_p]
+    L.cp3_conv2d_forward_workspace_bytes.restype = ctypes.c_size_t
+    L.cp3_conv2d_forward_workspace_bytes.argtypes = [_S]
+    L.cp3_conv2d_forward.argtypes = [_S] + [_F] * 5 + [ctypes.c_void_p, ctypes.c_size_t,
+                                                        ctypes.c_void_p]
     L.cp4_count_exceeding.argtypes = [_F, _F, ctypes.c_size_t, ctypes.c_float,
                                       ctypes.POINTER(ctypes.c_longlong), ctypes.c_void_p]
     L.cp4_random_uniform.argtypes = [_F, ctypes.c_size_t, ctypes.c_ulonglong, ctypes.c_void_p]
@@ -320,6 +326,52 @@ def recompose(FK, FC, FH, FW, stream=None):
     check(lib().cp4_recompose(ctypes.byref(s), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
                               _ptr(K), _stream(stream)))
     return K
+
+
+def cp3_shape_for(x_shape, K0, K1, K2, pad):
+    """tensor_shape of the 3-factor CP op: K0 [C,R], K1 [Y,X,R], K2 [R,T]
+    (Kernels/cp_fused_nchw.cc:20-24); Rank is the CP rank."""
+    N, _, H, W = x_shape
+    assert K1.shape[2] == K0.shape[1] == K2.shape[0]
+    return Shape(N=N, H=H, W=W, pad=pad, T=K2.shape[1], C=K0.shape[0], Y=K1.shape[0],
+                 X=K1.shape[1], Rank=K0.shape[1])
+
+
+def cp3_expand_factors(K0, K1, K2, stream=None):
+    """The CP4 factors (FK, FC, FH, FW) of rank Y*R that compute the same convolution."""
+    s = cp3_shape_for((0, 0, 1, 1), K0, K1, K2, 0)
+    Q = s.Y * s.Rank
+    out = [torch.empty((d, Q), device=K0.device, dtype=torch.float32)
+           for d in (s.T, s.C, s.Y, s.X)]
+    check(lib().cp3_expand_factors(ctypes.byref(s), _ptr(K0), _ptr(K1), _ptr(K2),
+                                   *[_ptr(o) for o in out], _stream(stream)))
+    return tuple(out)
+
+
+def cp3_fold_gradients(dFK, dFC, dFW, Y, stream=None):
+    """(dK0, dK1, dK2) from the gradients of the expanded CP4 factors."""
+    Q = dFK.shape[1]
+    assert Q % Y == 0
+    s = Shape(T=dFK.shape[0], C=dFC.shape[0], Y=Y, X=dFW.shape[0], Rank=Q // Y)
+    dK0 = torch.empty((s.C, s.Rank), device=dFK.device, dtype=torch.float32)
+    dK1 = torch.empty((s.Y, s.X, s.Rank), device=dFK.device, dtype=torch.float32)
+    dK2 = torch.empty((s.Rank, s.T), device=dFK.device, dtype=torch.float32)
+    check(lib().cp3_fold_gradients(ctypes.byref(s), _ptr(dFK), _ptr(dFC), _ptr(dFW), _ptr(dK0),
+                                   _ptr(dK1), _ptr(dK2), _stream(stream)))
+    return dK0, dK1, dK2
+
+
+def cp3_conv2d_forward(x, K0, K1, K2, pad=1, out=None, stream=None):
+    s = cp3_shape_for(x.shape, K0, K1, K2, pad)
+    assert x.shape[1] == s.C
+    y = out if out is not None else torch.empty((s.N, s.T, s.H, s.W), device=x.device,
+                                                dtype=torch.float32)
+    nbytes = lib().cp3_conv2d_forward_workspace_bytes(ctypes.byref(s))
+    ws = torch.empty(nbytes, device=x.device, dtype=torch.uint8)
+    check(lib().cp3_conv2d_forward(ctypes.byref(s), _ptr(x), _ptr(K0), _ptr(K1), _ptr(K2),
+                                   _ptr(y), ctypes.c_void_p(ws.data_ptr()), nbytes,
+                                   _stream(stream)))
+    return y
 
 
 def count_exceeding(a, b, tol, stream=None):

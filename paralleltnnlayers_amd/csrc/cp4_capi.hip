@@ -648,6 +648,70 @@ cp4_status cp4_recompose(const cp4_shape* shape, const float* FK,
   return CP4_OK;
 }
 
+// ---- 3-factor CP sibling op ---------------------------------------------------
+
+namespace {
+size_t cp3_align(size_t floats) { return (floats + 63) & ~(size_t)63; }   // 256-byte slices
+
+cp4_status cp3_check(const cp4_shape* s) {
+  if (!s) return fail(CP4_ERR_NULL_POINTER, "shape is NULL");
+  if (!s->T || !s->C || !s->Y || !s->X || !s->Rank)
+    return fail(CP4_ERR_SHAPE, "T, C, Y, X and Rank must be >= 1");
+  if ((unsigned long long)s->Y * s->Rank > 65535ull)
+    return fail(CP4_ERR_SHAPE, "Y * Rank must be <= 65535");
+  return CP4_OK;
+}
+}  // namespace
+
+cp4_status cp3_expand_factors(const cp4_shape* shape, const float* K0, const float* K1,
+                              const float* K2, float* FK, float* FC, float* FH, float* FW,
+                              cp4_stream stream) {
+  cp4_status rc = cp3_check(shape);
+  if (rc != CP4_OK) return rc;
+  if (!K0 || !K1 || !K2 || !FK || !FC || !FH || !FW)
+    return fail(CP4_ERR_NULL_POINTER, "a data pointer is NULL");
+  CP4_HIP(cp4::cp3_expand_launch(*shape, K0, K1, K2, FK, FC, FH, FW, as_stream(stream)));
+  return CP4_OK;
+}
+
+cp4_status cp3_fold_gradients(const cp4_shape* shape, const float* dFK, const float* dFC,
+                              const float* dFW, float* dK0, float* dK1, float* dK2,
+                              cp4_stream stream) {
+  cp4_status rc = cp3_check(shape);
+  if (rc != CP4_OK) return rc;
+  if (!dFK || !dFC || !dFW || !dK0 || !dK1 || !dK2)
+    return fail(CP4_ERR_NULL_POINTER, "a data pointer is NULL");
+  CP4_HIP(cp4::cp3_fold_launch(*shape, dFK, dFC, dFW, dK0, dK1, dK2, as_stream(stream)));
+  return CP4_OK;
+}
+
+size_t cp3_conv2d_forward_workspace_bytes(const cp4_shape* s) {
+  if (!s) return 0;
+  const size_t Q = (size_t)s->Y * s->Rank;
+  return sizeof(float) * (cp3_align(s->T * Q) + cp3_align(s->C * Q) + cp3_align(s->Y * Q) +
+                          cp3_align(s->X * Q));
+}
+
+cp4_status cp3_conv2d_forward(const cp4_shape* shape, const float* x, const float* K0,
+                              const float* K1, const float* K2, float* y, void* workspace,
+                              size_t workspace_bytes, cp4_stream stream) {
+  cp4_status rc = cp3_check(shape);
+  if (rc != CP4_OK) return rc;
+  if (!workspace || workspace_bytes < cp3_conv2d_forward_workspace_bytes(shape))
+    return fail(CP4_ERR_WORKSPACE, "workspace missing or smaller than "
+                                   "cp3_conv2d_forward_workspace_bytes(shape)");
+  const size_t Q = (size_t)shape->Y * shape->Rank;
+  float* FK = static_cast<float*>(workspace);
+  float* FC = FK + cp3_align(shape->T * Q);
+  float* FH = FC + cp3_align(shape->C * Q);
+  float* FW = FH + cp3_align(shape->Y * Q);
+  rc = cp3_expand_factors(shape, K0, K1, K2, FK, FC, FH, FW, stream);
+  if (rc != CP4_OK) return rc;
+  cp4_shape wide = *shape;
+  wide.Rank = (unsigned)Q;
+  return cp4_conv2d_forward(&wide, x, FK, FC, FH, FW, y, stream);
+}
+
 cp4_status cp4_count_exceeding(const float* A, const float* B, size_t n,
                                float tol, long long* count, cp4_stream stream) {
   if (!count) return fail(CP4_ERR_NULL_POINTER, "count is NULL");

@@ -100,6 +100,13 @@ hipError_t count_exceeding_launch(const float* A, const float* B, size_t n,
                                   hipStream_t);
 hipError_t random_uniform_launch(float* dst, size_t n, unsigned long long seed,
                                  hipStream_t);
+// 3-factor CP sibling op: its factors as a CP4 of rank Y*Rank (s.Rank is the CP
+// rank), and the fold of the CP4 factor gradients back onto the three factors.
+hipError_t cp3_expand_launch(const cp4_shape& s, const float* K0, const float* K1,
+                             const float* K2, float* FK, float* FC, float* FH, float* FW,
+                             hipStream_t);
+hipError_t cp3_fold_launch(const cp4_shape& s, const float* dFK, const float* dFC,
+                           const float* dFW, float* dK0, float* dK1, float* dK2, hipStream_t);
 hipError_t copy_f32_launch(float* dst, const float* src, size_t n, hipStream_t);
 // Fill kernel rather than a memset node, so that callers may capture the
 // empty-batch paths into a graph like every other launch.

@@ -93,6 +93,63 @@ __global__ __launch_bounds__(256) void bias_act_kernel(float* __restrict__ y,
   }
 }
 
+// 3-factor CP (pointwise K0 [C,R], depthwise K1 [Y,X,R], pointwise K2 [R,T];
+// Kernels/cp_fused_nchw.cc:20-24) written as a CP4 of rank Y*R: rank q = i*R + r
+// stands for row i of the depthwise filter of rank r,
+//   FC'[c,q] = K0[c,r]   FH'[y,q] = (y == i)   FW'[x,q] = K1[i,x,r]   FK'[t,q] = K2[r,t].
+// The unit column taps only multiply by one and add zeros, so the CP4 kernels
+// compute sum_r K2[r,t] sum_{i,x} K1[i,x,r] sum_c K0[c,r] x[...] with no extra rounding.
+__global__ __launch_bounds__(256) void cp3_expand_kernel(
+    const float* __restrict__ K0, const float* __restrict__ K1, const float* __restrict__ K2,
+    float* __restrict__ FK, float* __restrict__ FC, float* __restrict__ FH,
+    float* __restrict__ FW, int T, int C, int Y, int X, int R) {
+  const size_t Q = (size_t)Y * R, total = (size_t)(T + C + Y + X) * Q;
+  for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * 256) {
+    const size_t q = idx % Q;
+    int row = (int)(idx / Q);
+    const int i = (int)(q / R), r = (int)(q % R);
+    if (row < T) {
+      FK[(size_t)row * Q + q] = K2[(size_t)r * T + row];
+    } else if ((row -= T) < C) {
+      FC[(size_t)row * Q + q] = K0[(size_t)row * R + r];
+    } else if ((row -= C) < Y) {
+      FH[(size_t)row * Q + q] = row == i ? 1.f : 0.f;
+    } else {
+      row -= Y;
+      FW[(size_t)row * Q + q] = K1[((size_t)i * X + row) * R + r];
+    }
+  }
+}
+
+// Gradients of the three CP factors from those of the expanded CP4 factors:
+// K0[c,r] and K2[r,t] appear in Y expanded columns each (summed in row order),
+// K1[i,x,r] in exactly one.
+__global__ __launch_bounds__(256) void cp3_fold_kernel(
+    const float* __restrict__ dFK, const float* __restrict__ dFC, const float* __restrict__ dFW,
+    float* __restrict__ dK0, float* __restrict__ dK1, float* __restrict__ dK2,
+    int T, int C, int Y, int X, int R) {
+  const size_t Q = (size_t)Y * R;
+  const size_t n0 = (size_t)C * R, n1 = (size_t)Y * X * R, n2 = (size_t)R * T;
+  for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < n0 + n1 + n2;
+       idx += (size_t)gridDim.x * 256) {
+    if (idx < n0) {
+      const size_t c = idx / R, r = idx % R;
+      float acc = 0.f;
+      for (int i = 0; i < Y; ++i) acc += dFC[c * Q + (size_t)i * R + r];
+      dK0[idx] = acc;
+    } else if (idx < n0 + n1) {
+      const size_t j = idx - n0, r = j % R, x = (j / R) % X, i = j / ((size_t)R * X);
+      dK1[j] = dFW[x * Q + i * R + r];
+    } else {
+      const size_t j = idx - n0 - n1, t = j % T, r = j / T;
+      float acc = 0.f;
+      for (int i = 0; i < Y; ++i) acc += dFK[t * Q + (size_t)i * R + r];
+      dK2[j] = acc;
+    }
+  }
+}
+
 unsigned grid_for(size_t n, unsigned cap) {
   const size_t g = (n + 255) / 256;
   return (unsigned)(g < 1 ? 1 : g > cap ? cap : g);
@@ -134,6 +191,24 @@ hipError_t bias_act_launch(float* y, const float* bias, int act, size_t N, size_
 hipError_t zero_f32_launch(float* dst, size_t n, hipStream_t st) {
   if (n == 0) return hipSuccess;
   zero_f32_kernel<<<grid_for(n, 2048), 256, 0, st>>>(dst, n);
+  return hipGetLastError();
+}
+
+hipError_t cp3_expand_launch(const cp4_shape& s, const float* K0, const float* K1,
+                             const float* K2, float* FK, float* FC, float* FH, float* FW,
+                             hipStream_t st) {
+  const size_t total = (size_t)(s.T + s.C + s.Y + s.X) * s.Y * s.Rank;
+  cp3_expand_kernel<<<grid_for(total, 4096), 256, 0, st>>>(K0, K1, K2, FK, FC, FH, FW, s.T, s.C,
+                                                          s.Y, s.X, s.Rank);
+  return hipGetLastError();
+}
+
+hipError_t cp3_fold_launch(const cp4_shape& s, const float* dFK, const float* dFC,
+                           const float* dFW, float* dK0, float* dK1, float* dK2,
+                           hipStream_t st) {
+  const size_t total = (size_t)s.Rank * (s.C + s.T + (size_t)s.Y * s.X);
+  cp3_fold_kernel<<<grid_for(total, 4096), 256, 0, st>>>(dFK, dFC, dFW, dK0, dK1, dK2, s.T, s.C,
+                                                        s.Y, s.X, s.Rank);
   return hipGetLastError();
 }
 

@@ -127,3 +127,46 @@ class CP4Conv2d(torch.nn.Module):
         """The recomposed [T,C,Y,X] filter (on the device, through cp4_recompose)."""
         return capi.recompose(self.FK.detach(), self.FC.detach(), self.FH.detach(),
                               self.FW.detach())
+
+
+class CP3Conv2dFunction(torch.autograd.Function):
+    """The 3-factor CP convolution of the reference's ``Conv2dCpFusedNchw`` op
+    (Kernels/cp_fused_nchw.cc:6-30; its Python definition is pointwise K0,
+    depthwise K1, pointwise K2, test/layers.py:265-282):
+
+        y[n,t] = sum_r K2[r,t] * (K1[:,:,r] (*) sum_c K0[c,r] x[n,c])
+
+    K0 [C,R], K1 [Y,X,R], K2 [R,T].  Runs on the fused CP4 kernels through the
+    library's exact rank-Y*R rewriting of the factors; the factor gradients are
+    folded back by the library as well.
+    """
+
+    @staticmethod
+    def forward(ctx, x, K0, K1, K2, pad):
+        if 2 * pad + 1 != K1.shape[0] or 2 * pad + 1 != K1.shape[1]:
+            raise ValueError("autograd binding needs 2*pad = Y-1 = X-1")
+        K0, K1, K2 = (t.contiguous().float() for t in (K0, K1, K2))
+        x = x.contiguous().float()
+        fac = capi.cp3_expand_factors(K0, K1, K2)
+        ctx.pad, ctx.Y = pad, K1.shape[0]
+        ctx.save_for_backward(x, *fac)
+        return capi.conv2d_forward(x, *fac, pad=pad)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, FK, FC, FH, FW = ctx.saved_tensors
+        dy = dy.contiguous().float()
+        dx = None
+        if ctx.needs_input_grad[0]:
+            dx = capi.conv2d_backward_data(dy, FK, FC, FH, FW, pad=ctx.pad)
+        grads = (None, None, None)
+        if any(ctx.needs_input_grad[1:4]):
+            dFK, dFC, _, dFW = capi.conv2d_backward_filter(x, dy, FK, FC, FH, FW, pad=ctx.pad)
+            grads = capi.cp3_fold_gradients(dFK, dFC, dFW, ctx.Y)
+            grads = tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad[1:4]))
+        return (dx,) + grads + (None,)
+
+
+def cp3_conv2d(x, K0, K1, K2, pad):
+    """Functional form of the differentiable 3-factor CP convolution (NCHW)."""
+    return CP3Conv2dFunction.apply(x, K0, K1, K2, pad)

@@ -18,7 +18,7 @@ def L():
 def declared_functions(header="capi.h"):
     text = open(os.path.join(ROOT, "include", "cp4", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(cp4_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(cp[34]_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_declares_the_three_passes():

@@ -224,3 +224,35 @@ def test_count_exceeding_semantics(oracle):
     b = a.copy(); b[2] = 0.05                   # a == 0 -> absolute error
     assert oracle.count_exceeding(a, b, 1e-1) == 0
     assert oracle.count_exceeding(a, b, 1e-2) == 1
+
+
+# ---- 3-factor CP sibling op ------------------------------------------------------
+
+@pytest.mark.parametrize("shape", [(1, 16, 32, 32, 3, 6, 16),     # test/test_conv2d_cp.py:12-15
+                                   (2, 5, 9, 7, 5, 4, 3),
+                                   (1, 3, 6, 6, 1, 2, 4)])
+def test_cp3_forward_vs_torch_dense_conv(oracle, shape):
+    """The reference's own check (test/test_conv2d_cp.py:20,27-31): the CP layer equals
+    the dense convolution with kernel einsum over the three factors."""
+    N, C, H, W, Y, R, T = shape
+    rng = np.random.default_rng(7)
+    x = rng.uniform(size=(N, C, H, W)).astype(np.float32)
+    K0 = rng.uniform(size=(C, R)).astype(np.float32)
+    K1 = rng.uniform(size=(Y, Y, R)).astype(np.float32)
+    K2 = rng.uniform(size=(R, T)).astype(np.float32)
+    dense = np.einsum("cr,ijr,rt->tcij", K0.astype(np.float64), K1.astype(np.float64),
+                      K2.astype(np.float64))
+    want = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(dense), padding=Y // 2).numpy()
+    close(oracle.cp3_forward(x, K0, K1, K2, Y // 2), want, 1e-5)
+
+
+def test_cp3_depthwise_tap_orientation(oracle):
+    """A single tap at (row 0, column 2) of a 3x3 depthwise filter reads the pixel one row
+    up and one column right: fails on a transposed or flipped K1."""
+    x = np.arange(25, dtype=np.float32).reshape(1, 1, 5, 5)
+    K1 = np.zeros((3, 3, 1), np.float32)
+    K1[0, 2, 0] = 1.0
+    y = oracle.cp3_forward(x, np.ones((1, 1), np.float32), K1, np.ones((1, 1), np.float32), 1)
+    want = np.zeros((5, 5), np.float32)
+    want[1:, :4] = x[0, 0, :4, 1:]
+    np.testing.assert_array_equal(y[0, 0], want)
