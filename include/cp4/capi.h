@@ -227,13 +227,23 @@ cp4_status cp3_expand_factors(const cp4_shape* shape, const float* K0,
 cp4_status cp3_fold_gradients(const cp4_shape* shape, const float* dFK,
                               const float* dFC, const float* dFW, float* dK0,
                               float* dK1, float* dK2, cp4_stream stream);
-/* Forward in one call; `workspace` (device memory, at least
- * cp3_conv2d_forward_workspace_bytes(shape) bytes) receives the expanded factors. */
+/* Forward and input gradient in one call each; `workspace` (device memory, at
+ * least cp3_conv2d_forward_workspace_bytes(shape) bytes, either pass) is scratch
+ * for rewritten factors.  With Rank <= 32 and a 1x1 or 3x3 filter the producer /
+ * consumer kernel applies K1 itself in its tap step (only K2 is transposed);
+ * other shapes run on the expanded factors.  The input gradient uses the
+ * reference's backward-data convention (flipped taps at offset +y-pad,
+ * Cuda_kernels/cp4Conv2dBackwardData.cu:79-87): the adjoint of the forward when
+ * 2*pad = Y-1 = X-1. */
 size_t cp3_conv2d_forward_workspace_bytes(const cp4_shape* shape);
 cp4_status cp3_conv2d_forward(const cp4_shape* shape, const float* x,
                               const float* K0, const float* K1, const float* K2,
                               float* y, void* workspace, size_t workspace_bytes,
                               cp4_stream stream);
+cp4_status cp3_conv2d_backward_data(const cp4_shape* shape, const float* dy,
+                                    const float* K0, const float* K1,
+                                    const float* K2, float* dx, void* workspace,
+                                    size_t workspace_bytes, cp4_stream stream);
 
 /* ---- test / bench utilities (Cuda_kernels/Utils.cuh:9-13) ---------------- */
 

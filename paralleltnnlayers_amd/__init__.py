@@ -13,6 +13,6 @@ from .capi import (Shape, Cp4Error, lib, library_path, conv2d_forward, conv2d_fo
                    time_forward, time_backward_data, time_backward_filter,
                    tune_forward, forward_variants, recompose, count_exceeding,
                    random_uniform, time_copy, cp3_shape_for, cp3_expand_factors,
-                   cp3_fold_gradients, cp3_conv2d_forward)
+                   cp3_fold_gradients, cp3_conv2d_forward, cp3_conv2d_backward_data)
 
 __all__ = [n for n in dir() if not n.startswith("_")]

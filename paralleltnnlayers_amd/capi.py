@@ -94,6 +94,7 @@ def lib():
     L.cp3_conv2d_forward_workspace_bytes.argtypes = [_S]
     L.cp3_conv2d_forward.argtypes = [_S] + [_F] * 5 + [ctypes.c_void_p, ctypes.c_size_t,
                                                         ctypes.c_void_p]
+    L.cp3_conv2d_backward_data.argtypes = L.cp3_conv2d_forward.argtypes
     L.cp4_count_exceeding.argtypes = [_F, _F, ctypes.c_size_t, ctypes.c_float,
                                       ctypes.POINTER(ctypes.c_longlong), ctypes.c_void_p]
     L.cp4_random_uniform.argtypes = [_F, ctypes.c_size_t, ctypes.c_ulonglong, ctypes.c_void_p]
@@ -361,17 +362,30 @@ def cp3_fold_gradients(dFK, dFC, dFW, Y, stream=None):
     return dK0, dK1, dK2
 
 
-def cp3_conv2d_forward(x, K0, K1, K2, pad=1, out=None, stream=None):
+def _cp3_pass(fn, s, src, K0, K1, K2, dst, workspace, stream):
+    nbytes = lib().cp3_conv2d_forward_workspace_bytes(ctypes.byref(s))
+    ws = workspace if workspace is not None else torch.empty(nbytes, device=src.device,
+                                                             dtype=torch.uint8)
+    assert ws.numel() * ws.element_size() >= nbytes
+    check(fn(ctypes.byref(s), _ptr(src), _ptr(K0), _ptr(K1), _ptr(K2), _ptr(dst),
+             ctypes.c_void_p(ws.data_ptr()), nbytes, _stream(stream)))
+    return dst
+
+
+def cp3_conv2d_forward(x, K0, K1, K2, pad=1, out=None, workspace=None, stream=None):
     s = cp3_shape_for(x.shape, K0, K1, K2, pad)
     assert x.shape[1] == s.C
     y = out if out is not None else torch.empty((s.N, s.T, s.H, s.W), device=x.device,
                                                 dtype=torch.float32)
-    nbytes = lib().cp3_conv2d_forward_workspace_bytes(ctypes.byref(s))
-    ws = torch.empty(nbytes, device=x.device, dtype=torch.uint8)
-    check(lib().cp3_conv2d_forward(ctypes.byref(s), _ptr(x), _ptr(K0), _ptr(K1), _ptr(K2),
-                                   _ptr(y), ctypes.c_void_p(ws.data_ptr()), nbytes,
-                                   _stream(stream)))
-    return y
+    return _cp3_pass(lib().cp3_conv2d_forward, s, x, K0, K1, K2, y, workspace, stream)
+
+
+def cp3_conv2d_backward_data(dy, K0, K1, K2, pad=1, out=None, workspace=None, stream=None):
+    s = cp3_shape_for(dy.shape, K0, K1, K2, pad)
+    assert dy.shape[1] == s.T
+    dx = out if out is not None else torch.empty((s.N, s.C, s.H, s.W), device=dy.device,
+                                                 dtype=torch.float32)
+    return _cp3_pass(lib().cp3_conv2d_backward_data, s, dy, K0, K1, K2, dx, workspace, stream)
 
 
 def count_exceeding(a, b, tol, stream=None):

@@ -692,16 +692,40 @@ size_t cp3_conv2d_forward_workspace_bytes(const cp4_shape* s) {
                           cp3_align(s->X * Q));
 }
 
-cp4_status cp3_conv2d_forward(const cp4_shape* shape, const float* x, const float* K0,
-                              const float* K1, const float* K2, float* y, void* workspace,
-                              size_t workspace_bytes, cp4_stream stream) {
+namespace {
+// The pass on the producer / consumer kernel's 2-D-tap build when that kernel is
+// the right one for the shape (whole-row strips that fit, enough channels to
+// fill its tiles, at most 256 input channels on large problems), else on the
+// expanded CP4 factors through the usual choice of variants.
+cp4_status cp3_run(const cp4_shape* shape, const float* in, const float* K0, const float* K1,
+                   const float* K2, float* out, void* workspace, size_t workspace_bytes,
+                   bool backward, cp4_stream stream) {
   cp4_status rc = cp3_check(shape);
   if (rc != CP4_OK) return rc;
+  rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return CP4_OK;
+  if (!in || !K0 || !K1 || !K2 || !out)
+    return fail(CP4_ERR_NULL_POINTER, "a data pointer is NULL");
   if (!workspace || workspace_bytes < cp3_conv2d_forward_workspace_bytes(shape))
     return fail(CP4_ERR_WORKSPACE, "workspace missing or smaller than "
                                    "cp3_conv2d_forward_workspace_bytes(shape)");
+  hipStream_t st = as_stream(stream);
   const size_t Q = (size_t)shape->Y * shape->Rank;
   float* FK = static_cast<float*>(workspace);
+
+  // K2 [R,T] as an out-channel factor [T,R]; K0 is an in-channel factor as it is
+  FwdArgs a = backward ? backward_data_args(*shape, in, FK, K0, nullptr, nullptr, out)
+                       : forward_args(*shape, in, FK, K0, nullptr, nullptr, out);
+  a.taps2d = K1;
+  const size_t pixels = (size_t)a.N * a.H * a.W;
+  if (cp4::fwd_pipe_taps2d_supported(a) && a.W <= 128 && a.Cin + a.Cout >= 24 &&
+      !(a.Cin > 256 && pixels > 8192)) {
+    CP4_HIP(cp4::transpose_f32_launch(K2, FK, (int)shape->Rank, (int)shape->T, st));
+    CP4_HIP(cp4::fwd_pipe_taps2d_launch(a, st));
+    return CP4_OK;
+  }
+
   float* FC = FK + cp3_align(shape->T * Q);
   float* FH = FC + cp3_align(shape->C * Q);
   float* FW = FH + cp3_align(shape->Y * Q);
@@ -709,7 +733,22 @@ cp4_status cp3_conv2d_forward(const cp4_shape* shape, const float* x, const floa
   if (rc != CP4_OK) return rc;
   cp4_shape wide = *shape;
   wide.Rank = (unsigned)Q;
-  return cp4_conv2d_forward(&wide, x, FK, FC, FH, FW, y, stream);
+  return backward ? cp4_conv2d_backward_data(&wide, in, FK, FC, FH, FW, out, stream)
+                  : cp4_conv2d_forward(&wide, in, FK, FC, FH, FW, out, stream);
+}
+}  // namespace
+
+cp4_status cp3_conv2d_forward(const cp4_shape* shape, const float* x, const float* K0,
+                              const float* K1, const float* K2, float* y, void* workspace,
+                              size_t workspace_bytes, cp4_stream stream) {
+  return cp3_run(shape, x, K0, K1, K2, y, workspace, workspace_bytes, false, stream);
+}
+
+cp4_status cp3_conv2d_backward_data(const cp4_shape* shape, const float* dy, const float* K0,
+                                    const float* K1, const float* K2, float* dx,
+                                    void* workspace, size_t workspace_bytes,
+                                    cp4_stream stream) {
+  return cp3_run(shape, dy, K0, K1, K2, dx, workspace, workspace_bytes, true, stream);
 }
 
 cp4_status cp4_count_exceeding(const float* A, const float* B, size_t n,

@@ -32,6 +32,9 @@ struct FwdArgs {
   // and accumulate != 0 adds to y instead of overwriting it.
   int ldf;
   int accumulate;
+  // 2-D-tap build of the producer / consumer kernel only: depthwise filter
+  // [Y, X, R] used instead of the outer product FH x FW (FH, FW unused then).
+  const float* taps2d;
 };
 
 
@@ -65,6 +68,9 @@ hipError_t fwd_pipe_rankpass_launch(const FwdArgs&, hipStream_t);
 // The same kernel on tiles of TH rows x Wt columns (wide planes).
 bool fwd_pipe_tiled_supported(const FwdArgs&);
 hipError_t fwd_pipe_tiled_launch(const FwdArgs&, hipStream_t);
+// The same kernel with a depthwise Y x X filter (FwdArgs::taps2d) in its tap step.
+bool fwd_pipe_taps2d_supported(const FwdArgs&);
+hipError_t fwd_pipe_taps2d_launch(const FwdArgs&, hipStream_t);
 // In-place y[n,k,:] = act(y[n,k,:] + bias[k]) for variants without the epilogue.
 hipError_t bias_act_launch(float* y, const float* bias, int act, size_t N, size_t K, size_t HW,
                            hipStream_t);
@@ -107,6 +113,8 @@ hipError_t cp3_expand_launch(const cp4_shape& s, const float* K0, const float* K
                              hipStream_t);
 hipError_t cp3_fold_launch(const cp4_shape& s, const float* dFK, const float* dFC,
                            const float* dFW, float* dK0, float* dK1, float* dK2, hipStream_t);
+// dst [cols, rows] = transpose of src [rows, cols]
+hipError_t transpose_f32_launch(const float* src, float* dst, int rows, int cols, hipStream_t);
 hipError_t copy_f32_launch(float* dst, const float* src, size_t n, hipStream_t);
 // Fill kernel rather than a memset node, so that callers may capture the
 // empty-batch paths into a graph like every other launch.

@@ -40,7 +40,7 @@
 // Cuda_kernels/cp4Conv2dForward.cu:84-133 (backward-data:
 // cp4Conv2dBackwardData.cu:57-108 through swapped factors and flipped taps).
 //
-// This file is compiled five times: as is; with CP4_PIPE_EPILOGUE defined, which
+// This file is compiled six times: as is; with CP4_PIPE_EPILOGUE defined, which
 // adds y = act(conv + bias[k]) to the stores (the bias of the lane's sixteen
 // output rows rides in registers next to the output-factor fragment) and exports
 // the entry points under the names fwd_pipe_epi_*; and with CP4_PIPE_IO16, where
@@ -55,7 +55,11 @@
 // columns (Wt a power of two, at least 64) instead of TH whole rows; the LDS
 // plane holds the tile plus its halo in rows of Wt + FS - 1 cells, so the taps
 // need no border masks (cells outside the image are stored as zeros) and every
-// 64-pixel output group is one row segment; entry points fwd_pipe_tiled_*.
+// 64-pixel output group is one row segment; entry points fwd_pipe_tiled_*;
+// and with CP4_PIPE_TAPS2D, for the 3-factor CP sibling op: the tap step weighs
+// the Y x X cells it reads with a depthwise filter FwdArgs::taps2d [Y, X, R]
+// instead of the outer product FH x FW (1x1 and 3x3 filters: 36 wave-uniform
+// weights per wave), entry points fwd_pipe_taps2d_*.
 #include <cstdlib>
 #include <type_traits>
 
@@ -429,6 +433,18 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     const bool split_roles = FS <= 5 && R <= 16 && nkb <= 4;   // (7x7: no registers to spare)
     const int wq = split_roles ? (wc >= 4 ? wc - 4 : 0) : wc;     // rank quad in the tap step
     // Tap weights of this wave's 4 ranks (wave-uniform values).
+#ifdef CP4_PIPE_TAPS2D
+    float w2[4][FS][FS];
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr)
+#pragma unroll
+      for (int ti = 0; ti < FS; ++ti)
+#pragma unroll
+        for (int j = 0; j < FS; ++j) {
+          const int ty = a.flip ? FS - 1 - ti : ti, tx = a.flip ? FS - 1 - j : j, r = 4 * wq + rr;
+          w2[rr][ti][j] = r < R ? a.taps2d[(ty * FS + tx) * ldf + r] : 0.f;
+        }
+#else
     float fh[4][FS], fw[4][FS];
 #pragma unroll
     for (int rr = 0; rr < 4; ++rr)
@@ -438,6 +454,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         fh[rr][j] = r < R ? a.FH[tap * ldf + r] : 0.f;
         fw[rr][j] = r < R ? a.FW[tap * ldf + r] : 0.f;
       }
+#endif
 #ifdef CP4_PIPE_TILED
     io_t* yn = reinterpret_cast<io_t*>(a.y) + (size_t)n * Cout * HW + (size_t)h0 * W + w0;
 #else
@@ -538,10 +555,15 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           float s = 0.f;
 #pragma unroll
           for (int ti = 0; ti < FS; ++ti) {
+#ifdef CP4_PIPE_TAPS2D
+#pragma unroll
+            for (int j = 0; j < FS; ++j) s += (in[j] ? w2[r0 + rr][ti][j] : 0.f) * av[rr][ti][j];
+#else
             float hs = 0.f;
 #pragma unroll
             for (int j = 0; j < FS; ++j) hs += (in[j] ? fw[r0 + rr][j] : 0.f) * av[rr][ti][j];
             s += fh[r0 + rr][ti] * hs;
+#endif
           }
           o[r0 + rr] = s;
         }
@@ -861,7 +883,10 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 
 }  // namespace
 
-#if defined(CP4_PIPE_TILED)
+#if defined(CP4_PIPE_TAPS2D)
+#define fwd_pipe_supported fwd_pipe_taps2d_supported
+#define fwd_pipe_launch fwd_pipe_taps2d_launch
+#elif defined(CP4_PIPE_TILED)
 #define fwd_pipe_supported fwd_pipe_tiled_supported
 #define fwd_pipe_launch fwd_pipe_tiled_launch
 #elif defined(CP4_PIPE_RANKPASS)
@@ -883,6 +908,9 @@ bool fwd_pipe_supported(const FwdArgs& a) {
   if (!fits_int_indexing(a.N, a.H, a.W)) return false;
   if ((size_t)a.Cin * a.H * a.W * sizeof(io_t) >= (1ull << 31)) return false;   // buffer offsets
   if (a.Y != a.X || !(a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7)) return false;
+#ifdef CP4_PIPE_TAPS2D
+  if (!a.taps2d || a.Y > 3) return false;        // 4 * Y * X weights per wave in registers
+#endif
   PipePlan pl;
   return plan(a, &pl);
 }
@@ -896,8 +924,12 @@ hipError_t fwd_pipe_launch(const FwdArgs& a, hipStream_t st) {
   switch (a.Y) {
     case 1: return launch_fs<1>(a, pl, st);
     case 3: return launch_fs<3>(a, pl, st);
+#ifdef CP4_PIPE_TAPS2D
+    default: return hipErrorInvalidValue;          // larger filters: the weights would spill
+#else
     case 5: return launch_fs<5>(a, pl, st);
     default: return launch_fs<7>(a, pl, st);
+#endif
   }
 }
 

@@ -150,6 +150,16 @@ __global__ __launch_bounds__(256) void cp3_fold_kernel(
   }
 }
 
+// dst[c, r] = src[r, c] (the [R,T] pointwise factor of the 3-factor CP op as a [T,R] one)
+__global__ __launch_bounds__(256) void transpose_f32_kernel(const float* __restrict__ src,
+                                                            float* __restrict__ dst, int rows,
+                                                            int cols) {
+  const size_t total = (size_t)rows * cols;
+  for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * 256)
+    dst[idx] = src[(idx % rows) * cols + idx / rows];
+}
+
 unsigned grid_for(size_t n, unsigned cap) {
   const size_t g = (n + 255) / 256;
   return (unsigned)(g < 1 ? 1 : g > cap ? cap : g);
@@ -209,6 +219,12 @@ hipError_t cp3_fold_launch(const cp4_shape& s, const float* dFK, const float* dF
   const size_t total = (size_t)s.Rank * (s.C + s.T + (size_t)s.Y * s.X);
   cp3_fold_kernel<<<grid_for(total, 4096), 256, 0, st>>>(dFK, dFC, dFW, dK0, dK1, dK2, s.T, s.C,
                                                         s.Y, s.X, s.Rank);
+  return hipGetLastError();
+}
+
+hipError_t transpose_f32_launch(const float* src, float* dst, int rows, int cols,
+                                hipStream_t st) {
+  transpose_f32_kernel<<<grid_for((size_t)rows * cols, 4096), 256, 0, st>>>(src, dst, rows, cols);
   return hipGetLastError();
 }
 

@@ -136,9 +136,9 @@ class CP3Conv2dFunction(torch.autograd.Function):
 
         y[n,t] = sum_r K2[r,t] * (K1[:,:,r] (*) sum_c K0[c,r] x[n,c])
 
-    K0 [C,R], K1 [Y,X,R], K2 [R,T].  Runs on the fused CP4 kernels through the
-    library's exact rank-Y*R rewriting of the factors; the factor gradients are
-    folded back by the library as well.
+    K0 [C,R], K1 [Y,X,R], K2 [R,T].  Forward and input gradient are the library's
+    cp3 passes; the factor gradients come from the CP4 backward-filter pass on the
+    library's exact rank-Y*R rewriting of the factors, folded back by the library.
     """
 
     @staticmethod
@@ -147,22 +147,22 @@ class CP3Conv2dFunction(torch.autograd.Function):
             raise ValueError("autograd binding needs 2*pad = Y-1 = X-1")
         K0, K1, K2 = (t.contiguous().float() for t in (K0, K1, K2))
         x = x.contiguous().float()
-        fac = capi.cp3_expand_factors(K0, K1, K2)
-        ctx.pad, ctx.Y = pad, K1.shape[0]
-        ctx.save_for_backward(x, *fac)
-        return capi.conv2d_forward(x, *fac, pad=pad)
+        ctx.pad = pad
+        ctx.save_for_backward(x, K0, K1, K2)
+        return capi.cp3_conv2d_forward(x, K0, K1, K2, pad=pad)
 
     @staticmethod
     def backward(ctx, dy):
-        x, FK, FC, FH, FW = ctx.saved_tensors
+        x, K0, K1, K2 = ctx.saved_tensors
         dy = dy.contiguous().float()
         dx = None
         if ctx.needs_input_grad[0]:
-            dx = capi.conv2d_backward_data(dy, FK, FC, FH, FW, pad=ctx.pad)
+            dx = capi.cp3_conv2d_backward_data(dy, K0, K1, K2, pad=ctx.pad)
         grads = (None, None, None)
         if any(ctx.needs_input_grad[1:4]):
+            FK, FC, FH, FW = capi.cp3_expand_factors(K0, K1, K2)
             dFK, dFC, _, dFW = capi.conv2d_backward_filter(x, dy, FK, FC, FH, FW, pad=ctx.pad)
-            grads = capi.cp3_fold_gradients(dFK, dFC, dFW, ctx.Y)
+            grads = capi.cp3_fold_gradients(dFK, dFC, dFW, K1.shape[0])
             grads = tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad[1:4]))
         return (dx,) + grads + (None,)
 

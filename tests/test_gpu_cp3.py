@@ -63,6 +63,42 @@ def test_cp3_forward_matches_oracle(cp4, oracle, dims):
     assert err.max() <= 1e-4 * np.abs(want).max()
 
 
+# shapes on the 2-D-tap build of the producer / consumer kernel (R <= 32, 3x3 or 1x1)
+NATIVE = [
+    (2, 64, 28, 28, 3, 16, 64),    # split consumer roles (R <= 16, at most 4 channel blocks)
+    (2, 256, 56, 56, 3, 32, 256),  # full rank tile, registers-resident factor slice
+    (3, 40, 13, 13, 3, 21, 72),    # odd plane, ragged channels and ranks
+    (1, 320, 14, 14, 3, 12, 300),  # factor fragments in LDS
+    (2, 16, 20, 20, 1, 8, 24),     # 1x1, one-chunk producers
+]
+
+
+@pytest.mark.parametrize("dims", NATIVE, ids=lambda d: "x".join(map(str, d)))
+def test_cp3_native_taps_agree_with_expanded_factors(cp4, oracle, dims):
+    """Forward and input gradient of the one-pass kernel against the same passes run on
+    the expanded CP4 factors (whose kernels the oracle pins), to the forward bar; the
+    forward of the smaller shapes also against the oracle directly."""
+    x, K0, K1, K2 = operands(dims)
+    N, C, H, W, Y, R, T = dims
+    pad = Y // 2
+    dK = [dev(a) for a in (K0, K1, K2)]
+    fac = cp4.cp3_expand_factors(*dK)
+    y = host(cp4.cp3_conv2d_forward(dev(x), *dK, pad=pad))
+    y_ref = host(cp4.conv2d_forward(dev(x), *fac, pad=pad))
+    assert np.abs(y - y_ref).max() <= 1e-5 * np.abs(y_ref).max()
+    if N * C * H * W * R <= 2 ** 24:
+        want = oracle.cp3_forward(x, K0, K1, K2, pad)
+        err = np.abs(y - want)
+        assert (err <= 1e-5 + 1e-4 * np.abs(want)).all() and err.max() <= 1e-4 * np.abs(want).max()
+    dy = np.random.default_rng(5).standard_normal((N, T, H, W)).astype(np.float32)
+    dx = host(cp4.cp3_conv2d_backward_data(dev(dy), *dK, pad=pad))
+    dx_ref = host(cp4.conv2d_backward_data(dev(dy), *fac, pad=pad))
+    assert np.abs(dx - dx_ref).max() <= 1e-5 * np.abs(dx_ref).max()
+    # adjoint identity ("same" padding): <dy, conv(x)> = <conv^T(dy), x>
+    lhs = float((dy.astype(np.float64) * y).sum()); rhs = float((dx.astype(np.float64) * x).sum())
+    assert abs(lhs - rhs) <= 1e-4 * max(abs(lhs), np.sqrt(float((dy ** 2).sum()) * float((y ** 2).sum())) * 1e-2)
+
+
 def test_cp3_expanded_factors_exact(cp4):
     _, K0, K1, K2 = operands((1, 7, 4, 4, 3, 5, 9))
     FK, FC, FH, FW = (host(t) for t in cp4.cp3_expand_factors(dev(K0), dev(K1), dev(K2)))
