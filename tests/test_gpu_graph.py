@@ -79,3 +79,45 @@ def test_empty_batch_gradients_capture(cp4):
         graph.replay()
         torch.cuda.synchronize()
         assert all(float(g.abs().max()) == 0.0 for g in grads)
+
+
+@pytest.mark.parametrize("dims", [(2, 64, 28, 28, 64, 3, 12), (2, 24, 14, 14, 24, 5, 6)],
+                         ids=lambda d: "x".join(map(str, d)))
+def test_cp3_passes_replay(cp4, dims):
+    """The 3-factor CP passes (factor rewriting kernels included) with a caller-owned
+    workspace: one-pass kernel with the depthwise tap step / expanded factors."""
+    N, C, H, W, T, Y, R = dims
+    pad = Y // 2
+    gen = torch.Generator(device="cuda").manual_seed(sum(dims))
+    mk = lambda *s: torch.randn(*s, device="cuda", generator=gen)
+    x, dy = mk(N, C, H, W), mk(N, T, H, W)
+    K = [mk(C, R), mk(Y, Y, R), mk(R, T)]
+    s = cp4.cp3_shape_for(x.shape, *K, pad)
+    import ctypes
+    nbytes = cp4.lib().cp3_conv2d_forward_workspace_bytes(ctypes.byref(s))
+    ws = [torch.empty(nbytes, device="cuda", dtype=torch.uint8) for _ in range(2)]
+    y, dx = torch.empty(N, T, H, W, device="cuda"), torch.empty(N, C, H, W, device="cuda")
+
+    def step():
+        cp4.cp3_conv2d_forward(x, *K, pad=pad, out=y, workspace=ws[0])
+        cp4.cp3_conv2d_backward_data(dy, *K, pad=pad, out=dx, workspace=ws[1])
+
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    torch.cuda.synchronize()
+    for replay in range(3):
+        x.copy_(mk(N, C, H, W))
+        dy.copy_(mk(N, T, H, W))
+        for k in K:
+            k.copy_(mk(*k.shape))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [y.clone(), dx.clone()]
+        y.zero_(), dx.zero_()
+        step()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("y", "dx"), got, (y, dx)):
+            assert (a - b).abs().max().item() <= 1e-6 * b.abs().max().item(), (replay, name)
