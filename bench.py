@@ -62,7 +62,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
-                 "(batch sharding across GPUs is design-only, see DESIGN.md)")
+                 "(the passes shard over the batch with one small all-reduce of the factor "
+                 "gradients; that is designed, not built)")
 
     import torch
 
