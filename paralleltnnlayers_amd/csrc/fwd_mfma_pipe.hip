@@ -830,6 +830,10 @@ bool plan(const FwdArgs& a, PipePlan* best) {
 bool plan(const FwdArgs& a, PipePlan* best) {
   double best_cost = 0;
   bool found = false;
+#ifdef CP4_PIPE_TUNE_TH
+  // measurement builds only: strip height from the environment
+  if (const char* th = getenv("CP4_PIPE_TH")) return layout(a, atoi(th), best);
+#endif
   for (int TH = 1; TH <= a.H; ++TH) {
     PipePlan pl;
     if (!layout(a, TH, &pl)) break;
