@@ -170,3 +170,27 @@ class CP3Conv2dFunction(torch.autograd.Function):
 def cp3_conv2d(x, K0, K1, K2, pad):
     """Functional form of the differentiable 3-factor CP convolution (NCHW)."""
     return CP3Conv2dFunction.apply(x, K0, K1, K2, pad)
+
+
+class CP3Conv2d(torch.nn.Module):
+    """A rank-R 3-factor CP convolution layer, "same" padding: pointwise K0 [C,R],
+    depthwise K1 [k,k,R], pointwise K2 [R,T] (the kernels of the reference's Python
+    layer, test/layers.py:285-294, in the fused op's layouts).  Factors start as
+    normal(0, s) with s chosen so that the equivalent dense filter
+    sum_r K0[c,r] K1[i,j,r] K2[r,t] has the variance of a Kaiming-normal one."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, rank, device="cuda"):
+        super().__init__()
+        if kernel_size % 2 != 1:
+            raise ValueError("kernel_size must be odd (same padding)")
+        self.pad = kernel_size // 2
+        fan_in = in_channels * kernel_size * kernel_size
+        # Var = R * s^6 for three independent N(0, s^2) factors; target 2 / fan_in
+        s = (2.0 / (fan_in * rank)) ** (1.0 / 6.0)
+        mk = lambda *d: torch.nn.Parameter(torch.randn(*d, device=device) * s)
+        self.K0 = mk(in_channels, rank)
+        self.K1 = mk(kernel_size, kernel_size, rank)
+        self.K2 = mk(rank, out_channels)
+
+    def forward(self, x):
+        return cp3_conv2d(x, self.K0, self.K1, self.K2, self.pad)

@@ -145,3 +145,24 @@ def test_cp3_rejects_small_workspace(cp4):
     rc = cp4.lib().cp3_conv2d_forward(ctypes.byref(s), p(x), p(K0), p(K1), p(K2), p(y), p(ws), 16,
                                       None)
     assert rc == 4      # CP4_ERR_WORKSPACE
+
+
+def test_cp3_layer_trains(cp4):
+    """A few SGD steps on the layer reduce a regression loss: forward, input gradient and
+    folded factor gradients fit together."""
+    from paralleltnnlayers_amd.torch_ops import CP3Conv2d
+    torch.manual_seed(0)
+    layer = CP3Conv2d(32, 48, 3, rank=12)
+    teacher = CP3Conv2d(32, 48, 3, rank=12)
+    x = torch.randn(4, 32, 16, 16, device="cuda")
+    with torch.no_grad():
+        target = teacher(x)
+    opt = torch.optim.SGD(layer.parameters(), lr=0.05)
+    losses = []
+    for _ in range(30):
+        opt.zero_grad()
+        loss = ((layer(x) - target) ** 2).mean()
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+    assert losses[-1] < 0.7 * losses[0], losses[::6]
