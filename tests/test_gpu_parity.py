@@ -251,6 +251,42 @@ def test_split_role_schedule_at_scale(cp4, oracle):
         assert_activation_close(host(cp4.conv2d_forward(xd, *f, pad=pad)), want, "forward")
 
 
+@pytest.mark.parametrize("dims", [(2, 64, 28, 28, 64, 3, 16), (2, 256, 28, 28, 256, 3, 32),
+                                  (2, 128, 14, 14, 128, 5, 16), (3, 5, 9, 9, 7, 3, 3),
+                                  (2, 48, 13, 13, 48, 3, 40)],
+                         ids=lambda d: "x".join(map(str, d)))
+def test_pointers_aligned_to_four_bytes_only(cp4, dims):
+    """The C ABI takes any float pointer: operands that start 4 bytes into an allocation
+    (no 8- or 16-byte alignment) give the results of the aligned call - bit-identical for
+    forward and backward-data, within fp32 summation order for the factor gradients."""
+    N, C, H, W, T, Y, R = dims
+    pad = Y // 2
+    gen = torch.Generator(device="cuda").manual_seed(sum(dims))
+    mk = lambda *s: torch.randn(*s, device="cuda", generator=gen)
+
+    def shifted(t):
+        buf = torch.empty(t.numel() + 1, device="cuda")
+        view = buf[1:].view(t.shape)
+        view.copy_(t)
+        assert view.data_ptr() % 8 == 4
+        return view
+
+    x, dy = mk(N, C, H, W), mk(N, T, H, W)
+    fac = [mk(d, R) for d in (T, C, Y, Y)]
+    y = cp4.conv2d_forward(x, *fac, pad=pad)
+    dx = cp4.conv2d_backward_data(dy, *fac, pad=pad)
+    grads = cp4.conv2d_backward_filter(x, dy, *fac, pad=pad)
+    xs, dys, facs = shifted(x), shifted(dy), [shifted(f) for f in fac]
+    ys = cp4.conv2d_forward(xs, *facs, pad=pad, out=shifted(torch.zeros_like(y)))
+    dxs = cp4.conv2d_backward_data(dys, *facs, pad=pad, out=shifted(torch.zeros_like(dx)))
+    gs = cp4.conv2d_backward_filter(xs, dys, *facs, pad=pad)
+    torch.cuda.synchronize()
+    assert torch.equal(ys, y) or (ys - y).abs().max() <= 1e-6 * y.abs().max()
+    assert torch.equal(dxs, dx) or (dxs - dx).abs().max() <= 1e-6 * dx.abs().max()
+    for a, b in zip(gs, grads):
+        assert (a - b).abs().max() <= 2e-6 * b.abs().max()
+
+
 def test_reference_single_case_against_dense_conv(cp4):
     """Cuda_kernels/test/test_cp4Conv.cpp.cu:14-44: CP4 forward vs a dense conv
     of the recomposed kernel, all-positive U(0,1] inputs, compared with the
