@@ -102,6 +102,7 @@ struct PipePlan {
   size_t lds_bytes;
   int Wt, lgWt, cols;       // tiled build: tile width, its log2, column tiles per row strip
   unsigned wl_magic;        // tiled build: 2^32 / (Wt + FS - 1) + 1, for the division by the row length
+  int split2;               // consumer waves split roles also above 16 ranks / 4 channel blocks
 #ifdef CP4_DEBUG_PHASES
   long long* dbg;
 #endif
@@ -398,13 +399,13 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // Output-factor fragment of this wave's 32-channel block kb = wc (reloaded per
     // item only when there are more blocks than consumer waves): lane holds row
     // 32*kb + l32, ranks 16*c + 8*hi + e.
-    u32x4 fkh[2], fkm[2], fkl[2];
+    // (slot 1: second block of a contraction wave in the wide split-role schedule)
+    u32x4 fkh[2][2], fkm[2][2], fkl[2][2];
 #ifdef CP4_PIPE_EPILOGUE
     float bs[16];                                  // bias of accumulator row v
     const bool relu = a.act != 0;
 #endif
-    auto load_fk = [&](int kb) {
-      const int k = 32 * kb + l32;
+    [[maybe_unused]] auto load_bias = [&](int kb) {
 #ifdef CP4_PIPE_EPILOGUE
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
@@ -412,6 +413,10 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         bs[v] = (a.bias && kk < Cout) ? a.bias[kk] : 0.f;
       }
 #endif
+    };
+    auto load_fk = [&](int kb, auto slot_c) {
+      constexpr int slot = decltype(slot_c)::value;
+      const int k = 32 * kb + l32;
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         float v[8];
@@ -420,21 +425,41 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           const int r = 16 * c + 8 * hi + e;
           v[e] = (k < Cout && r < R) ? a.Fout[(size_t)k * ldf + r] : 0.f;
         }
-        split8(v, fkh[c], fkm[c], fkl[c]);
+        split8(v, fkh[slot][c], fkm[slot][c], fkl[slot][c]);
       }
     };
+    constexpr std::integral_constant<int, 0> slot0{};
+    constexpr std::integral_constant<int, 1> slot1{};
     const bool fk_cached = nkb <= kCons;
-    if (fk_cached && wc < nkb) load_fk(wc);
     // With at most 16 ranks and at most 4 channel blocks only four waves have
     // ranks in the tap step and only four have a block to contract: the roles
     // are then split - waves 4-7 run the taps (rank quad wc - 4), waves 0-3 the
     // contractions - so that the tap step of one group overlaps the contraction
     // of the previous one, and the contraction skips the empty upper rank chunk.
-    const bool split_roles = FS <= 5 && R <= 16 && nkb <= 4;   // (7x7: no registers to spare)
-    const int wq = split_roles ? (wc >= 4 ? wc - 4 : 0) : wc;     // rank quad in the tap step
+    // Above that, up to 8 channel blocks (wide split): a tap wave takes two rank
+    // quads (wq and wq + 4), a contraction wave two channel blocks (wc and
+    // wc + 4, both output-factor fragments in registers).
+    const bool split_narrow = FS <= 5 && R <= 16 && nkb <= 4;  // (7x7: no registers to spare)
+#if defined(CP4_PIPE_TAPS2D) || defined(CP4_PIPE_EPILOGUE)
+    // (twice the 2-D weights would not fit; nor would the bias rows next to two
+    // output-factor fragments)
+    const bool split_wide = false;
+#else
+    // It pays with six or more channel blocks, or once the groups of a strip form a
+    // pipeline (a single group gains nothing from overlapping with its neighbours).
+    const bool split_wide = !split_narrow && pl.split2 && FS <= 3 && nkb <= 8 &&   // (5x5: registers)
+                            (nkb >= 6 || ngroups >= 3);
+#endif
+    const bool split_roles = split_narrow || split_wide;
+    const int wq = split_roles ? (wc >= 4 ? wc - 4 : 0) : wc;     // (first) rank quad in the tap step
+    if (!split_wide && fk_cached && wc < nkb) {
+      load_fk(wc, slot0);
+      load_bias(wc);
+    }
     // Tap weights of this wave's 4 ranks (wave-uniform values).
 #ifdef CP4_PIPE_TAPS2D
-    float w2[4][FS][FS];
+    constexpr int NTQ = 1;
+    float w2[NTQ][4][FS][FS];
 #pragma unroll
     for (int rr = 0; rr < 4; ++rr)
 #pragma unroll
@@ -442,18 +467,27 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #pragma unroll
         for (int j = 0; j < FS; ++j) {
           const int ty = a.flip ? FS - 1 - ti : ti, tx = a.flip ? FS - 1 - j : j, r = 4 * wq + rr;
-          w2[rr][ti][j] = r < R ? a.taps2d[(ty * FS + tx) * ldf + r] : 0.f;
+          w2[0][rr][ti][j] = r < R ? a.taps2d[(ty * FS + tx) * ldf + r] : 0.f;
         }
 #else
-    float fh[4][FS], fw[4][FS];
+#ifdef CP4_PIPE_EPILOGUE
+    constexpr int NTQ = 1;
+#else
+    constexpr int NTQ = FS <= 3 ? 2 : 1;           // quads a tap wave may take (wide split)
+#endif
+    float fh[NTQ][4][FS], fw[NTQ][4][FS];
+    auto load_taps = [&](auto qi_c) {
+      constexpr int qi = decltype(qi_c)::value;
 #pragma unroll
-    for (int rr = 0; rr < 4; ++rr)
+      for (int rr = 0; rr < 4; ++rr)
 #pragma unroll
-      for (int j = 0; j < FS; ++j) {
-        const int tap = a.flip ? FS - 1 - j : j, r = 4 * wq + rr;
-        fh[rr][j] = r < R ? a.FH[tap * ldf + r] : 0.f;
-        fw[rr][j] = r < R ? a.FW[tap * ldf + r] : 0.f;
-      }
+        for (int j = 0; j < FS; ++j) {
+          const int tap = a.flip ? FS - 1 - j : j, r = 4 * (wq + 4 * qi) + rr;
+          fh[qi][rr][j] = r < R ? a.FH[tap * ldf + r] : 0.f;
+          fw[qi][rr][j] = r < R ? a.FW[tap * ldf + r] : 0.f;
+        }
+    };
+    load_taps(std::integral_constant<int, 0>{});
 #endif
 #ifdef CP4_PIPE_TILED
     io_t* yn = reinterpret_cast<io_t*>(a.y) + (size_t)n * Cout * HW + (size_t)h0 * W + w0;
@@ -501,7 +535,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         ++frontier;
       return frontier > need;
     };
-    auto taps = [&](int i, unsigned char* cb) {
+    auto taps = [&](int i, unsigned char* cb, auto ntq_c) {
       const int g = rev ? ngroups - 1 - i : i;
       {
         const int need = need_of(i);
@@ -539,7 +573,10 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #endif
       // the LDS reads of RBT ranks go out together, then their arithmetic
       constexpr int RBT = FS <= 3 ? 4 : (FS == 5 ? 2 : 1);
-      const float* ab = As + (size_t)(4 * wq) * QA + h * RL;
+#pragma unroll
+      for (int qi = 0; qi < decltype(ntq_c)::value; ++qi) {
+      const int q = wq + 4 * qi;                   // this pass's rank quad
+      const float* ab = As + (size_t)(4 * q) * QA + h * RL;
       float o[4];
 #pragma unroll
       for (int r0 = 0; r0 < 4; r0 += RBT) {
@@ -557,12 +594,12 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           for (int ti = 0; ti < FS; ++ti) {
 #ifdef CP4_PIPE_TAPS2D
 #pragma unroll
-            for (int j = 0; j < FS; ++j) s += (in[j] ? w2[r0 + rr][ti][j] : 0.f) * av[rr][ti][j];
+            for (int j = 0; j < FS; ++j) s += (in[j] ? w2[qi][r0 + rr][ti][j] : 0.f) * av[rr][ti][j];
 #else
             float hs = 0.f;
 #pragma unroll
-            for (int j = 0; j < FS; ++j) hs += (in[j] ? fw[r0 + rr][j] : 0.f) * av[rr][ti][j];
-            s += fh[r0 + rr][ti] * hs;
+            for (int j = 0; j < FS; ++j) hs += (in[j] ? fw[qi][r0 + rr][j] : 0.f) * av[rr][ti][j];
+            s += fh[qi][r0 + rr][ti] * hs;
 #endif
           }
           o[r0 + rr] = s;
@@ -581,11 +618,12 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       }
       // plane ((part*2 + chunk)*2 + hi)*2 + parity, 512 B each; entry lane >> 1;
       // this quad is the low or high 8 bytes of the 16-byte entry
-      unsigned char* dst = cb + ((((wq >> 2) * 2 + ((wq >> 1) & 1)) * 2 + (lane & 1)) * 512) +
-                           (lane >> 1) * 16 + (wq & 1) * 8;
+      unsigned char* dst = cb + ((((q >> 2) * 2 + ((q >> 1) & 1)) * 2 + (lane & 1)) * 512) +
+                           (lane >> 1) * 16 + (q & 1) * 8;
       *reinterpret_cast<u32x2*>(dst) = ph;
       *reinterpret_cast<u32x2*>(dst + 8 * 512) = pm;
       *reinterpret_cast<u32x2*>(dst + 16 * 512) = pl2;
+      }
       STAMPX(3 + 4 * i)
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       if (lane == 0)
@@ -595,19 +633,38 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // Contraction ranks -> the 32 output channels of block kb for pixel group g
     // from fragment tile cb (nch rank chunks of 16), epilogue, stores.
     auto contract_block = [&](const unsigned char* cb, int g, int kb, auto nch, bool signal,
-                              int step) {
+                              int step, auto slot_c, auto seq_c) {
+      constexpr int slot = decltype(slot_c)::value;
       f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
 #pragma unroll
       for (int c = 0; c < decltype(nch)::value; ++c) {
         const unsigned char* bp = cb + ((c * 2 + hi) * 2) * 512 + l32 * 16;
-        const u32x4 b0h = *reinterpret_cast<const u32x4*>(bp);
-        const u32x4 b1h = *reinterpret_cast<const u32x4*>(bp + 512);
-        const u32x4 b0m = *reinterpret_cast<const u32x4*>(bp + 8 * 512);
-        const u32x4 b1m = *reinterpret_cast<const u32x4*>(bp + 9 * 512);
-        const u32x4 b0l = *reinterpret_cast<const u32x4*>(bp + 16 * 512);
-        const u32x4 b1l = *reinterpret_cast<const u32x4*>(bp + 17 * 512);
-        acc0 = mfma_split(fkh[c], fkm[c], fkl[c], b0h, b0m, b0l, acc0);
-        acc1 = mfma_split(fkh[c], fkm[c], fkl[c], b1h, b1m, b1l, acc1);
+        if constexpr (decltype(seq_c)::value) {
+          // wide split (two output-factor fragments in registers): one pixel
+          // parity's fragments live at a time
+          {
+            const u32x4 b0h = *reinterpret_cast<const u32x4*>(bp);
+            const u32x4 b0m = *reinterpret_cast<const u32x4*>(bp + 8 * 512);
+            const u32x4 b0l = *reinterpret_cast<const u32x4*>(bp + 16 * 512);
+            acc0 = mfma_split(fkh[slot][c], fkm[slot][c], fkl[slot][c], b0h, b0m, b0l, acc0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          {
+            const u32x4 b1h = *reinterpret_cast<const u32x4*>(bp + 512);
+            const u32x4 b1m = *reinterpret_cast<const u32x4*>(bp + 9 * 512);
+            const u32x4 b1l = *reinterpret_cast<const u32x4*>(bp + 17 * 512);
+            acc1 = mfma_split(fkh[slot][c], fkm[slot][c], fkl[slot][c], b1h, b1m, b1l, acc1);
+          }
+        } else {
+          const u32x4 b0h = *reinterpret_cast<const u32x4*>(bp);
+          const u32x4 b1h = *reinterpret_cast<const u32x4*>(bp + 512);
+          const u32x4 b0m = *reinterpret_cast<const u32x4*>(bp + 8 * 512);
+          const u32x4 b1m = *reinterpret_cast<const u32x4*>(bp + 9 * 512);
+          const u32x4 b0l = *reinterpret_cast<const u32x4*>(bp + 16 * 512);
+          const u32x4 b1l = *reinterpret_cast<const u32x4*>(bp + 17 * 512);
+          acc0 = mfma_split(fkh[slot][c], fkm[slot][c], fkl[slot][c], b0h, b0m, b0l, acc0);
+          acc1 = mfma_split(fkh[slot][c], fkm[slot][c], fkl[slot][c], b1h, b1m, b1l, acc1);
+        }
         __builtin_amdgcn_sched_barrier(0);     // one chunk's fragments live at a time
       }
       if (signal) {
@@ -703,6 +760,56 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       }
     };
 
+    constexpr std::integral_constant<int, 1> one{};
+    constexpr std::integral_constant<int, 2> two{};
+    [[maybe_unused]] constexpr std::integral_constant<bool, true> yes{};
+    constexpr std::integral_constant<bool, false> no{};
+    if (split_wide) {
+      // As the narrow split below, with two rank quads per tap wave and up to two
+      // channel blocks per contraction wave; the tile is free again once every
+      // contraction wave has read it for its last block.
+      const int ncw = nkb < 4 ? nkb : 4;           // contraction waves with a block
+      if (wc >= 4) {
+        if constexpr (NTQ == 2) {
+          // (up to 16 ranks: the second rank chunk is never read, one quad each)
+          if (R > 16) load_taps(std::integral_constant<int, 1>{});
+          for (int i = 0; i < ngroups; ++i) {
+            if (i >= 3) wait_ge(&cdone[(i - 3) & 3], ncw * (((i - 3) >> 2) + 1));
+            if (R > 16)
+              taps(i, Cb + (i % 3) * kCcBuf, two);
+            else
+              taps(i, Cb + (i % 3) * kCcBuf, one);
+          }
+        }
+      } else if (wc < nkb) {
+        const bool second = wc + 4 < nkb;
+        load_fk(wc, slot0);
+        if (second) load_fk(wc + 4, slot1);
+        if (!second) load_bias(wc);
+        for (int i = 0; i < ngroups; ++i) {
+          const int g = rev ? ngroups - 1 - i : i;
+          const unsigned char* cb = Cb + (i % 3) * kCcBuf;
+          wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1));
+          STAMPX(4 + 4 * i)
+          if (second) load_bias(wc);
+          if (R <= 16) {
+            contract_block(cb, g, wc, one, !second, i, slot0, yes);
+          } else {
+            contract_block(cb, g, wc, two, !second, i, slot0, yes);
+          }
+          if (second) {
+            load_bias(wc + 4);
+            if (R <= 16) {
+              contract_block(cb, g, wc + 4, one, true, i, slot1, yes);
+            } else {
+              contract_block(cb, g, wc + 4, two, true, i, slot1, yes);
+            }
+          }
+          STAMP(5 + 4 * i)
+        }
+      }
+      return;
+    }
     if (split_roles) {
       // The tile of step i is i % 3; the tap waves write it after every
       // contraction wave has read it for step i - 3.  cdone[s] counts one per
@@ -712,13 +819,13 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       if (wc >= 4) {
         for (int i = 0; i < ngroups; ++i) {
           if (i >= 3) wait_ge(&cdone[(i - 3) & 3], nkb * (((i - 3) >> 2) + 1));
-          taps(i, Cb + (i % 3) * kCcBuf);
+          taps(i, Cb + (i % 3) * kCcBuf, one);
         }
       } else if (wc < nkb) {
         for (int i = 0; i < ngroups; ++i) {
           const int g = rev ? ngroups - 1 - i : i;
           wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1));
-          contract_block(Cb + (i % 3) * kCcBuf, g, wc, std::integral_constant<int, 1>{}, true, i);
+          contract_block(Cb + (i % 3) * kCcBuf, g, wc, one, true, i, slot0, no);
         }
       }
       return;
@@ -731,7 +838,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     unsigned char* cb_cur = Cb;
     unsigned char* cb_next = Cb + kCcBuf;
     unsigned char* cb_free = Cb + 2 * kCcBuf;
-    taps(0, cb_cur);
+    taps(0, cb_cur, one);
     for (int i = 0; i < ngroups; ++i) {
       const int g = rev ? ngroups - 1 - i : i;
       wait_ge(&arrivals[i & 3], kCons * ((i >> 2) + 1));
@@ -739,15 +846,18 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       // tap step i+1 goes first when its blocks are there (keeps the stores of
       // consecutive groups close), else after this group's contraction
       const bool early = i + 1 < ngroups && ready(i + 1);
-      if (early) taps(i + 1, cb_next);
+      if (early) taps(i + 1, cb_next, one);
       // ---- rank -> output-channel contraction for this wave's blocks --------
       const unsigned char* cb = cb_cur;
       for (int kb = wc; kb < nkb; kb += kCons) {
-        if (!fk_cached) load_fk(kb);
-        contract_block(cb, g, kb, std::integral_constant<int, 2>{}, false, i);
+        if (!fk_cached) {
+          load_fk(kb, slot0);
+          load_bias(kb);
+        }
+        contract_block(cb, g, kb, two, false, i, slot0, no);
       }
       STAMP(5 + 4 * i)
-      if (i + 1 < ngroups && !early) taps(i + 1, cb_next);
+      if (i + 1 < ngroups && !early) taps(i + 1, cb_next, one);
       unsigned char* tmp = cb_cur;
       cb_cur = cb_next;
       cb_next = cb_free;
@@ -839,7 +949,8 @@ bool plan(const FwdArgs& a, PipePlan* best) {
     if (!layout(a, TH, &pl)) break;
     const double rounds = (pl.nWG + 255) / 256;
     const double cost = rounds * ((double)(TH + a.Y - 1) * a.Cin + (double)TH * a.Cout);
-    if (!found || cost < best_cost) {
+    // on equal cost (1x1 filters: no halo rows) the taller strip: fewer workgroups
+    if (!found || cost <= best_cost) {
       best_cost = cost;
       *best = pl;
       found = true;
@@ -922,6 +1033,10 @@ bool fwd_pipe_supported(const FwdArgs& a) {
 hipError_t fwd_pipe_launch(const FwdArgs& a, hipStream_t st) {
   PipePlan pl;
   if (!plan(a, &pl)) return hipErrorInvalidValue;
+  pl.split2 = 1;
+#ifdef CP4_PIPE_TUNE_TH
+  if (const char* e = getenv("CP4_PIPE_SPLIT2")) pl.split2 = atoi(e);
+#endif
 #ifdef CP4_DEBUG_PHASES
   pl.dbg = getenv("CP4_DBG_PTR") ? reinterpret_cast<long long*>(strtoull(getenv("CP4_DBG_PTR"), nullptr, 10)) : nullptr;
 #endif

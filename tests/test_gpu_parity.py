@@ -201,6 +201,13 @@ EDGE = [
     (3, 16, 30, 34, 2, 96, 5, 5, 9),      # 5x5, several groups per strip
     (2, 64, 6, 288, 1, 128, 3, 3, 16),    # long rows: five groups per strip, fragment tiles reused
     (1, 32, 3, 576, 0, 64, 1, 1, 8),      # ten groups per strip
+    # more than 16 ranks or more than 4 channel blocks, 1x1 / 3x3: wide role split (a
+    # tap wave takes two rank quads, a contraction wave two channel blocks)
+    (2, 64, 6, 288, 1, 160, 3, 3, 20),    # five blocks (one wave with two), ranks end inside quad 5
+    (1, 128, 4, 320, 1, 256, 3, 3, 32),   # eight blocks, 32 ranks, five groups per strip
+    (2, 32, 5, 200, 0, 200, 1, 1, 12),    # 1x1, seven blocks (the last partly filled), one rank chunk
+    (1, 64, 13, 13, 1, 224, 3, 3, 24),    # odd plane: per-pixel stores, one group per strip
+    (1, 320, 3, 210, 1, 72, 3, 3, 28),    # factor fragments in LDS, three blocks, four groups
     # wide planes: tiles of TH rows x Wt columns (producer/consumer kernel, tiled build)
     (1, 16, 9, 200, 1, 32, 3, 3, 8),      # four column tiles, the last one 8 columns wide
     (2, 24, 5, 131, 2, 16, 5, 5, 12),     # odd width across three tiles, 5x5
@@ -249,6 +256,26 @@ def test_split_role_schedule_at_scale(cp4, oracle):
     xd = dev(x)
     for _ in range(3):      # a race would not show on every launch
         assert_activation_close(host(cp4.conv2d_forward(xd, *f, pad=pad)), want, "forward")
+
+
+def test_wide_role_split_at_scale(cp4, oracle):
+    """More workgroups than compute units, seven groups per strip, 32 ranks and 8
+    channel blocks (the ResNet-stage shape at a small batch), forward and
+    backward-data: the tap waves run up to three groups ahead of the contraction
+    waves and the fragment tiles are reused."""
+    N, C, H, W, pad, T, Y, R = 5, 256, 56, 56, 1, 256, 3, 32
+    rng = np.random.default_rng(7)
+    x = np.maximum(rng.standard_normal((N, C, H, W)), 0).astype(np.float32)
+    dy = rng.standard_normal((N, T, H, W)).astype(np.float32)
+    fac = [(rng.standard_normal((d, R)) / np.sqrt(R)).astype(np.float32) for d in (T, C, Y, Y)]
+    f = [dev(v) for v in fac]
+    want = oracle.forward(x, *fac, pad)
+    want_dx = oracle.backward_data(dy, *fac, pad)
+    xd, dyd = dev(x), dev(dy)
+    for _ in range(3):      # a race would not show on every launch
+        assert_activation_close(host(cp4.conv2d_forward(xd, *f, pad=pad)), want, "forward")
+        assert_activation_close(host(cp4.conv2d_backward_data(dyd, *f, pad=pad)), want_dx,
+                                "backward-data")
 
 
 @pytest.mark.parametrize("dims", [(2, 64, 28, 28, 64, 3, 16), (2, 256, 28, 28, 256, 3, 32),
