@@ -92,6 +92,9 @@ constexpr int kCcBuf = 24 * 512;             // bytes of one Cc fragment tile (6
 constexpr size_t kLdsLimit = 160 * 1024;
 constexpr int kSpinLimit = 1 << 22;
 constexpr int kMaxBlk = 64;                  // per-block progress words in LDS
+#ifndef CP4_PIPE_SLEEP
+#define CP4_PIPE_SLEEP 1
+#endif
 
 struct PipePlan {
   int TH, strips, nWG;
@@ -116,7 +119,7 @@ __device__ __forceinline__ int wait_ge(int* word, int want) {
   for (int it = 0; it < kSpinLimit; ++it) {
     v = __hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
     if (v >= want) break;
-    __builtin_amdgcn_s_sleep(1);
+    __builtin_amdgcn_s_sleep(CP4_PIPE_SLEEP);
   }
   return v;
 }
@@ -224,6 +227,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   if (wave < kProd) {
     // =========================== producers ==================================
     const int bsel = wave % NB, cq = wave / NB;    // block within the round, channel split
+#ifdef CP4_PIPE_PPRIO
+    __builtin_amdgcn_s_setprio(CP4_PIPE_PPRIO);
+#endif
     const int nrounds = (nblk + NB - 1) / NB;
     // lane's channel 16*(cpq*cq + chunk) + 8*hi + e
     // (PAD: Cin is not a multiple of 64; channel groups past Cin count as zero)
