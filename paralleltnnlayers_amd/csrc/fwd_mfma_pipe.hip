@@ -90,11 +90,8 @@ constexpr int kProd = 8, kCons = 8;          // producer / consumer waves (4 per
 constexpr int kRP = 32;
 constexpr int kCcBuf = 24 * 512;             // bytes of one Cc fragment tile (64 pixels)
 constexpr size_t kLdsLimit = 160 * 1024;
-constexpr int kSpinLimit = 1 << 22;
+constexpr int kSpinLimit = 1 << 19;      // about a quarter of a second at the longest nap
 constexpr int kMaxBlk = 64;                  // per-block progress words in LDS
-#ifndef CP4_PIPE_SLEEP
-#define CP4_PIPE_SLEEP 1
-#endif
 
 struct PipePlan {
   int TH, strips, nWG;
@@ -119,7 +116,11 @@ __device__ __forceinline__ int wait_ge(int* word, int want) {
   for (int it = 0; it < kSpinLimit; ++it) {
     v = __hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
     if (v >= want) break;
-    __builtin_amdgcn_s_sleep(CP4_PIPE_SLEEP);
+    // short naps at first (a wait that is about to end costs little latency),
+    // longer ones after that (fewer polls between the producers' LDS traffic)
+    if (it < 6) __builtin_amdgcn_s_sleep(1);
+    else if (it < 12) __builtin_amdgcn_s_sleep(4);
+    else __builtin_amdgcn_s_sleep(16);
   }
   return v;
 }
@@ -227,9 +228,6 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   if (wave < kProd) {
     // =========================== producers ==================================
     const int bsel = wave % NB, cq = wave / NB;    // block within the round, channel split
-#ifdef CP4_PIPE_PPRIO
-    __builtin_amdgcn_s_setprio(CP4_PIPE_PPRIO);
-#endif
     const int nrounds = (nblk + NB - 1) / NB;
     // lane's channel 16*(cpq*cq + chunk) + 8*hi + e
     // (PAD: Cin is not a multiple of 64; channel groups past Cin count as zero)
@@ -435,7 +433,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       }
     };
     constexpr std::integral_constant<int, 0> slot0{};
-    constexpr std::integral_constant<int, 1> slot1{};
+    [[maybe_unused]] constexpr std::integral_constant<int, 1> slot1{};
     const bool fk_cached = nkb <= kCons;
     // With at most 16 ranks and at most 4 channel blocks only four waves have
     // ranks in the tap step and only four have a block to contract: the roles
@@ -770,6 +768,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     constexpr std::integral_constant<int, 2> two{};
     [[maybe_unused]] constexpr std::integral_constant<bool, true> yes{};
     constexpr std::integral_constant<bool, false> no{};
+#ifndef CP4_PIPE_TAPS2D
     if (split_wide) {
       // As the narrow split below, with two rank quads per tap wave and up to two
       // channel blocks per contraction wave; the tile is free again once every
@@ -816,6 +815,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       }
       return;
     }
+#endif
     if (split_roles) {
       // The tile of step i is i % 3; the tap waves write it after every
       // contraction wave has read it for step i - 3.  cdone[s] counts one per
