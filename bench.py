@@ -39,7 +39,7 @@ FACTORS = ("FK", "FC", "FH", "FW")
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs, scaled by the plain copy kernel's reading (see
 # profiles/): {workload: bytes}.  None until measured for the current kernel.
-MEASURED_TRAFFIC = {"C3": 212.7e6}   # fwd_pipe_kernel<3,4,2,false,4>: 109.7 MB fetched + 103.0 MB written
+MEASURED_TRAFFIC = {"C3": 213.5e6}   # fwd_pipe_kernel<3,4,2,false,4>: 110.5 MB fetched + 103.1 MB written
 
 
 def main():
