@@ -451,8 +451,10 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #else
     // It pays with six or more channel blocks, or once the groups of a strip form a
     // pipeline (a single group gains nothing from overlapping with its neighbours).
+    // Not for the accumulating rank pass: its stores read y first, and a
+    // contraction wave would wait for that twice per group, one block after the other.
     const bool split_wide = !split_narrow && pl.split2 && FS <= 3 && nkb <= 8 &&   // (5x5: registers)
-                            (nkb >= 6 || ngroups >= 3);
+                            (nkb >= 6 || ngroups >= 3) && !a.accumulate;
 #endif
     const bool split_roles = split_narrow || split_wide;
     const int wq = split_roles ? (wc >= 4 ? wc - 4 : 0) : wc;     // (first) rank quad in the tap step
