@@ -936,7 +936,8 @@ bool plan(const FwdArgs& a, PipePlan* best) {
       // last column counted whole
       const double cost = rounds * ((double)(TH + a.Y - 1) * (pl.Wt + a.Y - 1) * a.Cin +
                                     (double)TH * pl.Wt * a.Cout);
-      if (!found || cost < best_cost) {
+      // on equal cost (1x1 filters: no halo) the larger tile: fewer workgroups
+      if (!found || cost <= best_cost) {
         best_cost = cost;
         *best = pl;
         found = true;
