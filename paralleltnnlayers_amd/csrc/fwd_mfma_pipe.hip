@@ -110,15 +110,15 @@ struct PipePlan {
 
 // Wait until *word >= want and return the value seen.  The writer is another
 // wave of this workgroup; the spin is bounded so that a logic error cannot hang
-// the device.
-__device__ __forceinline__ int wait_ge(int* word, int want) {
+// the device.  With `backoff` the naps between polls grow (64, 256, then 1024
+// cycles): fewer polls between the producers' LDS traffic on long strips; on
+// the shortest strips the wake-up latency of a long nap would cost more.
+__device__ __forceinline__ int wait_ge(int* word, int want, bool backoff) {
   int v = 0;
   for (int it = 0; it < kSpinLimit; ++it) {
     v = __hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
     if (v >= want) break;
-    // short naps at first (a wait that is about to end costs little latency),
-    // longer ones after that (fewer polls between the producers' LDS traffic)
-    if (it < 6) __builtin_amdgcn_s_sleep(1);
+    if (!backoff || it < 6) __builtin_amdgcn_s_sleep(1);
     else if (it < 12) __builtin_amdgcn_s_sleep(4);
     else __builtin_amdgcn_s_sleep(16);
   }
@@ -200,6 +200,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   const int QLEN = (pl.TH + FS - 1) * W;
 #endif
   const int nblk = (QLEN + 31) >> 5;             // 32-pixel producer blocks
+  const bool backoff = nblk >= 4;                // growing naps in the spin waits
 
   // ---- prologue: clear the progress words; above 256 input channels the input
   // factor does not fit the producers' registers and goes to LDS, pre-split ----
@@ -367,7 +368,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           for (int v = 0; v < 16; ++v)
             dst[(8 * (v >> 2) + (v & 3)) * QA] = valid ? acc[v] : 0.f;
         } else {
-          wait_ge(bf, cq);
+          wait_ge(bf, cq, backoff);
           // read all, then add, then write all: one LDS round trip per half, not
           // one per element
 #pragma unroll
@@ -546,7 +547,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       {
         const int need = need_of(i);
         while (frontier <= need) {
-          wait_ge(&flags[frontier], NQ);
+          wait_ge(&flags[frontier], NQ, backoff);
           ++frontier;
         }
       }
@@ -781,7 +782,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           // (up to 16 ranks: the second rank chunk is never read, one quad each)
           if (R > 16) load_taps(std::integral_constant<int, 1>{});
           for (int i = 0; i < ngroups; ++i) {
-            if (i >= 3) wait_ge(&cdone[(i - 3) & 3], ncw * (((i - 3) >> 2) + 1));
+            if (i >= 3) wait_ge(&cdone[(i - 3) & 3], ncw * (((i - 3) >> 2) + 1), backoff);
             if (R > 16)
               taps(i, Cb + (i % 3) * kCcBuf, two);
             else
@@ -796,7 +797,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         for (int i = 0; i < ngroups; ++i) {
           const int g = rev ? ngroups - 1 - i : i;
           const unsigned char* cb = Cb + (i % 3) * kCcBuf;
-          wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1));
+          wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1), backoff);
           STAMPX(4 + 4 * i)
           if (second) load_bias(wc);
           if (R <= 16) {
@@ -826,13 +827,13 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       // missing one); like the arrivals, a slot cannot run a whole cycle ahead.
       if (wc >= 4) {
         for (int i = 0; i < ngroups; ++i) {
-          if (i >= 3) wait_ge(&cdone[(i - 3) & 3], nkb * (((i - 3) >> 2) + 1));
+          if (i >= 3) wait_ge(&cdone[(i - 3) & 3], nkb * (((i - 3) >> 2) + 1), backoff);
           taps(i, Cb + (i % 3) * kCcBuf, one);
         }
       } else if (wc < nkb) {
         for (int i = 0; i < ngroups; ++i) {
           const int g = rev ? ngroups - 1 - i : i;
-          wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1));
+          wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1), backoff);
           contract_block(Cb + (i % 3) * kCcBuf, g, wc, one, true, i, slot0, no);
         }
       }
@@ -849,7 +850,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     taps(0, cb_cur, one);
     for (int i = 0; i < ngroups; ++i) {
       const int g = rev ? ngroups - 1 - i : i;
-      wait_ge(&arrivals[i & 3], kCons * ((i >> 2) + 1));
+      wait_ge(&arrivals[i & 3], kCons * ((i >> 2) + 1), backoff);
       STAMPX(4 + 4 * i)
       // tap step i+1 goes first when its blocks are there (keeps the stores of
       // consecutive groups close), else after this group's contraction
