@@ -454,8 +454,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // pipeline (a single group gains nothing from overlapping with its neighbours).
     // Not for the accumulating rank pass: its stores read y first, and a
     // contraction wave would wait for that twice per group, one block after the other.
-    const bool split_wide = !split_narrow && pl.split2 && FS <= 3 && nkb <= 8 &&   // (5x5: registers)
-                            (nkb >= 6 || ngroups >= 3) && !a.accumulate;
+    // (5x5: the weights of a second rank quad do not fit - up to 16 ranks only)
+    const bool split_wide = !split_narrow && pl.split2 && (FS <= 3 || (FS == 5 && R <= 16)) &&
+                            nkb <= 8 && (nkb >= 6 || ngroups >= 3) && !a.accumulate;
 #endif
     const bool split_roles = split_narrow || split_wide;
     const int wq = split_roles ? (wc >= 4 ? wc - 4 : 0) : wc;     // (first) rank quad in the tap step
@@ -778,16 +779,19 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       // contraction wave has read it for its last block.
       const int ncw = nkb < 4 ? nkb : 4;           // contraction waves with a block
       if (wc >= 4) {
+        // (up to 16 ranks: the second rank chunk is never read, one quad each)
         if constexpr (NTQ == 2) {
-          // (up to 16 ranks: the second rank chunk is never read, one quad each)
           if (R > 16) load_taps(std::integral_constant<int, 1>{});
-          for (int i = 0; i < ngroups; ++i) {
-            if (i >= 3) wait_ge(&cdone[(i - 3) & 3], ncw * (((i - 3) >> 2) + 1), backoff);
-            if (R > 16)
+        }
+        for (int i = 0; i < ngroups; ++i) {
+          if (i >= 3) wait_ge(&cdone[(i - 3) & 3], ncw * (((i - 3) >> 2) + 1), backoff);
+          if constexpr (NTQ == 2) {
+            if (R > 16) {
               taps(i, Cb + (i % 3) * kCcBuf, two);
-            else
-              taps(i, Cb + (i % 3) * kCcBuf, one);
+              continue;
+            }
           }
+          taps(i, Cb + (i % 3) * kCcBuf, one);
         }
       } else if (wc < nkb) {
         const bool second = wc + 4 < nkb;

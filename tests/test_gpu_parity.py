@@ -208,6 +208,7 @@ EDGE = [
     (2, 32, 5, 200, 0, 200, 1, 1, 12),    # 1x1, seven blocks (the last partly filled), one rank chunk
     (1, 64, 13, 13, 1, 224, 3, 3, 24),    # odd plane: per-pixel stores, one group per strip
     (1, 320, 3, 210, 1, 72, 3, 3, 28),    # factor fragments in LDS, three blocks, four groups
+    (2, 64, 10, 90, 2, 200, 5, 5, 12),    # 5x5 with up to 16 ranks: one quad per tap wave, seven blocks
     # wide planes: tiles of TH rows x Wt columns (producer/consumer kernel, tiled build)
     (1, 16, 9, 200, 1, 32, 3, 3, 8),      # four column tiles, the last one 8 columns wide
     (2, 24, 5, 131, 2, 16, 5, 5, 12),     # odd width across three tiles, 5x5
