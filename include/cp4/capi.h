@@ -7,9 +7,19 @@
  * Plain pointers and sizes only.  Every data pointer is a DEVICE pointer to
  * contiguous fp32; activations are NCHW, the four factor matrices row-major
  * [dim, Rank] in the reference's argument order (out-channel FK = "FT",
- * in-channel FC, height FH = "FY", width FW = "FX").  Nothing here keeps global
- * state between calls, so calls on different streams may overlap.  Functions
+ * in-channel FC, height FH = "FY", width FW = "FX").  The passes keep no state
+ * between calls, so calls on different streams may overlap; what the library
+ * does keep per process is listed where it is set: the tuner's choices
+ * (cp4_tune_*), the bound of the in-kernel waits (cp4_set_spin_limit) and, on
+ * each device, the sticky fault record read by cp4_device_status.  Functions
  * return a status code and never exit the process.
+ *
+ * Non-finite inputs: the matrix-core kernels form every product from exact
+ * three-way splits of the fp32 operands, and Inf - trunc(Inf) is NaN.  An Inf or
+ * NaN in an activation or a factor therefore yields NaN in every output element
+ * whose sum it enters - also where plain fp32 arithmetic would give +-Inf or, for
+ * 0 * Inf, NaN anyway - and leaves all other elements exact.  Finite inputs
+ * whose products overflow fp32 behave like fp32 (+-Inf).
  */
 #ifndef CP4_CAPI_H
 #define CP4_CAPI_H
@@ -32,7 +42,8 @@ typedef enum cp4_status {
   CP4_ERR_SHAPE = 2,       /* zero dim, sizes beyond the documented limits ... */
   CP4_ERR_HIP = 3,         /* a HIP runtime call failed; see cp4_last_error_message */
   CP4_ERR_WORKSPACE = 4,   /* workspace missing or too small */
-  CP4_ERR_UNSUPPORTED = 5  /* requested kernel variant cannot run this shape */
+  CP4_ERR_UNSUPPORTED = 5, /* requested kernel variant cannot run this shape */
+  CP4_ERR_DEVICE = 6       /* a kernel gave up a wait between its waves: outputs incomplete */
 } cp4_status;
 
 /* A hipStream_t passed as void*; NULL is the default stream. */
@@ -41,6 +52,32 @@ typedef void* cp4_stream;
 const char* cp4_status_string(cp4_status);
 /* Detail of the calling thread's last failure ("" if none). */
 const char* cp4_last_error_message(void);
+
+/* ---- device-side failures --------------------------------------------------
+ * The producer / consumer kernels (the default for most shapes of forward and
+ * backward-data) hand work between the waves of a workgroup through counters in
+ * LDS and wait for them with a bounded number of polls.  A wait that runs out -
+ * which takes a bug in the library or a wave stalled for about a quarter of a
+ * second - never lets its wave go on: the wave records the fault on the device,
+ * the workgroup's other waves stop waiting, and the waves that gave up store
+ * nothing further, so the outputs of that launch are incomplete rather than
+ * silently wrong.  Launches are asynchronous, so the launch itself still
+ * returns CP4_OK; the record is sticky until somebody reads it:
+ *
+ * cp4_device_status synchronises `stream`, reads and clears the current device's
+ * record and returns CP4_ERR_DEVICE if a wait has run out since the last call
+ * (CP4_OK otherwise).  detail, if not NULL, receives {flag, workgroup, wave, wait
+ * site}.  The cp4_time_* and cp4_tune_* loops, which synchronise anyway, call it
+ * themselves and return its status; so do the synchronous C++ launchers of
+ * cp4conv2d.h.
+ *
+ * cp4_set_spin_limit sets the number of polls after which a wait gives up, for
+ * every later launch of the process (0: the default, 2^19).  For fault-injection
+ * tests of callers' error handling: with a limit of 1 the first wait of every
+ * workgroup runs out, every wave still ends normally, and cp4_device_status
+ * reports the fault. */
+cp4_status cp4_device_status(cp4_stream stream, int* detail);
+void cp4_set_spin_limit(int polls);
 
 /* ---- the three passes --------------------------------------------------- */
 
@@ -150,6 +187,16 @@ cp4_status cp4_time_forward(const cp4_shape* shape, const float* x,
                             const float* FW, float* y, unsigned warmup,
                             unsigned profcount, float* mean_us,
                             cp4_stream stream);
+/* The same loop over `nsets` distinct input / output buffer sets taken in turn
+ * (launch i uses xs[i % nsets], ys[i % nsets]; host arrays of device pointers).
+ * The reference's loop re-launches on one set, whose 2 x 103 MB at the
+ * ResNet-stage shape stay in the part's 256 MB memory-side cache; with enough sets
+ * to exceed it every launch streams from and to HBM, as a training step does. */
+cp4_status cp4_time_forward_sets(const cp4_shape* shape, const float* const* xs,
+                                 float* const* ys, unsigned nsets, const float* FK,
+                                 const float* FC, const float* FH, const float* FW,
+                                 unsigned warmup, unsigned profcount, float* mean_us,
+                                 cp4_stream stream);
 cp4_status cp4_time_backward_data(const cp4_shape* shape, const float* dy,
                                   const float* FK, const float* FC,
                                   const float* FH, const float* FW, float* dx,
@@ -182,13 +229,32 @@ cp4_status cp4_conv2d_forward_variant(const cp4_shape* shape, const float* x,
                                       float* y, int variant,
                                       cp4_stream stream);
 /* Times every variant that supports `shape` (warmup + profcount launches
- * each) on the caller's buffers, remembers the fastest for this shape for the
- * rest of the process and reports it. */
+ * each) on the caller's buffers - the producer / consumer variants once per
+ * strip height (tile height x width for wide planes) up to 16 rows and with the
+ * consumers' role split on and off - remembers the fastest for this shape for the
+ * rest of the process (a process-wide table behind a mutex; cp4_tune_clear
+ * empties it) and reports it.  cp4_tune_backward_data does the same for that
+ * pass, cp4_tune_backward_filter chooses between that pass's two variants.
+ * cp4_tuned_choice reports what a shape would run with now: the variant, the
+ * tuned tile (rows, columns; 0 = the kernel's own planner) and the role split. */
 cp4_status cp4_tune_forward(const cp4_shape* shape, const float* x,
                             const float* FK, const float* FC, const float* FH,
                             const float* FW, float* y, unsigned warmup,
                             unsigned profcount, int* best_variant,
                             float* best_us, cp4_stream stream);
+cp4_status cp4_tune_backward_data(const cp4_shape* shape, const float* dy,
+                                  const float* FK, const float* FC, const float* FH,
+                                  const float* FW, float* dx, unsigned warmup,
+                                  unsigned profcount, int* best_variant,
+                                  float* best_us, cp4_stream stream);
+cp4_status cp4_tune_backward_filter(const cp4_shape* shape, const float* x, const float* dy,
+                                    const float* FK, const float* FC, const float* FH,
+                                    const float* FW, float* dFK, float* dFC, float* dFH,
+                                    float* dFW, void* workspace, size_t workspace_bytes,
+                                    unsigned warmup, unsigned profcount, int* best_variant,
+                                    float* best_us, cp4_stream stream);
+cp4_status cp4_tuned_choice(const cp4_shape* shape, int backward_data, int* variant,
+                            int* tile_rows, int* tile_cols, int* role_split);
 void cp4_tune_clear(void);
 
 /* ---- device allocator / copy helpers (the reference's Tensor uses

@@ -10,8 +10,10 @@ from .capi import (Shape, Cp4Error, lib, library_path, conv2d_forward, conv2d_fo
                    conv2d_backward_data_bf16, conv2d_backward_filter_bf16, bf16_supported,
                    conv2d_backward_data, conv2d_backward_filter,
                    conv2d_backward_filter_full, backward_filter_workspace_bytes,
-                   time_forward, time_backward_data, time_backward_filter,
-                   tune_forward, forward_variants, recompose, count_exceeding,
+                   time_forward, time_forward_sets, time_backward_data, time_backward_filter,
+                   tune_forward, tune_backward_data, tune_backward_filter, tuned_choice,
+                   tune_clear, device_status, device_status_detail, set_spin_limit,
+                   forward_variants, recompose, count_exceeding,
                    random_uniform, time_copy, cp3_shape_for, cp3_expand_factors,
                    cp3_fold_gradients, cp3_conv2d_forward, cp3_conv2d_backward_data)
 

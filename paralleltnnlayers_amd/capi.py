@@ -10,8 +10,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# CP4_LIBRARY points at another build of the same library (A/B timing of kernels).
-_LIB = os.environ.get("CP4_LIBRARY") or os.path.join(_HERE, "csrc", "libcp4conv.so")
+_LIB = os.path.join(_HERE, "csrc", "libcp4conv.so")
 
 
 class Cp4Error(RuntimeError):
@@ -31,7 +30,8 @@ class Shape(ctypes.Structure):
 
 
 # status codes of cp4_status
-OK, ERR_NULL_POINTER, ERR_SHAPE, ERR_HIP, ERR_WORKSPACE, ERR_UNSUPPORTED = range(6)
+(OK, ERR_NULL_POINTER, ERR_SHAPE, ERR_HIP, ERR_WORKSPACE, ERR_UNSUPPORTED,
+ ERR_DEVICE) = range(7)
 
 _lib = None
 _F = ctypes.c_void_p          # const float* / float* (device)
@@ -81,12 +81,23 @@ def lib():
     timing = [ctypes.c_uint, ctypes.c_uint, ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
     L.cp4_time_forward.argtypes = fwd + timing
     L.cp4_time_backward_data.argtypes = fwd + timing
+    L.cp4_time_forward_sets.argtypes = [_S, ctypes.POINTER(ctypes.c_void_p),
+                                        ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint,
+                                        _F, _F, _F, _F] + timing
     L.cp4_time_backward_filter.argtypes = bwf + timing
     L.cp4_forward_variant_supported.argtypes = [_S, ctypes.c_int]
     L.cp4_tune_forward.argtypes = fwd + [ctypes.c_uint, ctypes.c_uint,
                                          ctypes.POINTER(ctypes.c_int),
                                          ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
+    L.cp4_tune_backward_data.argtypes = L.cp4_tune_forward.argtypes
+    L.cp4_tune_backward_filter.argtypes = bwf + [ctypes.c_uint, ctypes.c_uint,
+                                                 ctypes.POINTER(ctypes.c_int),
+                                                 ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
+    L.cp4_tuned_choice.argtypes = [_S, ctypes.c_int] + [ctypes.POINTER(ctypes.c_int)] * 4
     L.cp4_tune_clear.restype = None
+    L.cp4_device_status.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
+    L.cp4_set_spin_limit.argtypes = [ctypes.c_int]
+    L.cp4_set_spin_limit.restype = None
     L.cp4_recompose.argtypes = [_S, _F, _F, _F, _F, _F, ctypes.c_void_p]
     L.cp3_expand_factors.argtypes = [_S] + [_F] * 7 + [ctypes.c_void_p]
     L.cp3_fold_gradients.argtypes = [_S] + [_F] * 6 + [ctypes.c_void_p]
@@ -240,10 +251,13 @@ def backward_filter_workspace_bytes(s):
 
 
 def _workspace(s, device, workspace):
+    """(tensor, its size in bytes): the caller's workspace of any dtype, or a new one."""
     need = backward_filter_workspace_bytes(s)
     if workspace is None:
         workspace = torch.empty(max(need, 4) // 4 + 1, device=device, dtype=torch.float32)
-    return workspace, workspace.numel() * 4
+    assert workspace.is_cuda and workspace.is_contiguous(), \
+        "the workspace must be a contiguous device tensor"
+    return workspace, workspace.numel() * workspace.element_size()
 
 
 def conv2d_backward_filter(x, dy, FK, FC, FH, FW, pad=1, workspace=None, stream=None,
@@ -277,6 +291,22 @@ def time_forward(x, FK, FC, FH, FW, y, pad, warmup=1, profcount=47, stream=None)
     check(lib().cp4_time_forward(ctypes.byref(s), _ptr(x), _ptr(FK), _ptr(FC), _ptr(FH),
                                  _ptr(FW), _ptr(y), warmup, profcount, ctypes.byref(us),
                                  _stream(stream)))
+    return us.value
+
+
+def time_forward_sets(xs, FK, FC, FH, FW, ys, pad, warmup=1, profcount=47, stream=None):
+    """The timed loop over several buffer sets taken in turn (launch i uses set
+    i % len(xs)): with a footprint beyond the memory-side cache every launch
+    streams from and to HBM."""
+    assert len(xs) == len(ys) >= 1
+    s = shape_for(xs[0].shape, FK, FC, FH, FW, pad)
+    n = len(xs)
+    xp = (ctypes.c_void_p * n)(*[_ptr(x) for x in xs])
+    yp = (ctypes.c_void_p * n)(*[_ptr(y) for y in ys])
+    us = ctypes.c_float()
+    check(lib().cp4_time_forward_sets(ctypes.byref(s), xp, yp, n, _ptr(FK), _ptr(FC), _ptr(FH),
+                                      _ptr(FW), warmup, profcount, ctypes.byref(us),
+                                      _stream(stream)))
     return us.value
 
 
@@ -319,6 +349,58 @@ def tune_forward(x, FK, FC, FH, FW, y, pad, warmup=1, profcount=10, stream=None)
                                  _ptr(FW), _ptr(y), warmup, profcount, ctypes.byref(best),
                                  ctypes.byref(us), _stream(stream)))
     return best.value, us.value
+
+
+def tune_backward_data(dy, FK, FC, FH, FW, dx, pad, warmup=1, profcount=10, stream=None):
+    s = shape_for(dy.shape, FK, FC, FH, FW, pad)
+    best, us = ctypes.c_int(-1), ctypes.c_float()
+    check(lib().cp4_tune_backward_data(ctypes.byref(s), _ptr(dy), _ptr(FK), _ptr(FC), _ptr(FH),
+                                       _ptr(FW), _ptr(dx), warmup, profcount,
+                                       ctypes.byref(best), ctypes.byref(us), _stream(stream)))
+    return best.value, us.value
+
+
+def tune_backward_filter(x, dy, FK, FC, FH, FW, pad, warmup=1, profcount=10, workspace=None,
+                         stream=None):
+    """(best variant: 0 general / 1 matrix-core, its mean us)."""
+    s = shape_for(x.shape, FK, FC, FH, FW, pad)
+    outs = [torch.empty_like(f) for f in (FK, FC, FH, FW)]
+    ws, ws_bytes = _workspace(s, x.device, workspace)
+    best, us = ctypes.c_int(-1), ctypes.c_float()
+    check(lib().cp4_tune_backward_filter(
+        ctypes.byref(s), _ptr(x), _ptr(dy), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
+        *[_ptr(o) for o in outs], ctypes.c_void_p(ws.data_ptr()), ws_bytes, warmup, profcount,
+        ctypes.byref(best), ctypes.byref(us), _stream(stream)))
+    return best.value, us.value
+
+
+def tuned_choice(s, backward_data=False):
+    """{'variant', 'tile_rows', 'tile_cols', 'role_split'} a shape would run with now."""
+    v = [ctypes.c_int() for _ in range(4)]
+    check(lib().cp4_tuned_choice(ctypes.byref(s), int(backward_data), *[ctypes.byref(i) for i in v]))
+    return dict(zip(("variant", "tile_rows", "tile_cols", "role_split"), (i.value for i in v)))
+
+
+def tune_clear():
+    lib().cp4_tune_clear()
+
+
+def device_status(stream=None):
+    """Synchronises the stream; raises Cp4Error(ERR_DEVICE) if a kernel gave up a
+    wait between its waves since the last call (the record is cleared)."""
+    check(lib().cp4_device_status(_stream(stream), None))
+
+
+def device_status_detail(stream=None):
+    """(status, [flag, workgroup, wave, wait site]) without raising."""
+    d = (ctypes.c_int * 4)()
+    st = lib().cp4_device_status(_stream(stream), d)
+    return st, list(d)
+
+
+def set_spin_limit(polls):
+    """Polls after which an in-kernel wait gives up (0: the default); fault injection."""
+    lib().cp4_set_spin_limit(int(polls))
 
 
 def recompose(FK, FC, FH, FW, stream=None):

@@ -17,6 +17,9 @@
 #include <cstdlib>
 
 #include "cp4_internal.h"
+#ifdef CP4_DEBUG_PHASES
+#include "cp4_debug.h"
+#endif
 #include "split_bf16.h"
 
 // Compiled a second time with CP4_BWF_IO16: x and dy are then bfloat16 in memory
@@ -1168,7 +1171,7 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   c.N = N; c.R = R; c.RP = p.RP; c.HW = HW; c.npb = p.npb;
   c.items = N * p.npb;
 #ifdef CP4_DEBUG_PHASES
-  c.dbg = getenv("CP4_DBG_PTR") ? reinterpret_cast<long long*>(strtoull(getenv("CP4_DBG_PTR"), nullptr, 10)) : nullptr;
+  c.dbg = debug_stamp_buffer();
 #endif
   const int cmax = a.C > a.T ? a.C : a.T;
   hipError_t e;
@@ -1242,7 +1245,7 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   g.act[1] = ax; g.Z[1] = G1; g.part[1] = pC; g.D[1] = a.C;
   g.N = N; g.R = R; g.RP = p.RP; g.HW = HW; g.PS = p.PS; g.cps = p.cps;
 #ifdef CP4_DEBUG_PHASES
-  g.dbg = getenv("CP4_DBG_PTR") ? reinterpret_cast<long long*>(strtoull(getenv("CP4_DBG_PTR"), nullptr, 10)) : nullptr;
+  g.dbg = debug_stamp_buffer();
 #endif
   const int dmax = a.T > a.C ? a.T : a.C;
   const dim3 ggrid(p.S, (dmax + 127) / 128, 2);

@@ -1,5 +1,6 @@
 // C ABI entry points: argument checks, kernel-variant choice, the PROFCOUNT
 // timing loops and the device allocator / copy helpers.
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <map>
@@ -13,6 +14,16 @@ namespace {
 using cp4::FwdArgs;
 
 thread_local char g_err[256] = "";
+
+// Sticky record of the first in-kernel wait that ran out on this device since the
+// last cp4_device_status: {nonzero, workgroup, wave, wait site}.  One copy per GPU.
+__device__ int g_device_fault[4];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_dev_mu;
+int* g_fault_ptr[kMaxDevices];
+int g_num_cus[kMaxDevices];
+std::atomic<int> g_spin_limit{0};
 
 cp4_status fail(cp4_status st, const char* what) {
   std::snprintf(g_err, sizeof(g_err), "%s", what);
@@ -29,6 +40,53 @@ cp4_status hip_fail(hipError_t e, const char* where) {
   } while (0)
 
 hipStream_t as_stream(cp4_stream s) { return static_cast<hipStream_t>(s); }
+
+// Address of this device's fault record (null if the runtime cannot say; the
+// kernels then run without one).
+int* fault_of_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lk(g_dev_mu);
+  if (!g_fault_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_device_fault)) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    g_fault_ptr[dev] = static_cast<int*>(p);
+  }
+  return g_fault_ptr[dev];
+}
+
+// The launch context every producer / consumer launch carries.
+void arm(FwdArgs& a) {
+  a.fault = fault_of_current_device();
+  a.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
+}
+
+// Synchronise `st`, read and clear the device's fault record.
+cp4_status device_status(hipStream_t st, int* detail) {
+  CP4_HIP(hipStreamSynchronize(st));
+  int rec[4] = {0, 0, 0, 0};
+  int* p = fault_of_current_device();
+  if (p) {
+    CP4_HIP(hipMemcpy(rec, p, sizeof(rec), hipMemcpyDeviceToHost));
+    if (rec[0]) {
+      const int zero[4] = {0, 0, 0, 0};
+      CP4_HIP(hipMemcpy(p, zero, sizeof(zero), hipMemcpyHostToDevice));
+    }
+  }
+  if (detail) memcpy(detail, rec, sizeof(rec));
+  if (!rec[0]) return CP4_OK;
+  std::snprintf(g_err, sizeof(g_err),
+                "a wait between waves ran out in workgroup %d, wave %d, wait site %d: the "
+                "outputs of launches since the last status check are incomplete",
+                rec[1], rec[2], rec[3]);
+  return CP4_ERR_DEVICE;
+}
 
 // Shape rules shared by the three passes.  N == 0 is a valid empty batch.
 cp4_status check_shape(const cp4_shape* s) {
@@ -107,69 +165,111 @@ const Variant kVariants[] = {
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
+// ---- choice of kernel variant and of its tile ------------------------------------
+
+// What runs a shape: a variant and, for the producer / consumer kernels, the tile
+// the tuner measured to be best (zeros: the kernel's own planner).
+struct Choice {
+  int variant;
+  int th, lgwt, split2;
+};
+
 using TuneKey = std::tuple<int, int, int, int, int, int, int, int, int, int>;
 std::mutex g_tune_mu;
-std::map<TuneKey, int> g_tuned;
+std::map<TuneKey, Choice> g_tuned;          // filled by cp4_tune_forward / _backward_data only
+std::map<TuneKey, int> g_tuned_filter;      // filled by cp4_tune_backward_filter only
 
 TuneKey key_of(const FwdArgs& a) {
   return TuneKey(a.N, a.Cin, a.Cout, a.H, a.W, a.pad, a.Y, a.X, a.R, a.flip);
 }
+TuneKey key_of(const cp4_shape& s) {
+  return TuneKey(s.N, s.C, s.T, s.H, s.W, s.pad, s.Y, s.X, s.Rank, 2);
+}
 
-int choose_variant(const FwdArgs& a) {
+int variant_named(const char* name) {
+  for (int v = 0; v < kNumVariants; ++v)
+    if (!strcmp(kVariants[v].name, name)) return v;
+  return -1;
+}
+bool is_variant(int v, const char* name) { return v >= 0 && !strcmp(kVariants[v].name, name); }
+
+// Thresholds of the untuned heuristic, each the measured crossover on MI355X.
+// Above 256 input channels the producer / consumer kernel keeps its factor in LDS
+// and its strips get short; from this many pixels on, the phase-by-phase split
+// kernel is then the faster one where it applies (even widths).
+constexpr long kPipeLdsFactorMaxPixels = 8192;
+constexpr int kPipeRegisterFactorMaxCin = 256;
+// Fewer channels than this on both sides together leave the 32 x 32 matrix tiles
+// almost empty: the VALU kernels, whose cost follows the real channel counts, win.
+constexpr int kMatrixMinChannels = 24;
+// Rows longer than this leave whole-row strips only a row or two (2 at W = 224):
+// tiles of TH x Wt pay less for their halo.
+constexpr int kWholeRowMaxWidth = 128;
+// Two rank passes read x twice and y once more; below this many activation
+// elements the fp32 matrix-core strip kernel is the faster one for ranks 33-64.
+constexpr long kTwoPassMinElements = 16l << 20;
+
+int heuristic_variant(const FwdArgs& a) {
+  // CP4_FORWARD_VARIANT=<name> overrides the heuristic where that variant can
+  // run the shape (profiling and A/B runs of unmodified callers).
+  if (const char* want = getenv("CP4_FORWARD_VARIANT")) {
+    const int v = variant_named(want);
+    if (v >= 0 && kVariants[v].supported(a)) return v;
+  }
+  int pick = -1;
+  for (int v = kNumVariants - 1; v >= 0 && pick < 0; --v)
+    if (kVariants[v].supported(a)) pick = v;
+  auto prefer = [&](const char* name) {
+    const int v = variant_named(name);
+    if (v >= 0 && kVariants[v].supported(a)) pick = v;
+  };
+  if (is_variant(pick, "mfma_bf16x3_pipe") && a.Cin > kPipeRegisterFactorMaxCin &&
+      (long)a.N * a.H * a.W > kPipeLdsFactorMaxPixels)
+    prefer("mfma_bf16x3_strip");
+  if (pick >= 0 && !strncmp(kVariants[pick].name, "mfma_bf16x3_pipe", 16) &&
+      a.Cin + a.Cout < kMatrixMinChannels) {
+    prefer("general_valu");
+    prefer("valu_rows");
+  }
+  if (is_variant(pick, "mfma_bf16x3_pipe") && a.W > kWholeRowMaxWidth)
+    prefer("mfma_bf16x3_pipe_tiled");
+  if (is_variant(pick, "mfma_bf16x3_pipe_2pass") &&
+      (long)a.N * a.H * a.W * (a.Cin + a.Cout) < kTwoPassMinElements)
+    prefer("mfma_f32_strip");
+  return pick;
+}
+
+Choice choose(const FwdArgs& a) {
   {
     std::lock_guard<std::mutex> lk(g_tune_mu);
     auto it = g_tuned.find(key_of(a));
     if (it != g_tuned.end()) return it->second;
   }
-  // CP4_FORWARD_VARIANT=<name> overrides the heuristic where that variant can
-  // run the shape (profiling and A/B runs of unmodified callers).
-  if (const char* want = getenv("CP4_FORWARD_VARIANT")) {
-    for (int v = 0; v < kNumVariants; ++v)
-      if (!strcmp(want, kVariants[v].name) && kVariants[v].supported(a)) return v;
-  }
-  int pick = -1;
-  for (int v = kNumVariants - 1; v >= 0 && pick < 0; --v)
-    if (kVariants[v].supported(a)) pick = v;
-  // Above 256 input channels the producer/consumer kernel keeps its factor in
-  // LDS and its strips get short; on large problems the phase-by-phase split
-  // kernel, where it applies (even widths), is then the faster one.
-  if (pick >= 0 && !strcmp(kVariants[pick].name, "mfma_bf16x3_pipe") && a.Cin > 256 &&
-      (long)a.N * a.H * a.W > 8192) {
-    for (int v = 0; v < kNumVariants; ++v)
-      if (!strcmp(kVariants[v].name, "mfma_bf16x3_strip") && kVariants[v].supported(a)) pick = v;
-  }
-  // A handful of channels on either side (3 -> 1, say) leaves the 32 x 32 matrix
-  // tiles almost empty: the general kernel, whose cost follows the real channel
-  // counts, is then as fast or faster.
-  if (pick >= 0 && !strncmp(kVariants[pick].name, "mfma_bf16x3_pipe", 16) &&
-      a.Cin + a.Cout < 24) {
-    for (int v = 0; v < kNumVariants; ++v)
-      if (!strcmp(kVariants[v].name, "general_valu") && kVariants[v].supported(a)) pick = v;
-  }
-  // Planes wider than 128 pixels: whole-row strips get short (2 rows at W = 224)
-  // and pay for it in halo rows; tiles of TH x Wt do better there.
-  if (pick >= 0 && !strcmp(kVariants[pick].name, "mfma_bf16x3_pipe") && a.W > 128) {
-    for (int v = 0; v < kNumVariants; ++v)
-      if (!strcmp(kVariants[v].name, "mfma_bf16x3_pipe_tiled") && kVariants[v].supported(a))
-        pick = v;
-  }
-  // Two rank passes read x twice and y once more: on small problems the fp32
-  // matrix-core strip kernel, where it applies, is the faster one for ranks 33-64.
-  if (pick >= 0 && !strcmp(kVariants[pick].name, "mfma_bf16x3_pipe_2pass") &&
-      (long)a.N * a.H * a.W * (a.Cin + a.Cout) < (16l << 20)) {
-    for (int v = 0; v < kNumVariants; ++v)
-      if (!strcmp(kVariants[v].name, "mfma_f32_strip") && kVariants[v].supported(a)) pick = v;
-  }
-  return pick;
+  return Choice{heuristic_variant(a), 0, 0, 0};
+}
+
+FwdArgs with_tile(const FwdArgs& a, const Choice& c) {
+  FwdArgs b = a;
+  b.tune_th = c.th;
+  b.tune_lgwt = c.lgwt;
+  b.tune_split2 = c.split2;
+  return b;
+}
+
+cp4_status run_choice(const FwdArgs& a0, const Choice& c, hipStream_t st) {
+  if (c.variant < 0 || c.variant >= kNumVariants)
+    return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape");
+  FwdArgs a = with_tile(a0, c);
+  if (!kVariants[c.variant].supported(a))
+    return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape");
+  arm(a);
+  CP4_HIP(kVariants[c.variant].launch(a, st));
+  return CP4_OK;
 }
 
 cp4_status run_forward_like(const FwdArgs& a, int variant, hipStream_t st) {
   if (a.N == 0) return CP4_OK;
-  if (variant < 0) variant = choose_variant(a);
-  if (variant < 0 || variant >= kNumVariants || !kVariants[variant].supported(a))
-    return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape");
-  CP4_HIP(kVariants[variant].launch(a, st));
-  return CP4_OK;
+  return run_choice(a, variant < 0 ? choose(a) : Choice{variant, 0, 0, 0}, st);
 }
 
 // One workspace size serves either backward-filter variant.
@@ -213,10 +313,31 @@ cp4_status time_loop(Launch&& launch, unsigned warmup, unsigned profcount,
   if (rc != CP4_OK) return rc;
   if (e != hipSuccess) return hip_fail(e, "timing loop");
   *mean_us = ms * 1e3f / (float)profcount;
-  return CP4_OK;
+  return device_status(st, nullptr);    // the launches are done: did any give up a wait?
 }
 
 }  // namespace
+
+namespace cp4 {
+int num_compute_units() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  std::lock_guard<std::mutex> lk(g_dev_mu);
+  if (!g_num_cus[dev]) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        n <= 0) {
+      (void)hipGetLastError();
+      n = 256;
+    }
+    g_num_cus[dev] = n;
+  }
+  return g_num_cus[dev];
+}
+}  // namespace cp4
 
 extern "C" {
 
@@ -228,6 +349,7 @@ const char* cp4_status_string(cp4_status s) {
     case CP4_ERR_HIP: return "HIP runtime error";
     case CP4_ERR_WORKSPACE: return "workspace missing or too small";
     case CP4_ERR_UNSUPPORTED: return "unsupported kernel variant for this shape";
+    case CP4_ERR_DEVICE: return "a kernel gave up a wait between its waves";
   }
   return "unknown status";
 }
@@ -279,13 +401,18 @@ cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
   FwdArgs plain = a;
   plain.bias = nullptr;
   plain.act = 0;
-  const int v = choose_variant(plain);
-  if (v < 0) return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape");
-  if (!strcmp(kVariants[v].name, "mfma_bf16x3_pipe") && cp4::fwd_pipe_epi_supported(a)) {
-    CP4_HIP(cp4::fwd_pipe_epi_launch(a, st));
-    return CP4_OK;
+  const Choice c = choose(plain);
+  if (c.variant < 0) return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape");
+  if (is_variant(c.variant, "mfma_bf16x3_pipe")) {
+    FwdArgs e = with_tile(a, c);
+    if (cp4::fwd_pipe_epi_supported(e)) {
+      arm(e);
+      CP4_HIP(cp4::fwd_pipe_epi_launch(e, st));
+      return CP4_OK;
+    }
   }
-  CP4_HIP(kVariants[v].launch(plain, st));
+  rc = run_choice(plain, c, st);
+  if (rc != CP4_OK) return rc;
   CP4_HIP(cp4::bias_act_launch(y, bias, activation, shape->N, shape->T,
                                (size_t)shape->H * shape->W, st));
   return CP4_OK;
@@ -334,6 +461,7 @@ cp4_status cp4_conv2d_forward_bf16(const cp4_shape* shape, const void* x_bf16,
                            static_cast<float*>(y_bf16));
   a.bias = bias;
   a.act = activation;
+  arm(a);
   if (!cp4::fwd_pipe_io16_supported(a))
     return fail(CP4_ERR_UNSUPPORTED, "bfloat16 I/O: shape not taken by the producer/consumer kernel");
   CP4_HIP(cp4::fwd_pipe_io16_launch(a, as_stream(stream)));
@@ -349,8 +477,9 @@ cp4_status cp4_conv2d_backward_data_bf16(const cp4_shape* shape, const void* dy_
   if (shape->N == 0) return CP4_OK;
   rc = check_forward_ptrs(dy_bf16, FK, FC, FH, FW, dx_bf16);
   if (rc != CP4_OK) return rc;
-  const FwdArgs a = backward_data_args(*shape, static_cast<const float*>(dy_bf16), FK, FC, FH, FW,
-                                       static_cast<float*>(dx_bf16));
+  FwdArgs a = backward_data_args(*shape, static_cast<const float*>(dy_bf16), FK, FC, FH, FW,
+                                 static_cast<float*>(dx_bf16));
+  arm(a);
   if (!cp4::fwd_pipe_io16_supported(a))
     return fail(CP4_ERR_UNSUPPORTED, "bfloat16 I/O: shape not taken by the producer/consumer kernel");
   CP4_HIP(cp4::fwd_pipe_io16_launch(a, as_stream(stream)));
@@ -402,6 +531,11 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
   a.dFK = dFK; a.dFC = dFC; a.dFH = dFH; a.dFW = dFW; a.workspace = workspace;
   a.N = s.N; a.C = s.C; a.T = s.T; a.H = s.H; a.W = s.W; a.pad = s.pad;
   a.Y = s.Y; a.X = s.X; a.R = s.Rank;
+  if (variant < 0) {
+    std::lock_guard<std::mutex> lk(g_tune_mu);
+    auto it = g_tuned_filter.find(key_of(s));
+    if (it != g_tuned_filter.end() && (it->second == 0 || mfma_ok)) variant = it->second;
+  }
   if (variant == 1 || (variant < 0 && mfma_ok)) CP4_HIP(cp4::bwd_filter_mfma_launch(a, st));
   else CP4_HIP(cp4::bwd_filter_launch(a, st));
   return CP4_OK;
@@ -483,6 +617,22 @@ cp4_status cp4_time_forward(const cp4_shape* shape, const float* x,
       warmup, profcount, mean_us, as_stream(stream));
 }
 
+cp4_status cp4_time_forward_sets(const cp4_shape* shape, const float* const* xs,
+                                 float* const* ys, unsigned nsets, const float* FK,
+                                 const float* FC, const float* FH, const float* FW,
+                                 unsigned warmup, unsigned profcount, float* mean_us,
+                                 cp4_stream stream) {
+  if (!xs || !ys) return fail(CP4_ERR_NULL_POINTER, "xs or ys is NULL");
+  if (nsets == 0) return fail(CP4_ERR_SHAPE, "nsets must be >= 1");
+  unsigned i = 0;
+  return time_loop(
+      [&] {
+        const unsigned k = i++ % nsets;
+        return cp4_conv2d_forward(shape, xs[k], FK, FC, FH, FW, ys[k], stream);
+      },
+      warmup, profcount, mean_us, as_stream(stream));
+}
+
 cp4_status cp4_time_backward_data(const cp4_shape* shape, const float* dy,
                                   const float* FK, const float* FC,
                                   const float* FH, const float* FW, float* dx,
@@ -528,6 +678,52 @@ cp4_status cp4_forward_variant_supported(const cp4_shape* shape, int variant) {
              : fail(CP4_ERR_UNSUPPORTED, "variant does not support this shape");
 }
 
+namespace {
+// Times every variant that can run the shape and, for the producer / consumer
+// kernels, every strip height (tile height and width) and role split they can
+// run it with; remembers the fastest.
+cp4_status tune_forward_like(const FwdArgs& a, unsigned warmup, unsigned profcount,
+                             int* best_variant, float* best_us, hipStream_t st) {
+  Choice best{-1, 0, 0, 0};
+  float best_t = 0.f;
+  auto consider = [&](const Choice& c) -> cp4_status {
+    if (!kVariants[c.variant].supported(with_tile(a, c))) return CP4_OK;
+    float us = 0.f;
+    const cp4_status rc =
+        time_loop([&] { return run_choice(a, c, st); }, warmup, profcount, &us, st);
+    if (rc != CP4_OK) return rc;
+    if (best.variant < 0 || us < best_t) {
+      best = c;
+      best_t = us;
+    }
+    return CP4_OK;
+  };
+  for (int v = 0; v < kNumVariants; ++v) {
+    if (!kVariants[v].supported(a)) continue;
+    cp4_status rc = consider(Choice{v, 0, 0, 0});     // the kernel's own planner
+    if (rc != CP4_OK) return rc;
+    const bool strips = is_variant(v, "mfma_bf16x3_pipe") || is_variant(v, "mfma_bf16x3_pipe_2pass");
+    const bool tiles = is_variant(v, "mfma_bf16x3_pipe_tiled");
+    if (!strips && !tiles) continue;
+    const int max_th = a.H < 16 ? a.H : 16;
+    for (int lgwt = tiles ? 6 : 0; lgwt <= (tiles ? 8 : 0); ++lgwt)
+      for (int th = 1; th <= max_th; ++th)
+        for (int split2 = 0; split2 <= 1; ++split2) {
+          rc = consider(Choice{v, th, lgwt, split2});
+          if (rc != CP4_OK) return rc;
+        }
+  }
+  if (best.variant < 0) return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape");
+  {
+    std::lock_guard<std::mutex> lk(g_tune_mu);
+    g_tuned[key_of(a)] = best;
+  }
+  if (best_variant) *best_variant = best.variant;
+  if (best_us) *best_us = best_t;
+  return CP4_OK;
+}
+}  // namespace
+
 cp4_status cp4_tune_forward(const cp4_shape* shape, const float* x,
                             const float* FK, const float* FC, const float* FH,
                             const float* FW, float* y, unsigned warmup,
@@ -538,31 +734,84 @@ cp4_status cp4_tune_forward(const cp4_shape* shape, const float* x,
   rc = check_forward_ptrs(x, FK, FC, FH, FW, y);
   if (rc != CP4_OK) return rc;
   if (shape->N == 0) return fail(CP4_ERR_SHAPE, "cannot tune an empty batch");
-  const FwdArgs a = forward_args(*shape, x, FK, FC, FH, FW, y);
+  return tune_forward_like(forward_args(*shape, x, FK, FC, FH, FW, y), warmup, profcount,
+                           best_variant, best_us, as_stream(stream));
+}
+
+cp4_status cp4_tune_backward_data(const cp4_shape* shape, const float* dy,
+                                  const float* FK, const float* FC, const float* FH,
+                                  const float* FW, float* dx, unsigned warmup,
+                                  unsigned profcount, int* best_variant,
+                                  float* best_us, cp4_stream stream) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  rc = check_forward_ptrs(dy, FK, FC, FH, FW, dx);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return fail(CP4_ERR_SHAPE, "cannot tune an empty batch");
+  return tune_forward_like(backward_data_args(*shape, dy, FK, FC, FH, FW, dx), warmup,
+                           profcount, best_variant, best_us, as_stream(stream));
+}
+
+cp4_status cp4_tune_backward_filter(const cp4_shape* shape, const float* x, const float* dy,
+                                    const float* FK, const float* FC, const float* FH,
+                                    const float* FW, float* dFK, float* dFC, float* dFH,
+                                    float* dFW, void* workspace, size_t workspace_bytes,
+                                    unsigned warmup, unsigned profcount, int* best_variant,
+                                    float* best_us, cp4_stream stream) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return fail(CP4_ERR_SHAPE, "cannot tune an empty batch");
   int best = -1;
   float best_t = 0.f;
-  for (int v = 0; v < kNumVariants; ++v) {
-    if (!kVariants[v].supported(a)) continue;
+  for (int v = 0; v < 2; ++v) {
     float us = 0.f;
-    rc = time_loop([&] { return run_forward_like(a, v, as_stream(stream)); },
-                   warmup, profcount, &us, as_stream(stream));
+    rc = time_loop(
+        [&] {
+          return cp4_conv2d_backward_filter_variant(shape, x, dy, FK, FC, FH, FW, dFK, dFC, dFH,
+                                                    dFW, workspace, workspace_bytes, v, stream);
+        },
+        warmup, profcount, &us, as_stream(stream));
+    if (rc == CP4_ERR_UNSUPPORTED) continue;
     if (rc != CP4_OK) return rc;
     if (best < 0 || us < best_t) { best = v; best_t = us; }
   }
   if (best < 0) return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape");
   {
     std::lock_guard<std::mutex> lk(g_tune_mu);
-    g_tuned[key_of(a)] = best;
+    g_tuned_filter[key_of(*shape)] = best;
   }
   if (best_variant) *best_variant = best;
   if (best_us) *best_us = best_t;
   return CP4_OK;
 }
 
+cp4_status cp4_tuned_choice(const cp4_shape* shape, int backward_data, int* variant,
+                            int* tile_rows, int* tile_cols, int* role_split) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  const FwdArgs a =
+      backward_data
+          ? backward_data_args(*shape, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr)
+          : forward_args(*shape, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr);
+  const Choice c = choose(a);
+  if (variant) *variant = c.variant;
+  if (tile_rows) *tile_rows = c.th;
+  if (tile_cols) *tile_cols = c.lgwt ? 1 << c.lgwt : 0;
+  if (role_split) *role_split = c.split2 == 1 ? 0 : 1;
+  return CP4_OK;
+}
+
 void cp4_tune_clear(void) {
   std::lock_guard<std::mutex> lk(g_tune_mu);
   g_tuned.clear();
+  g_tuned_filter.clear();
 }
+
+cp4_status cp4_device_status(cp4_stream stream, int* detail) {
+  return device_status(as_stream(stream), detail);
+}
+
+void cp4_set_spin_limit(int polls) { g_spin_limit.store(polls > 0 ? polls : 0); }
 
 cp4_status cp4_set_device(int ordinal) {
   CP4_HIP(hipSetDevice(ordinal));
@@ -718,6 +967,7 @@ cp4_status cp3_run(const cp4_shape* shape, const float* in, const float* K0, con
   FwdArgs a = backward ? backward_data_args(*shape, in, FK, K0, nullptr, nullptr, out)
                        : forward_args(*shape, in, FK, K0, nullptr, nullptr, out);
   a.taps2d = K1;
+  arm(a);
   const size_t pixels = (size_t)a.N * a.H * a.W;
   if (cp4::fwd_pipe_taps2d_supported(a) && a.W <= 128 && a.Cin + a.Cout >= 24 &&
       !(a.Cin > 256 && pixels > 8192)) {

@@ -35,7 +35,18 @@ struct FwdArgs {
   // 2-D-tap build of the producer / consumer kernel only: depthwise filter
   // [Y, X, R] used instead of the outer product FH x FW (FH, FW unused then).
   const float* taps2d;
+  // Producer / consumer kernel: a tuned strip height (tile height in the tiled
+  // build), log2 of the tile width (tiled build) and role split (1: off) that
+  // replace the planner's choice; 0 leaves it to the planner.
+  int tune_th, tune_lgwt, tune_split2;
+  // Producer / consumer kernel: polls before a wait between waves gives up
+  // (0: the default) and the device's fault record, four ints (may be null).
+  int spin_limit;
+  int* fault;
 };
+
+// Compute units of the current device (256 when no device can be asked).
+int num_compute_units();
 
 
 // The matrix-core kernels index pixels, strips and work items with 32-bit

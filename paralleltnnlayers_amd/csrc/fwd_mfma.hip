@@ -30,6 +30,9 @@
 #include <type_traits>
 
 #include "cp4_internal.h"
+#ifdef CP4_DEBUG_PHASES
+#include "cp4_debug.h"
+#endif
 
 namespace cp4 {
 namespace {
@@ -573,15 +576,16 @@ bool layout(const FwdArgs& a, int TH, StripPlan* pl) {
   return true;
 }
 
-// Strip height: fewest rounds of 256 workgroups times the per-strip matrix work
+// Strip height: fewest rounds of one workgroup per compute unit times the per-strip matrix work
 // (halo rows repeat the channel->rank contraction).
 bool plan(const FwdArgs& a, StripPlan* best) {
   double best_cost = 0;
   bool found = false;
+  const int cus = num_compute_units();
   for (int TH = 1; TH <= a.H; ++TH) {
     StripPlan pl;
     if (!layout(a, TH, &pl)) break;
-    const double rounds = (pl.nWG + 255) / 256;
+    const double rounds = (pl.nWG + cus - 1) / cus;
     const double cost = rounds * ((double)(TH + a.Y - 1) * a.Cin + (double)TH * a.Cout);
     if (!found || cost < best_cost) {
       best_cost = cost;
@@ -643,8 +647,8 @@ hipError_t fwd_mfma_launch(const FwdArgs& a, hipStream_t st) {
   StripPlan pl;
   if (!plan(a, &pl)) return hipErrorInvalidValue;
 #ifdef CP4_DEBUG_PHASES
-  if (getenv("CP4_FWD_PHASES")) pl.phases = atoi(getenv("CP4_FWD_PHASES"));
-  pl.dbg = getenv("CP4_DBG_PTR") ? reinterpret_cast<long long*>(strtoull(getenv("CP4_DBG_PTR"), nullptr, 10)) : nullptr;
+  pl.phases = debug_phase_limit(pl.phases);
+  pl.dbg = debug_stamp_buffer();
 #endif
   return a.R <= 32 ? launch_rb<1>(a, pl, st) : launch_rb<2>(a, pl, st);
 }

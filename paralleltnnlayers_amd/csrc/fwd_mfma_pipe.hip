@@ -65,6 +65,9 @@
 
 #include "cp4_internal.h"
 #include "split_bf16.h"
+#ifdef CP4_DEBUG_PHASES
+#include "cp4_debug.h"
+#endif
 
 #ifdef CP4_PIPE_IO16
 #define CP4_PIPE_EPILOGUE 1
@@ -90,7 +93,7 @@ constexpr int kProd = 8, kCons = 8;          // producer / consumer waves (4 per
 constexpr int kRP = 32;
 constexpr int kCcBuf = 24 * 512;             // bytes of one Cc fragment tile (64 pixels)
 constexpr size_t kLdsLimit = 160 * 1024;
-constexpr int kSpinLimit = 1 << 19;      // about a quarter of a second at the longest nap
+constexpr int kSpinLimit = 1 << 19;      // default bound of a wait: about a quarter of a second at the longest nap
 constexpr int kMaxBlk = 64;                  // per-block progress words in LDS
 
 struct PipePlan {
@@ -103,9 +106,19 @@ struct PipePlan {
   int Wt, lgWt, cols;       // tiled build: tile width, its log2, column tiles per row strip
   unsigned wl_magic;        // tiled build: 2^32 / (Wt + FS - 1) + 1, for the division by the row length
   int split2;               // consumer waves split roles also above 16 ranks / 4 channel blocks
+  int spin_limit;           // polls before a wait between waves gives up
 #ifdef CP4_DEBUG_PHASES
   long long* dbg;
 #endif
+};
+
+// What a wait needs besides its word: the bound on its polls, the workgroup's
+// abort word in LDS, the device's sticky fault record and who is asking.
+struct WaitCtx {
+  int limit;       // polls before a wait gives up
+  int* abort;      // LDS: set by the first wave of the workgroup that gives up
+  int* fault;      // global, 4 ints: code, workgroup, wave, wait site (null: not recorded)
+  int wg, wave;
 };
 
 // Wait until *word >= want and return the value seen.  The writer is another
@@ -113,16 +126,33 @@ struct PipePlan {
 // the device.  With `backoff` the naps between polls grow (64, 256, then 1024
 // cycles): fewer polls between the producers' LDS traffic on long strips; on
 // the shortest strips the wake-up latency of a long nap would cost more.
-__device__ __forceinline__ int wait_ge(int* word, int want, bool backoff) {
+// A wait that runs out never lets its wave go on with unfinished data: the wave
+// records the fault for the host (first one wins; cp4_device_status reports it),
+// raises the workgroup's abort word, which ends the other waves' waits early, and
+// ends there - none of its later stores happen.  No barrier follows the
+// prologue, so a wave may end on its own.
+__device__ __forceinline__ int wait_ge(int* word, int want, bool backoff, const WaitCtx& cx,
+                                       int site) {
   int v = 0;
-  for (int it = 0; it < kSpinLimit; ++it) {
+  for (int it = 0; it < cx.limit; ++it) {
     v = __hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (v >= want) break;
+    if (v >= want) return v;
     if (!backoff || it < 6) __builtin_amdgcn_s_sleep(1);
     else if (it < 12) __builtin_amdgcn_s_sleep(4);
     else __builtin_amdgcn_s_sleep(16);
+    if ((it & 63) == 63 &&
+        __hip_atomic_load(cx.abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP))
+      break;
   }
-  return v;
+  if ((threadIdx.x & 63) == 0) {
+    __hip_atomic_store(cx.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (cx.fault && atomicCAS(cx.fault, 0, 1) == 0) {
+      cx.fault[1] = cx.wg;
+      cx.fault[2] = cx.wave;
+      cx.fault[3] = site;
+    }
+  }
+  __builtin_amdgcn_endpgm();
 }
 
 // NQ: channel splits of the producers (4: quarters, two blocks per round; 1: up to
@@ -136,7 +166,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   unsigned char* Fb = ldsb + pl.fin_off;     // Fin fragments [chunk][part][hi][r] x 16 B (CPQ == 0)
   unsigned char* Cb = ldsb + pl.cc_off;      // 3 x Cc fragment tiles
   // [0..kMaxBlk) quarters done per block (sweep order), then 4 consumer arrival
-  // counters, then the 4 contraction counters of the split-role schedule
+  // counters, then the 4 contraction counters of the split-role schedule, then
+  // the abort word
   int* flags = reinterpret_cast<int*>(ldsb + pl.flag_off);
 
   const int per = (pl.nWG + 7) >> 3;
@@ -154,6 +185,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const WaitCtx wx{pl.spin_limit, flags + kMaxBlk + 8, a.fault, t, wave};
 #ifdef CP4_DEBUG_PHASES
 #define STAMP(i) if (pl.dbg && lane == 0 && (i) < 32) { pl.dbg[((size_t)t * 16 + wave) * 32 + (i)] = wall_clock64(); }
 #if CP4_DEBUG_PHASES > 1
@@ -207,7 +239,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   constexpr bool FLDS = CPQ == 0;
   constexpr int NB = kProd / NQ;                   // blocks per producer round
   const int cpq = FLDS ? (Cin + 63) >> 6 : CPQ;    // 16-channel chunks per channel split
-  if (tid < kMaxBlk + 8) flags[tid] = 0;
+  if (tid < kMaxBlk + 16) flags[tid] = 0;
   if (FLDS) {
     for (int it = tid; it < 8 * cpq * 32; it += kThreads) {
       const int o = it >> 5, r = it & 31;          // channel octet (of the padded count), rank
@@ -368,7 +400,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           for (int v = 0; v < 16; ++v)
             dst[(8 * (v >> 2) + (v & 3)) * QA] = valid ? acc[v] : 0.f;
         } else {
-          wait_ge(bf, cq, backoff);
+          wait_ge(bf, cq, backoff, wx, 1);
           // read all, then add, then write all: one LDS round trip per half, not
           // one per element
 #pragma unroll
@@ -398,9 +430,6 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   } else {
     // =========================== consumers ==================================
     const int wc = wave - kProd;                   // 0..7: rank quad in the tap step
-#ifdef CP4_PIPE_PRIO
-    __builtin_amdgcn_s_setprio(CP4_PIPE_PRIO);
-#endif
     // Output-factor fragment of this wave's 32-channel block kb = wc (reloaded per
     // item only when there are more blocks than consumer waves): lane holds row
     // 32*kb + l32, ranks 16*c + 8*hi + e.
@@ -548,7 +577,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       {
         const int need = need_of(i);
         while (frontier <= need) {
-          wait_ge(&flags[frontier], NQ, backoff);
+          wait_ge(&flags[frontier], NQ, backoff, wx, 2);
           ++frontier;
         }
       }
@@ -784,7 +813,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           if (R > 16) load_taps(std::integral_constant<int, 1>{});
         }
         for (int i = 0; i < ngroups; ++i) {
-          if (i >= 3) wait_ge(&cdone[(i - 3) & 3], ncw * (((i - 3) >> 2) + 1), backoff);
+          if (i >= 3) wait_ge(&cdone[(i - 3) & 3], ncw * (((i - 3) >> 2) + 1), backoff, wx, 3);
           if constexpr (NTQ == 2) {
             if (R > 16) {
               taps(i, Cb + (i % 3) * kCcBuf, two);
@@ -801,7 +830,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         for (int i = 0; i < ngroups; ++i) {
           const int g = rev ? ngroups - 1 - i : i;
           const unsigned char* cb = Cb + (i % 3) * kCcBuf;
-          wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1), backoff);
+          wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1), backoff, wx, 4);
           STAMPX(4 + 4 * i)
           if (second) load_bias(wc);
           if (R <= 16) {
@@ -831,13 +860,13 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       // missing one); like the arrivals, a slot cannot run a whole cycle ahead.
       if (wc >= 4) {
         for (int i = 0; i < ngroups; ++i) {
-          if (i >= 3) wait_ge(&cdone[(i - 3) & 3], nkb * (((i - 3) >> 2) + 1), backoff);
+          if (i >= 3) wait_ge(&cdone[(i - 3) & 3], nkb * (((i - 3) >> 2) + 1), backoff, wx, 5);
           taps(i, Cb + (i % 3) * kCcBuf, one);
         }
       } else if (wc < nkb) {
         for (int i = 0; i < ngroups; ++i) {
           const int g = rev ? ngroups - 1 - i : i;
-          wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1), backoff);
+          wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1), backoff, wx, 6);
           contract_block(Cb + (i % 3) * kCcBuf, g, wc, one, true, i, slot0, no);
         }
       }
@@ -854,7 +883,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     taps(0, cb_cur, one);
     for (int i = 0; i < ngroups; ++i) {
       const int g = rev ? ngroups - 1 - i : i;
-      wait_ge(&arrivals[i & 3], kCons * ((i >> 2) + 1), backoff);
+      wait_ge(&arrivals[i & 3], kCons * ((i >> 2) + 1), backoff, wx, 7);
       STAMPX(4 + 4 * i)
       // tap step i+1 goes first when its blocks are there (keeps the stores of
       // consecutive groups close), else after this group's contraction
@@ -890,7 +919,7 @@ int round_up(int v, int m) { return (v + m - 1) / m * m; }
   const size_t a_bytes = (size_t)kRP * QA * sizeof(float);
   // above 256 input channels: pre-split factor fragments, 192 B per (padded) channel
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
-  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 8) * sizeof(int);
+  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 16) * sizeof(int);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
@@ -912,7 +941,7 @@ bool layout_tiled(const FwdArgs& a, int TH, int lgWt, PipePlan* pl) {
   const long QA = round_up((int)QLEN, 64) + 8;
   const size_t a_bytes = (size_t)kRP * QA * sizeof(float);
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
-  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 8) * sizeof(int);
+  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 16) * sizeof(int);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
@@ -932,11 +961,15 @@ bool layout_tiled(const FwdArgs& a, int TH, int lgWt, PipePlan* pl) {
 bool plan(const FwdArgs& a, PipePlan* best) {
   double best_cost = 0;
   bool found = false;
+  // a tuned tile (cp4_tune_forward) replaces the cost model
+  if (a.tune_th > 0 && a.tune_lgwt >= 6 && a.tune_lgwt <= 8)
+    return a.tune_th <= a.H && layout_tiled(a, a.tune_th, a.tune_lgwt, best);
+  const int cus = num_compute_units();
   for (int lgWt = 6; lgWt <= 8; ++lgWt)
     for (int TH = 1; TH <= a.H; ++TH) {
       PipePlan pl;
       if (!layout_tiled(a, TH, lgWt, &pl)) break;
-      const double rounds = (pl.nWG + 255) / 256;
+      const double rounds = (pl.nWG + cus - 1) / cus;
       // cells read per channel and cells written per channel, with the tiles of the
       // last column counted whole
       const double cost = rounds * ((double)(TH + a.Y - 1) * (pl.Wt + a.Y - 1) * a.Cin +
@@ -954,14 +987,13 @@ bool plan(const FwdArgs& a, PipePlan* best) {
 bool plan(const FwdArgs& a, PipePlan* best) {
   double best_cost = 0;
   bool found = false;
-#ifdef CP4_PIPE_TUNE_TH
-  // measurement builds only: strip height from the environment
-  if (const char* th = getenv("CP4_PIPE_TH")) return layout(a, atoi(th), best);
-#endif
+  // a tuned strip height (cp4_tune_forward) replaces the cost model
+  if (a.tune_th > 0) return a.tune_th <= a.H && layout(a, a.tune_th, best);
+  const int cus = num_compute_units();
   for (int TH = 1; TH <= a.H; ++TH) {
     PipePlan pl;
     if (!layout(a, TH, &pl)) break;
-    const double rounds = (pl.nWG + 255) / 256;
+    const double rounds = (pl.nWG + cus - 1) / cus;
     const double cost = rounds * ((double)(TH + a.Y - 1) * a.Cin + (double)TH * a.Cout);
     // on equal cost (1x1 filters: no halo rows) the taller strip: fewer workgroups
     if (!found || cost <= best_cost) {
@@ -1047,12 +1079,10 @@ bool fwd_pipe_supported(const FwdArgs& a) {
 hipError_t fwd_pipe_launch(const FwdArgs& a, hipStream_t st) {
   PipePlan pl;
   if (!plan(a, &pl)) return hipErrorInvalidValue;
-  pl.split2 = 1;
-#ifdef CP4_PIPE_TUNE_TH
-  if (const char* e = getenv("CP4_PIPE_SPLIT2")) pl.split2 = atoi(e);
-#endif
+  pl.split2 = a.tune_split2 != 1;               // 0: the kernel's own rule, 1: off, 2: as 0
+  pl.spin_limit = a.spin_limit > 0 ? a.spin_limit : kSpinLimit;
 #ifdef CP4_DEBUG_PHASES
-  pl.dbg = getenv("CP4_DBG_PTR") ? reinterpret_cast<long long*>(strtoull(getenv("CP4_DBG_PTR"), nullptr, 10)) : nullptr;
+  pl.dbg = debug_stamp_buffer();
 #endif
   switch (a.Y) {
     case 1: return launch_fs<1>(a, pl, st);

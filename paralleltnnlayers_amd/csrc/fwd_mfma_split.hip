@@ -28,6 +28,9 @@
 #include <cstdlib>
 
 #include "cp4_internal.h"
+#ifdef CP4_DEBUG_PHASES
+#include "cp4_debug.h"
+#endif
 
 namespace cp4 {
 namespace {
@@ -415,15 +418,16 @@ bool layout(const FwdArgs& a, int TH, SplitPlan* pl) {
   return true;
 }
 
-// Strip height: fewest rounds of 256 workgroups times the rows each strip
+// Strip height: fewest rounds of one workgroup per compute unit times the rows each strip
 // reads (with halo) and writes.
 bool plan(const FwdArgs& a, SplitPlan* best) {
   double best_cost = 0;
   bool found = false;
+  const int cus = num_compute_units();
   for (int TH = 1; TH <= a.H; ++TH) {
     SplitPlan pl;
     if (!layout(a, TH, &pl)) break;
-    const double rounds = (pl.nWG + 255) / 256;
+    const double rounds = (pl.nWG + cus - 1) / cus;
     const double cost = rounds * ((double)(TH + a.Y - 1) * a.Cin + (double)TH * a.Cout);
     if (!found || cost < best_cost) {
       best_cost = cost;
@@ -461,7 +465,7 @@ hipError_t fwd_split_launch(const FwdArgs& a, hipStream_t st) {
   SplitPlan pl;
   if (!plan(a, &pl)) return hipErrorInvalidValue;
 #ifdef CP4_DEBUG_PHASES
-  pl.dbg = getenv("CP4_DBG_PTR") ? reinterpret_cast<long long*>(strtoull(getenv("CP4_DBG_PTR"), nullptr, 10)) : nullptr;
+  pl.dbg = debug_stamp_buffer();
 #endif
   switch (a.Y) {
     case 1: return launch_fs<1>(a, pl, st);

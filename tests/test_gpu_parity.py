@@ -5,8 +5,9 @@ Tolerances (written out here as the bar for this path):
   forward / backward-data : |a-b| <= 1e-5 + 1e-4*|b| elementwise, and
                             max|a-b| <= 1e-4 * max|b| so that small-magnitude
                             outputs cannot pass vacuously;
-  backward-filter         : |a-b| <= 1e-3*|b| + 1e-4*max|b| elementwise, and
-                            max|a-b| <= 1e-3 * max|b|.
+  backward-filter         : |a-b| <= 1e-3*|b| + 1e-6*max|b| elementwise (the
+                            floor only keeps entries that cancel to ~0 from
+                            dividing by nothing), and max|a-b| <= 1e-3 * max|b|.
 """
 import os
 
@@ -50,7 +51,7 @@ def assert_activation_close(got, want, what=""):
 def assert_gradient_close(got, want, what=""):
     scale = float(np.abs(want).max())
     err = np.abs(got - want)
-    assert np.all(err <= 1e-3 * np.abs(want) + 1e-4 * scale), f"{what}: elementwise {err.max():.3e}"
+    assert np.all(err <= 1e-3 * np.abs(want) + 1e-6 * scale), f"{what}: elementwise {err.max():.3e}"
     assert err.max() <= 1e-3 * scale, f"{what}: normalised {err.max() / scale:.3e}"
 
 
