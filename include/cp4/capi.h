@@ -157,6 +157,26 @@ cp4_status cp4_conv2d_backward_filter(const cp4_shape* shape, const float* x,
                                       size_t workspace_bytes,
                                       cp4_stream stream);
 
+/* cp4_conv2d_backward_filter for callers that cannot allocate.  It has no
+ * counterpart in the reference; it is for code under HIP graph capture, tight
+ * serving loops and harnesses that forbid hipMalloc, which cannot provide the
+ * workspace above.  Same arguments without the workspace, same kernels, same
+ * results bit for bit: the planes and partial sums live in a static device array
+ * inside the library instead (CP4_NOALLOC_SCRATCH_BYTES per GPU the library runs
+ * on, held until the process ends; its address is looked up once per device on
+ * the first call there).  The call allocates and frees nothing.  Shapes whose
+ * cp4_conv2d_backward_filter_workspace_bytes exceeds the array return
+ * CP4_ERR_WORKSPACE (config C5, N64 C256 K256 14x14 R64, needs 23.6 MB and fits).
+ * All calls on one GPU share the array: calls that overlap in time on one GPU -
+ * different streams, or different host threads - race; serialise them. */
+#define CP4_NOALLOC_SCRATCH_BYTES (32u << 20)
+size_t cp4_noalloc_scratch_bytes(void);
+cp4_status cp4_conv2d_backward_filter_noalloc(const cp4_shape* shape, const float* x,
+                                              const float* dy, const float* FK,
+                                              const float* FC, const float* FH,
+                                              const float* FW, float* dFK, float* dFC,
+                                              float* dFH, float* dFW, cp4_stream stream);
+
 /* Same, with the kernel variant chosen by the caller: -1 library's choice,
  * 0 general (any shape), 1 matrix-core path (CP4_ERR_UNSUPPORTED if the shape
  * does not qualify). */

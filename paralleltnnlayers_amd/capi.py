@@ -77,6 +77,8 @@ def lib():
     bwf = [_S] + [_F] * 10 + [ctypes.c_void_p, ctypes.c_size_t]
     L.cp4_conv2d_backward_filter.argtypes = bwf + [ctypes.c_void_p]
     L.cp4_conv2d_backward_filter_variant.argtypes = bwf + [ctypes.c_int, ctypes.c_void_p]
+    L.cp4_conv2d_backward_filter_noalloc.argtypes = [_S] + [_F] * 10 + [ctypes.c_void_p]
+    L.cp4_noalloc_scratch_bytes.restype = ctypes.c_size_t
     L.cp4_conv2d_backward_filter_full.argtypes = [_S, _F, _F, _F, ctypes.c_int, ctypes.c_void_p]
     timing = [ctypes.c_uint, ctypes.c_uint, ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
     L.cp4_time_forward.argtypes = fwd + timing
@@ -271,6 +273,17 @@ def conv2d_backward_filter(x, dy, FK, FC, FH, FW, pad=1, workspace=None, stream=
         ctypes.byref(s), _ptr(x), _ptr(dy), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
         *[_ptr(o) for o in outs], ctypes.c_void_p(ws.data_ptr()), ws_bytes, variant,
         _stream(stream)))
+    return tuple(outs)
+
+
+def conv2d_backward_filter_noalloc(x, dy, FK, FC, FH, FW, outs, pad=1, stream=None):
+    """The factor gradients into the caller's `outs` = (dFK, dFC, dFH, dFW) through the
+    entry point that allocates nothing (the library's static scratch)."""
+    s = shape_for(x.shape, FK, FC, FH, FW, pad)
+    assert tuple(dy.shape) == (s.N, s.T, s.H, s.W) and x.shape[1] == s.C
+    check(lib().cp4_conv2d_backward_filter_noalloc(
+        ctypes.byref(s), _ptr(x), _ptr(dy), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
+        *[_ptr(o) for o in outs], _stream(stream)))
     return tuple(outs)
 
 

@@ -19,9 +19,18 @@ thread_local char g_err[256] = "";
 // last cp4_device_status: {nonzero, workgroup, wave, wait site}.  One copy per GPU.
 __device__ int g_device_fault[4];
 
+// Scratch of cp4_conv2d_backward_filter_noalloc: the planes and partial sums the
+// backward-filter kernels otherwise keep in the caller's workspace.  Every GPU the
+// library runs on holds its own copy, at its own address, until the process ends.
+// In host code the array's name is only a stand-in for those copies: the address
+// to hand to kernels comes from hipGetSymbolAddress (scratch_of_current_device).
+constexpr size_t kScratchBytes = (size_t)CP4_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
 constexpr int kMaxDevices = 64;
 std::mutex g_dev_mu;
 int* g_fault_ptr[kMaxDevices];
+void* g_scratch_ptr[kMaxDevices];
 int g_num_cus[kMaxDevices];
 std::atomic<int> g_spin_limit{0};
 
@@ -59,6 +68,24 @@ int* fault_of_current_device() {
     g_fault_ptr[dev] = static_cast<int*>(p);
   }
   return g_fault_ptr[dev];
+}
+
+// Address of the current device's copy of `scratch`: looked up once per device,
+// with that device current, and kept.
+cp4_status scratch_of_current_device(void** out) {
+  int dev = -1;
+  CP4_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(CP4_ERR_UNSUPPORTED, "device ordinal beyond the library's table");
+  std::lock_guard<std::mutex> lk(g_dev_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    CP4_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(CP4_ERR_HIP, "hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return CP4_OK;
 }
 
 // The launch context every producer / consumer launch carries.
@@ -539,6 +566,33 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
   if (variant == 1 || (variant < 0 && mfma_ok)) CP4_HIP(cp4::bwd_filter_mfma_launch(a, st));
   else CP4_HIP(cp4::bwd_filter_launch(a, st));
   return CP4_OK;
+}
+
+size_t cp4_noalloc_scratch_bytes(void) { return kScratchBytes; }
+
+cp4_status cp4_conv2d_backward_filter_noalloc(const cp4_shape* shape, const float* x,
+                                              const float* dy, const float* FK,
+                                              const float* FC, const float* FH,
+                                              const float* FW, float* dFK, float* dFC,
+                                              float* dFH, float* dFW, cp4_stream stream) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  const size_t need = shape->N ? filter_workspace(*shape) : 0;
+  if (need > kScratchBytes) {
+    std::snprintf(g_err, sizeof(g_err),
+                  "this shape needs %zu bytes of scratch, the library's static scratch holds "
+                  "%zu: use cp4_conv2d_backward_filter with a workspace",
+                  need, kScratchBytes);
+    return CP4_ERR_WORKSPACE;
+  }
+  void* ws = nullptr;
+  rc = scratch_of_current_device(&ws);
+  if (rc != CP4_OK) return rc;
+  // The kernels write every scratch word before they read it (planes, then
+  // per-workgroup partial sums, then the fixed-order reduce), so nothing has to be
+  // cleared between calls; two calls in flight on one GPU would share the array.
+  return cp4_conv2d_backward_filter_variant(shape, x, dy, FK, FC, FH, FW, dFK, dFC, dFH, dFW,
+                                            ws, kScratchBytes, -1, stream);
 }
 
 int cp4_bf16_backward_filter_supported(const cp4_shape* shape) {
