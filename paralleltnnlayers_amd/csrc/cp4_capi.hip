@@ -184,6 +184,7 @@ hipError_t fwd_pipe2_launch(const FwdArgs& a, hipStream_t st) {
 // Order = preference of the untuned heuristic, last to first.
 const Variant kVariants[] = {
     {"general_valu", cp4::fwd_general_supported, cp4::fwd_general_launch},
+    {"dense_small_valu", cp4::fwd_dense_small_supported, cp4::fwd_dense_small_launch},
     {"mfma_f32_strip", cp4::fwd_mfma_supported, cp4::fwd_mfma_launch},
     {"mfma_bf16x3_strip", cp4::fwd_split_supported, cp4::fwd_split_launch},
     {"mfma_bf16x3_pipe_tiled", cp4::fwd_pipe_tiled_supported, cp4::fwd_pipe_tiled_launch},
@@ -226,9 +227,29 @@ bool is_variant(int v, const char* name) { return v >= 0 && !strcmp(kVariants[v]
 // kernel is then the faster one where it applies (even widths).
 constexpr long kPipeLdsFactorMaxPixels = 8192;
 constexpr int kPipeRegisterFactorMaxCin = 256;
-// Fewer channels than this on both sides together leave the 32 x 32 matrix tiles
-// almost empty: the VALU kernels, whose cost follows the real channel counts, win.
+// Fewer channels than this on both sides together and a rank of one or two leave
+// the 32 x 32 matrix tiles almost empty: the general VALU kernel, whose cost
+// follows the real counts, wins (N1 C3 K128 512x512 R1: 28 against 31 us; at rank
+// 16 the matrix-core kernels win at every channel count: N1 C3 K16 512x512 27
+// against 36 us, N8 C8 K8 256x256 47 against 73 us).
 constexpr int kMatrixMinChannels = 24;
+constexpr int kMatrixMinRank = 2;
+// The recomposed-filter kernel against the kernel that would run otherwise:
+// estimated microseconds per 2^18 pixels, fitted to measurements on MI355X.
+// Recomposed: bound by its LDS segment reads (Cin * FS * (FS + 3) / 4 per pixel)
+// more than by its Cout * Cin * FS^2 multiply-adds.  Matrix-core kernels: about
+// 18 us whatever the (small) channel counts.  General VALU kernel: grows with the
+// factored order's R * (Cin + Cout + Y + X).  (N1 512x512 3x3 R16: C16 K1 14
+// against 25 us matrix-core, C128 K1 107 against 43; 17x17 C3 K1: 24 against 240
+// us general at R16, 22 against 13 at R1.)
+double dense_small_estimate(const FwdArgs& a) {
+  return 8.0 + 0.155 * a.Cin * a.Y * (a.X + 3) / 4.0 + 0.0025 * a.Cout * a.Cin * a.Y * a.X;
+}
+constexpr double kMatrixSmallChannelEstimate = 26.0;
+double general_estimate(const FwdArgs& a) {
+  return 10.0 + 0.3 * a.R * (a.Cin + a.Cout + a.Y + a.X);
+}
+
 // Rows longer than this leave whole-row strips only a row or two (2 at W = 224):
 // tiles of TH x Wt pay less for their halo.
 constexpr int kWholeRowMaxWidth = 128;
@@ -245,7 +266,7 @@ int heuristic_variant(const FwdArgs& a) {
   }
   int pick = -1;
   for (int v = kNumVariants - 1; v >= 0 && pick < 0; --v)
-    if (kVariants[v].supported(a)) pick = v;
+    if (kVariants[v].supported(a) && !is_variant(v, "dense_small_valu")) pick = v;
   auto prefer = [&](const char* name) {
     const int v = variant_named(name);
     if (v >= 0 && kVariants[v].supported(a)) pick = v;
@@ -254,15 +275,20 @@ int heuristic_variant(const FwdArgs& a) {
       (long)a.N * a.H * a.W > kPipeLdsFactorMaxPixels)
     prefer("mfma_bf16x3_strip");
   if (pick >= 0 && !strncmp(kVariants[pick].name, "mfma_bf16x3_pipe", 16) &&
-      a.Cin + a.Cout < kMatrixMinChannels) {
+      a.Cin + a.Cout < kMatrixMinChannels && a.R <= kMatrixMinRank)
     prefer("general_valu");
-    prefer("valu_rows");
-  }
   if (is_variant(pick, "mfma_bf16x3_pipe") && a.W > kWholeRowMaxWidth)
     prefer("mfma_bf16x3_pipe_tiled");
   if (is_variant(pick, "mfma_bf16x3_pipe_2pass") &&
       (long)a.N * a.H * a.W * (a.Cin + a.Cout) < kTwoPassMinElements)
     prefer("mfma_f32_strip");
+  // A handful of channels on both sides: the recomposed filter costs fewer
+  // multiply-adds per pixel than the factor-by-factor order.
+  if (cp4::fwd_dense_small_supported(a)) {
+    const bool matrix = pick >= 0 && !strncmp(kVariants[pick].name, "mfma_", 5);
+    if (dense_small_estimate(a) <= (matrix ? kMatrixSmallChannelEstimate : general_estimate(a)))
+      prefer("dense_small_valu");
+  }
   return pick;
 }
 

@@ -60,6 +60,9 @@ inline bool fits_int_indexing(int N, int H, int W) {
 
 bool fwd_general_supported(const FwdArgs&);
 hipError_t fwd_general_launch(const FwdArgs&, hipStream_t);
+// Recomposed-filter direct convolution for very few channels on both sides.
+bool fwd_dense_small_supported(const FwdArgs&);
+hipError_t fwd_dense_small_launch(const FwdArgs&, hipStream_t);
 bool fwd_mfma_supported(const FwdArgs&);
 hipError_t fwd_mfma_launch(const FwdArgs&, hipStream_t);
 bool fwd_split_supported(const FwdArgs&);

@@ -41,7 +41,8 @@ __global__ __launch_bounds__(kThreads) void fwd_general_kernel(FwdArgs a) {
       for (int rr = 0; rr < RB; ++rr) acc[rr] = 0.f;
       if (gh >= 0 && gh < a.H && gw >= 0 && gw < a.W) {
         const float* xp = xn + (size_t)gh * a.W + gw;
-        for (int c = 0; c < a.Cin; ++c) {
+#pragma unroll 4
+        for (int c = 0; c < a.Cin; ++c) {     // (unrolled: the scalar factor loads of four channels overlap)
           const float v = xp[c * HW];
           const float* f = a.Fin + (size_t)c * R + r0;
 #pragma unroll
@@ -82,7 +83,8 @@ __global__ __launch_bounds__(kThreads) void fwd_general_kernel(FwdArgs a) {
     // 4. rank -> output-channel contraction
     if (h0 + h < a.H && w0 + w < a.W) {
       float* yp = a.y + (size_t)n * a.Cout * HW + (size_t)(h0 + h) * a.W + w0 + w;
-      for (int k = 0; k < a.Cout; ++k) {
+#pragma unroll 4
+      for (int k = 0; k < a.Cout; ++k) {      // (unrolled: four rows of the factor in flight)
         const float* f = a.Fout + (size_t)k * R + r0;
         float s = 0.f;
 #pragma unroll
@@ -100,11 +102,17 @@ size_t lds_floats(const FwdArgs& a, int rb) {
   const size_t HT = kTH + a.Y - 1, WT = kTW + a.X - 1;
   return (size_t)rb * (HT * WT + kTH * WT);
 }
-constexpr size_t kLdsBudget = 64 * 1024;
+// More LDS per workgroup costs occupancy, a second rank block re-reads and
+// re-writes y: with many output channels the second costs more (N1 C3 K96
+// 224x224 11x11 R16: 80 us in one block of 70 KB, 99 us in two), with few the
+// first (N1 C3 K1 512x512 17x17 R16: 239 against 126 us).
+constexpr size_t kLdsBudget = 64 * 1024, kLdsBudgetManyOutputs = 96 * 1024;
+constexpr int kManyOutputs = 32;
 
 int pick_rank_block(const FwdArgs& a) {
+  const size_t budget = a.Cout >= kManyOutputs ? kLdsBudgetManyOutputs : kLdsBudget;
   int rb = 32;
-  while (rb > 1 && (rb / 2 >= a.R || lds_floats(a, rb) * 4 > kLdsBudget)) rb /= 2;
+  while (rb > 1 && (rb / 2 >= a.R || lds_floats(a, rb) * 4 > budget)) rb /= 2;
   return rb;
 }
 
@@ -115,19 +123,27 @@ bool fwd_general_supported(const FwdArgs& a) {
          (a.H + kTH - 1) / kTH <= 65535;
 }
 
+template <int RB>
+hipError_t launch_rb(const FwdArgs& a, size_t smem, hipStream_t s) {
+  const void* fn = reinterpret_cast<const void*>(fwd_general_kernel<RB>);
+  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  if (e != hipSuccess) return e;
+  const dim3 grid((a.W + kTW - 1) / kTW, (a.H + kTH - 1) / kTH, a.N);
+  fwd_general_kernel<RB><<<grid, kThreads, smem, s>>>(a);
+  return hipGetLastError();
+}
+
 hipError_t fwd_general_launch(const FwdArgs& a, hipStream_t s) {
   const int rb = pick_rank_block(a);
-  const dim3 grid((a.W + kTW - 1) / kTW, (a.H + kTH - 1) / kTH, a.N);
   const size_t smem = lds_floats(a, rb) * sizeof(float);
   switch (rb) {
-    case 32: fwd_general_kernel<32><<<grid, kThreads, smem, s>>>(a); break;
-    case 16: fwd_general_kernel<16><<<grid, kThreads, smem, s>>>(a); break;
-    case 8: fwd_general_kernel<8><<<grid, kThreads, smem, s>>>(a); break;
-    case 4: fwd_general_kernel<4><<<grid, kThreads, smem, s>>>(a); break;
-    case 2: fwd_general_kernel<2><<<grid, kThreads, smem, s>>>(a); break;
-    default: fwd_general_kernel<1><<<grid, kThreads, smem, s>>>(a); break;
+    case 32: return launch_rb<32>(a, smem, s);
+    case 16: return launch_rb<16>(a, smem, s);
+    case 8: return launch_rb<8>(a, smem, s);
+    case 4: return launch_rb<4>(a, smem, s);
+    case 2: return launch_rb<2>(a, smem, s);
+    default: return launch_rb<1>(a, smem, s);
   }
-  return hipGetLastError();
 }
 
 }  // namespace cp4
