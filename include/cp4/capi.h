@@ -196,6 +196,57 @@ cp4_status cp4_conv2d_backward_filter_full(const cp4_shape* shape,
                                            float* dK, int accumulate,
                                            cp4_stream stream);
 
+/* ---- layer geometry: stride, explicit padding, an output plane of its own ---
+ * The reference's kernels are stride 1 with an H x W output; its layer library
+ * passes strides and padding = "SAME" / "VALID" on to the framework's convolutions
+ * (test/layers.py:264-279).  With a cp4_geometry the operator is
+ *   y[n,t,ho,wo] = sum_{c,r} FK[t,r] FC[c,r] sum_{i,j} FH[i,r] FW[j,r]
+ *                  x[n,c, stride_h*ho + i - pad_top, stride_w*wo + j - pad_left]
+ * on an out_h x out_w output plane; reads outside the image are zero (so the
+ * padding after the image is implied by the output size).  shape->pad is not
+ * used by the _ex entry points; shape->H, W describe x.  Limits: strides >= 1,
+ * pad_top <= Y - 1, pad_left <= X - 1, every output window overlapping the padded
+ * image (stride*(out-1) - pad < image size).  cp4_geometry_same / _valid /
+ * _symmetric fill in the three usual cases: the framework's "SAME" (out =
+ * ceil(in / stride), the smaller half of the zeros before the image - on even
+ * sizes not the symmetric padding of a PyTorch layer), "VALID" (no zeros) and
+ * `pad` zeros on every side (out = (in + 2 pad - filter) / stride + 1). */
+typedef struct cp4_geometry {
+  unsigned stride_h, stride_w, pad_top, pad_left, out_h, out_w;
+} cp4_geometry;
+cp4_status cp4_geometry_same(const cp4_shape* shape, unsigned stride_h, unsigned stride_w,
+                             cp4_geometry* g);
+cp4_status cp4_geometry_valid(const cp4_shape* shape, unsigned stride_h, unsigned stride_w,
+                              cp4_geometry* g);
+cp4_status cp4_geometry_symmetric(const cp4_shape* shape, unsigned stride_h, unsigned stride_w,
+                                  unsigned pad_h, unsigned pad_w, cp4_geometry* g);
+/* Forward x[N,C,H,W] -> y[N,T,out_h,out_w] = act(conv + bias) (bias [T] or NULL,
+ * activation a cp4_activation).  Only the kept outputs are filtered, contracted
+ * and stored: the producer / consumer kernel's strided build (square 1/3/5/7
+ * filters, Rank <= 32), else the general kernel. */
+cp4_status cp4_conv2d_forward_ex(const cp4_shape* shape, const cp4_geometry* g, const float* x,
+                                 const float* FK, const float* FC, const float* FH,
+                                 const float* FW, const float* bias, int activation, float* y,
+                                 cp4_stream stream);
+/* The two gradients of that map: dx[N,C,H,W] (the exact adjoint, whatever the
+ * padding) from dy[N,T,out_h,out_w], and the four factor gradients.  Both first
+ * spread dy out with zeros to stride 1 in `workspace` (device memory of at least
+ * cp4_conv2d_backward_ex_workspace_bytes, which also covers the factor pass's own
+ * planes) and then run the stride-1 kernels, so their cost is that of the
+ * stride-1 layer. */
+size_t cp4_conv2d_backward_ex_workspace_bytes(const cp4_shape* shape, const cp4_geometry* g);
+cp4_status cp4_conv2d_backward_data_ex(const cp4_shape* shape, const cp4_geometry* g,
+                                       const float* dy, const float* FK, const float* FC,
+                                       const float* FH, const float* FW, float* dx,
+                                       void* workspace, size_t workspace_bytes,
+                                       cp4_stream stream);
+cp4_status cp4_conv2d_backward_filter_ex(const cp4_shape* shape, const cp4_geometry* g,
+                                         const float* x, const float* dy, const float* FK,
+                                         const float* FC, const float* FH, const float* FW,
+                                         float* dFK, float* dFC, float* dFH, float* dFW,
+                                         void* workspace, size_t workspace_bytes,
+                                         cp4_stream stream);
+
 /* ---- timed launches: the reference's PROFCOUNT loop ---------------------- */
 
 /* Replace the event-timed loops of cp4Conv2dForward.cu:245-327 and

@@ -250,6 +250,207 @@ void cp4o_backward_filter_factor_direct(const cp4o_shape* s, int which,
     }
 }
 
+/* ------------------------------------------------------------------------ */
+/* (1b) layer geometry: stride and an output plane of its own                 */
+/* ------------------------------------------------------------------------ */
+
+/* The reference's kernels are stride 1 with an H x W output; its Python layer
+ * passes strides and padding = "SAME" / "VALID" to the framework's convolutions
+ * (test/layers.py:264-279).  With stride (sh, sw), pad_top / pad_left zero rows /
+ * columns before the image and an out_h x out_w output plane the operator is
+ *   Out[n,t,ho,wo] = sum_{c,r} FK[t,r] FC[c,r] sum_{y,x} FH[y,r] FW[x,r]
+ *                    In[n,c, sh*ho + y - pad_top, sw*wo + x - pad_left]
+ * (reads outside the image are zero), the forward formula of
+ * cp4Conv2dForward.cu:84-133 with the anchor sh*ho, sw*wo in place of h, w.
+ * s->pad is not used by the functions of this section.  Pinned in
+ * tests/test_oracle.py against torch float64 conv2d(stride, padding) and its
+ * autograd on the recomposed kernel (tests/golden/make_golden.py). */
+typedef struct cp4o_geometry {
+  unsigned stride_h, stride_w, pad_top, pad_left, out_h, out_w;
+} cp4o_geometry;
+
+void cp4o_forward_geom_direct(const cp4o_shape* s, const cp4o_geometry* g, const float* In,
+                              const float* FK, const float* FC, const float* FH,
+                              const float* FW, float* Out) {
+  const long N = s->N, H = s->H, W = s->W, T = s->T, C = s->C, Y = s->Y, X = s->X, R = s->Rank;
+  const long SH = g->stride_h, SW = g->stride_w, PT = g->pad_top, PL = g->pad_left,
+             HO = g->out_h, WO = g->out_w;
+#pragma omp parallel for collapse(2) schedule(dynamic)
+  for (long n = 0; n < N; ++n)
+    for (long t = 0; t < T; ++t)
+      for (long ho = 0; ho < HO; ++ho)
+        for (long wo = 0; wo < WO; ++wo) {
+          double acc = 0.0;
+          for (long r = 0; r < R; ++r) {
+            double cacc = 0.0;
+            for (long c = 0; c < C; ++c) {
+              const float* ip = In + (n * C + c) * H * W;
+              double pix = 0.0;
+              for (long y = 0; y < Y; ++y)
+                for (long x = 0; x < X; ++x)
+                  pix += rd(ip, SH * ho + y - PT, SW * wo + x - PL, H, W) *
+                         (double)FH[y * R + r] * (double)FW[x * R + r];
+              cacc += pix * (double)FC[c * R + r];
+            }
+            acc += cacc * (double)FK[t * R + r];
+          }
+          Out[((n * T + t) * HO + ho) * WO + wo] = (float)acc;
+        }
+}
+
+/* The adjoint of the map above in In: dX[n,c,h,w] = sum over every (t, ho, wo, y, x)
+ * with sh*ho + y - pad_top = h and sw*wo + x - pad_left = w of
+ * dY[n,t,ho,wo] K[t,c,y,x].  For stride 1, out = H x W and 2*pad = Y - 1 this is
+ * cp4Conv2dBackwardData.cu:57-108. */
+void cp4o_backward_data_geom_direct(const cp4o_shape* s, const cp4o_geometry* g,
+                                    const float* dY, const float* FK, const float* FC,
+                                    const float* FH, const float* FW, float* dX) {
+  const long N = s->N, H = s->H, W = s->W, T = s->T, C = s->C, Y = s->Y, X = s->X, R = s->Rank;
+  const long SH = g->stride_h, SW = g->stride_w, PT = g->pad_top, PL = g->pad_left,
+             HO = g->out_h, WO = g->out_w;
+#pragma omp parallel for collapse(2) schedule(dynamic)
+  for (long n = 0; n < N; ++n)
+    for (long c = 0; c < C; ++c)
+      for (long h = 0; h < H; ++h)
+        for (long w = 0; w < W; ++w) {
+          double acc = 0.0;
+          for (long r = 0; r < R; ++r) {
+            double tacc = 0.0;
+            for (long t = 0; t < T; ++t) {
+              const float* gp = dY + (n * T + t) * HO * WO;
+              double pix = 0.0;
+              for (long y = 0; y < Y; ++y) {
+                const long hn = h + PT - y;
+                if (hn < 0 || hn % SH) continue;
+                for (long x = 0; x < X; ++x) {
+                  const long wn = w + PL - x;
+                  if (wn < 0 || wn % SW) continue;
+                  pix += rd(gp, hn / SH, wn / SW, HO, WO) * (double)FH[y * R + r] *
+                         (double)FW[x * R + r];
+                }
+              }
+              tacc += pix * (double)FK[t * R + r];
+            }
+            acc += tacc * (double)FC[c * R + r];
+          }
+          dX[((n * C + c) * H + h) * W + w] = (float)acc;
+        }
+}
+
+/* The factor gradients of the map above, the 8-deep sums of
+ * cp4Conv2dBackwardFilter.cu:64-257 with the strided anchor; `which` and the
+ * += convention as in cp4o_backward_filter_factor_direct. */
+void cp4o_backward_filter_geom_direct(const cp4o_shape* s, const cp4o_geometry* g, int which,
+                                      float* dF, const float* In, const float* dY,
+                                      const float* FK, const float* FC, const float* FH,
+                                      const float* FW) {
+  const long N = s->N, H = s->H, W = s->W, T = s->T, C = s->C, Y = s->Y, X = s->X, R = s->Rank;
+  const long SH = g->stride_h, SW = g->stride_w, PT = g->pad_top, PL = g->pad_left,
+             HO = g->out_h, WO = g->out_w;
+  const long D = which == 0 ? T : which == 1 ? C : which == 2 ? Y : X;
+#pragma omp parallel for collapse(2) schedule(dynamic)
+  for (long d = 0; d < D; ++d)
+    for (long r = 0; r < R; ++r) {
+      double acc = 0.0;
+      for (long n = 0; n < N; ++n)
+        for (long t = 0; t < T; ++t) {
+          if (which == 0 && t != d) continue;
+          for (long c = 0; c < C; ++c) {
+            if (which == 1 && c != d) continue;
+            const float* ip = In + (n * C + c) * H * W;
+            const float* gp = dY + (n * T + t) * HO * WO;
+            for (long y = 0; y < Y; ++y) {
+              if (which == 2 && y != d) continue;
+              for (long x = 0; x < X; ++x) {
+                if (which == 3 && x != d) continue;
+                double f = 1.0;
+                if (which != 0) f *= (double)FK[t * R + r];
+                if (which != 1) f *= (double)FC[c * R + r];
+                if (which != 2) f *= (double)FH[y * R + r];
+                if (which != 3) f *= (double)FW[x * R + r];
+                double sum = 0.0;
+                for (long ho = 0; ho < HO; ++ho)
+                  for (long wo = 0; wo < WO; ++wo)
+                    sum += (double)gp[ho * WO + wo] *
+                           rd(ip, SH * ho + y - PT, SW * wo + x - PL, H, W);
+                acc += sum * f;
+              }
+            }
+          }
+        }
+      dF[d * R + r] += (float)acc;
+    }
+}
+
+/* The forward map above, factor by factor (1x1 by FC, strided depthwise 1-D by FH,
+ * strided depthwise 1-D by FW, 1x1 by FK): what full-size results are compared
+ * with.  Checked against cp4o_forward_geom_direct in tests/test_oracle.py. */
+int cp4o_forward_geom_unfused(const cp4o_shape* s, const cp4o_geometry* g, const float* In,
+                              const float* FK, const float* FC, const float* FH,
+                              const float* FW, float* Out) {
+  const long N = s->N, H = s->H, W = s->W, T = s->T, C = s->C, Y = s->Y, X = s->X, R = s->Rank;
+  const long SH = g->stride_h, SW = g->stride_w, PT = g->pad_top, PL = g->pad_left,
+             HO = g->out_h, WO = g->out_w, HW = H * W;
+  int fail = 0;
+#pragma omp parallel
+  {
+    float* a = (float*)malloc(sizeof(float) * (size_t)(R * HW));
+    float* b = (float*)malloc(sizeof(float) * (size_t)(R * HO * W));
+    float* cc = (float*)malloc(sizeof(float) * (size_t)(R * HO * WO));
+    if (!a || !b || !cc) {
+#pragma omp atomic write
+      fail = 1;
+    }
+#pragma omp for schedule(dynamic)
+    for (long n = 0; n < N; ++n) {
+      if (!a || !b || !cc) continue;
+      const float* xn = In + n * C * HW;
+      for (long r = 0; r < R; ++r) {
+        float* ar = a + r * HW;
+        for (long p = 0; p < HW; ++p) ar[p] = 0.f;
+        for (long c = 0; c < C; ++c) {
+          const float f = FC[c * R + r];
+          const float* xp = xn + c * HW;
+          for (long p = 0; p < HW; ++p) ar[p] += f * xp[p];
+        }
+        float* br = b + r * HO * W;
+        for (long ho = 0; ho < HO; ++ho)
+          for (long w = 0; w < W; ++w) {
+            float v = 0.f;
+            for (long y = 0; y < Y; ++y) {
+              const long h = SH * ho + y - PT;
+              if (h >= 0 && h < H) v += FH[y * R + r] * ar[h * W + w];
+            }
+            br[ho * W + w] = v;
+          }
+        float* cr = cc + r * HO * WO;
+        for (long ho = 0; ho < HO; ++ho)
+          for (long wo = 0; wo < WO; ++wo) {
+            float v = 0.f;
+            for (long x = 0; x < X; ++x) {
+              const long w = SW * wo + x - PL;
+              if (w >= 0 && w < W) v += FW[x * R + r] * br[ho * W + w];
+            }
+            cr[ho * WO + wo] = v;
+          }
+      }
+      for (long t = 0; t < T; ++t) {
+        float* op = Out + (n * T + t) * HO * WO;
+        for (long p = 0; p < HO * WO; ++p) op[p] = 0.f;
+        for (long r = 0; r < R; ++r) {
+          const float f = FK[t * R + r];
+          const float* cr = cc + r * HO * WO;
+          for (long p = 0; p < HO * WO; ++p) op[p] += f * cr[p];
+        }
+      }
+    }
+    free(a);
+    free(b);
+    free(cc);
+  }
+  return fail;
+}
+
 /* Number of elements whose symmetric relative error exceeds tol; absolute
  * error when either value is zero (Utils.cu:143-156). */
 long cp4o_count_exceeding(const float* A, const float* B, size_t n, float tol) {

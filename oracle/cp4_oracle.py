@@ -125,6 +125,69 @@ def backward_filter(x, dy, FK, FC, FH, FW, pad, direct=False):
     return tuple(outs)
 
 
+class Geometry(ctypes.Structure):
+    """stride, zero rows / columns before the image, output plane (cp4o_geometry)."""
+    _fields_ = [(k, ctypes.c_uint) for k in
+                ("stride_h", "stride_w", "pad_top", "pad_left", "out_h", "out_w")]
+
+
+def geometry_same(H, W, Y, X, stride):
+    """The framework's padding="SAME" that the reference's layers ask for
+    (test/layers.py:264-279): out = ceil(in / stride); as many zeros as the last
+    window needs, the smaller half of them before the image."""
+    sh, sw = (stride, stride) if isinstance(stride, int) else stride
+    ho, wo = -(-H // sh), -(-W // sw)
+    th, tw = max((ho - 1) * sh + Y - H, 0), max((wo - 1) * sw + X - W, 0)
+    return Geometry(sh, sw, th // 2, tw // 2, ho, wo)
+
+
+def geometry_valid(H, W, Y, X, stride):
+    sh, sw = (stride, stride) if isinstance(stride, int) else stride
+    return Geometry(sh, sw, 0, 0, (H - Y) // sh + 1, (W - X) // sw + 1)
+
+
+def geometry_symmetric(H, W, Y, X, stride, pad):
+    """pad zeros on every side: out = (in + 2 pad - filter) / stride + 1."""
+    sh, sw = (stride, stride) if isinstance(stride, int) else stride
+    return Geometry(sh, sw, pad, pad, (H + 2 * pad - Y) // sh + 1, (W + 2 * pad - X) // sw + 1)
+
+
+def forward_geom(x, FK, FC, FH, FW, g, direct=False):
+    x, FK, FC, FH, FW = map(_f32, (x, FK, FC, FH, FW))
+    s = shape_of(x.shape, FK, FC, FH, FW, 0)
+    y = np.empty((s.N, s.T, g.out_h, g.out_w), np.float32)
+    fn = lib().cp4o_forward_geom_direct if direct else lib().cp4o_forward_geom_unfused
+    rc = fn(ctypes.byref(s), ctypes.byref(g), _fp(x), _fp(FK), _fp(FC), _fp(FH), _fp(FW), _fp(y))
+    assert direct or rc == 0
+    return y
+
+
+def backward_data_geom(dy, x_hw, FK, FC, FH, FW, g):
+    """dx [N,C,H,W] of the strided map for dy [N,T,out_h,out_w]; x_hw = (H, W)."""
+    dy, FK, FC, FH, FW = map(_f32, (dy, FK, FC, FH, FW))
+    N, T = dy.shape[:2]
+    assert dy.shape[2:] == (g.out_h, g.out_w)
+    s = Shape(N=N, H=x_hw[0], W=x_hw[1], pad=0, T=T, C=FC.shape[0], Y=FH.shape[0],
+              X=FW.shape[0], Rank=FK.shape[1])
+    dx = np.empty((N, s.C, s.H, s.W), np.float32)
+    lib().cp4o_backward_data_geom_direct(ctypes.byref(s), ctypes.byref(g), _fp(dy), _fp(FK),
+                                         _fp(FC), _fp(FH), _fp(FW), _fp(dx))
+    return dx
+
+
+def backward_filter_geom(x, dy, FK, FC, FH, FW, g):
+    """(dFK, dFC, dFH, dFW) of the strided map."""
+    x, dy, FK, FC, FH, FW = map(_f32, (x, dy, FK, FC, FH, FW))
+    s = shape_of(x.shape, FK, FC, FH, FW, 0)
+    assert dy.shape == (s.N, s.T, g.out_h, g.out_w)
+    outs = [np.zeros_like(f) for f in (FK, FC, FH, FW)]
+    for which, o in enumerate(outs):
+        lib().cp4o_backward_filter_geom_direct(
+            ctypes.byref(s), ctypes.byref(g), ctypes.c_int(which), _fp(o), _fp(x), _fp(dy),
+            _fp(FK), _fp(FC), _fp(FH), _fp(FW))
+    return tuple(outs)
+
+
 def backward_filter_full(x, dy, Y, X, pad):
     """Dense filter gradient dK[T,C,Y,X] (cp4Conv2dBackwardFilter.cu:23-59)."""
     x, dy = _f32(x), _f32(dy)

@@ -29,6 +29,15 @@ class Shape(ctypes.Structure):
         return "Shape(" + ", ".join(f"{k}={getattr(self, k)}" for k, _ in self._fields_) + ")"
 
 
+class Geometry(ctypes.Structure):
+    """cp4_geometry: stride, zero rows / columns before the image, output plane."""
+    _fields_ = [(k, ctypes.c_uint) for k in
+                ("stride_h", "stride_w", "pad_top", "pad_left", "out_h", "out_w")]
+
+    def __repr__(self):
+        return "Geometry(" + ", ".join(f"{k}={getattr(self, k)}" for k, _ in self._fields_) + ")"
+
+
 # status codes of cp4_status
 (OK, ERR_NULL_POINTER, ERR_SHAPE, ERR_HIP, ERR_WORKSPACE, ERR_UNSUPPORTED,
  ERR_DEVICE) = range(7)
@@ -65,6 +74,17 @@ def lib():
     L.cp4_conv2d_backward_data.argtypes = fwd + [ctypes.c_void_p]
     L.cp4_conv2d_forward_bias_act.argtypes = [_S, _F, _F, _F, _F, _F, _F, ctypes.c_int, _F,
                                               ctypes.c_void_p]
+    _G = ctypes.POINTER(Geometry)
+    L.cp4_geometry_same.argtypes = [_S, ctypes.c_uint, ctypes.c_uint, _G]
+    L.cp4_geometry_valid.argtypes = [_S, ctypes.c_uint, ctypes.c_uint, _G]
+    L.cp4_geometry_symmetric.argtypes = [_S] + [ctypes.c_uint] * 4 + [_G]
+    L.cp4_conv2d_forward_ex.argtypes = [_S, _G] + [_F] * 6 + [ctypes.c_int, _F, ctypes.c_void_p]
+    L.cp4_conv2d_backward_ex_workspace_bytes.restype = ctypes.c_size_t
+    L.cp4_conv2d_backward_ex_workspace_bytes.argtypes = [_S, _G]
+    L.cp4_conv2d_backward_data_ex.argtypes = [_S, _G] + [_F] * 6 + [ctypes.c_void_p, ctypes.c_size_t,
+                                                                    ctypes.c_void_p]
+    L.cp4_conv2d_backward_filter_ex.argtypes = [_S, _G] + [_F] * 10 + [ctypes.c_void_p,
+                                                                       ctypes.c_size_t, ctypes.c_void_p]
     L.cp4_bf16_supported.argtypes = [_S, ctypes.c_int]
     L.cp4_conv2d_forward_bf16.argtypes = [_S, ctypes.c_void_p, _F, _F, _F, _F, _F, ctypes.c_int,
                                           ctypes.c_void_p, ctypes.c_void_p]
@@ -185,6 +205,75 @@ def conv2d_forward_bias_act(x, FK, FC, FH, FW, bias=None, activation=None, pad=1
         _ptr(bias) if bias is not None else None, ACTIVATIONS[activation], _ptr(y),
         _stream(stream)))
     return y
+
+
+def geometry(s, stride=1, padding="same"):
+    """cp4_geometry of a layer on shape `s`: padding "same" (the framework's rule the
+    reference's layers use, test/layers.py:264-279), "valid", an int or an (h, w)
+    pair of zeros on every side."""
+    sh, sw = (stride, stride) if isinstance(stride, int) else stride
+    g = Geometry()
+    if padding == "same":
+        check(lib().cp4_geometry_same(ctypes.byref(s), sh, sw, ctypes.byref(g)))
+    elif padding == "valid":
+        check(lib().cp4_geometry_valid(ctypes.byref(s), sh, sw, ctypes.byref(g)))
+    else:
+        ph, pw = (padding, padding) if isinstance(padding, int) else padding
+        check(lib().cp4_geometry_symmetric(ctypes.byref(s), sh, sw, ph, pw, ctypes.byref(g)))
+    return g
+
+
+def conv2d_forward_ex(x, FK, FC, FH, FW, g, bias=None, activation=None, out=None, stream=None):
+    """Forward with a stride / explicit padding / an output plane of its own."""
+    s = shape_for(x.shape, FK, FC, FH, FW, 0)
+    assert x.shape[1] == s.C and FC.shape[1] == s.Rank
+    y = out if out is not None else torch.empty((s.N, s.T, g.out_h, g.out_w), device=x.device,
+                                                dtype=torch.float32)
+    check(lib().cp4_conv2d_forward_ex(
+        ctypes.byref(s), ctypes.byref(g), _ptr(x), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
+        _ptr(bias) if bias is not None else None, ACTIVATIONS[activation], _ptr(y),
+        _stream(stream)))
+    return y
+
+
+def backward_ex_workspace_bytes(s, g):
+    return int(lib().cp4_conv2d_backward_ex_workspace_bytes(ctypes.byref(s), ctypes.byref(g)))
+
+
+def _ex_workspace(s, g, device, workspace):
+    need = backward_ex_workspace_bytes(s, g)
+    if workspace is None:
+        workspace = torch.empty(need + 256, device=device, dtype=torch.uint8)
+        off = (-workspace.data_ptr()) % 256
+        workspace = workspace[off:off + need]
+    return workspace, workspace.numel() * workspace.element_size()
+
+
+def conv2d_backward_data_ex(dy, x_hw, FK, FC, FH, FW, g, out=None, workspace=None, stream=None):
+    """dx [N,C,H,W] of the layer with geometry g for dy [N,T,out_h,out_w]; x_hw = (H, W)."""
+    N, T = dy.shape[:2]
+    assert tuple(dy.shape[2:]) == (g.out_h, g.out_w) and FK.shape[0] == T
+    s = Shape(N=N, H=x_hw[0], W=x_hw[1], pad=0, T=T, C=FC.shape[0], Y=FH.shape[0], X=FW.shape[0],
+              Rank=FK.shape[1])
+    dx = out if out is not None else torch.empty((N, s.C, s.H, s.W), device=dy.device,
+                                                 dtype=torch.float32)
+    ws, nbytes = _ex_workspace(s, g, dy.device, workspace)
+    check(lib().cp4_conv2d_backward_data_ex(
+        ctypes.byref(s), ctypes.byref(g), _ptr(dy), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW), _ptr(dx),
+        ctypes.c_void_p(ws.data_ptr()), nbytes, _stream(stream)))
+    return dx
+
+
+def conv2d_backward_filter_ex(x, dy, FK, FC, FH, FW, g, workspace=None, stream=None):
+    """(dFK, dFC, dFH, dFW) of the layer with geometry g."""
+    s = shape_for(x.shape, FK, FC, FH, FW, 0)
+    assert tuple(dy.shape) == (s.N, s.T, g.out_h, g.out_w) and x.shape[1] == s.C
+    outs = [torch.empty_like(f) for f in (FK, FC, FH, FW)]
+    ws, nbytes = _ex_workspace(s, g, x.device, workspace)
+    check(lib().cp4_conv2d_backward_filter_ex(
+        ctypes.byref(s), ctypes.byref(g), _ptr(x), _ptr(dy), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
+        *[_ptr(o) for o in outs], ctypes.c_void_p(ws.data_ptr()), nbytes, _stream(stream)))
+    return tuple(outs)
 
 
 def _ptr16(t):

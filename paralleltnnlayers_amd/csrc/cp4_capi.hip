@@ -687,6 +687,222 @@ cp4_status cp4_conv2d_backward_filter_full(const cp4_shape* shape,
   return CP4_OK;
 }
 
+// ---- layer geometry ---------------------------------------------------------
+
+namespace {
+cp4_status check_geometry(const cp4_shape* s, const cp4_geometry* g) {
+  cp4_status rc = check_shape(s);
+  if (rc != CP4_OK) return rc;
+  if (!g) return fail(CP4_ERR_NULL_POINTER, "geometry is NULL");
+  if (!g->stride_h || !g->stride_w || !g->out_h || !g->out_w)
+    return fail(CP4_ERR_SHAPE, "strides and output sizes must be >= 1");
+  if (g->stride_h > 1024u || g->stride_w > 1024u)
+    return fail(CP4_ERR_SHAPE, "strides must be <= 1024");
+  if (g->pad_top > s->Y - 1 || g->pad_left > s->X - 1)
+    return fail(CP4_ERR_SHAPE, "pad_top must be <= Y - 1 and pad_left <= X - 1");
+  if ((unsigned long long)g->out_h * g->out_w >= (1ull << 31))
+    return fail(CP4_ERR_SHAPE, "out_h*out_w must be below 2^31");
+  // the last window still starts inside the padded image
+  if ((unsigned long long)g->stride_h * (g->out_h - 1) >= (unsigned long long)s->H + g->pad_top ||
+      (unsigned long long)g->stride_w * (g->out_w - 1) >= (unsigned long long)s->W + g->pad_left)
+    return fail(CP4_ERR_SHAPE, "the output plane reaches past the padded image");
+  return CP4_OK;
+}
+bool is_reference_geometry(const cp4_shape& s, const cp4_geometry& g) {
+  return g.stride_h == 1 && g.stride_w == 1 && g.pad_top == g.pad_left && g.out_h == s.H &&
+         g.out_w == s.W;
+}
+void set_geometry(FwdArgs& a, const cp4_geometry& g) {
+  a.sh = (int)g.stride_h; a.sw = (int)g.stride_w; a.pt = (int)g.pad_top; a.pl = (int)g.pad_left;
+  a.Ho = (int)g.out_h; a.Wo = (int)g.out_w;
+}
+// A launch with a geometry: the strided build of the producer / consumer kernel
+// where it applies and the matrix tiles are not mostly padding, else the general kernel.
+cp4_status run_geometry(FwdArgs a, hipStream_t st) {
+  if (a.N == 0) return CP4_OK;
+  arm(a);
+  if (cp4::fwd_pipe_strided_supported(a) && a.Cin + a.Cout >= kMatrixMinChannels) {
+    CP4_HIP(cp4::fwd_pipe_strided_launch(a, st));
+    return CP4_OK;
+  }
+  if (!cp4::fwd_general_supported(a))
+    return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape and geometry");
+  CP4_HIP(cp4::fwd_general_launch(a, st));
+  return CP4_OK;
+}
+// Stride-1 canvas that carries the strided layer (backward-filter): pad P on every
+// side, x set in at (ot, ol), dy spread out with zeros from the origin.
+struct Canvas {
+  unsigned P, ot, ol, Hc, Wc;
+  bool x_in_place, dy_in_place;
+};
+Canvas canvas_of(const cp4_shape& s, const cp4_geometry& g) {
+  Canvas c;
+  c.P = g.pad_top > g.pad_left ? g.pad_top : g.pad_left;
+  c.ot = c.P - g.pad_top;
+  c.ol = c.P - g.pad_left;
+  const unsigned hu = g.stride_h * (g.out_h - 1) + 1, wu = g.stride_w * (g.out_w - 1) + 1;
+  c.Hc = c.ot + s.H > hu ? c.ot + s.H : hu;
+  c.Wc = c.ol + s.W > wu ? c.ol + s.W : wu;
+  c.x_in_place = c.ot == 0 && c.ol == 0 && c.Hc == s.H && c.Wc == s.W;
+  c.dy_in_place = g.stride_h == 1 && g.stride_w == 1 && g.out_h == c.Hc && g.out_w == c.Wc;
+  return c;
+}
+size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+}  // namespace
+
+cp4_status cp4_geometry_same(const cp4_shape* s, unsigned sh, unsigned sw, cp4_geometry* g) {
+  cp4_status rc = check_shape(s);
+  if (rc != CP4_OK) return rc;
+  if (!g) return fail(CP4_ERR_NULL_POINTER, "geometry is NULL");
+  if (!sh || !sw) return fail(CP4_ERR_SHAPE, "strides must be >= 1");
+  g->stride_h = sh; g->stride_w = sw;
+  g->out_h = (s->H + sh - 1) / sh;
+  g->out_w = (s->W + sw - 1) / sw;
+  const long th = (long)(g->out_h - 1) * sh + s->Y - s->H, tw = (long)(g->out_w - 1) * sw + s->X - s->W;
+  g->pad_top = th > 0 ? (unsigned)(th / 2) : 0;
+  g->pad_left = tw > 0 ? (unsigned)(tw / 2) : 0;
+  return CP4_OK;
+}
+
+cp4_status cp4_geometry_valid(const cp4_shape* s, unsigned sh, unsigned sw, cp4_geometry* g) {
+  cp4_status rc = check_shape(s);
+  if (rc != CP4_OK) return rc;
+  if (!g) return fail(CP4_ERR_NULL_POINTER, "geometry is NULL");
+  if (!sh || !sw) return fail(CP4_ERR_SHAPE, "strides must be >= 1");
+  if (s->H < s->Y || s->W < s->X) return fail(CP4_ERR_SHAPE, "the filter is larger than the image");
+  *g = cp4_geometry{sh, sw, 0, 0, (s->H - s->Y) / sh + 1, (s->W - s->X) / sw + 1};
+  return CP4_OK;
+}
+
+cp4_status cp4_geometry_symmetric(const cp4_shape* s, unsigned sh, unsigned sw, unsigned ph,
+                                  unsigned pw, cp4_geometry* g) {
+  cp4_status rc = check_shape(s);
+  if (rc != CP4_OK) return rc;
+  if (!g) return fail(CP4_ERR_NULL_POINTER, "geometry is NULL");
+  if (!sh || !sw) return fail(CP4_ERR_SHAPE, "strides must be >= 1");
+  if (s->H + 2 * ph < s->Y || s->W + 2 * pw < s->X)
+    return fail(CP4_ERR_SHAPE, "the filter is larger than the padded image");
+  *g = cp4_geometry{sh, sw, ph, pw, (s->H + 2 * ph - s->Y) / sh + 1, (s->W + 2 * pw - s->X) / sw + 1};
+  return CP4_OK;
+}
+
+cp4_status cp4_conv2d_forward_ex(const cp4_shape* shape, const cp4_geometry* g, const float* x,
+                                 const float* FK, const float* FC, const float* FH,
+                                 const float* FW, const float* bias, int activation, float* y,
+                                 cp4_stream stream) {
+  if (activation != CP4_ACT_NONE && activation != CP4_ACT_RELU)
+    return fail(CP4_ERR_UNSUPPORTED, "activation must be CP4_ACT_NONE or CP4_ACT_RELU");
+  cp4_status rc = check_geometry(shape, g);
+  if (rc != CP4_OK) return rc;
+  if (is_reference_geometry(*shape, *g)) {
+    cp4_shape s = *shape;
+    s.pad = g->pad_top;
+    return cp4_conv2d_forward_bias_act(&s, x, FK, FC, FH, FW, bias, activation, y, stream);
+  }
+  if (shape->N == 0) return CP4_OK;
+  rc = check_forward_ptrs(x, FK, FC, FH, FW, y);
+  if (rc != CP4_OK) return rc;
+  FwdArgs a = forward_args(*shape, x, FK, FC, FH, FW, y);
+  set_geometry(a, *g);
+  hipStream_t st = as_stream(stream);
+  rc = run_geometry(a, st);
+  if (rc != CP4_OK) return rc;
+  if (bias || activation != CP4_ACT_NONE)
+    CP4_HIP(cp4::bias_act_launch(y, bias, activation, shape->N, shape->T,
+                                 (size_t)g->out_h * g->out_w, st));
+  return CP4_OK;
+}
+
+size_t cp4_conv2d_backward_ex_workspace_bytes(const cp4_shape* shape, const cp4_geometry* g) {
+  if (check_geometry(shape, g) != CP4_OK || shape->N == 0) return 0;
+  const Canvas c = canvas_of(*shape, *g);
+  cp4_shape sc = *shape;
+  sc.H = c.Hc; sc.W = c.Wc; sc.pad = c.P;
+  const size_t plane = (size_t)c.Hc * c.Wc * sizeof(float);
+  // backward-filter: canvas x (unless in place), canvas dy, the stride-1 pass's workspace;
+  // backward-data needs only dy spread out, which is no larger than canvas dy
+  return align256(c.x_in_place ? 0 : (size_t)shape->N * shape->C * plane) +
+         align256((size_t)shape->N * shape->T * plane) + filter_workspace(sc);
+}
+
+cp4_status cp4_conv2d_backward_data_ex(const cp4_shape* shape, const cp4_geometry* g,
+                                       const float* dy, const float* FK, const float* FC,
+                                       const float* FH, const float* FW, float* dx,
+                                       void* workspace, size_t workspace_bytes,
+                                       cp4_stream stream) {
+  cp4_status rc = check_geometry(shape, g);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return CP4_OK;
+  rc = check_forward_ptrs(dy, FK, FC, FH, FW, dx);
+  if (rc != CP4_OK) return rc;
+  const cp4_shape& s = *shape;
+  hipStream_t st = as_stream(stream);
+  // dx[h,w] = sum_{i,j} K[i,j] dyu[h + pad_top - i, w + pad_left - j] with dyu = dy spread
+  // out with zeros: a stride-1 pass over dyu with the taps in reverse order, Y - 1 - pad_top
+  // zeros before it and an H x W output.
+  const unsigned hu = g->stride_h * (g->out_h - 1) + 1, wu = g->stride_w * (g->out_w - 1) + 1;
+  const float* src = dy;
+  if (g->stride_h > 1 || g->stride_w > 1) {
+    const size_t need = (size_t)s.N * s.T * hu * wu * sizeof(float);
+    if (!workspace || workspace_bytes < need)
+      return fail(CP4_ERR_WORKSPACE, "workspace smaller than cp4_conv2d_backward_ex_workspace_bytes");
+    CP4_HIP(cp4::embed_launch(dy, static_cast<float*>(workspace), (size_t)s.N * s.T, (int)g->out_h,
+                              (int)g->out_w, (int)hu, (int)wu, 0, 0, (int)g->stride_h,
+                              (int)g->stride_w, st));
+    src = static_cast<const float*>(workspace);
+  }
+  cp4_shape su = s;
+  su.H = hu; su.W = wu;
+  FwdArgs a = backward_data_args(su, src, FK, FC, FH, FW, dx);
+  a.sh = 1; a.sw = 1;
+  a.pt = (int)(s.Y - 1 - g->pad_top);
+  a.pl = (int)(s.X - 1 - g->pad_left);
+  a.Ho = (int)s.H; a.Wo = (int)s.W;
+  return run_geometry(a, st);
+}
+
+cp4_status cp4_conv2d_backward_filter_ex(const cp4_shape* shape, const cp4_geometry* g,
+                                         const float* x, const float* dy, const float* FK,
+                                         const float* FC, const float* FH, const float* FW,
+                                         float* dFK, float* dFC, float* dFH, float* dFW,
+                                         void* workspace, size_t workspace_bytes,
+                                         cp4_stream stream) {
+  cp4_status rc = check_geometry(shape, g);
+  if (rc != CP4_OK) return rc;
+  const cp4_shape& s = *shape;
+  const Canvas c = canvas_of(s, *g);
+  cp4_shape sc = s;
+  sc.H = c.Hc; sc.W = c.Wc; sc.pad = c.P;
+  if (s.N == 0 || (c.x_in_place && c.dy_in_place))
+    return cp4_conv2d_backward_filter(&sc, x, dy, FK, FC, FH, FW, dFK, dFC, dFH, dFW, workspace,
+                                      workspace_bytes, stream);
+  if (!x || !dy) return fail(CP4_ERR_NULL_POINTER, "x or dy is NULL");
+  if (!workspace || workspace_bytes < cp4_conv2d_backward_ex_workspace_bytes(shape, g))
+    return fail(CP4_ERR_WORKSPACE, "workspace smaller than cp4_conv2d_backward_ex_workspace_bytes");
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0)
+    return fail(CP4_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  // The stride-1 layer on the canvas computes y1[sh*ho, sw*wo] = y[ho, wo]; with dy
+  // spread out with zeros the loss and so the factor gradients are the same.
+  hipStream_t st = as_stream(stream);
+  unsigned char* w = static_cast<unsigned char*>(workspace);
+  const size_t plane = (size_t)c.Hc * c.Wc * sizeof(float);
+  const float* xc = x;
+  if (!c.x_in_place) {
+    CP4_HIP(cp4::embed_launch(x, reinterpret_cast<float*>(w), (size_t)s.N * s.C, (int)s.H, (int)s.W,
+                              (int)c.Hc, (int)c.Wc, (int)c.ot, (int)c.ol, 1, 1, st));
+    xc = reinterpret_cast<const float*>(w);
+    w += align256((size_t)s.N * s.C * plane);
+  }
+  float* dyc = reinterpret_cast<float*>(w);
+  CP4_HIP(cp4::embed_launch(dy, dyc, (size_t)s.N * s.T, (int)g->out_h, (int)g->out_w, (int)c.Hc,
+                            (int)c.Wc, 0, 0, (int)g->stride_h, (int)g->stride_w, st));
+  w += align256((size_t)s.N * s.T * plane);
+  const size_t used = (size_t)(w - static_cast<unsigned char*>(workspace));
+  return cp4_conv2d_backward_filter(&sc, xc, dyc, FK, FC, FH, FW, dFK, dFC, dFH, dFW, w,
+                                    workspace_bytes - used, stream);
+}
+
 cp4_status cp4_time_forward(const cp4_shape* shape, const float* x,
                             const float* FK, const float* FC, const float* FH,
                             const float* FW, float* y, unsigned warmup,

@@ -43,7 +43,21 @@ struct FwdArgs {
   // (0: the default) and the device's fault record, four ints (may be null).
   int spin_limit;
   int* fault;
+  // Layer geometry beyond the reference's (stride 1, `pad` zeros before the image,
+  // an H x W output): output pixel (ho, wo) reads x at (sh*ho + i - pt, sw*wo + j - pl),
+  // the output plane is Ho x Wo.  sh == 0: the reference's geometry, the other
+  // fields unused.  Only kernels that say so take sh != 0.
+  int sh, sw, pt, pl, Ho, Wo;
 };
+
+// The geometry of a launch with the defaults filled in.
+struct Geometry {
+  int sh, sw, pt, pl, Ho, Wo;
+};
+inline Geometry geometry_of(const FwdArgs& a) {
+  if (a.sh == 0) return Geometry{1, 1, a.pad, a.pad, a.H, a.W};
+  return Geometry{a.sh, a.sw, a.pt, a.pl, a.Ho, a.Wo};
+}
 
 // Compute units of the current device (256 when no device can be asked).
 int num_compute_units();
@@ -82,6 +96,10 @@ hipError_t fwd_pipe_rankpass_launch(const FwdArgs&, hipStream_t);
 // The same kernel on tiles of TH rows x Wt columns (wide planes).
 bool fwd_pipe_tiled_supported(const FwdArgs&);
 hipError_t fwd_pipe_tiled_launch(const FwdArgs&, hipStream_t);
+// The same kernel for a stride or an output plane of its own (FwdArgs::sh ...
+// all filled in by the caller).
+bool fwd_pipe_strided_supported(const FwdArgs&);
+hipError_t fwd_pipe_strided_launch(const FwdArgs&, hipStream_t);
 // The same kernel with a depthwise Y x X filter (FwdArgs::taps2d) in its tap step.
 bool fwd_pipe_taps2d_supported(const FwdArgs&);
 hipError_t fwd_pipe_taps2d_launch(const FwdArgs&, hipStream_t);
@@ -127,6 +145,10 @@ hipError_t cp3_expand_launch(const cp4_shape& s, const float* K0, const float* K
                              hipStream_t);
 hipError_t cp3_fold_launch(const cp4_shape& s, const float* dFK, const float* dFC,
                            const float* dFW, float* dK0, float* dK1, float* dK2, hipStream_t);
+// dst[plane][ot + sh*u][ol + sw*v] = src[plane][u][v] on `planes` planes of h x w
+// set into canvases of Hc x Wc; every other canvas cell is written as zero.
+hipError_t embed_launch(const float* src, float* dst, size_t planes, int h, int w, int Hc, int Wc,
+                        int ot, int ol, int sh, int sw, hipStream_t);
 // dst [cols, rows] = transpose of src [rows, cols]
 hipError_t transpose_f32_launch(const float* src, float* dst, int rows, int cols, hipStream_t);
 hipError_t copy_f32_launch(float* dst, const float* src, size_t n, hipStream_t);

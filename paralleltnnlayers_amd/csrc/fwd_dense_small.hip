@@ -179,7 +179,7 @@ __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, De
 
 bool plan(const FwdArgs& a, DensePlan* pl) {
   if (a.Y != a.X || !(a.Y & 1) || a.Y > 17 || a.pad > a.Y - 1) return false;
-  if (a.Cout > 8 || a.ldf || a.accumulate) return false;
+  if (a.Cout > 8 || a.ldf || a.accumulate || a.sh) return false;
   const long nw = (long)a.Cout * a.Cin * a.Y * a.X;
   if (nw > kMaxWeights) return false;
   const long nf = (long)a.R * (a.Cout + a.Cin + a.Y + a.X);

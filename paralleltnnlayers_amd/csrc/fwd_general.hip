@@ -1,5 +1,5 @@
 // General forward / backward-data kernel: any rank, channel counts, odd or
-// even filter size and pad; VALU arithmetic, LDS-tiled.
+// even filter size, pad, stride and output size; VALU arithmetic, LDS-tiled.
 //
 // One workgroup owns an 8 x 32 output tile of one image and walks the rank in
 // blocks of RB.  Per rank block:
@@ -19,15 +19,16 @@ namespace {
 constexpr int kTH = 8, kTW = 32, kThreads = kTH * kTW;
 
 template <int RB>
-__global__ __launch_bounds__(kThreads) void fwd_general_kernel(FwdArgs a) {
+__global__ __launch_bounds__(kThreads) void fwd_general_kernel(FwdArgs a, Geometry g) {
   extern __shared__ float lds[];
-  const int HT = kTH + a.Y - 1, WT = kTW + a.X - 1;
+  // input cells under a tile of kTH x kTW outputs: rows, columns
+  const int HT = g.sh * (kTH - 1) + a.Y, WT = g.sw * (kTW - 1) + a.X;
   const int nA = HT * WT, nB = kTH * WT;
   float* As = lds;            // [RB][HT*WT]
   float* Bs = lds + RB * nA;  // [RB][kTH*WT]
-  const int n = blockIdx.z, h0 = blockIdx.y * kTH, w0 = blockIdx.x * kTW;
+  const int n = blockIdx.z, h0 = blockIdx.y * kTH, w0 = blockIdx.x * kTW;   // output coordinates
   const int tid = threadIdx.x;
-  const size_t HW = (size_t)a.H * a.W;
+  const size_t HW = (size_t)a.H * a.W, HWo = (size_t)g.Ho * g.Wo;
   const float* xn = a.x + (size_t)n * a.Cin * HW;
   const int R = a.R;
 
@@ -35,7 +36,7 @@ __global__ __launch_bounds__(kThreads) void fwd_general_kernel(FwdArgs a) {
     // 1. channel -> rank contraction on the halo tile
     for (int q = tid; q < nA; q += kThreads) {
       const int hh = q / WT, ww = q - hh * WT;
-      const int gh = h0 + hh - a.pad, gw = w0 + ww - a.pad;
+      const int gh = g.sh * h0 + hh - g.pt, gw = g.sw * w0 + ww - g.pl;
       float acc[RB];
 #pragma unroll
       for (int rr = 0; rr < RB; ++rr) acc[rr] = 0.f;
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(kThreads) void fwd_general_kernel(FwdArgs a) {
         if (r0 + rr < R)
           for (int i = 0; i < a.Y; ++i)
             s += a.FH[(a.flip ? a.Y - 1 - i : i) * R + r0 + rr] *
-                 As[rr * nA + (h + i) * WT + ww];
+                 As[rr * nA + (g.sh * h + i) * WT + ww];
         Bs[rr * nB + q] = s;
       }
     }
@@ -77,20 +78,20 @@ __global__ __launch_bounds__(kThreads) void fwd_general_kernel(FwdArgs a) {
       if (r0 + rr < R)
         for (int j = 0; j < a.X; ++j)
           s += a.FW[(a.flip ? a.X - 1 - j : j) * R + r0 + rr] *
-               Bs[rr * nB + h * WT + w + j];
+               Bs[rr * nB + h * WT + g.sw * w + j];
       cc[rr] = s;
     }
     // 4. rank -> output-channel contraction
-    if (h0 + h < a.H && w0 + w < a.W) {
-      float* yp = a.y + (size_t)n * a.Cout * HW + (size_t)(h0 + h) * a.W + w0 + w;
+    if (h0 + h < g.Ho && w0 + w < g.Wo) {
+      float* yp = a.y + (size_t)n * a.Cout * HWo + (size_t)(h0 + h) * g.Wo + w0 + w;
 #pragma unroll 4
       for (int k = 0; k < a.Cout; ++k) {      // (unrolled: four rows of the factor in flight)
         const float* f = a.Fout + (size_t)k * R + r0;
         float s = 0.f;
 #pragma unroll
         for (int rr = 0; rr < RB; ++rr) s += cc[rr] * (r0 + rr < R ? f[rr] : 0.f);
-        if (r0 > 0) s += yp[k * HW];
-        yp[k * HW] = s;
+        if (r0 > 0) s += yp[k * HWo];
+        yp[k * HWo] = s;
       }
     }
     __syncthreads();
@@ -99,7 +100,8 @@ __global__ __launch_bounds__(kThreads) void fwd_general_kernel(FwdArgs a) {
 
 // LDS floats needed for a rank block of rb.
 size_t lds_floats(const FwdArgs& a, int rb) {
-  const size_t HT = kTH + a.Y - 1, WT = kTW + a.X - 1;
+  const Geometry g = geometry_of(a);
+  const size_t HT = (size_t)g.sh * (kTH - 1) + a.Y, WT = (size_t)g.sw * (kTW - 1) + a.X;
   return (size_t)rb * (HT * WT + kTH * WT);
 }
 // More LDS per workgroup costs occupancy, a second rank block re-reads and
@@ -120,7 +122,7 @@ int pick_rank_block(const FwdArgs& a) {
 
 bool fwd_general_supported(const FwdArgs& a) {
   return lds_floats(a, 1) * 4 <= kLdsBudget && a.N <= 65535 &&
-         (a.H + kTH - 1) / kTH <= 65535;
+         (geometry_of(a).Ho + kTH - 1) / kTH <= 65535;
 }
 
 template <int RB>
@@ -128,8 +130,9 @@ hipError_t launch_rb(const FwdArgs& a, size_t smem, hipStream_t s) {
   const void* fn = reinterpret_cast<const void*>(fwd_general_kernel<RB>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (e != hipSuccess) return e;
-  const dim3 grid((a.W + kTW - 1) / kTW, (a.H + kTH - 1) / kTH, a.N);
-  fwd_general_kernel<RB><<<grid, kThreads, smem, s>>>(a);
+  const Geometry g = geometry_of(a);
+  const dim3 grid((g.Wo + kTW - 1) / kTW, (g.Ho + kTH - 1) / kTH, a.N);
+  fwd_general_kernel<RB><<<grid, kThreads, smem, s>>>(a, g);
   return hipGetLastError();
 }
 

@@ -635,7 +635,7 @@ hipError_t launch_rb(const FwdArgs& a, const StripPlan& pl, hipStream_t st) {
 }  // namespace
 
 bool fwd_mfma_supported(const FwdArgs& a) {
-  if (a.R > 64 || (a.W & 1) || (a.Cin & 1)) return false;
+  if (a.R > 64 || (a.W & 1) || (a.Cin & 1) || a.sh) return false;
   if (!fits_int_indexing(a.N, a.H, a.W)) return false;
   if (a.x && (reinterpret_cast<uintptr_t>(a.x) & 7)) return false;
   if (a.y && (reinterpret_cast<uintptr_t>(a.y) & 7)) return false;

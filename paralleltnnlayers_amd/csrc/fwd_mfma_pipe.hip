@@ -40,7 +40,7 @@
 // Cuda_kernels/cp4Conv2dForward.cu:84-133 (backward-data:
 // cp4Conv2dBackwardData.cu:57-108 through swapped factors and flipped taps).
 //
-// This file is compiled six times: as is; with CP4_PIPE_EPILOGUE defined, which
+// This file is compiled seven times: as is; with CP4_PIPE_EPILOGUE defined, which
 // adds y = act(conv + bias[k]) to the stores (the bias of the lane's sixteen
 // output rows rides in registers next to the output-factor fragment) and exports
 // the entry points under the names fwd_pipe_epi_*; and with CP4_PIPE_IO16, where
@@ -59,7 +59,12 @@
 // and with CP4_PIPE_TAPS2D, for the 3-factor CP sibling op: the tap step weighs
 // the Y x X cells it reads with a depthwise filter FwdArgs::taps2d [Y, X, R]
 // instead of the outer product FH x FW (1x1 and 3x3 filters: 36 wave-uniform
-// weights per wave), entry points fwd_pipe_taps2d_*.
+// weights per wave), entry points fwd_pipe_taps2d_*;
+// and with CP4_PIPE_STRIDED, for layers with a stride or an output plane that is
+// not the input's (FwdArgs::sh ...): a strip is TH rows of the OUTPUT, its LDS
+// plane the sh*(TH-1) + Y input rows under them; the tap step of output pixel
+// (ho, wo) reads the plane at row sh*ho, column sw*wo - pl, so only the kept
+// outputs are filtered, contracted and stored; entry points fwd_pipe_strided_*.
 #include <cstdlib>
 #include <type_traits>
 
@@ -203,13 +208,19 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #endif
   const int l32 = lane & 31, hi = lane >> 5;
   const int H = a.H, W = a.W, HW = H * W, R = a.R, Cin = a.Cin, Cout = a.Cout;
+#ifdef CP4_PIPE_STRIDED
+  // output plane, stride, zeros before the image; h0 counts output rows
+  const int Ho = a.Ho, Wo = a.Wo, HWo = Ho * Wo, SH = a.sh, SW = a.sw, PT = a.pt, PL = a.pl;
+#else
+  [[maybe_unused]] const int Ho = H, Wo = W, HWo = HW;
+#endif
   const int QA = pl.QA;
 #ifdef CP4_PIPE_RANKPASS
   const int ldf = a.ldf ? a.ldf : R;             // row stride of the factor matrices
 #else
   const int ldf = R;
 #endif
-  const int rows = min(pl.TH, H - h0);
+  const int rows = min(pl.TH, Ho - h0);
 #ifdef CP4_PIPE_TILED
   const int Wt = pl.Wt, lgWt = pl.lgWt, WL = Wt + FS - 1;   // tile width, LDS row length
   const int wcols = min(Wt, W - w0);             // tile columns inside the image
@@ -217,19 +228,24 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   const int gshift = 0;
   const int ngroups = nvalid >> 6;
 #else
-  const int nvalid = rows * W;                   // output pixels inside the image
+  const int nvalid = rows * Wo;                  // output pixels inside the image
   // 64-pixel output groups start `gshift` pixels before the strip so that their
   // boundaries fall on 128-byte lines of y (pixel h0*W + 64*g - gshift is a
   // multiple of 32); pixels before the strip are computed and not stored.
-  const int gshift = (h0 * W) & 31;
+  const int gshift = (h0 * Wo) & 31;
   const int ngroups = (nvalid + gshift + 63) >> 6;
 #endif
   const int nkb = (Cout + 31) >> 5;
 #ifdef CP4_PIPE_TILED
   const int QLEN = (pl.TH + FS - 1) * WL;
 #else
+#ifdef CP4_PIPE_STRIDED
+  const int qbase = (SH * h0 - PT) * W;          // global flat pixel of LDS column 0
+  const int QLEN = (SH * (pl.TH - 1) + FS) * W;
+#else
   const int qbase = (h0 - a.pad) * W;            // global flat pixel of LDS column 0
   const int QLEN = (pl.TH + FS - 1) * W;
+#endif
 #endif
   const int nblk = (QLEN + 31) >> 5;             // 32-pixel producer blocks
   const bool backoff = nblk >= 4;                // growing naps in the spin waits
@@ -529,12 +545,12 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #ifdef CP4_PIPE_TILED
     io_t* yn = reinterpret_cast<io_t*>(a.y) + (size_t)n * Cout * HW + (size_t)h0 * W + w0;
 #else
-    io_t* yn = reinterpret_cast<io_t*>(a.y) + (size_t)n * Cout * HW + (size_t)h0 * W;
+    io_t* yn = reinterpret_cast<io_t*>(a.y) + (size_t)n * Cout * HWo + (size_t)h0 * Wo;
 #endif
     [[maybe_unused]] const bool accumulate = a.accumulate != 0;
     const bool pair_stores =                       // one store per pixel pair is legal
-        ((W | HW) & 1) == 0 && (reinterpret_cast<uintptr_t>(a.y) & (2 * kIoBytes - 1)) == 0;
-#ifndef CP4_PIPE_TILED
+        ((Wo | HWo) & 1) == 0 && (reinterpret_cast<uintptr_t>(a.y) & (2 * kIoBytes - 1)) == 0;
+#if !defined(CP4_PIPE_TILED) && !defined(CP4_PIPE_STRIDED)
     const int reach = (FS - 1) * (W + 1);          // how far past a pixel its taps read in A
 #endif
 
@@ -554,6 +570,14 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       // h .. h + FS - 1, columns w .. w + 62 + FS
       const int h = (64 * i) >> lgWt, w = (64 * i) & (Wt - 1);
       const int last = ((h + FS - 1) * WL + w + 63 + FS - 1) >> 5;
+      return last > nblk - 1 ? nblk - 1 : last;
+#elif defined(CP4_PIPE_STRIDED)
+      // group g holds output pixels 64*g - gshift ... + 63 of the strip: its taps
+      // read the plane rows SH*h ... SH*h + FS - 1 of its first to last output row h
+      const int g = rev ? ngroups - 1 - i : i;
+      const int pf = max(64 * g - gshift, 0), pz = min(64 * g - gshift + 63, nvalid - 1);
+      if (rev) return nblk - 1 - ((SH * (pf / Wo) * W) >> 5);
+      const int last = ((SH * (pz / Wo) + FS - 1) * W + W - 1) >> 5;
       return last > nblk - 1 ? nblk - 1 : last;
 #else
       const int g = rev ? ngroups - 1 - i : i;
@@ -594,6 +618,20 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       for (int j = 0; j < FS; ++j) {
         in[j] = true;
         off[j] = w + j;
+      }
+#elif defined(CP4_PIPE_STRIDED)
+      const int RL = W;
+      // lanes before or past the strip's outputs: any valid pixel (not stored)
+      const int p = min(max(64 * g - gshift + lane, 0), nvalid - 1);
+      const int ho = p / Wo, wo = p - ho * Wo;
+      const int h = SH * ho;                             // plane row of the first tap row
+      int off[FS];
+      bool in[FS];
+#pragma unroll
+      for (int j = 0; j < FS; ++j) {
+        const int ww = SW * wo + j - PL;
+        in[j] = ww >= 0 && ww < W;
+        off[j] = ww < 0 ? 0 : (ww >= W ? W - 1 : ww);      // clamped: weight is 0 there
       }
 #else
       const int RL = W;
@@ -734,7 +772,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       const int pofs = p;
       const bool pin0 = p >= 0 && p < nvalid, pin1 = p + 1 >= 0 && p + 1 < nvalid;
 #endif
-      io_t* rowbase = yn + (size_t)(32 * kb) * HW;
+      io_t* rowbase = yn + (size_t)(32 * kb) * HWo;
       // the lane's pixel pair as one store: float2, or two bfloat16 in a dword
       auto store_pair = [&](io_t* dst, float v0, float v1) {
 #ifdef CP4_PIPE_IO16
@@ -767,29 +805,29 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       if (pair_stores) {
         // W and H*W even, y aligned to a pair: p is even and the pair is one store
         if (pin0) {
-          const unsigned lofs = (unsigned)(4 * hi * HW + pofs);
+          const unsigned lofs = (unsigned)(4 * hi * HWo + pofs);
           if (32 * kb + 32 <= Cout) {
 #pragma unroll
             for (int v = 0; v < 16; ++v)
-              store_pair(rowbase + (size_t)(8 * (v >> 2) + (v & 3)) * HW + lofs, acc0[v], acc1[v]);
+              store_pair(rowbase + (size_t)(8 * (v >> 2) + (v & 3)) * HWo + lofs, acc0[v], acc1[v]);
           } else {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
               const int kk = 8 * (v >> 2) + (v & 3);         // + 4*hi is in lofs
               if (32 * kb + kk + 4 * hi < Cout)
-                store_pair(rowbase + (size_t)kk * HW + lofs, acc0[v], acc1[v]);
+                store_pair(rowbase + (size_t)kk * HWo + lofs, acc0[v], acc1[v]);
             }
           }
         }
       } else {
         // odd widths or planes: the two pixels are stored and bounded one by one
         const bool in0 = pin0, in1 = pin1;
-        const long lofs = (long)(4 * hi) * HW + pofs;
+        const long lofs = (long)(4 * hi) * HWo + pofs;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int kk = 8 * (v >> 2) + (v & 3);
           if (32 * kb + kk + 4 * hi < Cout) {
-            io_t* rp = rowbase + (size_t)kk * HW + lofs;
+            io_t* rp = rowbase + (size_t)kk * HWo + lofs;
             if (in0) store_one(rp, acc0[v]);
             if (in1) store_one(rp + 1, acc1[v]);
           }
@@ -933,7 +971,47 @@ int round_up(int v, int m) { return (v + m - 1) / m * m; }
   return true;
 }
 
-#ifdef CP4_PIPE_TILED
+#ifdef CP4_PIPE_STRIDED
+// Strip of TH output rows: plane of the sh * (TH - 1) + Y input rows under them.
+bool layout_strided(const FwdArgs& a, int TH, PipePlan* pl) {
+  const long QLEN = ((long)a.sh * (TH - 1) + a.Y) * a.W;
+  const long QA = round_up((int)QLEN, 64) + 8;
+  const size_t a_bytes = (size_t)kRP * QA * sizeof(float);
+  const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
+  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 16) * sizeof(int);
+  if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
+  if (bytes > kLdsLimit) return false;
+  pl->TH = TH;
+  pl->strips = (a.Ho + TH - 1) / TH;
+  pl->nWG = a.N * pl->strips;
+  pl->QA = (int)QA;
+  pl->fin_off = (int)a_bytes;
+  pl->cc_off = (int)(a_bytes + fin_bytes);
+  pl->flag_off = (int)(a_bytes + fin_bytes + 3 * kCcBuf);
+  pl->lds_bytes = bytes;
+  return true;
+}
+bool plan(const FwdArgs& a, PipePlan* best) {
+  double best_cost = 0;
+  bool found = false;
+  if (a.tune_th > 0) return a.tune_th <= a.Ho && layout_strided(a, a.tune_th, best);
+  const int cus = num_compute_units();
+  for (int TH = 1; TH <= a.Ho; ++TH) {
+    PipePlan pl;
+    if (!layout_strided(a, TH, &pl)) break;
+    const double rounds = (pl.nWG + cus - 1) / cus;
+    // cells read per channel and cells written per channel
+    const double cost = rounds * (((double)a.sh * (TH - 1) + a.Y) * a.W * a.Cin +
+                                  (double)TH * a.Wo * a.Cout);
+    if (!found || cost <= best_cost) {
+      best_cost = cost;
+      *best = pl;
+      found = true;
+    }
+  }
+  return found;
+}
+#elif defined(CP4_PIPE_TILED)
 // Tile of TH rows x Wt columns: plane of (TH + Y - 1) rows of Wt + Y - 1 cells.
 bool layout_tiled(const FwdArgs& a, int TH, int lgWt, PipePlan* pl) {
   const int Wt = 1 << lgWt, WL = Wt + a.Y - 1;
@@ -983,7 +1061,8 @@ bool plan(const FwdArgs& a, PipePlan* best) {
     }
   return found;
 }
-#else
+#endif
+#if !defined(CP4_PIPE_TILED) && !defined(CP4_PIPE_STRIDED)
 bool plan(const FwdArgs& a, PipePlan* best) {
   double best_cost = 0;
   bool found = false;
@@ -1044,7 +1123,10 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 
 }  // namespace
 
-#if defined(CP4_PIPE_TAPS2D)
+#if defined(CP4_PIPE_STRIDED)
+#define fwd_pipe_supported fwd_pipe_strided_supported
+#define fwd_pipe_launch fwd_pipe_strided_launch
+#elif defined(CP4_PIPE_TAPS2D)
 #define fwd_pipe_supported fwd_pipe_taps2d_supported
 #define fwd_pipe_launch fwd_pipe_taps2d_launch
 #elif defined(CP4_PIPE_TILED)
@@ -1067,6 +1149,14 @@ bool fwd_pipe_supported(const FwdArgs& a) {
   if (a.accumulate || a.ldf) return false;       // only the rank-pass build has these
 #endif
   if (!fits_int_indexing(a.N, a.H, a.W)) return false;
+#ifdef CP4_PIPE_STRIDED
+  // the caller fills in the whole geometry; every output row reads at least one image row
+  if (a.sh < 1 || a.sw < 1 || a.Ho < 1 || a.Wo < 1 || a.pt < 0 || a.pl < 0) return false;
+  if (!fits_int_indexing(a.N, a.Ho, a.Wo)) return false;
+  if ((size_t)a.Cout * a.Ho * a.Wo * sizeof(io_t) >= (1ull << 31)) return false;
+#else
+  if (a.sh) return false;                        // only the strided build takes a geometry
+#endif
   if ((size_t)a.Cin * a.H * a.W * sizeof(io_t) >= (1ull << 31)) return false;   // buffer offsets
   if (a.Y != a.X || !(a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7)) return false;
 #ifdef CP4_PIPE_TAPS2D

@@ -452,7 +452,7 @@ hipError_t launch_fs(const FwdArgs& a, const SplitPlan& pl, hipStream_t st) {
 }  // namespace
 
 bool fwd_split_supported(const FwdArgs& a) {
-  if (a.R > kRP || (a.W & 1) || (a.Cin & 63)) return false;
+  if (a.R > kRP || (a.W & 1) || (a.Cin & 63) || a.sh) return false;
   if (!fits_int_indexing(a.N, a.H, a.W)) return false;
   if (a.Y != a.X || !(a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7)) return false;
   if (a.x && (reinterpret_cast<uintptr_t>(a.x) & 7)) return false;

@@ -77,6 +77,26 @@ __global__ __launch_bounds__(256) void zero_f32_kernel(float* __restrict__ dst, 
     dst[i] = 0.f;
 }
 
+// dst[plane][ot + sh*h][ol + sw*w] = src[plane][h][w], every other cell of dst zero:
+// a plane set into a larger canvas, its pixels spread sh x sw apart (zero
+// insertion).  One pass that writes every cell of dst.
+__global__ __launch_bounds__(256) void embed_kernel(const float* __restrict__ src,
+                                                    float* __restrict__ dst, size_t planes, int h,
+                                                    int w, int Hc, int Wc, int ot, int ol, int sh,
+                                                    int sw) {
+  const size_t total = planes * Hc * Wc;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (size_t)gridDim.x * 256) {
+    const int v = (int)(i % Wc), u = (int)((i / Wc) % Hc);
+    const size_t p = i / ((size_t)Wc * Hc);
+    const int du = u - ot, dv = v - ol;
+    float val = 0.f;
+    if (du >= 0 && dv >= 0 && du % sh == 0 && dv % sw == 0 && du / sh < h && dv / sw < w)
+      val = src[(p * h + du / sh) * w + dv / sw];
+    dst[i] = val;
+  }
+}
+
 // one workgroup per (image, channel) plane segment: the bias is a scalar
 __global__ __launch_bounds__(256) void bias_act_kernel(float* __restrict__ y,
                                                        const float* __restrict__ bias, int act,
@@ -201,6 +221,14 @@ hipError_t bias_act_launch(float* y, const float* bias, int act, size_t N, size_
 hipError_t zero_f32_launch(float* dst, size_t n, hipStream_t st) {
   if (n == 0) return hipSuccess;
   zero_f32_kernel<<<grid_for(n, 2048), 256, 0, st>>>(dst, n);
+  return hipGetLastError();
+}
+
+hipError_t embed_launch(const float* src, float* dst, size_t planes, int h, int w, int Hc, int Wc,
+                        int ot, int ol, int sh, int sw, hipStream_t st) {
+  const size_t total = planes * Hc * Wc;
+  if (total == 0) return hipSuccess;
+  embed_kernel<<<grid_for(total, 8192), 256, 0, st>>>(src, dst, planes, h, w, Hc, Wc, ot, ol, sh, sw);
   return hipGetLastError();
 }
 

@@ -8,10 +8,11 @@ PyTorch only owns the tensors and the stream; all arithmetic is in the HIP
 library, and there is no eager fallback.
 
 Factor layout is the C ABI's: FK [T,R], FC [C,R], FH [Y,R], FW [X,R].
-Gradients are exact for "same" padding (2*pad = Y-1 = X-1), the only case in
-which the reference's backward-data formula (flipped taps at offset +y-pad,
-Cuda_kernels/cp4Conv2dBackwardData.cu:79-87) is the adjoint of its forward;
-other paddings are refused for autograd use.
+For "same" padding at stride 1 (2*pad = Y-1 = X-1) the reference's three passes
+run as they are; that is the only case in which its backward-data formula
+(flipped taps at offset +y-pad, Cuda_kernels/cp4Conv2dBackwardData.cu:79-87) is
+the adjoint of its forward.  Strides and every other padding go through the
+library's geometry entry points (cp4_conv2d_forward_ex and its exact gradients).
 """
 import torch
 
@@ -79,19 +80,61 @@ class CP4Conv2dFunction(torch.autograd.Function):
         return (dx,) + grads + (None, dbias, None)
 
 
-def cp4_conv2d(x, FK, FC, FH, FW, pad, bias=None, activation=None, stride=1):
+class CP4Conv2dGeometryFunction(torch.autograd.Function):
+    """The layer with a stride, explicit padding or an output plane of its own
+    (cp4_conv2d_forward_ex and its two gradients; float32)."""
+
+    @staticmethod
+    def forward(ctx, x, FK, FC, FH, FW, geom, bias=None, activation=None):
+        x, FK, FC, FH, FW = (t.contiguous().float() for t in (x, FK, FC, FH, FW))
+        if bias is not None:
+            bias = bias.contiguous().float()
+        y = capi.conv2d_forward_ex(x, FK, FC, FH, FW, geom, bias, activation)
+        ctx.geom = geom
+        ctx.relu = capi.ACTIVATIONS[activation] == 1
+        ctx.save_for_backward(x, FK, FC, FH, FW, y if ctx.relu else None)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, FK, FC, FH, FW, y = ctx.saved_tensors
+        dy = dy.contiguous().float()
+        if ctx.relu:
+            dy = dy * (y > 0)
+        dbias = dy.sum(dim=(0, 2, 3)) if ctx.needs_input_grad[6] else None
+        dx = None
+        if ctx.needs_input_grad[0]:
+            dx = capi.conv2d_backward_data_ex(dy, x.shape[2:], FK, FC, FH, FW, ctx.geom)
+        grads = (None, None, None, None)
+        if any(ctx.needs_input_grad[1:5]):
+            grads = capi.conv2d_backward_filter_ex(x, dy, FK, FC, FH, FW, ctx.geom)
+            grads = tuple(g if need else None
+                          for g, need in zip(grads, ctx.needs_input_grad[1:5]))
+        return (dx,) + grads + (None, dbias, None)
+
+
+def cp4_conv2d(x, FK, FC, FH, FW, pad, bias=None, activation=None, stride=1, padding=None):
     """Functional form: differentiable fused CP4 convolution (NCHW), with the
     optional bias [T] and activation ("relu") fused into the forward stores.
 
-    The kernels are stride 1 (as the reference's, whose tensor_shape has no stride
-    field).  ``stride`` > 1 keeps every stride-th row and column of that result -
-    for "same" padding exactly the strided convolution the reference's Python
-    layers build with ``strides`` (test/layers.py:264-277) - at the cost of
-    computing the skipped outputs; autograd scatters the upstream gradient back
-    into the full-resolution one.
+    ``pad`` zeros on every side, stride 1 and 2*pad = Y - 1 is the reference's own
+    layer and runs its three passes (bfloat16 activations included).  A ``stride``,
+    ``padding`` = "same" (the framework's rule of the reference's Python layers,
+    test/layers.py:264-279: out = ceil(in / stride), on even sizes one more zero
+    after the image than before it), "valid", an int or an (h, w) pair run the
+    strided kernels: only the kept outputs are computed.
     """
-    y = CP4Conv2dFunction.apply(x, FK, FC, FH, FW, pad, bias, activation)
-    return y if stride == 1 else y[:, :, ::stride, ::stride]
+    if padding is None:
+        padding = pad
+    y_taps, x_taps = FH.shape[0], FW.shape[0]
+    plain = stride == 1 and (
+        (isinstance(padding, int) and 2 * padding + 1 == y_taps == x_taps) or
+        (padding == "same" and y_taps == x_taps and y_taps % 2 == 1))
+    if plain:
+        return CP4Conv2dFunction.apply(x, FK, FC, FH, FW, y_taps // 2, bias, activation)
+    s = capi.shape_for(x.shape, FK, FC, FH, FW, 0)
+    geom = capi.geometry(s, stride, padding)
+    return CP4Conv2dGeometryFunction.apply(x, FK, FC, FH, FW, geom, bias, activation)
 
 
 class CP4Conv2d(torch.nn.Module):
@@ -104,11 +147,12 @@ class CP4Conv2d(torch.nn.Module):
     """
 
     def __init__(self, in_channels, out_channels, kernel_size, rank, device="cuda", bias=False,
-                 activation=None, stride=1):
+                 activation=None, stride=1, padding=None):
         super().__init__()
-        if kernel_size % 2 != 1:
-            raise ValueError("kernel_size must be odd (same padding)")
+        if kernel_size % 2 != 1 and padding is None:
+            raise ValueError("kernel_size must be odd for the default padding")
         self.pad = kernel_size // 2
+        self.padding = padding
         fan_in = in_channels * kernel_size * kernel_size
         # Var[K] = R * s^8 for four independent N(0, s^2) factors; target 2 / fan_in
         s = (2.0 / (fan_in * rank)) ** 0.125
@@ -121,7 +165,7 @@ class CP4Conv2d(torch.nn.Module):
 
     def forward(self, x):
         return cp4_conv2d(x, self.FK, self.FC, self.FH, self.FW, self.pad, self.bias,
-                          self.activation, self.stride)
+                          self.activation, self.stride, self.padding)
 
     def dense_filter(self):
         """The recomposed [T,C,Y,X] filter (on the device, through cp4_recompose)."""

@@ -113,3 +113,25 @@ def test_workload_byte_counts():
         assert algorithmic_bytes(WORKLOADS[k]) == v
     assert minimal_flops(WORKLOADS["C3"]) == 3326869504
     assert minimal_flops(WORKLOADS["C5"]) == 1673068544
+
+
+def test_geometry_helpers_need_no_device(L):
+    """cp4_geometry_same / _valid / _symmetric and the checks of the _ex entry points."""
+    from paralleltnnlayers_amd import capi
+    s = capi.Shape(N=1, H=8, W=9, pad=0, T=2, C=2, Y=3, X=3, Rank=2)
+    g = capi.geometry(s, 2, "same")          # even size: no zeros before the image
+    assert (g.pad_top, g.pad_left, g.out_h, g.out_w) == (0, 1, 4, 5)
+    g = capi.geometry(s, 2, "valid")
+    assert (g.pad_top, g.pad_left, g.out_h, g.out_w) == (0, 0, 3, 4)
+    g = capi.geometry(s, (2, 1), 1)
+    assert (g.stride_h, g.stride_w, g.pad_top, g.out_h, g.out_w) == (2, 1, 1, 4, 9)
+    one = ctypes.c_void_p(256)               # never dereferenced: checks fail first
+    bad = capi.Geometry(2, 2, 3, 0, 4, 4)    # pad_top > Y - 1
+    assert L.cp4_conv2d_forward_ex(ctypes.byref(s), ctypes.byref(bad), one, one, one, one, one,
+                                   None, 0, one, None) == capi.ERR_SHAPE
+    far = capi.Geometry(2, 2, 0, 0, 40, 4)   # the output plane reaches past the image
+    assert L.cp4_conv2d_forward_ex(ctypes.byref(s), ctypes.byref(far), one, one, one, one, one,
+                                   None, 0, one, None) == capi.ERR_SHAPE
+    assert L.cp4_conv2d_forward_ex(ctypes.byref(s), None, one, one, one, one, one, None, 0, one,
+                                   None) == capi.ERR_NULL_POINTER
+    assert capi.backward_ex_workspace_bytes(s, capi.geometry(s, 2, "same")) > 0

@@ -57,11 +57,17 @@ def test_only_requested_gradients(ops):
     assert fac[0].grad is not None and all(f.grad is None for f in fac[1:]) and x.grad is None
 
 
-def test_non_same_padding_is_refused(ops):
-    x = torch.randn(1, 8, 6, 6, device="cuda")
-    fac = [torch.randn(d, 4, device="cuda") for d in (8, 8, 3, 3)]
-    with pytest.raises(ValueError):
-        ops.cp4_conv2d(x, *fac, 0)
+def test_padding_other_than_same_gives_the_smaller_output(ops):
+    """pad = 0 with a 3x3 filter: the layer's output is (H - 2) x (W - 2), as a dense
+    convolution's, and differentiable (the geometry entry points)."""
+    x = torch.randn(1, 8, 6, 6, device="cuda", requires_grad=True)
+    fac = [torch.randn(d, 4, device="cuda", requires_grad=True) for d in (8, 8, 3, 3)]
+    y = ops.cp4_conv2d(x, *fac, 0)
+    want = torch.nn.functional.conv2d(x.detach(), recomposed(*[f.detach() for f in fac]))
+    assert y.shape == want.shape == (1, 8, 4, 4)
+    assert (y.detach() - want).abs().max() <= 1e-4 * want.abs().max()
+    y.sum().backward()
+    assert x.grad is not None and all(f.grad is not None for f in fac)
 
 
 def test_layer_trains(ops):

@@ -256,3 +256,73 @@ def test_cp3_depthwise_tap_orientation(oracle):
     want = np.zeros((5, 5), np.float32)
     want[1:, :4] = x[0, 0, :4, 1:]
     np.testing.assert_array_equal(y[0, 0], want)
+
+
+# ---- layer geometry: stride, explicit padding, an output plane of its own ----
+GEOM = np.load(os.path.join(os.path.dirname(__file__), "golden", "cp4_golden_geometry.npz"))
+GEOM_CASES = sorted({k.split(".")[0] for k in GEOM.files})
+
+
+def geom_gold(oracle, name):
+    g = {k: GEOM[f"{name}.{k}"] for k in
+         ("x", "dy", "FK", "FC", "FH", "FW", "y", "dx", "dFK", "dFC", "dFH", "dFW")}
+    g["geometry"] = oracle.Geometry(*[int(v) for v in GEOM[name + ".geometry"]])
+    return g
+
+
+@pytest.mark.parametrize("name", GEOM_CASES)
+def test_geometry_forward_golden(oracle, name):
+    g = geom_gold(oracle, name)
+    f = [g[k] for k in ("FK", "FC", "FH", "FW")]
+    close(oracle.forward_geom(g["x"], *f, g["geometry"], direct=True), g["y"], 2e-5)
+    close(oracle.forward_geom(g["x"], *f, g["geometry"], direct=False), g["y"], 2e-5)
+
+
+@pytest.mark.parametrize("name", GEOM_CASES)
+def test_geometry_backward_golden(oracle, name):
+    g = geom_gold(oracle, name)
+    f = [g[k] for k in ("FK", "FC", "FH", "FW")]
+    dx = oracle.backward_data_geom(g["dy"], g["x"].shape[2:], *f, g["geometry"])
+    close(dx, g["dx"], 2e-5)
+    grads = oracle.backward_filter_geom(g["x"], g["dy"], *f, g["geometry"])
+    for got, k in zip(grads, ("dFK", "dFC", "dFH", "dFW")):
+        close(got, g[k], 1e-4)
+
+
+def test_geometry_same_padding_formula(oracle):
+    """The framework's SAME rule on an even size: 8 -> 4 at stride 2 with a 3x3
+    filter pads 0 before and 1 after, so window o starts at input row 2o; the
+    symmetric padding=1 of a same-named PyTorch layer starts it at 2o - 1."""
+    g = oracle.geometry_same(8, 8, 3, 3, 2)
+    assert (g.pad_top, g.pad_left, g.out_h, g.out_w) == (0, 0, 4, 4)
+    g = oracle.geometry_same(9, 7, 3, 3, 2)
+    assert (g.pad_top, g.pad_left, g.out_h, g.out_w) == (1, 1, 5, 4)
+    g = oracle.geometry_same(13, 13, 7, 7, 3)
+    assert (g.pad_top, g.out_h) == (3, 5)
+    g = oracle.geometry_valid(11, 12, 5, 5, 2)
+    assert (g.pad_top, g.out_h, g.out_w) == (0, 4, 4)
+    # an impulse at input row 2, column 2 under SAME / stride 2 / 3x3 on 8x8: output
+    # (1, 1) sees it through tap (0, 0), output (0, 0) through tap (2, 2)
+    x = np.zeros((1, 1, 8, 8), np.float32)
+    x[0, 0, 2, 2] = 1.0
+    FK = np.ones((1, 1), np.float32)
+    FC = np.ones((1, 1), np.float32)
+    FH = np.array([[1.0], [10.0], [100.0]], np.float32)
+    FW = np.array([[1.0], [2.0], [3.0]], np.float32)
+    y = oracle.forward_geom(x, FK, FC, FH, FW, oracle.geometry_same(8, 8, 3, 3, 2), direct=True)
+    assert y[0, 0, 1, 1] == 1.0 and y[0, 0, 0, 0] == 300.0 and y[0, 0, 1, 0] == 3.0 \
+        and y[0, 0, 0, 1] == 100.0
+
+
+def test_geometry_reduces_to_the_reference_case(oracle):
+    """Stride 1, pad zeros before, an H x W output: the reference's own operator."""
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((2, 3, 6, 7)).astype(np.float32)
+    dy = rng.standard_normal((2, 4, 6, 7)).astype(np.float32)
+    f = [rng.standard_normal((d, 3)).astype(np.float32) for d in (4, 3, 3, 3)]
+    g = oracle.Geometry(1, 1, 1, 1, 6, 7)
+    close(oracle.forward_geom(x, *f, g, direct=True), oracle.forward(x, *f, 1, direct=True), 1e-6)
+    close(oracle.backward_data_geom(dy, (6, 7), *f, g), oracle.backward_data(dy, *f, 1, direct=True), 1e-6)
+    for a, b in zip(oracle.backward_filter_geom(x, dy, *f, g),
+                    oracle.backward_filter(x, dy, *f, 1, direct=True)):
+        close(a, b, 1e-6)
