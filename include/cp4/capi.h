@@ -121,6 +121,21 @@ cp4_status cp4_conv2d_backward_data_bf16(const cp4_shape* shape, const void* dy_
                                          const float* FK, const float* FC,
                                          const float* FH, const float* FW,
                                          void* dx_bf16, cp4_stream stream);
+/* The same two passes with IEEE half-precision (fp16) activations in memory: a
+ * half is exactly two bfloat16 parts, so the products with the fp32 factors are
+ * still exact; y / dx are rounded once, to nearest-even (values beyond 65504
+ * become infinities, as in any fp16 store).  Same shape limits as the bfloat16
+ * entry points (cp4_bf16_supported answers for both).  There is no fp16
+ * backward-filter entry: widen x and dy and use the fp32 one. */
+cp4_status cp4_conv2d_forward_f16(const cp4_shape* shape, const void* x_f16,
+                                  const float* FK, const float* FC,
+                                  const float* FH, const float* FW,
+                                  const float* bias, int activation,
+                                  void* y_f16, cp4_stream stream);
+cp4_status cp4_conv2d_backward_data_f16(const cp4_shape* shape, const void* dy_f16,
+                                        const float* FK, const float* FC,
+                                        const float* FH, const float* FW,
+                                        void* dx_f16, cp4_stream stream);
 /* Backward-filter with bfloat16 x and dy in memory; factors, gradients, the
  * workspace (cp4_conv2d_backward_filter_workspace_bytes) and all arithmetic stay
  * fp32.  Matrix-core path only: Rank <= 64, C and T multiples of 16
@@ -381,6 +396,41 @@ cp4_status cp3_conv2d_backward_data(const cp4_shape* shape, const float* dy,
                                     const float* K0, const float* K1,
                                     const float* K2, float* dx, void* workspace,
                                     size_t workspace_bytes, cp4_stream stream);
+
+/* ---- reshaped-CP sibling op -------------------------------------------------
+ * Stands where the reference registers its TensorFlow op Conv2dRcpFusedNchw
+ * (Kernels/rcp_fused_nchw.cc:6-12, launcher Conv2dRcpFusedNchwKernelLauncher :32; a
+ * generated kernel for the single shape 1 x (4,4) x 32 x 32, rank 11; defined by
+ * test/test_conv2d_rcp.py:38-41 and the layer test/layers.py:687-760): the C = S0*S1
+ * input channels are the pairs (a,b) of a grid, the T = T0*T1 output channels the
+ * pairs (x,y), and
+ *   y[n,(x,y),h,w] = sum_{a,b,i,j,r} K0[a,x,r] K1[b,y,r] KC[i,j,r] x[n,(a,b),h+i-pad,w+j-pad]
+ * with K0 [S0,T0,Rank], K1 [S1,T1,Rank], KC [Y,X,Rank], channel (a,b) = a*S1 + b.
+ * Each rank couples every input channel with every output channel, so there is no
+ * [N,Rank,H,W] intermediate to pass through as in the CP ops; for the channel
+ * counts the op is meant for (16 in the reference) the cheaper order is the dense
+ * filter, recomposed on the device, in a direct convolution (the recomposed-filter
+ * kernel of the CP4 passes).  Square odd filters up to 17x17, pad <= Y - 1,
+ * 8*C*Y*X <= 8192; CP4_ERR_UNSUPPORTED beyond.  shape->C and shape->T must equal
+ * S0*S1 and T0*T1.  `workspace`: device memory of rcp_conv2d_workspace_bytes (the
+ * dense filter and, for the factor gradients, its gradient).  The input gradient
+ * follows the reference's backward-data convention (reversed taps at offset
+ * +y-pad): the adjoint of the forward when 2*pad = Y-1 = X-1. */
+typedef struct rcp_dims {
+  unsigned S0, S1, T0, T1;
+} rcp_dims;
+size_t rcp_conv2d_workspace_bytes(const cp4_shape* shape, const rcp_dims* dims);
+cp4_status rcp_conv2d_forward(const cp4_shape* shape, const rcp_dims* dims, const float* x,
+                              const float* K0, const float* K1, const float* KC, float* y,
+                              void* workspace, size_t workspace_bytes, cp4_stream stream);
+cp4_status rcp_conv2d_backward_data(const cp4_shape* shape, const rcp_dims* dims, const float* dy,
+                                    const float* K0, const float* K1, const float* KC, float* dx,
+                                    void* workspace, size_t workspace_bytes, cp4_stream stream);
+cp4_status rcp_conv2d_backward_filter(const cp4_shape* shape, const rcp_dims* dims,
+                                      const float* x, const float* dy, const float* K0,
+                                      const float* K1, const float* KC, float* dK0, float* dK1,
+                                      float* dKC, void* workspace, size_t workspace_bytes,
+                                      cp4_stream stream);
 
 /* ---- test / bench utilities (Cuda_kernels/Utils.cuh:9-13) ---------------- */
 

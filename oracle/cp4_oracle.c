@@ -15,6 +15,9 @@
  *        comparator     Cuda_kernels/Utils.cu:143-156
  *        3-factor CP    test/layers.py:265-282 (forward only; its gradients are
  *                       checked against float64 autograd in the GPU tests)
+ *        reshaped CP    test/test_conv2d_rcp.py:38-41 (forward only, likewise)
+ *        strides etc.   test/layers.py:264-279 (section 1b: all three passes with a
+ *                       stride, explicit padding and an output plane of its own)
  *
  *  (2) "unfused" functions: the factor-by-factor sequence
  *        1x1 conv by FC -> depthwise 1-D conv by FH -> depthwise 1-D conv by
@@ -449,6 +452,51 @@ int cp4o_forward_geom_unfused(const cp4o_shape* s, const cp4o_geometry* g, const
     free(cc);
   }
   return fail;
+}
+
+/* ------------------------------------------------------------------------ */
+/* (1c) reshaped-CP sibling op                                               */
+/* ------------------------------------------------------------------------ */
+
+/* The reference's third fused op, Conv2dRcpFusedNchw (Kernels/rcp_fused_nchw.cc:6-12,
+ * a generated kernel for the single shape 1 x (4,4) x 32 x 32, rank 11), as its test
+ * defines it (test/test_conv2d_rcp.py:38-41): the input channels are the pairs (a, b)
+ * of an S0 x S1 grid, the output channels the pairs (x, y) of a T0 x T1 grid, and the
+ * dense filter is einsum('axr,byr,hwr->hwabxy') of K0 [S0,T0,R], K1 [S1,T1,R],
+ * KC [Y,X,R], used in a "SAME" convolution:
+ *   Out[n,(x,y),h,w] = sum_{a,b,i,j,r} K0[a,x,r] K1[b,y,r] KC[i,j,r]
+ *                      In[n,(a,b),h+i-pad,w+j-pad]
+ * with channel (a,b) = a*S1 + b and (x,y) = x*T1 + y (row-major reshapes).  s->C must
+ * be S0*S1 and s->T = T0*T1.  Pinned in tests/test_oracle.py against torch's dense
+ * conv2d on that einsum. */
+void rcpo_forward_direct(const cp4o_shape* s, unsigned S0, unsigned S1, unsigned T0,
+                         unsigned T1, const float* In, const float* K0, const float* K1,
+                         const float* KC, float* Out) {
+  const long N = s->N, H = s->H, W = s->W, P = s->pad, Y = s->Y, X = s->X, R = s->Rank;
+  const long C = (long)S0 * S1, T = (long)T0 * T1;
+#pragma omp parallel for collapse(2) schedule(dynamic)
+  for (long n = 0; n < N; ++n)
+    for (long t = 0; t < T; ++t) {
+      const long x = t / T1, y = t % T1;
+      for (long h = 0; h < H; ++h)
+        for (long w = 0; w < W; ++w) {
+          double acc = 0.0;
+          for (long r = 0; r < R; ++r) {
+            double cacc = 0.0;
+            for (long c = 0; c < C; ++c) {
+              const long a = c / S1, b = c % S1;
+              const float* ip = In + (n * C + c) * H * W;
+              double pix = 0.0;
+              for (long i = 0; i < Y; ++i)
+                for (long j = 0; j < X; ++j)
+                  pix += rd(ip, h + i - P, w + j - P, H, W) * (double)KC[(i * X + j) * R + r];
+              cacc += pix * (double)K0[(a * T0 + x) * R + r] * (double)K1[(b * T1 + y) * R + r];
+            }
+            acc += cacc;
+          }
+          Out[((n * T + t) * H + h) * W + w] = (float)acc;
+        }
+    }
 }
 
 /* Number of elements whose symmetric relative error exceeds tol; absolute

@@ -92,6 +92,21 @@ def cp3_forward(x, K0, K1, K2, pad):
     return y
 
 
+def rcp_forward(x, K0, K1, KC, pad):
+    """Reshaped-CP forward: K0 [S0,T0,R], K1 [S1,T1,R], KC [Y,X,R]; x has S0*S1 channels."""
+    x, K0, K1, KC = map(_f32, (x, K0, K1, KC))
+    N, C, H, W = x.shape
+    S0, T0, R = K0.shape
+    S1, T1, _ = K1.shape
+    assert C == S0 * S1 and K1.shape[2] == R and KC.shape[2] == R
+    s = Shape(N=N, H=H, W=W, pad=pad, T=T0 * T1, C=C, Y=KC.shape[0], X=KC.shape[1], Rank=R)
+    y = np.empty((N, s.T, H, W), np.float32)
+    lib().rcpo_forward_direct(ctypes.byref(s), ctypes.c_uint(S0), ctypes.c_uint(S1),
+                              ctypes.c_uint(T0), ctypes.c_uint(T1), _fp(x), _fp(K0), _fp(K1),
+                              _fp(KC), _fp(y))
+    return y
+
+
 def backward_data(dy, FK, FC, FH, FW, pad, direct=False):
     dy, FK, FC, FH, FW = map(_f32, (dy, FK, FC, FH, FW))
     N, T, H, W = dy.shape

@@ -38,6 +38,11 @@ class Geometry(ctypes.Structure):
         return "Geometry(" + ", ".join(f"{k}={getattr(self, k)}" for k, _ in self._fields_) + ")"
 
 
+class RcpDims(ctypes.Structure):
+    """rcp_dims: the channel grids of the reshaped-CP op (C = S0*S1, T = T0*T1)."""
+    _fields_ = [(k, ctypes.c_uint) for k in ("S0", "S1", "T0", "T1")]
+
+
 # status codes of cp4_status
 (OK, ERR_NULL_POINTER, ERR_SHAPE, ERR_HIP, ERR_WORKSPACE, ERR_UNSUPPORTED,
  ERR_DEVICE) = range(7)
@@ -85,6 +90,18 @@ def lib():
                                                                     ctypes.c_void_p]
     L.cp4_conv2d_backward_filter_ex.argtypes = [_S, _G] + [_F] * 10 + [ctypes.c_void_p,
                                                                        ctypes.c_size_t, ctypes.c_void_p]
+    _D = ctypes.POINTER(RcpDims)
+    L.rcp_conv2d_workspace_bytes.restype = ctypes.c_size_t
+    L.rcp_conv2d_workspace_bytes.argtypes = [_S, _D]
+    L.rcp_conv2d_forward.argtypes = [_S, _D] + [_F] * 5 + [ctypes.c_void_p, ctypes.c_size_t,
+                                                           ctypes.c_void_p]
+    L.rcp_conv2d_backward_data.argtypes = L.rcp_conv2d_forward.argtypes
+    L.rcp_conv2d_backward_filter.argtypes = [_S, _D] + [_F] * 8 + [ctypes.c_void_p, ctypes.c_size_t,
+                                                                   ctypes.c_void_p]
+    L.cp4_conv2d_forward_f16.argtypes = [_S, ctypes.c_void_p, _F, _F, _F, _F, _F, ctypes.c_int,
+                                         ctypes.c_void_p, ctypes.c_void_p]
+    L.cp4_conv2d_backward_data_f16.argtypes = [_S, ctypes.c_void_p, _F, _F, _F, _F,
+                                               ctypes.c_void_p, ctypes.c_void_p]
     L.cp4_bf16_supported.argtypes = [_S, ctypes.c_int]
     L.cp4_conv2d_forward_bf16.argtypes = [_S, ctypes.c_void_p, _F, _F, _F, _F, _F, ctypes.c_int,
                                           ctypes.c_void_p, ctypes.c_void_p]
@@ -276,9 +293,86 @@ def conv2d_backward_filter_ex(x, dy, FK, FC, FH, FW, g, workspace=None, stream=N
     return tuple(outs)
 
 
-def _ptr16(t):
-    assert t.is_cuda and t.is_contiguous() and t.dtype == torch.bfloat16
+def _ptr16(t, dtype=torch.bfloat16):
+    assert t.is_cuda and t.is_contiguous() and t.dtype == dtype
     return ctypes.c_void_p(t.data_ptr())
+
+
+def conv2d_forward_f16(x, FK, FC, FH, FW, bias=None, activation=None, pad=1, out=None,
+                       stream=None):
+    """float16 x -> float16 y = act(conv(x) + bias); fp32 factors, bias and arithmetic."""
+    s = shape_for(x.shape, FK, FC, FH, FW, pad)
+    assert x.shape[1] == s.C and FC.shape[1] == s.Rank
+    y = out if out is not None else torch.empty((s.N, s.T, s.H, s.W), device=x.device,
+                                                dtype=torch.float16)
+    check(lib().cp4_conv2d_forward_f16(
+        ctypes.byref(s), _ptr16(x, torch.float16), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
+        _ptr(bias) if bias is not None else None, ACTIVATIONS[activation],
+        _ptr16(y, torch.float16), _stream(stream)))
+    return y
+
+
+def conv2d_backward_data_f16(dy, FK, FC, FH, FW, pad=1, out=None, stream=None):
+    """float16 dy -> float16 dx; fp32 factors and arithmetic."""
+    s = shape_for(dy.shape, FK, FC, FH, FW, pad)
+    assert dy.shape[1] == s.T
+    dx = out if out is not None else torch.empty((s.N, s.C, s.H, s.W), device=dy.device,
+                                                 dtype=torch.float16)
+    check(lib().cp4_conv2d_backward_data_f16(
+        ctypes.byref(s), _ptr16(dy, torch.float16), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
+        _ptr16(dx, torch.float16), _stream(stream)))
+    return dx
+
+
+def _rcp_shape(act_shape, K0, K1, KC, pad):
+    N, _, H, W = act_shape
+    S0, T0, R = K0.shape
+    S1, T1, _ = K1.shape
+    assert K1.shape[2] == R and KC.shape[2] == R
+    s = Shape(N=N, H=H, W=W, pad=pad, T=T0 * T1, C=S0 * S1, Y=KC.shape[0], X=KC.shape[1], Rank=R)
+    return s, RcpDims(S0, S1, T0, T1)
+
+
+def _rcp_workspace(s, d, device):
+    n = int(lib().rcp_conv2d_workspace_bytes(ctypes.byref(s), ctypes.byref(d)))
+    return torch.empty(n + 256, device=device, dtype=torch.uint8), n + 256
+
+
+def rcp_conv2d_forward(x, K0, K1, KC, pad=1, out=None, stream=None):
+    """Reshaped-CP op: x [N,S0*S1,H,W], K0 [S0,T0,R], K1 [S1,T1,R], KC [Y,X,R] -> [N,T0*T1,H,W]."""
+    s, d = _rcp_shape(x.shape, K0, K1, KC, pad)
+    assert x.shape[1] == s.C
+    y = out if out is not None else torch.empty((s.N, s.T, s.H, s.W), device=x.device,
+                                                dtype=torch.float32)
+    ws, n = _rcp_workspace(s, d, x.device)
+    check(lib().rcp_conv2d_forward(ctypes.byref(s), ctypes.byref(d), _ptr(x), _ptr(K0), _ptr(K1),
+                                   _ptr(KC), _ptr(y), ctypes.c_void_p(ws.data_ptr()), n,
+                                   _stream(stream)))
+    return y
+
+
+def rcp_conv2d_backward_data(dy, K0, K1, KC, pad=1, out=None, stream=None):
+    s, d = _rcp_shape(dy.shape, K0, K1, KC, pad)
+    assert dy.shape[1] == s.T
+    dx = out if out is not None else torch.empty((s.N, s.C, s.H, s.W), device=dy.device,
+                                                 dtype=torch.float32)
+    ws, n = _rcp_workspace(s, d, dy.device)
+    check(lib().rcp_conv2d_backward_data(ctypes.byref(s), ctypes.byref(d), _ptr(dy), _ptr(K0),
+                                         _ptr(K1), _ptr(KC), _ptr(dx),
+                                         ctypes.c_void_p(ws.data_ptr()), n, _stream(stream)))
+    return dx
+
+
+def rcp_conv2d_backward_filter(x, dy, K0, K1, KC, pad=1, stream=None):
+    """(dK0, dK1, dKC)."""
+    s, d = _rcp_shape(x.shape, K0, K1, KC, pad)
+    assert tuple(dy.shape) == (s.N, s.T, s.H, s.W)
+    outs = [torch.empty_like(t) for t in (K0, K1, KC)]
+    ws, n = _rcp_workspace(s, d, x.device)
+    check(lib().rcp_conv2d_backward_filter(
+        ctypes.byref(s), ctypes.byref(d), _ptr(x), _ptr(dy), _ptr(K0), _ptr(K1), _ptr(KC),
+        *[_ptr(o) for o in outs], ctypes.c_void_p(ws.data_ptr()), n, _stream(stream)))
+    return tuple(outs)
 
 
 def bf16_supported(s, backward_data=False):

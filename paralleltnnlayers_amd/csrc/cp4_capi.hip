@@ -243,7 +243,9 @@ constexpr int kMatrixMinRank = 2;
 // against 25 us matrix-core, C128 K1 107 against 43; 17x17 C3 K1: 24 against 240
 // us general at R16, 22 against 13 at R1.)
 double dense_small_estimate(const FwdArgs& a) {
-  return 8.0 + 0.155 * a.Cin * a.Y * (a.X + 3) / 4.0 + 0.0025 * a.Cout * a.Cin * a.Y * a.X;
+  const int groups = (a.Cout + 7) / 8;       // the segment reads repeat per group of 8 outputs
+  return 8.0 + 0.155 * groups * a.Cin * a.Y * (a.X + 3) / 4.0 +
+         0.0025 * a.Cout * a.Cin * a.Y * a.X;
 }
 constexpr double kMatrixSmallChannelEstimate = 26.0;
 double general_estimate(const FwdArgs& a) {
@@ -536,6 +538,48 @@ cp4_status cp4_conv2d_backward_data_bf16(const cp4_shape* shape, const void* dy_
   if (!cp4::fwd_pipe_io16_supported(a))
     return fail(CP4_ERR_UNSUPPORTED, "bfloat16 I/O: shape not taken by the producer/consumer kernel");
   CP4_HIP(cp4::fwd_pipe_io16_launch(a, as_stream(stream)));
+  return CP4_OK;
+}
+
+cp4_status cp4_conv2d_forward_f16(const cp4_shape* shape, const void* x_f16,
+                                   const float* FK, const float* FC,
+                                   const float* FH, const float* FW,
+                                   const float* bias, int activation,
+                                   void* y_f16, cp4_stream stream) {
+  if (activation != CP4_ACT_NONE && activation != CP4_ACT_RELU)
+    return fail(CP4_ERR_UNSUPPORTED, "activation must be CP4_ACT_NONE or CP4_ACT_RELU");
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return CP4_OK;
+  rc = check_forward_ptrs(x_f16, FK, FC, FH, FW, y_f16);
+  if (rc != CP4_OK) return rc;
+  // the kernel reads FwdArgs::x / y as 16-bit elements
+  FwdArgs a = forward_args(*shape, static_cast<const float*>(x_f16), FK, FC, FH, FW,
+                           static_cast<float*>(y_f16));
+  a.bias = bias;
+  a.act = activation;
+  arm(a);
+  if (!cp4::fwd_pipe_iof16_supported(a))
+    return fail(CP4_ERR_UNSUPPORTED, "half-precision I/O: shape not taken by the producer/consumer kernel");
+  CP4_HIP(cp4::fwd_pipe_iof16_launch(a, as_stream(stream)));
+  return CP4_OK;
+}
+
+cp4_status cp4_conv2d_backward_data_f16(const cp4_shape* shape, const void* dy_f16,
+                                         const float* FK, const float* FC,
+                                         const float* FH, const float* FW,
+                                         void* dx_f16, cp4_stream stream) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return CP4_OK;
+  rc = check_forward_ptrs(dy_f16, FK, FC, FH, FW, dx_f16);
+  if (rc != CP4_OK) return rc;
+  FwdArgs a = backward_data_args(*shape, static_cast<const float*>(dy_f16), FK, FC, FH, FW,
+                                 static_cast<float*>(dx_f16));
+  arm(a);
+  if (!cp4::fwd_pipe_iof16_supported(a))
+    return fail(CP4_ERR_UNSUPPORTED, "half-precision I/O: shape not taken by the producer/consumer kernel");
+  CP4_HIP(cp4::fwd_pipe_iof16_launch(a, as_stream(stream)));
   return CP4_OK;
 }
 
@@ -1295,6 +1339,93 @@ cp4_status cp3_conv2d_backward_data(const cp4_shape* shape, const float* dy, con
                                     void* workspace, size_t workspace_bytes,
                                     cp4_stream stream) {
   return cp3_run(shape, dy, K0, K1, K2, dx, workspace, workspace_bytes, true, stream);
+}
+
+// ---- reshaped-CP sibling op ------------------------------------------------------
+
+namespace {
+cp4_status rcp_check(const cp4_shape* s, const rcp_dims* d) {
+  cp4_status rc = check_shape(s);
+  if (rc != CP4_OK) return rc;
+  if (!d) return fail(CP4_ERR_NULL_POINTER, "dims is NULL");
+  if (!d->S0 || !d->S1 || !d->T0 || !d->T1 ||
+      (unsigned long long)d->S0 * d->S1 != s->C || (unsigned long long)d->T0 * d->T1 != s->T)
+    return fail(CP4_ERR_SHAPE, "S0*S1 must equal C and T0*T1 must equal T");
+  return CP4_OK;
+}
+size_t rcp_filter_floats(const cp4_shape& s) { return (size_t)s.T * s.C * s.Y * s.X; }
+
+// One dense pass of the op on the recomposed filter in `K`.
+cp4_status rcp_dense_pass(const cp4_shape& s, const float* in, float* out, const float* K,
+                          bool backward, hipStream_t st) {
+  FwdArgs a{};
+  a.x = in; a.y = out; a.dense = K;
+  a.N = s.N; a.Cin = backward ? s.T : s.C; a.Cout = backward ? s.C : s.T;
+  a.H = s.H; a.W = s.W; a.pad = s.pad; a.Y = s.Y; a.X = s.X; a.R = s.Rank;
+  if (!cp4::fwd_dense_small_supported(a))
+    return fail(CP4_ERR_UNSUPPORTED,
+                "reshaped-CP op: square odd filters up to 17x17, pad <= Y-1, 8*C*Y*X <= 8192");
+  CP4_HIP(cp4::fwd_dense_small_launch(a, st));
+  return CP4_OK;
+}
+}  // namespace
+
+size_t rcp_conv2d_workspace_bytes(const cp4_shape* s, const rcp_dims* d) {
+  if (rcp_check(s, d) != CP4_OK) return 0;
+  return 2 * align256(rcp_filter_floats(*s) * sizeof(float));
+}
+
+cp4_status rcp_conv2d_forward(const cp4_shape* shape, const rcp_dims* d, const float* x,
+                              const float* K0, const float* K1, const float* KC, float* y,
+                              void* workspace, size_t workspace_bytes, cp4_stream stream) {
+  cp4_status rc = rcp_check(shape, d);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return CP4_OK;
+  if (!x || !K0 || !K1 || !KC || !y) return fail(CP4_ERR_NULL_POINTER, "a data pointer is NULL");
+  if (!workspace || workspace_bytes < rcp_conv2d_workspace_bytes(shape, d))
+    return fail(CP4_ERR_WORKSPACE, "workspace smaller than rcp_conv2d_workspace_bytes");
+  hipStream_t st = as_stream(stream);
+  float* K = static_cast<float*>(workspace);
+  CP4_HIP(cp4::rcp_recompose_launch(K0, K1, KC, K, d->S0, d->S1, d->T0, d->T1, shape->Y, shape->X,
+                                    shape->Rank, 0, st));
+  return rcp_dense_pass(*shape, x, y, K, false, st);
+}
+
+cp4_status rcp_conv2d_backward_data(const cp4_shape* shape, const rcp_dims* d, const float* dy,
+                                    const float* K0, const float* K1, const float* KC, float* dx,
+                                    void* workspace, size_t workspace_bytes, cp4_stream stream) {
+  cp4_status rc = rcp_check(shape, d);
+  if (rc != CP4_OK) return rc;
+  if (shape->N == 0) return CP4_OK;
+  if (!dy || !K0 || !K1 || !KC || !dx) return fail(CP4_ERR_NULL_POINTER, "a data pointer is NULL");
+  if (!workspace || workspace_bytes < rcp_conv2d_workspace_bytes(shape, d))
+    return fail(CP4_ERR_WORKSPACE, "workspace smaller than rcp_conv2d_workspace_bytes");
+  hipStream_t st = as_stream(stream);
+  float* K = static_cast<float*>(workspace);
+  CP4_HIP(cp4::rcp_recompose_launch(K0, K1, KC, K, d->S0, d->S1, d->T0, d->T1, shape->Y, shape->X,
+                                    shape->Rank, 1, st));
+  return rcp_dense_pass(*shape, dy, dx, K, true, st);
+}
+
+cp4_status rcp_conv2d_backward_filter(const cp4_shape* shape, const rcp_dims* d, const float* x,
+                                      const float* dy, const float* K0, const float* K1,
+                                      const float* KC, float* dK0, float* dK1, float* dKC,
+                                      void* workspace, size_t workspace_bytes,
+                                      cp4_stream stream) {
+  cp4_status rc = rcp_check(shape, d);
+  if (rc != CP4_OK) return rc;
+  if (!K0 || !K1 || !KC || !dK0 || !dK1 || !dKC)
+    return fail(CP4_ERR_NULL_POINTER, "a factor or gradient pointer is NULL");
+  if (!workspace || workspace_bytes < rcp_conv2d_workspace_bytes(shape, d))
+    return fail(CP4_ERR_WORKSPACE, "workspace smaller than rcp_conv2d_workspace_bytes");
+  hipStream_t st = as_stream(stream);
+  // dense filter gradient (cp4Conv2dBackwardFilter.cu:23-59), then the chain rule
+  float* dK = static_cast<float*>(workspace) + align256(rcp_filter_floats(*shape) * sizeof(float)) / sizeof(float);
+  rc = cp4_conv2d_backward_filter_full(shape, x, dy, dK, 0, stream);
+  if (rc != CP4_OK) return rc;
+  CP4_HIP(cp4::rcp_fold_launch(dK, K0, K1, KC, dK0, dK1, dKC, d->S0, d->S1, d->T0, d->T1, shape->Y,
+                               shape->X, shape->Rank, st));
+  return CP4_OK;
 }
 
 cp4_status cp4_count_exceeding(const float* A, const float* B, size_t n,

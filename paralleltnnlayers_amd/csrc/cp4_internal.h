@@ -48,6 +48,9 @@ struct FwdArgs {
   // the output plane is Ho x Wo.  sh == 0: the reference's geometry, the other
   // fields unused.  Only kernels that say so take sh != 0.
   int sh, sw, pt, pl, Ho, Wo;
+  // Recomposed-filter kernel only: the dense filter [Cout, Cin, Y, X] itself, taps in
+  // the order the pass reads them; the four factors are unused then.
+  const float* dense;
 };
 
 // The geometry of a launch with the defaults filled in.
@@ -90,6 +93,9 @@ hipError_t fwd_pipe_epi_launch(const FwdArgs&, hipStream_t);
 // 16-bit elements; factors and bias stay fp32), epilogue included.
 bool fwd_pipe_io16_supported(const FwdArgs&);
 hipError_t fwd_pipe_io16_launch(const FwdArgs&, hipStream_t);
+// The same with IEEE half-precision x and y in memory.
+bool fwd_pipe_iof16_supported(const FwdArgs&);
+hipError_t fwd_pipe_iof16_launch(const FwdArgs&, hipStream_t);
 // The same kernel honouring FwdArgs::ldf and FwdArgs::accumulate (rank passes).
 bool fwd_pipe_rankpass_supported(const FwdArgs&);
 hipError_t fwd_pipe_rankpass_launch(const FwdArgs&, hipStream_t);
@@ -149,6 +155,15 @@ hipError_t cp3_fold_launch(const cp4_shape& s, const float* dFK, const float* dF
 // set into canvases of Hc x Wc; every other canvas cell is written as zero.
 hipError_t embed_launch(const float* src, float* dst, size_t planes, int h, int w, int Hc, int Wc,
                         int ot, int ol, int sh, int sw, hipStream_t);
+// Reshaped-CP sibling op: its dense filter (transposed != 0: the input-gradient
+// pass's filter [C][T][Y][X], taps reversed) and the fold of a dense filter
+// gradient [T][C][Y][X] back onto K0 [S0,T0,R], K1 [S1,T1,R], KC [Y,X,R].
+hipError_t rcp_recompose_launch(const float* K0, const float* K1, const float* KC, float* out,
+                                int S0, int S1, int T0, int T1, int Y, int X, int R,
+                                int transposed, hipStream_t);
+hipError_t rcp_fold_launch(const float* dK, const float* K0, const float* K1, const float* KC,
+                           float* dK0, float* dK1, float* dKC, int S0, int S1, int T0, int T1,
+                           int Y, int X, int R, hipStream_t);
 // dst [cols, rows] = transpose of src [rows, cols]
 hipError_t transpose_f32_launch(const float* src, float* dst, int rows, int cols, hipStream_t);
 hipError_t copy_f32_launch(float* dst, const float* src, size_t n, hipStream_t);

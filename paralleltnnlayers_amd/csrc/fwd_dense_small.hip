@@ -11,7 +11,9 @@
 // only where the recomposed order is the cheaper one.
 //
 // One workgroup (256 threads) owns `tpw` vertically adjacent tiles of 16 rows x
-// 64 columns of one image:
+// 64 columns of one image and up to eight output channels (more output channels:
+// more workgroups).  With FwdArgs::dense the filter K is given instead of the
+// factors (the reshaped-CP sibling op recomposes its own):
 //   prologue  the four factors go to LDS, then every workgroup recomposes K into
 //             LDS itself (Cout*Cin*Y*X*R multiply-adds: a few thousand, no scratch
 //             memory, no extra launch; the tiles of a workgroup share it)
@@ -38,40 +40,51 @@ struct DensePlan {
   int cc;        // input channels per chunk
   int tile_w;    // LDS row length of the tile (floats, odd: conflict-free segment reads)
   int tpw;       // tiles per workgroup, down the image
+  int wfloats;   // LDS floats set aside for a workgroup's filter (a multiple of 4)
   size_t lds_bytes;
 };
 
 template <int FS, int KO>
 __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, DensePlan pl) {
   extern __shared__ float lds[];
-  const int Cin = a.Cin, Cout = a.Cout, R = a.R, H = a.H, W = a.W;
+  const int Cin = a.Cin, R = a.R, H = a.H, W = a.W;
+  // output channels in groups of eight, one group per workgroup (blockIdx.z = image, group)
+  const int ngrp = (a.Cout + 7) >> 3;
+  const int n = blockIdx.z / ngrp, k0 = 8 * (blockIdx.z - n * ngrp);
+  const int Cout = min(8, a.Cout - k0);               // channels of this group
   const int nw = Cout * Cin * FS * FS;
   float* wts = lds;                                   // [Cout][Cin][FS][FS]
-  float* tile = lds + ((nw + 3) & ~3);                // [cc][kTH + FS - 1][tile_w]
+  float* tile = lds + pl.wfloats;                     // [cc][kTH + FS - 1][tile_w]
   const int tid = threadIdx.x;
-  const int n = blockIdx.z, w0 = blockIdx.x * kTW;
+  const int w0 = blockIdx.x * kTW;
   const size_t HW = (size_t)H * W;
 
-  // the factors once through LDS (they alias the tile, which is loaded later) ...
-  float* fo = tile;                                   // Fout [Cout][R]
-  float* fi = fo + Cout * R;                          // Fin  [Cin][R]
-  float* fh = fi + Cin * R;                           // FH   [FS][R]
-  float* fw = fh + FS * R;                            // FW   [FS][R]
-  for (int q = tid; q < Cout * R; q += kThreads) fo[q] = a.Fout[q];
-  for (int q = tid; q < Cin * R; q += kThreads) fi[q] = a.Fin[q];
-  for (int q = tid; q < FS * R; q += kThreads) {
-    fh[q] = a.FH[q];
-    fw[q] = a.FW[q];
-  }
-  __syncthreads();
-  // ... and the recomposed filter, taps already in the order this pass reads them
-  for (int q = tid; q < nw; q += kThreads) {
-    const int j = q % FS, i = (q / FS) % FS, c = (q / (FS * FS)) % Cin, k = q / (FS * FS * Cin);
-    const int ti = a.flip ? FS - 1 - i : i, tj = a.flip ? FS - 1 - j : j;
-    const float *p0 = fo + k * R, *p1 = fi + c * R, *p2 = fh + ti * R, *p3 = fw + tj * R;
-    float s = 0.f;
-    for (int r = 0; r < R; ++r) s += p0[r] * p1[r] * p2[r] * p3[r];
-    wts[q] = s;
+  if (a.dense) {
+    // the filter is given: [Cout][Cin][FS][FS], taps in the order this pass reads them
+    const float* src = a.dense + (size_t)k0 * Cin * FS * FS;
+    for (int q = tid; q < nw; q += kThreads) wts[q] = src[q];
+  } else {
+    // the factors once through LDS (they alias the tile, which is loaded later) ...
+    float* fo = tile;                                 // Fout [Cout][R]
+    float* fi = fo + Cout * R;                        // Fin  [Cin][R]
+    float* fh = fi + Cin * R;                         // FH   [FS][R]
+    float* fw = fh + FS * R;                          // FW   [FS][R]
+    for (int q = tid; q < Cout * R; q += kThreads) fo[q] = a.Fout[(size_t)k0 * R + q];
+    for (int q = tid; q < Cin * R; q += kThreads) fi[q] = a.Fin[q];
+    for (int q = tid; q < FS * R; q += kThreads) {
+      fh[q] = a.FH[q];
+      fw[q] = a.FW[q];
+    }
+    __syncthreads();
+    // ... and the recomposed filter, taps already in the order this pass reads them
+    for (int q = tid; q < nw; q += kThreads) {
+      const int j = q % FS, i = (q / FS) % FS, c = (q / (FS * FS)) % Cin, k = q / (FS * FS * Cin);
+      const int ti = a.flip ? FS - 1 - i : i, tj = a.flip ? FS - 1 - j : j;
+      const float *p0 = fo + k * R, *p1 = fi + c * R, *p2 = fh + ti * R, *p3 = fw + tj * R;
+      float s = 0.f;
+      for (int r = 0; r < R; ++r) s += p0[r] * p1[r] * p2[r] * p3[r];
+      wts[q] = s;
+    }
   }
 
   constexpr int kUnrollI = FS <= 5 ? FS : 1;         // filter rows unrolled only for small filters
@@ -158,7 +171,7 @@ __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, De
 
     const int h = h0 + ty, w = w0 + kPX * tx;
     if (h < H && w < W) {
-      float* yp = a.y + (size_t)n * Cout * HW + (size_t)h * W + w;
+      float* yp = a.y + ((size_t)n * a.Cout + k0) * HW + (size_t)h * W + w;
       const bool vec = vec_out && w + kPX <= W;
 #pragma unroll
       for (int k = 0; k < KO; ++k) {
@@ -179,12 +192,14 @@ __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, De
 
 bool plan(const FwdArgs& a, DensePlan* pl) {
   if (a.Y != a.X || !(a.Y & 1) || a.Y > 17 || a.pad > a.Y - 1) return false;
-  if (a.Cout > 8 || a.ldf || a.accumulate || a.sh) return false;
-  const long nw = (long)a.Cout * a.Cin * a.Y * a.X;
+  if (a.ldf || a.accumulate || a.sh) return false;
+  const int kgrp = a.Cout < 8 ? a.Cout : 8;           // output channels of a workgroup
+  const long ngrp = (a.Cout + 7) / 8;
+  const long nw = (long)kgrp * a.Cin * a.Y * a.X;
   if (nw > kMaxWeights) return false;
-  const long nf = (long)a.R * (a.Cout + a.Cin + a.Y + a.X);
+  const long nf = a.dense ? 0 : (long)a.R * (kgrp + a.Cin + a.Y + a.X);
   if (nf > kMaxFactorFloats) return false;
-  if (a.N > 65535) return false;
+  if ((long)a.N * ngrp > 65535) return false;
   // odd row length: the four-column segments of neighbouring threads fall on
   // different LDS banks
   const int tile_w = (kTW + a.Y - 1) | 1;
@@ -197,7 +212,7 @@ bool plan(const FwdArgs& a, DensePlan* pl) {
   // enough workgroups to fill the device a few times over, each amortising its
   // filter recomposition over several tiles
   const long row_tiles = (a.H + kTH - 1) / kTH, col_tiles = (a.W + kTW - 1) / kTW;
-  const long tiles = row_tiles * col_tiles * a.N;
+  const long tiles = row_tiles * col_tiles * a.N * ngrp;
   long tpw = tiles / (8l * num_compute_units());
   if (tpw < 1) tpw = 1;
   if (tpw > row_tiles) tpw = row_tiles;
@@ -206,7 +221,8 @@ bool plan(const FwdArgs& a, DensePlan* pl) {
   pl->cc = cc;
   pl->tile_w = tile_w;
   pl->tpw = (int)tpw;
-  pl->lds_bytes = (size_t)((nw + 3) & ~3l) * sizeof(float) + tile_bytes;
+  pl->wfloats = (int)((nw + 3) & ~3l);
+  pl->lds_bytes = (size_t)pl->wfloats * sizeof(float) + tile_bytes;
   return true;
 }
 
@@ -216,7 +232,8 @@ hipError_t launch_as(const FwdArgs& a, const DensePlan& pl, hipStream_t st) {
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds_bytes);
   if (e != hipSuccess) return e;
   const int row_tiles = (a.H + kTH - 1) / kTH;
-  const dim3 grid((a.W + kTW - 1) / kTW, (row_tiles + pl.tpw - 1) / pl.tpw, a.N);
+  const dim3 grid((a.W + kTW - 1) / kTW, (row_tiles + pl.tpw - 1) / pl.tpw,
+                  a.N * ((a.Cout + 7) / 8));
   fwd_dense_small_kernel<FS, KO><<<grid, kThreads, pl.lds_bytes, st>>>(a, pl);
   return hipGetLastError();
 }
@@ -226,7 +243,7 @@ hipError_t launch_ko(const FwdArgs& a, const DensePlan& pl, hipStream_t st) {
   if (a.Cout <= 1) return launch_as<FS, 1>(a, pl, st);
   if (a.Cout <= 2) return launch_as<FS, 2>(a, pl, st);
   if (a.Cout <= 4) return launch_as<FS, 4>(a, pl, st);
-  return launch_as<FS, 8>(a, pl, st);
+  return launch_as<FS, 8>(a, pl, st);              // groups of eight, the last one may be short
 }
 
 }  // namespace

@@ -47,7 +47,9 @@
 // x and y are bfloat16 in memory (factors, bias and all arithmetic stay fp32):
 // a bf16 activation is its own high part, so the channel contraction needs
 // neither the split nor the three MFMAs of the lower parts, and y is rounded to
-// nearest-even as pixel pairs (entry points fwd_pipe_io16_*, epilogue included);
+// nearest-even as pixel pairs (entry points fwd_pipe_io16_*, epilogue included;
+// CP4_PIPE_IO16=2: IEEE half precision instead - a half is two bfloat16 parts, five
+// MFMAs per chunk - entry points fwd_pipe_iof16_*);
 // and with CP4_PIPE_RANKPASS, the build behind the two-pass variant for ranks
 // 33-64: factor matrices with a row stride of their own (FwdArgs::ldf) and stores
 // that add to y (FwdArgs::accumulate), entry points fwd_pipe_rankpass_*;
@@ -82,9 +84,13 @@ namespace cp4 {
 namespace {
 
 #ifdef CP4_PIPE_IO16
-using io_t = unsigned short;     // bfloat16 bits
+using io_t = unsigned short;     // bfloat16 bits (CP4_PIPE_IO16 == 2: IEEE half bits)
 __device__ __forceinline__ unsigned short to_io(float v) {
+#if CP4_PIPE_IO16 == 2
+  return __builtin_bit_cast(unsigned short, static_cast<_Float16>(v));   // round to nearest even
+#else
   return __builtin_bit_cast(unsigned short, static_cast<__bf16>(v));   // round to nearest even
+#endif
 }
 #else
 using io_t = float;
@@ -359,7 +365,30 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       const unsigned xpn = geom(r + 1 < nrounds ? r + 1 : r, jn, qan, validn);
       f32x16 acc = (f32x16)(0.f);
       auto step = [&](int ch, int u) {
-#ifdef CP4_PIPE_IO16
+#if CP4_PIPE_IO16 == 2
+        // half-precision activations: 11 significand bits are two bfloat16 parts
+        // (h + m exactly, l = 0), so five of the six partial products remain
+        float xv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          xv[e] = (float)__builtin_bit_cast(_Float16, (unsigned short)xb[u][e]);
+        u32x4 xh, xm, xl;
+        split8(xv, xh, xm, xl);
+        if (FLDS) {
+          const u32x4* fp = fbase + (size_t)(ch + u) * (6 * 32);
+          acc = mfma16(fp[128], xh, acc);
+          acc = mfma16(fp[64], xm, acc);
+          acc = mfma16(fp[64], xh, acc);
+          acc = mfma16(fp[0], xm, acc);
+          acc = mfma16(fp[0], xh, acc);
+        } else {
+          acc = mfma16(fl[FLDS ? 0 : ch + u], xh, acc);
+          acc = mfma16(fm[FLDS ? 0 : ch + u], xm, acc);
+          acc = mfma16(fm[FLDS ? 0 : ch + u], xh, acc);
+          acc = mfma16(fh[FLDS ? 0 : ch + u], xm, acc);
+          acc = mfma16(fh[FLDS ? 0 : ch + u], xh, acc);
+        }
+#elif defined(CP4_PIPE_IO16)
         // the activations are bfloat16 already: pack pairs, multiply by the three
         // factor parts (smallest first)
         u32x4 xh;
@@ -1135,6 +1164,9 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 #elif defined(CP4_PIPE_RANKPASS)
 #define fwd_pipe_supported fwd_pipe_rankpass_supported
 #define fwd_pipe_launch fwd_pipe_rankpass_launch
+#elif defined(CP4_PIPE_IO16) && CP4_PIPE_IO16 == 2
+#define fwd_pipe_supported fwd_pipe_iof16_supported
+#define fwd_pipe_launch fwd_pipe_iof16_launch
 #elif defined(CP4_PIPE_IO16)
 #define fwd_pipe_supported fwd_pipe_io16_supported
 #define fwd_pipe_launch fwd_pipe_io16_launch

@@ -97,6 +97,79 @@ __global__ __launch_bounds__(256) void embed_kernel(const float* __restrict__ sr
   }
 }
 
+// Reshaped-CP op: its dense filter from K0 [S0,T0,R], K1 [S1,T1,R], KC [Y,X,R]
+// (test/test_conv2d_rcp.py:38-39): K[(x,y),(a,b),i,j] = sum_r K0[a,x,r] K1[b,y,r] KC[i,j,r].
+// transposed == 0: out[T][C][Y][X]; != 0: the filter of the input-gradient pass,
+// out[C][T][Y][X] with the taps reversed.
+__global__ __launch_bounds__(256) void rcp_recompose_kernel(
+    const float* __restrict__ K0, const float* __restrict__ K1, const float* __restrict__ KC,
+    float* __restrict__ out, int S0, int S1, int T0, int T1, int Y, int X, int R, int transposed) {
+  const int C = S0 * S1, T = T0 * T1;
+  const size_t total = (size_t)T * C * Y * X;
+  for (size_t q = (size_t)blockIdx.x * 256 + threadIdx.x; q < total; q += (size_t)gridDim.x * 256) {
+    const int j = (int)(q % X), i = (int)((q / X) % Y);
+    const int inner = (int)((q / ((size_t)X * Y)) % (transposed ? T : C));
+    const int outer = (int)(q / ((size_t)X * Y * (transposed ? T : C)));
+    const int t = transposed ? inner : outer, c = transposed ? outer : inner;
+    const int ti = transposed ? Y - 1 - i : i, tj = transposed ? X - 1 - j : j;
+    const int a = c / S1, b = c % S1, x = t / T1, y = t % T1;
+    const float *p0 = K0 + (size_t)(a * T0 + x) * R, *p1 = K1 + (size_t)(b * T1 + y) * R,
+                *p2 = KC + (size_t)(ti * X + tj) * R;
+    float s = 0.f;
+    for (int r = 0; r < R; ++r) s += p0[r] * p1[r] * p2[r];
+    out[q] = s;
+  }
+}
+
+// Chain rule from the dense filter gradient dK [T][C][Y][X] to the three factors:
+// element e of [dK0 | dK1 | dKC] sums dK times the other two factors, fixed order.
+__global__ __launch_bounds__(256) void rcp_fold_kernel(
+    const float* __restrict__ dK, const float* __restrict__ K0, const float* __restrict__ K1,
+    const float* __restrict__ KC, float* __restrict__ dK0, float* __restrict__ dK1,
+    float* __restrict__ dKC, int S0, int S1, int T0, int T1, int Y, int X, int R) {
+  const int C = S0 * S1;
+  const int n0 = S0 * T0 * R, n1 = S1 * T1 * R, n2 = Y * X * R;
+  for (int e = blockIdx.x * 256 + threadIdx.x; e < n0 + n1 + n2; e += gridDim.x * 256) {
+    float s = 0.f;
+    if (e < n0) {
+      const int r = e % R, x = (e / R) % T0, a = e / (R * T0);
+      for (int b = 0; b < S1; ++b)
+        for (int y = 0; y < T1; ++y) {
+          const float f1 = K1[(size_t)(b * T1 + y) * R + r];
+          const float* g = dK + ((size_t)(x * T1 + y) * C + a * S1 + b) * Y * X;
+          float u = 0.f;
+          for (int ij = 0; ij < Y * X; ++ij) u += g[ij] * KC[(size_t)ij * R + r];
+          s += f1 * u;
+        }
+      dK0[e] = s;
+    } else if (e < n0 + n1) {
+      const int q = e - n0, r = q % R, y = (q / R) % T1, b = q / (R * T1);
+      for (int a = 0; a < S0; ++a)
+        for (int x = 0; x < T0; ++x) {
+          const float f0 = K0[(size_t)(a * T0 + x) * R + r];
+          const float* g = dK + ((size_t)(x * T1 + y) * C + a * S1 + b) * Y * X;
+          float u = 0.f;
+          for (int ij = 0; ij < Y * X; ++ij) u += g[ij] * KC[(size_t)ij * R + r];
+          s += f0 * u;
+        }
+      dK1[q] = s;
+    } else {
+      const int q = e - n0 - n1, r = q % R, ij = q / R;
+      for (int a = 0; a < S0; ++a)
+        for (int x = 0; x < T0; ++x) {
+          const float f0 = K0[(size_t)(a * T0 + x) * R + r];
+          float u = 0.f;
+          for (int b = 0; b < S1; ++b)
+            for (int y = 0; y < T1; ++y)
+              u += dK[((size_t)(x * T1 + y) * C + a * S1 + b) * Y * X + ij] *
+                   K1[(size_t)(b * T1 + y) * R + r];
+          s += f0 * u;
+        }
+      dKC[q] = s;
+    }
+  }
+}
+
 // one workgroup per (image, channel) plane segment: the bias is a scalar
 __global__ __launch_bounds__(256) void bias_act_kernel(float* __restrict__ y,
                                                        const float* __restrict__ bias, int act,
@@ -221,6 +294,24 @@ hipError_t bias_act_launch(float* y, const float* bias, int act, size_t N, size_
 hipError_t zero_f32_launch(float* dst, size_t n, hipStream_t st) {
   if (n == 0) return hipSuccess;
   zero_f32_kernel<<<grid_for(n, 2048), 256, 0, st>>>(dst, n);
+  return hipGetLastError();
+}
+
+hipError_t rcp_recompose_launch(const float* K0, const float* K1, const float* KC, float* out,
+                                int S0, int S1, int T0, int T1, int Y, int X, int R,
+                                int transposed, hipStream_t st) {
+  const size_t total = (size_t)S0 * S1 * T0 * T1 * Y * X;
+  rcp_recompose_kernel<<<grid_for(total, 4096), 256, 0, st>>>(K0, K1, KC, out, S0, S1, T0, T1, Y, X,
+                                                             R, transposed);
+  return hipGetLastError();
+}
+
+hipError_t rcp_fold_launch(const float* dK, const float* K0, const float* K1, const float* KC,
+                           float* dK0, float* dK1, float* dKC, int S0, int S1, int T0, int T1,
+                           int Y, int X, int R, hipStream_t st) {
+  const size_t total = (size_t)R * (S0 * T0 + S1 * T1 + Y * X);
+  rcp_fold_kernel<<<grid_for(total, 4096), 256, 0, st>>>(dK, K0, K1, KC, dK0, dK1, dKC, S0, S1, T0,
+                                                        T1, Y, X, R);
   return hipGetLastError();
 }
 

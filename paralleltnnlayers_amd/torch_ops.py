@@ -36,6 +36,20 @@ class CP4Conv2dFunction(torch.autograd.Function):
         if bias is not None:
             bias = bias.contiguous().float()
         s = capi.shape_for(x.shape, FK, FC, FH, FW, pad)
+        ctx.half = x.dtype == torch.float16
+        if ctx.half:
+            # half-precision activations: forward and input gradient on the library's
+            # float16 entry points, the factor gradients on widened copies
+            x = x.contiguous()
+            ctx.pad, ctx.bf16, ctx.shape = pad, False, s
+            ctx.relu = capi.ACTIVATIONS[activation] == 1
+            if capi.bf16_supported(s):
+                y = capi.conv2d_forward_f16(x, FK, FC, FH, FW, bias, activation, pad=pad)
+            else:
+                y = capi.conv2d_forward_bias_act(x.float(), FK, FC, FH, FW, bias, activation,
+                                                 pad=pad).half()
+            ctx.save_for_backward(x, FK, FC, FH, FW, y if ctx.relu else None)
+            return y
         ctx.bf16 = x.dtype == torch.bfloat16
         ctx.fwd16 = ctx.bf16 and capi.bf16_supported(s)
         x = x.contiguous() if ctx.bf16 else x.contiguous().float()
@@ -61,6 +75,19 @@ class CP4Conv2dFunction(torch.autograd.Function):
         dbias = dy.float().sum(dim=(0, 2, 3)) if ctx.needs_input_grad[6] else None
         dy16 = ctx.bf16 and dy.dtype == torch.bfloat16
         dx = None
+        if ctx.half:
+            if ctx.needs_input_grad[0]:
+                if dy.dtype == torch.float16 and capi.bf16_supported(s, backward_data=True):
+                    dx = capi.conv2d_backward_data_f16(dy, FK, FC, FH, FW, pad=ctx.pad)
+                else:
+                    dx = capi.conv2d_backward_data(dy.float(), FK, FC, FH, FW, pad=ctx.pad).half()
+            grads = (None, None, None, None)
+            if any(ctx.needs_input_grad[1:5]):
+                grads = capi.conv2d_backward_filter(x.float(), dy.float(), FK, FC, FH, FW,
+                                                    pad=ctx.pad)
+                grads = tuple(g if need else None
+                              for g, need in zip(grads, ctx.needs_input_grad[1:5]))
+            return (dx,) + grads + (None, dbias, None)
         if ctx.needs_input_grad[0]:
             if dy16 and capi.bf16_supported(s, backward_data=True):
                 dx = capi.conv2d_backward_data_bf16(dy, FK, FC, FH, FW, pad=ctx.pad)
@@ -238,3 +265,41 @@ class CP3Conv2d(torch.nn.Module):
 
     def forward(self, x):
         return cp3_conv2d(x, self.K0, self.K1, self.K2, self.pad)
+
+
+class RCPConv2dFunction(torch.autograd.Function):
+    """The reshaped-CP convolution of the reference's ``Conv2dRcpFusedNchw`` op
+    (Kernels/rcp_fused_nchw.cc:6-12; test/test_conv2d_rcp.py:38-41):
+
+        y[n,(x,y)] = sum_r sum_{a,b} K0[a,x,r] K1[b,y,r] * (KC[:,:,r] (*) x[n,(a,b)])
+
+    K0 [S0,T0,R], K1 [S1,T1,R], KC [Y,X,R]; x has S0*S1 channels, y T0*T1.  All three
+    passes are the library's rcp entry points."""
+
+    @staticmethod
+    def forward(ctx, x, K0, K1, KC, pad):
+        if 2 * pad + 1 != KC.shape[0] or 2 * pad + 1 != KC.shape[1]:
+            raise ValueError("autograd binding needs 2*pad = Y-1 = X-1")
+        K0, K1, KC = (t.contiguous().float() for t in (K0, K1, KC))
+        x = x.contiguous().float()
+        ctx.pad = pad
+        ctx.save_for_backward(x, K0, K1, KC)
+        return capi.rcp_conv2d_forward(x, K0, K1, KC, pad=pad)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, K0, K1, KC = ctx.saved_tensors
+        dy = dy.contiguous().float()
+        dx = None
+        if ctx.needs_input_grad[0]:
+            dx = capi.rcp_conv2d_backward_data(dy, K0, K1, KC, pad=ctx.pad)
+        grads = (None, None, None)
+        if any(ctx.needs_input_grad[1:4]):
+            grads = capi.rcp_conv2d_backward_filter(x, dy, K0, K1, KC, pad=ctx.pad)
+            grads = tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad[1:4]))
+        return (dx,) + grads + (None,)
+
+
+def rcp_conv2d(x, K0, K1, KC, pad):
+    """Functional form of the differentiable reshaped-CP convolution (NCHW)."""
+    return RCPConv2dFunction.apply(x, K0, K1, KC, pad)

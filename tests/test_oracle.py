@@ -326,3 +326,31 @@ def test_geometry_reduces_to_the_reference_case(oracle):
     for a, b in zip(oracle.backward_filter_geom(x, dy, *f, g),
                     oracle.backward_filter(x, dy, *f, 1, direct=True)):
         close(a, b, 1e-6)
+
+
+# ---- reshaped-CP sibling op ---------------------------------------------------
+@pytest.mark.parametrize("dims", [(1, 4, 4, 4, 4, 8, 8, 3, 11), (2, 2, 3, 3, 2, 6, 7, 3, 4),
+                                  (1, 3, 2, 2, 5, 5, 6, 5, 3)],
+                         ids=lambda d: "x".join(map(str, d)))
+def test_rcp_forward_matches_the_dense_einsum(oracle, dims):
+    """The reference's own check of its reshaped-CP op (test/test_conv2d_rcp.py:38-45):
+    a SAME convolution with einsum('axr,byr,hwr->hwabxy') reshaped to [h,w,in,out]."""
+    N, S0, S1, T0, T1, H, W, Y, R = dims
+    g = torch.Generator().manual_seed(sum(dims))
+    x = torch.rand(N, S0 * S1, H, W, generator=g, dtype=torch.float64)
+    K0 = torch.rand(S0, T0, R, generator=g, dtype=torch.float64)
+    K1 = torch.rand(S1, T1, R, generator=g, dtype=torch.float64)
+    KC = torch.randn(Y, Y, R, generator=g, dtype=torch.float64)
+    K = torch.einsum("axr,byr,hwr->hwabxy", K0, K1, KC).reshape(Y, Y, S0 * S1, T0 * T1)
+    want = F.conv2d(x, K.permute(3, 2, 0, 1), padding=Y // 2).numpy()
+    got = oracle.rcp_forward(x.numpy(), K0.numpy(), K1.numpy(), KC.numpy(), Y // 2)
+    close(got, want.astype(np.float32), 2e-5)
+    # an impulse in channel (a, b) = (1, 0) reaches output channel (x, y) through
+    # K0[1, x] K1[0, y] only: pins the row-major channel pairing
+    if S0 > 1:
+        xi = np.zeros((1, S0 * S1, H, W), np.float32)
+        xi[0, 1 * S1 + 0, H // 2, W // 2] = 1.0
+        yi = oracle.rcp_forward(xi, K0.numpy(), K1.numpy(), KC.numpy(), Y // 2)
+        t = (T0 - 1) * T1 + (T1 - 1)
+        centre = float((K0[1, T0 - 1] * K1[0, T1 - 1] * KC[Y // 2, Y // 2]).sum())
+        assert abs(yi[0, t, H // 2, W // 2] - centre) <= 1e-5 * max(abs(centre), 1.0)
