@@ -397,6 +397,19 @@ cp4_status cp3_conv2d_backward_data(const cp4_shape* shape, const float* dy,
                                     const float* K2, float* dx, void* workspace,
                                     size_t workspace_bytes, cp4_stream stream);
 
+/* The factor gradients of the 3-factor op in one call: dK0 [C,Rank], dK1 [Y,X,Rank],
+ * dK2 [Rank,T].  `workspace`: cp3_conv2d_backward_filter_workspace_bytes.  With more
+ * than 32 expanded ranks (Y*Rank), where the matrix-core backward-filter applies and
+ * a plane pair fits LDS (H*W up to about 8000), the pass runs on Rank planes with
+ * K1 applied as it is - the channel contractions and gradient products do a Y-th
+ * of the work of the rewriting; other shapes run cp3_expand_factors, the CP4 pass
+ * at rank Y*Rank and cp3_fold_gradients. */
+size_t cp3_conv2d_backward_filter_workspace_bytes(const cp4_shape* shape);
+cp4_status cp3_conv2d_backward_filter(const cp4_shape* shape, const float* x, const float* dy,
+                                      const float* K0, const float* K1, const float* K2,
+                                      float* dK0, float* dK1, float* dK2, void* workspace,
+                                      size_t workspace_bytes, cp4_stream stream);
+
 /* ---- reshaped-CP sibling op -------------------------------------------------
  * Stands where the reference registers its TensorFlow op Conv2dRcpFusedNchw
  * (Kernels/rcp_fused_nchw.cc:6-12, launcher Conv2dRcpFusedNchwKernelLauncher :32; a

@@ -18,6 +18,7 @@ from .capi import (Shape, Geometry, geometry, conv2d_forward_ex, conv2d_backward
                    tune_clear, device_status, device_status_detail, set_spin_limit,
                    forward_variants, recompose, count_exceeding,
                    random_uniform, time_copy, cp3_shape_for, cp3_expand_factors,
-                   cp3_fold_gradients, cp3_conv2d_forward, cp3_conv2d_backward_data)
+                   cp3_fold_gradients, cp3_conv2d_forward, cp3_conv2d_backward_data,
+                   cp3_conv2d_backward_filter)
 
 __all__ = [n for n in dir() if not n.startswith("_")]

@@ -145,6 +145,10 @@ def lib():
     L.cp3_conv2d_forward.argtypes = [_S] + [_F] * 5 + [ctypes.c_void_p, ctypes.c_size_t,
                                                         ctypes.c_void_p]
     L.cp3_conv2d_backward_data.argtypes = L.cp3_conv2d_forward.argtypes
+    L.cp3_conv2d_backward_filter_workspace_bytes.restype = ctypes.c_size_t
+    L.cp3_conv2d_backward_filter_workspace_bytes.argtypes = [_S]
+    L.cp3_conv2d_backward_filter.argtypes = [_S] + [_F] * 8 + [ctypes.c_void_p, ctypes.c_size_t,
+                                                              ctypes.c_void_p]
     L.cp4_count_exceeding.argtypes = [_F, _F, ctypes.c_size_t, ctypes.c_float,
                                       ctypes.POINTER(ctypes.c_longlong), ctypes.c_void_p]
     L.cp4_random_uniform.argtypes = [_F, ctypes.c_size_t, ctypes.c_ulonglong, ctypes.c_void_p]
@@ -664,6 +668,20 @@ def cp3_conv2d_backward_data(dy, K0, K1, K2, pad=1, out=None, workspace=None, st
     dx = out if out is not None else torch.empty((s.N, s.C, s.H, s.W), device=dy.device,
                                                  dtype=torch.float32)
     return _cp3_pass(lib().cp3_conv2d_backward_data, s, dy, K0, K1, K2, dx, workspace, stream)
+
+
+def cp3_conv2d_backward_filter(x, dy, K0, K1, K2, pad=1, stream=None):
+    """(dK0 [C,R], dK1 [Y,X,R], dK2 [R,T]) of the 3-factor CP op."""
+    s = cp3_shape_for(x.shape, K0, K1, K2, pad)
+    assert tuple(dy.shape) == (s.N, s.T, s.H, s.W)
+    outs = [torch.empty_like(t) for t in (K0, K1, K2)]
+    n = int(lib().cp3_conv2d_backward_filter_workspace_bytes(ctypes.byref(s)))
+    ws = torch.empty(n + 512, device=x.device, dtype=torch.uint8)
+    off = (-ws.data_ptr()) % 256
+    check(lib().cp3_conv2d_backward_filter(
+        ctypes.byref(s), _ptr(x), _ptr(dy), _ptr(K0), _ptr(K1), _ptr(K2),
+        *[_ptr(o) for o in outs], ctypes.c_void_p(ws.data_ptr() + off), n, _stream(stream)))
+    return tuple(outs)
 
 
 def count_exceeding(a, b, tol, stream=None):

@@ -469,6 +469,56 @@ __global__ __launch_bounds__(256) void taps_plane_kernel(
   }
 }
 
+// The 3-factor CP op's tap step (test/layers.py:265-282: a depthwise Y x X filter
+// K1 [Y,X,R] between the two pointwise factors): one workgroup per (image, rank)
+// plane in LDS, Cc = K1 (*) A, G1 = the adjoint taps of G3, and the plane's
+// Y*X tap-gradient partials part[n][i*X+j][r] = <G3, shift_(i,j) A>.
+__global__ __launch_bounds__(256) void taps2d_plane_kernel(
+    const float* __restrict__ A, const float* __restrict__ G3, const float* __restrict__ K1,
+    float* __restrict__ Cc, float* __restrict__ G1, float* __restrict__ part, int R, int H, int W,
+    int Y, int X, int P) {
+  extern __shared__ float pl[];
+  const int HW = H * W, YX = Y * X;
+  float *sA = pl, *sG = pl + HW;
+  float* red = pl + 2 * HW;                       // [Y*X][4] wave partials
+  float* wk = red + 4 * YX;                       // this rank's filter
+  const int plane = blockIdx.x, r = plane % R, n = plane / R;
+  const size_t base = (size_t)plane * HW;
+  for (int p = threadIdx.x; p < HW; p += 256) {
+    sA[p] = A[base + p];
+    sG[p] = G3[base + p];
+  }
+  for (int t = threadIdx.x; t < YX; t += 256) wk[t] = K1[(size_t)t * R + r];
+  __syncthreads();
+  for (int p = threadIdx.x; p < HW; p += 256) {
+    const int h = p / W, w = p - h * W;
+    float cc = 0.f, g1 = 0.f;
+    for (int i = 0; i < Y; ++i)
+      for (int j = 0; j < X; ++j) {
+        const float k = wk[i * X + j];
+        const int hf = h + i - P, wf = w + j - P, hb = h - i + P, wb = w - j + P;
+        if (hf >= 0 && hf < H && wf >= 0 && wf < W) cc += k * sA[hf * W + wf];
+        if (hb >= 0 && hb < H && wb >= 0 && wb < W) g1 += k * sG[hb * W + wb];
+      }
+    Cc[base + p] = cc;
+    G1[base + p] = g1;
+  }
+  for (int t = 0; t < YX; ++t) {
+    const int oi = t / X - P, oj = t % X - P;
+    float acc = 0.f;
+    for (int p = threadIdx.x; p < HW; p += 256) {
+      const int h = p / W, w = p - h * W, hh = h + oi, ww = w + oj;
+      if (hh >= 0 && hh < H && ww >= 0 && ww < W) acc += sG[p] * sA[hh * W + ww];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off, 64);
+    if ((threadIdx.x & 63) == 0) red[t * 4 + (threadIdx.x >> 6)] = acc;
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < YX; t += 256)
+    part[((size_t)n * YX + t) * R + r] = ((red[t * 4] + red[t * 4 + 1]) + red[t * 4 + 2]) + red[t * 4 + 3];
+}
+
 // Sum of v over the 64 lanes, valid in lane 63: a shift-and-add scan inside each
 // row of 16 lanes, then the row totals passed on to the following rows, all as
 // data-parallel-primitive moves (no LDS traffic).  Lanes a move does not reach
@@ -1126,7 +1176,10 @@ Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R, int pad) 
   p.St = p.column_taps ? N * column_segments(W, Y, pad)
                        : (p.plane_taps ? N : (N < 8 ? N : 8));
   p.plane = (size_t)N * R * HW;
-  p.part_elems = (size_t)p.S * R * ((size_t)T + C) + (size_t)p.St * R * ((size_t)Y + X);
+  // (tap partials: Y + X per plane, Y * X with the 3-factor op's depthwise filter)
+  const size_t taps = (size_t)Y * X > (size_t)Y + X ? (size_t)Y * X : (size_t)Y + X;
+  const size_t st_max = p.St > N ? p.St : N;
+  p.part_elems = (size_t)p.S * R * ((size_t)T + C) + st_max * R * taps;
   return p;
 }
 
@@ -1145,6 +1198,14 @@ bool bwd_filter_mfma_supported(const cp4_shape& s) {
          (size_t)(s.C > s.T ? s.C : s.T) * (s.Rank <= 32 ? 32 : 64) * 4 <= 160 * 1024 &&
          s.Y + s.X <= 65535;
 }
+
+#ifndef CP4_BWF_IO16
+// The depthwise-filter tap step keeps two planes and Y*X partial sums in LDS.
+bool bwd_filter_mfma_taps2d_supported(const cp4_shape& s) {
+  return bwd_filter_mfma_supported(s) &&
+         ((size_t)s.H * s.W * 2 + 5 * (size_t)s.Y * s.X) * sizeof(float) <= 64 * 1024;
+}
+#endif
 
 size_t bwd_filter_mfma_workspace_bytes(const cp4_shape& s) {
   const Plan p = make_plan(s.N, s.C, s.T, s.H, s.W, s.Y, s.X, s.Rank, s.pad);
@@ -1210,7 +1271,14 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   }
 
   const bool wave_taps = p.wave_taps, column_taps = p.column_taps;
-  if (column_taps) {
+  if (a.taps2d) {
+    const size_t tsm = ((size_t)HW * 2 + 5 * (size_t)a.Y * a.X) * sizeof(float);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(taps2d_plane_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)tsm);
+    if (e != hipSuccess) return e;
+    taps2d_plane_kernel<<<N * R, 256, tsm, st>>>(A, G3, a.taps2d, Cc, G1, pH, R, a.H, a.W, a.Y,
+                                                 a.X, a.pad);
+  } else if (column_taps) {
     switch (a.Y) {
       case 1: e = launch_taps_column<1>(A, G3, a, Cc, G1, pH, pW, st); break;
       case 3: e = launch_taps_column<3>(A, G3, a, Cc, G1, pH, pW, st); break;
@@ -1276,9 +1344,10 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
 
   ReduceArgs r{};
   const float* parts[4] = {pK, pC, pH, pW};
-  float* outs[4] = {a.dFK, a.dFC, a.dFH, a.dFW};
-  const int counts[4] = {a.T * R, a.C * R, a.Y * R, a.X * R};
-  const int Ss[4] = {p.S, p.S, p.St, p.St};
+  float* outs[4] = {a.dFK, a.dFC, a.taps2d ? a.dtaps2d : a.dFH, a.dFW};
+  const int counts[4] = {a.T * R, a.C * R, a.taps2d ? a.Y * a.X * R : a.Y * R,
+                         a.taps2d ? 0 : a.X * R};
+  const int Ss[4] = {p.S, p.S, a.taps2d ? N : p.St, p.St};
   int maxc = 0;
   for (int i = 0; i < 4; ++i) {
     r.part[i] = parts[i]; r.out[i] = outs[i]; r.count[i] = counts[i]; r.S[i] = Ss[i];

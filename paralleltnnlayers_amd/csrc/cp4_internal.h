@@ -119,12 +119,17 @@ struct BwdFilterArgs {
   float *dFK, *dFC, *dFH, *dFW;
   void* workspace;
   int N, C, T, H, W, pad, Y, X, R;
+  // Matrix-core variant only, 3-factor CP op: a depthwise filter [Y, X, R] in place
+  // of FH x FW and its gradient (FH, FW, dFH, dFW unused then).
+  const float* taps2d;
+  float* dtaps2d;
 };
 // general (VALU, any shape) and matrix-core variants
 size_t bwd_filter_workspace_bytes(const cp4_shape&);
 hipError_t bwd_filter_launch(const BwdFilterArgs&, hipStream_t);
 bool bwd_filter_mfma_supported(const cp4_shape&);
 size_t bwd_filter_mfma_workspace_bytes(const cp4_shape&);
+bool bwd_filter_mfma_taps2d_supported(const cp4_shape&);   // with BwdFilterArgs::taps2d
 hipError_t bwd_filter_mfma_launch(const BwdFilterArgs&, hipStream_t);
 // The same with bfloat16 x and dy in memory (BwdFilterArgs::x / dy point at 16-bit
 // elements); split-bf16 kernels only: C and T multiples of 16.

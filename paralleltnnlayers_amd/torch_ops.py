@@ -207,9 +207,8 @@ class CP3Conv2dFunction(torch.autograd.Function):
 
         y[n,t] = sum_r K2[r,t] * (K1[:,:,r] (*) sum_c K0[c,r] x[n,c])
 
-    K0 [C,R], K1 [Y,X,R], K2 [R,T].  Forward and input gradient are the library's
-    cp3 passes; the factor gradients come from the CP4 backward-filter pass on the
-    library's exact rank-Y*R rewriting of the factors, folded back by the library.
+    K0 [C,R], K1 [Y,X,R], K2 [R,T].  All three passes are the library's cp3 entry
+    points.
     """
 
     @staticmethod
@@ -231,9 +230,7 @@ class CP3Conv2dFunction(torch.autograd.Function):
             dx = capi.cp3_conv2d_backward_data(dy, K0, K1, K2, pad=ctx.pad)
         grads = (None, None, None)
         if any(ctx.needs_input_grad[1:4]):
-            FK, FC, FH, FW = capi.cp3_expand_factors(K0, K1, K2)
-            dFK, dFC, _, dFW = capi.conv2d_backward_filter(x, dy, FK, FC, FH, FW, pad=ctx.pad)
-            grads = capi.cp3_fold_gradients(dFK, dFC, dFW, K1.shape[0])
+            grads = capi.cp3_conv2d_backward_filter(x, dy, K0, K1, K2, pad=ctx.pad)
             grads = tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad[1:4]))
         return (dx,) + grads + (None,)
 

@@ -166,3 +166,32 @@ def test_cp3_layer_trains(cp4):
         opt.step()
         losses.append(loss.item())
     assert losses[-1] < 0.7 * losses[0], losses[::6]
+
+
+@pytest.mark.parametrize("dims", SHAPES + [(4, 64, 56, 56, 3, 16, 64), (2, 32, 12, 12, 3, 40, 48)],
+                         ids=lambda d: "x".join(map(str, d)))
+def test_cp3_backward_filter_entry_point(cp4, dims):
+    """cp3_conv2d_backward_filter (K1 applied as it is where the matrix-core pass takes
+    the shape, the rank-Y*R rewriting elsewhere) against the rewriting spelled out
+    through the C ABI - cp3_expand_factors, the CP4 pass, cp3_fold_gradients - and
+    against float64 autograd of the dense convolution."""
+    x, K0, K1, K2 = operands(dims)
+    pad = dims[4] // 2
+    xd, k0, k1, k2 = (dev(a) for a in (x, K0, K1, K2))
+    dy = torch.randn((dims[0], dims[6], dims[2], dims[3]), device="cuda",
+                     generator=torch.Generator("cuda").manual_seed(5))
+    got = cp4.cp3_conv2d_backward_filter(xd, dy, k0, k1, k2, pad=pad)
+    FK, FC, FH, FW = cp4.cp3_expand_factors(k0, k1, k2)
+    dFK, dFC, _, dFW = cp4.conv2d_backward_filter(xd, dy, FK, FC, FH, FW, pad=pad)
+    via = cp4.cp3_fold_gradients(dFK, dFC, dFW, K1.shape[0])
+    ref = [torch.from_numpy(a).double().requires_grad_() for a in (x, K0, K1, K2)]
+    dense = torch.einsum("cr,ijr,rt->tcij", ref[1], ref[2], ref[3])
+    (F.conv2d(ref[0], dense, padding=pad) * dy.cpu().double()).sum().backward()
+    for name, g, v, r in zip(("dK0", "dK1", "dK2"), got, via, ref[1:]):
+        w = r.grad.numpy()
+        assert np.abs(host(g) - w).max() <= 1e-3 * np.abs(w).max(), name + " vs float64"
+        assert np.abs(host(g) - host(v)).max() <= 1e-4 * np.abs(w).max(), name + " vs rewriting"
+    # bit-reproducible: no floating-point atomics on either path
+    again = cp4.cp3_conv2d_backward_filter(xd, dy, k0, k1, k2, pad=pad)
+    for a, b in zip(got, again):
+        assert torch.equal(a, b)
