@@ -156,29 +156,34 @@ struct Variant {
   bool (*supported)(const FwdArgs&);
   hipError_t (*launch)(const FwdArgs&, hipStream_t);
 };
-// Ranks 33 to 64 on the producer / consumer kernel (which holds 32): the sum over
-// ranks splits, so the kernel runs on ranks [0, 32) and then on the rest with
-// y += - the factor pointers moved 32 columns in, the row stride unchanged.
+// More than 32 ranks on the producer / consumer kernel (which holds 32): the sum
+// over ranks splits, so the kernel runs on ranks [0, 32), then on [32, 64) with
+// y +=, and so on - the factor pointers moved 32 columns in per pass, the row
+// stride unchanged.  Every pass reads x again (and y, after the first).
+constexpr int kMaxRankPasses = 8;     // ranks up to 256
+int rank_passes(const FwdArgs& a) { return (a.R + 31) / 32; }
 FwdArgs rank_pass(const FwdArgs& a, int pass) {
   FwdArgs b = a;
   b.ldf = a.R;
-  if (pass == 0) {
-    b.R = 32;
-  } else {
-    b.R = a.R - 32;
-    b.Fin += 32; b.Fout += 32; b.FH += 32; b.FW += 32;
-    b.accumulate = 1;
-  }
+  const int r0 = 32 * pass;
+  b.R = a.R - r0 < 32 ? a.R - r0 : 32;
+  b.Fin += r0; b.Fout += r0; b.FH += r0; b.FW += r0;
+  b.accumulate = pass > 0;
   return b;
 }
 bool fwd_pipe2_supported(const FwdArgs& a) {
-  return a.R > 32 && a.R <= 64 && !a.ldf && !a.accumulate && !a.bias && !a.act &&
-         cp4::fwd_pipe_rankpass_supported(rank_pass(a, 0)) &&
-         cp4::fwd_pipe_rankpass_supported(rank_pass(a, 1));
+  if (a.R <= 32 || rank_passes(a) > kMaxRankPasses || a.ldf || a.accumulate || a.bias || a.act)
+    return false;
+  // (the passes differ in their rank count only: the first and the last decide)
+  return cp4::fwd_pipe_rankpass_supported(rank_pass(a, 0)) &&
+         cp4::fwd_pipe_rankpass_supported(rank_pass(a, rank_passes(a) - 1));
 }
 hipError_t fwd_pipe2_launch(const FwdArgs& a, hipStream_t st) {
-  const hipError_t e = cp4::fwd_pipe_rankpass_launch(rank_pass(a, 0), st);
-  return e != hipSuccess ? e : cp4::fwd_pipe_rankpass_launch(rank_pass(a, 1), st);
+  for (int p = 0; p < rank_passes(a); ++p) {
+    const hipError_t e = cp4::fwd_pipe_rankpass_launch(rank_pass(a, p), st);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }
 
 // Order = preference of the untuned heuristic, last to first.
@@ -189,7 +194,7 @@ const Variant kVariants[] = {
     {"mfma_bf16x3_strip", cp4::fwd_split_supported, cp4::fwd_split_launch},
     {"mfma_bf16x3_pipe_tiled", cp4::fwd_pipe_tiled_supported, cp4::fwd_pipe_tiled_launch},
     {"mfma_bf16x3_pipe", cp4::fwd_pipe_supported, cp4::fwd_pipe_launch},
-    {"mfma_bf16x3_pipe_2pass", fwd_pipe2_supported, fwd_pipe2_launch},
+    {"mfma_bf16x3_pipe_rank_passes", fwd_pipe2_supported, fwd_pipe2_launch},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -281,7 +286,7 @@ int heuristic_variant(const FwdArgs& a) {
     prefer("general_valu");
   if (is_variant(pick, "mfma_bf16x3_pipe") && a.W > kWholeRowMaxWidth)
     prefer("mfma_bf16x3_pipe_tiled");
-  if (is_variant(pick, "mfma_bf16x3_pipe_2pass") &&
+  if (is_variant(pick, "mfma_bf16x3_pipe_rank_passes") && a.R <= 64 &&
       (long)a.N * a.H * a.W * (a.Cin + a.Cout) < kTwoPassMinElements)
     prefer("mfma_f32_strip");
   // A handful of channels on both sides: the recomposed filter costs fewer
@@ -327,11 +332,35 @@ cp4_status run_forward_like(const FwdArgs& a, int variant, hipStream_t st) {
   return run_choice(a, variant < 0 ? choose(a) : Choice{variant, 0, 0, 0}, st);
 }
 
-// One workspace size serves either backward-filter variant.
+// Backward-filter with more than 64 ranks on the matrix-core kernels (which hold
+// 64): the gradient columns of a rank depend on that rank's factor columns only,
+// so the pass runs once per tile of 64 ranks on compact copies of the factor
+// columns and its gradients are copied back into their columns.
+constexpr unsigned kFilterRankTile = 64;
+cp4_shape filter_rank_tile(const cp4_shape& s, unsigned r0) {
+  cp4_shape t = s;
+  t.Rank = s.Rank - r0 < kFilterRankTile ? s.Rank - r0 : kFilterRankTile;
+  return t;
+}
+size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+bool filter_rank_tiles_supported(const cp4_shape& s) {
+  return s.Rank > kFilterRankTile && cp4::bwd_filter_mfma_supported(filter_rank_tile(s, 0)) &&
+         cp4::bwd_filter_mfma_supported(filter_rank_tile(s, (s.Rank - 1) / kFilterRankTile * kFilterRankTile));
+}
+size_t filter_rank_tile_floats(const cp4_shape& s) {   // compact factors or gradients of a tile
+  return align256((size_t)(s.T + s.C + s.Y + s.X) * kFilterRankTile * sizeof(float)) / sizeof(float);
+}
+
+// One workspace size serves every backward-filter variant.
 size_t filter_workspace(const cp4_shape& s) {
   size_t b = cp4::bwd_filter_workspace_bytes(s);
   if (cp4::bwd_filter_mfma_supported(s)) {
     const size_t m = cp4::bwd_filter_mfma_workspace_bytes(s);
+    if (m > b) b = m;
+  }
+  if (filter_rank_tiles_supported(s)) {
+    const size_t m = 2 * filter_rank_tile_floats(s) * sizeof(float) +
+                     cp4::bwd_filter_mfma_workspace_bytes(filter_rank_tile(s, 0));
     if (m > b) b = m;
   }
   return b;
@@ -618,9 +647,11 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
   if (!workspace || workspace_bytes < filter_workspace(s))
     return fail(CP4_ERR_WORKSPACE,
                 "workspace smaller than cp4_conv2d_backward_filter_workspace_bytes");
-  const bool mfma_ok = cp4::bwd_filter_mfma_supported(s) &&
-                       ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) |
+  const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) |
                          reinterpret_cast<uintptr_t>(workspace)) & 7) == 0;
+  const bool tiles_ok = filter_rank_tiles_supported(s) && aligned &&
+                        (reinterpret_cast<uintptr_t>(workspace) & 255) == 0;
+  const bool mfma_ok = (cp4::bwd_filter_mfma_supported(s) && aligned) || tiles_ok;
   if (variant > 1 || (variant == 1 && !mfma_ok))
     return fail(CP4_ERR_UNSUPPORTED, "backward-filter variant cannot run this shape");
   cp4::BwdFilterArgs a{};
@@ -632,6 +663,36 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
     std::lock_guard<std::mutex> lk(g_tune_mu);
     auto it = g_tuned_filter.find(key_of(s));
     if (it != g_tuned_filter.end() && (it->second == 0 || mfma_ok)) variant = it->second;
+  }
+  if ((variant == 1 || (variant < 0 && mfma_ok)) && tiles_ok) {
+    float* cf = static_cast<float*>(workspace);                 // compact factors of a tile
+    float* cg = cf + filter_rank_tile_floats(s);                // compact gradients
+    void* inner = cg + filter_rank_tile_floats(s);
+    const int R = (int)s.Rank;
+    const float* fac[4] = {FK, FC, FH, FW};
+    float* grad[4] = {dFK, dFC, dFH, dFW};
+    const int rows[4] = {(int)s.T, (int)s.C, (int)s.Y, (int)s.X};
+    for (unsigned r0 = 0; r0 < s.Rank; r0 += kFilterRankTile) {
+      const cp4_shape t = filter_rank_tile(s, r0);
+      const int rt = (int)t.Rank;
+      float *f[4], *g[4];
+      size_t off = 0;
+      for (int i = 0; i < 4; ++i) {
+        f[i] = cf + off;
+        g[i] = cg + off;
+        off += (size_t)rows[i] * rt;
+        CP4_HIP(cp4::copy_columns_launch(fac[i] + r0, R, f[i], rt, rows[i], rt, st));
+      }
+      cp4::BwdFilterArgs b = a;
+      b.FK = f[0]; b.FC = f[1]; b.FH = f[2]; b.FW = f[3];
+      b.dFK = g[0]; b.dFC = g[1]; b.dFH = g[2]; b.dFW = g[3];
+      b.R = rt;
+      b.workspace = inner;
+      CP4_HIP(cp4::bwd_filter_mfma_launch(b, st));
+      for (int i = 0; i < 4; ++i)
+        CP4_HIP(cp4::copy_columns_launch(g[i], rt, grad[i] + r0, R, rows[i], rt, st));
+    }
+    return CP4_OK;
   }
   if (variant == 1 || (variant < 0 && mfma_ok)) CP4_HIP(cp4::bwd_filter_mfma_launch(a, st));
   else CP4_HIP(cp4::bwd_filter_launch(a, st));
@@ -792,7 +853,6 @@ Canvas canvas_of(const cp4_shape& s, const cp4_geometry& g) {
   c.dy_in_place = g.stride_h == 1 && g.stride_w == 1 && g.out_h == c.Hc && g.out_w == c.Wc;
   return c;
 }
-size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
 }  // namespace
 
 cp4_status cp4_geometry_same(const cp4_shape* s, unsigned sh, unsigned sw, cp4_geometry* g) {
@@ -1042,7 +1102,7 @@ cp4_status tune_forward_like(const FwdArgs& a, unsigned warmup, unsigned profcou
     if (!kVariants[v].supported(a)) continue;
     cp4_status rc = consider(Choice{v, 0, 0, 0});     // the kernel's own planner
     if (rc != CP4_OK) return rc;
-    const bool strips = is_variant(v, "mfma_bf16x3_pipe") || is_variant(v, "mfma_bf16x3_pipe_2pass");
+    const bool strips = is_variant(v, "mfma_bf16x3_pipe") || is_variant(v, "mfma_bf16x3_pipe_rank_passes");
     const bool tiles = is_variant(v, "mfma_bf16x3_pipe_tiled");
     if (!strips && !tiles) continue;
     const int max_th = a.H < 16 ? a.H : 16;

@@ -156,6 +156,9 @@ hipError_t cp3_expand_launch(const cp4_shape& s, const float* K0, const float* K
                              hipStream_t);
 hipError_t cp3_fold_launch(const cp4_shape& s, const float* dFK, const float* dFC,
                            const float* dFW, float* dK0, float* dK1, float* dK2, hipStream_t);
+// dst[row*ld_dst + c] = src[row*ld_src + c], c < cols (column blocks of factor matrices)
+hipError_t copy_columns_launch(const float* src, int ld_src, float* dst, int ld_dst, int rows,
+                               int cols, hipStream_t);
 // dst[plane][ot + sh*u][ol + sw*v] = src[plane][u][v] on `planes` planes of h x w
 // set into canvases of Hc x Wc; every other canvas cell is written as zero.
 hipError_t embed_launch(const float* src, float* dst, size_t planes, int h, int w, int Hc, int Wc,

@@ -170,6 +170,18 @@ __global__ __launch_bounds__(256) void rcp_fold_kernel(
   }
 }
 
+// dst[row*ld_dst + c] = src[row*ld_src + c] for c < cols: a column block of a
+// row-major matrix copied to or from a compact one.
+__global__ __launch_bounds__(256) void copy_columns_kernel(const float* __restrict__ src,
+                                                           int ld_src, float* __restrict__ dst,
+                                                           int ld_dst, int rows, int cols) {
+  const int total = rows * cols;
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
+    const int row = i / cols, c = i - row * cols;
+    dst[(size_t)row * ld_dst + c] = src[(size_t)row * ld_src + c];
+  }
+}
+
 // one workgroup per (image, channel) plane segment: the bias is a scalar
 __global__ __launch_bounds__(256) void bias_act_kernel(float* __restrict__ y,
                                                        const float* __restrict__ bias, int act,
@@ -312,6 +324,14 @@ hipError_t rcp_fold_launch(const float* dK, const float* K0, const float* K1, co
   const size_t total = (size_t)R * (S0 * T0 + S1 * T1 + Y * X);
   rcp_fold_kernel<<<grid_for(total, 4096), 256, 0, st>>>(dK, K0, K1, KC, dK0, dK1, dKC, S0, S1, T0,
                                                         T1, Y, X, R);
+  return hipGetLastError();
+}
+
+hipError_t copy_columns_launch(const float* src, int ld_src, float* dst, int ld_dst, int rows,
+                               int cols, hipStream_t st) {
+  if (rows <= 0 || cols <= 0) return hipSuccess;
+  copy_columns_kernel<<<grid_for((size_t)rows * cols, 1024), 256, 0, st>>>(src, ld_src, dst, ld_dst,
+                                                                          rows, cols);
   return hipGetLastError();
 }
 

@@ -400,3 +400,37 @@ def test_timed_launch_and_tuner(cp4):
         y4 = cp4.conv2d_forward(x, *f, pad=w.pad, variant=best)   # explicit non-default stream
     s.synchronize()
     assert torch.equal(y3, y4)
+
+
+# ------------------------------------------------ ranks beyond a kernel's tile ----
+@pytest.mark.parametrize("R", [33, 48, 64, 65, 96, 128, 200])
+def test_ranks_beyond_one_tile(cp4, oracle, R):
+    """Ranks above 32 (forward / backward-data: passes of 32 ranks on the producer /
+    consumer kernel) and above 64 (backward-filter: the matrix-core pass per tile of 64
+    ranks): all three passes, every variant that takes the shape, against the oracle."""
+    rng = np.random.default_rng(R)
+    N, C, H, W, T, Y = 2, 64, 28, 28, 96, 3
+    a = {"x": rng.standard_normal((N, C, H, W), dtype=np.float32),
+         "dy": rng.standard_normal((N, T, H, W), dtype=np.float32)}
+    for k, d in (("FK", T), ("FC", C), ("FH", Y), ("FW", Y)):
+        a[k] = rng.standard_normal((d, R), dtype=np.float32) * np.float32((R * C) ** -0.25)
+    f = {k: dev(a[k]) for k in FACTORS}
+    fa = [a[k] for k in FACTORS]
+    x, dy = dev(a["x"]), dev(a["dy"])
+    want = oracle.forward(a["x"], *fa, 1)
+    names = dict((v, n) for v, n, _ in cp4.forward_variants())
+    vs = variants_for(cp4, x.shape, f, 1)
+    assert any(names[v] == "mfma_bf16x3_pipe_rank_passes" for v in vs)
+    for v in vs:
+        assert_activation_close(host(cp4.conv2d_forward(x, *f.values(), pad=1, variant=v)), want,
+                                f"R={R} forward {names[v]}")
+    assert_activation_close(host(cp4.conv2d_backward_data(dy, *f.values(), pad=1)),
+                            oracle.backward_data(a["dy"], *fa, 1), f"R={R} backward-data")
+    wants = oracle.backward_filter(a["x"], a["dy"], *fa, 1)
+    fv = filter_variants(cp4, x, dy, list(f.values()), 1)
+    assert 1 in fv, "the matrix-core backward-filter must take every rank here"
+    for variant in fv:
+        grads = cp4.conv2d_backward_filter(x, dy, *f.values(), pad=1, variant=variant)
+        for g, wnt, k in zip(grads, wants, FACTORS):
+            assert_gradient_close(host(g), wnt, f"R={R} d{k} variant {variant}")
+    cp4.device_status()
