@@ -63,6 +63,9 @@ def main():
     ap.add_argument("--cold-sets", type=int, default=4,
                     help="distinct x / y buffer sets of the rotating (HBM-streaming) leg of a "
                          "forward workload; 0 skips the leg")
+    ap.add_argument("--cold-only", action="store_true",
+                    help="run only the rotating leg (profiling: every launch of the process "
+                         "then streams from and to HBM); prints that leg's figures")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-passes", action="store_true", help="skip the five-workload table")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -130,6 +133,16 @@ def main():
         return
     host, d = device_inputs(w)
     nbytes = algorithmic_bytes(w)
+    if args.cold_only:
+        assert w.pass_ == "forward" and args.cold_sets > 0
+        f = [d[k] for k in FACTORS]
+        xs = [d["x"]] + [d["x"].clone() for _ in range(args.cold_sets - 1)]
+        ys = [torch.empty((w.N, w.T, w.H, w.W), device="cuda") for _ in xs]
+        cus = cp4.time_forward_sets(xs, *f, ys, w.pad, args.warmup, args.steps)
+        print(json.dumps({"workload": w.name, "sets": len(xs), "us_per_launch": round(cus, 2),
+                          "GB/s": round(nbytes / cus / 1e3, 1),
+                          "hbm_frac": round(nbytes / cus / 1e3 / HBM_PEAK_GBS, 4)}))
+        return
     us, wall = timed(w, d, args.warmup, args.steps, args.settle_ms)
     value = nbytes * args.steps / wall / 1e9
     achieved = nbytes / us / 1e3

@@ -41,6 +41,7 @@ struct DensePlan {
   int tile_w;    // LDS row length of the tile (floats, odd: conflict-free segment reads)
   int tpw;       // tiles per workgroup, down the image
   int wfloats;   // LDS floats set aside for a workgroup's filter (a multiple of 4)
+  int cols, rowgroups, ntiles;   // tile columns, groups of tpw tile rows, workgroups with work
   size_t lds_bytes;
 };
 
@@ -48,15 +49,23 @@ template <int FS, int KO>
 __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, DensePlan pl) {
   extern __shared__ float lds[];
   const int Cin = a.Cin, R = a.R, H = a.H, W = a.W;
-  // output channels in groups of eight, one group per workgroup (blockIdx.z = image, group)
+  // Workgroup b runs on XCD b % 8, each with an L2 of its own: tile ids are permuted
+  // so that an XCD gets a contiguous range - horizontally adjacent tiles, which
+  // share their halo columns' cache lines, then meet in one L2 (with the plain
+  // x-fastest grid the kernel fetched 2.1 times its input).
+  const int per = (pl.ntiles + 7) >> 3;
+  const int t = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  if (t >= pl.ntiles) return;                         // whole workgroup, before any barrier
+  const int bx = t % pl.cols, by = (t / pl.cols) % pl.rowgroups, bz = t / (pl.cols * pl.rowgroups);
+  // output channels in groups of eight, one group per workgroup (bz = image, group)
   const int ngrp = (a.Cout + 7) >> 3;
-  const int n = blockIdx.z / ngrp, k0 = 8 * (blockIdx.z - n * ngrp);
+  const int n = bz / ngrp, k0 = 8 * (bz - n * ngrp);
   const int Cout = min(8, a.Cout - k0);               // channels of this group
   const int nw = Cout * Cin * FS * FS;
   float* wts = lds;                                   // [Cout][Cin][FS][FS]
   float* tile = lds + pl.wfloats;                     // [cc][kTH + FS - 1][tile_w]
   const int tid = threadIdx.x;
-  const int w0 = blockIdx.x * kTW;
+  const int w0 = bx * kTW;
   const size_t HW = (size_t)H * W;
 
   if (a.dense) {
@@ -97,7 +106,7 @@ __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, De
   const float* xn = a.x + (size_t)n * Cin * HW;
 
   for (int tr = 0; tr < pl.tpw; ++tr) {
-    const int h0 = (blockIdx.y * pl.tpw + tr) * kTH;
+    const int h0 = (by * pl.tpw + tr) * kTH;
     if (h0 >= H) break;
     float acc[KO][kPX];
 #pragma unroll
@@ -199,7 +208,7 @@ bool plan(const FwdArgs& a, DensePlan* pl) {
   if (nw > kMaxWeights) return false;
   const long nf = a.dense ? 0 : (long)a.R * (kgrp + a.Cin + a.Y + a.X);
   if (nf > kMaxFactorFloats) return false;
-  if ((long)a.N * ngrp > 65535) return false;
+
   // odd row length: the four-column segments of neighbouring threads fall on
   // different LDS banks
   const int tile_w = (kTW + a.Y - 1) | 1;
@@ -209,15 +218,20 @@ bool plan(const FwdArgs& a, DensePlan* pl) {
   if (cc > a.Cin) cc = a.Cin;
   size_t tile_bytes = cc * per_channel;
   if (tile_bytes < (size_t)nf * sizeof(float)) tile_bytes = (size_t)nf * sizeof(float);
-  // enough workgroups to fill the device a few times over, each amortising its
+  // enough workgroups to fill the device sixteen times over, each amortising its
   // filter recomposition over several tiles
   const long row_tiles = (a.H + kTH - 1) / kTH, col_tiles = (a.W + kTW - 1) / kTW;
   const long tiles = row_tiles * col_tiles * a.N * ngrp;
-  long tpw = tiles / (8l * num_compute_units());
+  long tpw = tiles / (16l * num_compute_units());
   if (tpw < 1) tpw = 1;
   if (tpw > row_tiles) tpw = row_tiles;
   if (tpw > 16) tpw = 16;
-  if ((row_tiles + tpw - 1) / tpw > 65535) return false;
+  const long rowgroups = (row_tiles + tpw - 1) / tpw;
+  const long ntiles = col_tiles * rowgroups * a.N * ngrp;
+  if (ntiles > (1l << 30)) return false;
+  pl->cols = (int)col_tiles;
+  pl->rowgroups = (int)rowgroups;
+  pl->ntiles = (int)ntiles;
   pl->cc = cc;
   pl->tile_w = tile_w;
   pl->tpw = (int)tpw;
@@ -231,9 +245,7 @@ hipError_t launch_as(const FwdArgs& a, const DensePlan& pl, hipStream_t st) {
   const void* fn = reinterpret_cast<const void*>(fwd_dense_small_kernel<FS, KO>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds_bytes);
   if (e != hipSuccess) return e;
-  const int row_tiles = (a.H + kTH - 1) / kTH;
-  const dim3 grid((a.W + kTW - 1) / kTW, (row_tiles + pl.tpw - 1) / pl.tpw,
-                  a.N * ((a.Cout + 7) / 8));
+  const unsigned grid = 8u * ((pl.ntiles + 7) / 8);
   fwd_dense_small_kernel<FS, KO><<<grid, kThreads, pl.lds_bytes, st>>>(a, pl);
   return hipGetLastError();
 }
