@@ -104,11 +104,20 @@ constexpr int kProd = 8, kCons = 8;          // producer / consumer waves (4 per
 constexpr int kRP = 32;
 constexpr int kCcBuf = 24 * 512;             // bytes of one Cc fragment tile (64 pixels)
 constexpr size_t kLdsLimit = 160 * 1024;
+#ifndef CP4_WHOLE_BLOCK_MIN
+#define CP4_WHOLE_BLOCK_MIN 16
+#endif
+// What a workgroup spends before its pipeline runs (first loads, factor
+// fragments, the consumers' wait for the first rows: 7-8 us), in the planners'
+// unit of one channel of one cell read or written (7-11 thousand per us).
+constexpr double kTileStartCost = 50000.0;
+constexpr int kWholeBlockMin = CP4_WHOLE_BLOCK_MIN;   // blocks per plane from which 17-64 channels go unsplit
 constexpr int kSpinLimit = 1 << 19;      // default bound of a wait: about a quarter of a second at the longest nap
 constexpr int kMaxBlk = 64;                  // per-block progress words in LDS
 
 struct PipePlan {
   int TH, strips, nWG;
+  int nblk;        // 32-pixel producer blocks of a workgroup's plane
   int QA;          // LDS row stride of A (floats)
   int fin_off;     // byte offsets inside LDS; factor fragments only above 256 input channels
   int cc_off;
@@ -254,6 +263,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #endif
 #endif
   const int nblk = (QLEN + 31) >> 5;             // 32-pixel producer blocks
+  const bool low16 = R <= 16;                    // the plane holds rank rows 0 ... 15 only
   const bool backoff = nblk >= 4;                // growing naps in the spin waits
 
   // ---- prologue: clear the progress words; above 256 input channels the input
@@ -442,14 +452,20 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         float* dst = &As[(4 * hi) * QA + qa];      // row 8*(v>>2) + (v&3) + 4*hi
         if (cq == 0) {
 #pragma unroll
-          for (int v = 0; v < 16; ++v)
+          for (int v = 0; v < 8; ++v)
             dst[(8 * (v >> 2) + (v & 3)) * QA] = valid ? acc[v] : 0.f;
+          if (!low16) {
+#pragma unroll
+            for (int v = 8; v < 16; ++v)
+              dst[(8 * (v >> 2) + (v & 3)) * QA] = valid ? acc[v] : 0.f;
+          }
         } else {
           wait_ge(bf, cq, backoff, wx, 1);
           // read all, then add, then write all: one LDS round trip per half, not
           // one per element
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
+            if (half == 1 && low16) break;
             float old[8];
 #pragma unroll
             for (int v = 0; v < 8; ++v) old[v] = dst[(8 * ((8 * half + v) >> 2) + (v & 3)) * QA];
@@ -680,7 +696,10 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #pragma unroll
       for (int qi = 0; qi < decltype(ntq_c)::value; ++qi) {
       const int q = wq + 4 * qi;                   // this pass's rank quad
-      const float* ab = As + (size_t)(4 * q) * QA + h * RL;
+      // (a quad past the last rank has zero weights; it reads quad 0's rows, the
+      // plane may end before its own, and writes zeros)
+      const bool live = 4 * q < R;
+      const float* ab = As + (size_t)(live ? 4 * q : 0) * QA + h * RL;
       float o[4];
 #pragma unroll
       for (int r0 = 0; r0 < 4; r0 += RBT) {
@@ -706,7 +725,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
             s += fh[qi][r0 + rr][ti] * hs;
 #endif
           }
-          o[r0 + rr] = s;
+          o[r0 + rr] = live ? s : 0.f;
         }
         if (RBT < 4) __builtin_amdgcn_sched_barrier(0);
       }
@@ -977,19 +996,24 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 
 int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
+// Rank rows of the A plane in LDS: the producers' 32 x 32 products carry 32, of
+// which the upper 16 are zero (and neither written nor read) up to 16 ranks.
+int plane_rows(const FwdArgs& a) { return a.R <= 16 ? 16 : kRP; }
+
 [[maybe_unused]] bool layout(const FwdArgs& a, int TH, PipePlan* pl) {
   const long QLEN = (long)(TH + a.Y - 1) * a.W;
   // the taps of the last (partly filled) 64-pixel group may read past QLEN; the
   // groups start up to 31 pixels before the strip, so they end up to 31 + 63 past it
   const long QA =
       round_up((int)(round_up(TH * a.W + 31, 64) + (long)(a.Y - 1) * (a.W + 1) + 1), 64) + 8;
-  const size_t a_bytes = (size_t)kRP * QA * sizeof(float);
+  const size_t a_bytes = (size_t)plane_rows(a) * QA * sizeof(float);
   // above 256 input channels: pre-split factor fragments, 192 B per (padded) channel
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
   const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 16) * sizeof(int);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
+  pl->nblk = (int)((QLEN + 31) / 32);
   pl->strips = (a.H + TH - 1) / TH;
   pl->nWG = a.N * pl->strips;
   pl->QA = (int)QA;
@@ -1005,12 +1029,13 @@ int round_up(int v, int m) { return (v + m - 1) / m * m; }
 bool layout_strided(const FwdArgs& a, int TH, PipePlan* pl) {
   const long QLEN = ((long)a.sh * (TH - 1) + a.Y) * a.W;
   const long QA = round_up((int)QLEN, 64) + 8;
-  const size_t a_bytes = (size_t)kRP * QA * sizeof(float);
+  const size_t a_bytes = (size_t)plane_rows(a) * QA * sizeof(float);
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
   const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 16) * sizeof(int);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
+  pl->nblk = (int)((QLEN + 31) / 32);
   pl->strips = (a.Ho + TH - 1) / TH;
   pl->nWG = a.N * pl->strips;
   pl->QA = (int)QA;
@@ -1031,7 +1056,7 @@ bool plan(const FwdArgs& a, PipePlan* best) {
     const double rounds = (pl.nWG + cus - 1) / cus;
     // cells read per channel and cells written per channel
     const double cost = rounds * (((double)a.sh * (TH - 1) + a.Y) * a.W * a.Cin +
-                                  (double)TH * a.Wo * a.Cout);
+                                  (double)TH * a.Wo * a.Cout + kTileStartCost);
     if (!found || cost <= best_cost) {
       best_cost = cost;
       *best = pl;
@@ -1046,12 +1071,13 @@ bool layout_tiled(const FwdArgs& a, int TH, int lgWt, PipePlan* pl) {
   const int Wt = 1 << lgWt, WL = Wt + a.Y - 1;
   const long QLEN = (long)(TH + a.Y - 1) * WL;
   const long QA = round_up((int)QLEN, 64) + 8;
-  const size_t a_bytes = (size_t)kRP * QA * sizeof(float);
+  const size_t a_bytes = (size_t)plane_rows(a) * QA * sizeof(float);
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
   const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 16) * sizeof(int);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
+  pl->nblk = (int)((QLEN + 31) / 32);
   pl->strips = (a.H + TH - 1) / TH;
   pl->Wt = Wt;
   pl->lgWt = lgWt;
@@ -1080,7 +1106,7 @@ bool plan(const FwdArgs& a, PipePlan* best) {
       // cells read per channel and cells written per channel, with the tiles of the
       // last column counted whole
       const double cost = rounds * ((double)(TH + a.Y - 1) * (pl.Wt + a.Y - 1) * a.Cin +
-                                    (double)TH * pl.Wt * a.Cout);
+                                    (double)TH * pl.Wt * a.Cout + kTileStartCost);
       // on equal cost (1x1 filters: no halo) the larger tile: fewer workgroups
       if (!found || cost <= best_cost) {
         best_cost = cost;
@@ -1102,7 +1128,8 @@ bool plan(const FwdArgs& a, PipePlan* best) {
     PipePlan pl;
     if (!layout(a, TH, &pl)) break;
     const double rounds = (pl.nWG + cus - 1) / cus;
-    const double cost = rounds * ((double)(TH + a.Y - 1) * a.Cin + (double)TH * a.Cout);
+    const double cost = rounds * ((double)(TH + a.Y - 1) * a.Cin + (double)TH * a.Cout +
+                                  kTileStartCost / a.W);
     // on equal cost (1x1 filters: no halo rows) the taller strip: fewer workgroups
     if (!found || cost <= best_cost) {
       best_cost = cost;
@@ -1147,6 +1174,21 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
   if (a.Cin <= 16)
     return (a.Cin & 15) ? launch_as<FS, 1, 1, true, 1>(a, pl, st)
                         : launch_as<FS, 1, 1, false, 1>(a, pl, st);
+  // On planes of many blocks the waves' arithmetic bounds the sweep, not the
+  // latency of one block, and the split's four chained LDS accumulations per block
+  // are half of the producers' instructions at 17-64 channels: there, too, every
+  // producer wave contracts whole blocks (N32 C32 112x112 R16: 63 -> 47 us).
+  if (a.Cin <= 64 && pl.nblk >= kWholeBlockMin) {
+    const bool padc = (a.Cin & 15) != 0;
+    switch ((a.Cin + 15) >> 4) {
+      case 2:
+        return padc ? launch_as<FS, 2, 2, true, 1>(a, pl, st) : launch_as<FS, 2, 2, false, 1>(a, pl, st);
+      case 3:
+        return padc ? launch_as<FS, 3, 1, true, 1>(a, pl, st) : launch_as<FS, 3, 1, false, 1>(a, pl, st);
+      default:
+        return padc ? launch_as<FS, 4, 2, true, 1>(a, pl, st) : launch_as<FS, 4, 2, false, 1>(a, pl, st);
+    }
+  }
   return (a.Cin & 63) ? launch_cpq<FS, true>(a, pl, st) : launch_cpq<FS, false>(a, pl, st);
 }
 
