@@ -316,13 +316,15 @@ cp4_status cp4_conv2d_forward_variant(const cp4_shape* shape, const float* x,
                                       cp4_stream stream);
 /* Times every variant that supports `shape` (warmup + profcount launches
  * each) on the caller's buffers - the producer / consumer variants once per
- * strip height (tile height x width for wide planes) up to 16 rows and with the
- * consumers' role split on and off - remembers the fastest for this shape for the
+ * strip height (tile height x width for wide planes) up to 16 rows and with each
+ * of the consumers' schedules (role split by the kernel's rule, off, whole pixel
+ * groups per wave) - remembers the fastest for this shape for the
  * rest of the process (a process-wide table behind a mutex; cp4_tune_clear
  * empties it) and reports it.  cp4_tune_backward_data does the same for that
  * pass, cp4_tune_backward_filter chooses between that pass's two variants.
  * cp4_tuned_choice reports what a shape would run with now: the variant, the
- * tuned tile (rows, columns; 0 = the kernel's own planner) and the role split. */
+ * tuned tile (rows, columns; 0 = the kernel's own planner) and the consumers'
+ * schedule (1 = the kernel's rule, 0 = no role split, 2 = whole groups per wave). */
 cp4_status cp4_tune_forward(const cp4_shape* shape, const float* x,
                             const float* FK, const float* FC, const float* FH,
                             const float* FW, float* y, unsigned warmup,
@@ -341,6 +343,11 @@ cp4_status cp4_tune_backward_filter(const cp4_shape* shape, const float* x, cons
                                     float* best_us, cp4_stream stream);
 cp4_status cp4_tuned_choice(const cp4_shape* shape, int backward_data, int* variant,
                             int* tile_rows, int* tile_cols, int* role_split);
+/* Enters a choice into the table as cp4_tune_forward / cp4_tune_backward_data
+ * would (one saved from an earlier process, say), in cp4_tuned_choice's terms.
+ * CP4_ERR_UNSUPPORTED if the variant does not take the shape with that tile. */
+cp4_status cp4_set_tuned_choice(const cp4_shape* shape, int backward_data, int variant,
+                                int tile_rows, int tile_cols, int schedule);
 void cp4_tune_clear(void);
 
 /* ---- device allocator / copy helpers (the reference's Tensor uses

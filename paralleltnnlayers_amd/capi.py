@@ -133,6 +133,7 @@ def lib():
                                                  ctypes.POINTER(ctypes.c_int),
                                                  ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
     L.cp4_tuned_choice.argtypes = [_S, ctypes.c_int] + [ctypes.POINTER(ctypes.c_int)] * 4
+    L.cp4_set_tuned_choice.argtypes = [_S] + [ctypes.c_int] * 5
     L.cp4_tune_clear.restype = None
     L.cp4_device_status.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
     L.cp4_set_spin_limit.argtypes = [ctypes.c_int]
@@ -579,6 +580,13 @@ def tuned_choice(s, backward_data=False):
     v = [ctypes.c_int() for _ in range(4)]
     check(lib().cp4_tuned_choice(ctypes.byref(s), int(backward_data), *[ctypes.byref(i) for i in v]))
     return dict(zip(("variant", "tile_rows", "tile_cols", "role_split"), (i.value for i in v)))
+
+
+def set_tuned_choice(s, variant, tile_rows=0, tile_cols=0, schedule=1, backward_data=False):
+    """Enters a choice into the tuner's table (tuned_choice's terms: schedule 1 = the
+    kernel's rule, 0 = no role split, 2 = whole pixel groups per consumer wave)."""
+    check(lib().cp4_set_tuned_choice(ctypes.byref(s), int(backward_data), int(variant),
+                                     int(tile_rows), int(tile_cols), int(schedule)))
 
 
 def tune_clear():

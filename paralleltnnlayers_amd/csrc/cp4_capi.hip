@@ -1108,7 +1108,7 @@ cp4_status tune_forward_like(const FwdArgs& a, unsigned warmup, unsigned profcou
     const int max_th = a.H < 16 ? a.H : 16;
     for (int lgwt = tiles ? 6 : 0; lgwt <= (tiles ? 8 : 0); ++lgwt)
       for (int th = 1; th <= max_th; ++th)
-        for (int split2 = 0; split2 <= 1; ++split2) {
+        for (int split2 = 0; split2 <= 2; ++split2) {   // 2: consumer waves with groups of their own
           rc = consider(Choice{v, th, lgwt, split2});
           if (rc != CP4_OK) return rc;
         }
@@ -1197,7 +1197,33 @@ cp4_status cp4_tuned_choice(const cp4_shape* shape, int backward_data, int* vari
   if (variant) *variant = c.variant;
   if (tile_rows) *tile_rows = c.th;
   if (tile_cols) *tile_cols = c.lgwt ? 1 << c.lgwt : 0;
-  if (role_split) *role_split = c.split2 == 1 ? 0 : 1;
+  if (role_split) *role_split = c.split2 == 1 ? 0 : (c.split2 == 2 ? 2 : 1);
+  return CP4_OK;
+}
+
+cp4_status cp4_set_tuned_choice(const cp4_shape* shape, int backward_data, int variant,
+                                int tile_rows, int tile_cols, int schedule) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (variant < 0 || variant >= kNumVariants) return fail(CP4_ERR_SHAPE, "variant out of range");
+  int lgwt = 0;
+  if (tile_cols) {
+    while ((1 << lgwt) < tile_cols) ++lgwt;
+    if ((1 << lgwt) != tile_cols || lgwt < 6 || lgwt > 8)
+      return fail(CP4_ERR_SHAPE, "tile_cols must be 0, 64, 128 or 256");
+  }
+  if (tile_rows < 0 || schedule < 0 || schedule > 2)
+    return fail(CP4_ERR_SHAPE, "tile_rows >= 0 and schedule 0, 1 or 2 expected");
+  const FwdArgs a =
+      backward_data
+          ? backward_data_args(*shape, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr)
+          : forward_args(*shape, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr);
+  // (schedule as cp4_tuned_choice reports it: 1 the kernel's rule, 0 no role split, 2 whole groups)
+  const Choice c{variant, tile_rows, lgwt, schedule == 1 ? 0 : (schedule == 0 ? 1 : 2)};
+  if (!kVariants[variant].supported(with_tile(a, c)))
+    return fail(CP4_ERR_UNSUPPORTED, "the variant does not take this shape with this tile");
+  std::lock_guard<std::mutex> lk(g_tune_mu);
+  g_tuned[key_of(a)] = c;
   return CP4_OK;
 }
 

@@ -104,6 +104,7 @@ constexpr int kProd = 8, kCons = 8;          // producer / consumer waves (4 per
 constexpr int kRP = 32;
 constexpr int kCcBuf = 24 * 512;             // bytes of one Cc fragment tile (64 pixels)
 constexpr size_t kLdsLimit = 160 * 1024;
+constexpr int kOwnGroupsMaxRank = 4;         // ranks up to which consumer waves take whole groups by default
 #ifndef CP4_WHOLE_BLOCK_MIN
 #define CP4_WHOLE_BLOCK_MIN 16
 #endif
@@ -126,6 +127,7 @@ struct PipePlan {
   int Wt, lgWt, cols;       // tiled build: tile width, its log2, column tiles per row strip
   unsigned wl_magic;        // tiled build: 2^32 / (Wt + FS - 1) + 1, for the division by the row length
   int split2;               // consumer waves split roles also above 16 ranks / 4 channel blocks
+  int own;                  // consumer waves take whole groups each (few ranks and channel blocks)
   int spin_limit;           // polls before a wait between waves gives up
 #ifdef CP4_DEBUG_PHASES
   long long* dbg;
@@ -534,7 +536,19 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // Above that, up to 8 channel blocks (wide split): a tap wave takes two rank
     // quads (wq and wq + 4), a contraction wave two channel blocks (wc and
     // wc + 4, both output-factor fragments in registers).
-    const bool split_narrow = FS <= 5 && R <= 16 && nkb <= 4;  // (7x7: no registers to spare)
+    // With at most 16 ranks and one or two channel blocks even that leaves most
+    // waves idle and every group's latency in series; a strip of many groups then
+    // runs them side by side instead (own groups): consumer wave wc takes groups
+    // wc, wc + 8, ... whole - the taps of all rank quads into a tile of its own,
+    // then the contractions - with no hand-over between consumer waves at all.
+    // (Only in the builds for up to 64 input channels, whose producers leave the
+    // registers for it.)
+#ifdef CP4_PIPE_TAPS2D
+    constexpr bool own_groups = false;
+#else
+    const bool own_groups = NQ == 1 && pl.own && ngroups >= 4;   // (the host checked ranks, blocks, filter)
+#endif
+    const bool split_narrow = !own_groups && FS <= 5 && R <= 16 && nkb <= 4;  // (7x7: no registers to spare)
 #if defined(CP4_PIPE_TAPS2D) || defined(CP4_PIPE_EPILOGUE)
     // (twice the 2-D weights would not fit; nor would the bias rows next to two
     // output-factor fragments)
@@ -641,65 +655,65 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         ++frontier;
       return frontier > need;
     };
-    auto taps = [&](int i, unsigned char* cb, auto ntq_c) {
-      const int g = rev ? ngroups - 1 - i : i;
-      {
-        const int need = need_of(i);
-        while (frontier <= need) {
-          wait_ge(&flags[frontier], NQ, backoff, wx, 2);
-          ++frontier;
-        }
-      }
-      STAMPX(2 + 4 * i)
+    // Where the taps of pixel group g read the plane: first plane row h of the
+    // lane's pixel, row length RL, and per tap column the (clamped) plane column
+    // and whether it lies inside the image.
+    struct TapPos {
+      int h, RL;
+      int off[FS];
+      bool in[FS];
+    };
+    auto tap_pos = [&](int g) {
+      TapPos tp;
 #ifdef CP4_PIPE_TILED
       // the plane carries the halo columns: tap (ti, j) of cell (h, w) is plane
       // cell (h + ti, w + j), no border cases
       const int p = 64 * g + lane;
-      const int h = p >> lgWt, w = p & (Wt - 1);
-      const int RL = WL;                           // row length of the plane
-      int off[FS];
-      bool in[FS];
+      const int w = p & (Wt - 1);
+      tp.h = p >> lgWt;
+      tp.RL = WL;                                  // row length of the plane
 #pragma unroll
       for (int j = 0; j < FS; ++j) {
-        in[j] = true;
-        off[j] = w + j;
+        tp.in[j] = true;
+        tp.off[j] = w + j;
       }
 #elif defined(CP4_PIPE_STRIDED)
-      const int RL = W;
+      tp.RL = W;
       // lanes before or past the strip's outputs: any valid pixel (not stored)
       const int p = min(max(64 * g - gshift + lane, 0), nvalid - 1);
       const int ho = p / Wo, wo = p - ho * Wo;
-      const int h = SH * ho;                             // plane row of the first tap row
-      int off[FS];
-      bool in[FS];
+      tp.h = SH * ho;                              // plane row of the first tap row
 #pragma unroll
       for (int j = 0; j < FS; ++j) {
         const int ww = SW * wo + j - PL;
-        in[j] = ww >= 0 && ww < W;
-        off[j] = ww < 0 ? 0 : (ww >= W ? W - 1 : ww);      // clamped: weight is 0 there
+        tp.in[j] = ww >= 0 && ww < W;
+        tp.off[j] = ww < 0 ? 0 : (ww >= W ? W - 1 : ww);   // clamped: weight is 0 there
       }
 #else
-      const int RL = W;
+      tp.RL = W;
       const int p = max(64 * g - gshift + lane, 0);      // lanes before the strip: any valid column
-      const int h = p / W, w = p - h * W;
-      int off[FS];
-      bool in[FS];
+      tp.h = p / W;
+      const int w = p - tp.h * W;
 #pragma unroll
       for (int j = 0; j < FS; ++j) {
         const int ww = w + j - a.pad;
-        in[j] = ww >= 0 && ww < W;
-        off[j] = ww < 0 ? 0 : (ww >= W ? W - 1 : ww);      // clamped: weight is 0 there
+        tp.in[j] = ww >= 0 && ww < W;
+        tp.off[j] = ww < 0 ? 0 : (ww >= W ? W - 1 : ww);   // clamped: weight is 0 there
       }
 #endif
+      return tp;
+    };
+    // The taps of rank quad q at the lane's pixel, split exactly and written into
+    // fragment tile cb.  wa / wb: the quad's weights (2-D taps: wa[rank][row][col];
+    // else rows wa[rank][row] and columns wb[rank][col]).
+    auto tap_quad = [&](const TapPos& tp, int q, const auto& wa, [[maybe_unused]] const auto& wb,
+                        unsigned char* cb) {
       // the LDS reads of RBT ranks go out together, then their arithmetic
       constexpr int RBT = FS <= 3 ? 4 : (FS == 5 ? 2 : 1);
-#pragma unroll
-      for (int qi = 0; qi < decltype(ntq_c)::value; ++qi) {
-      const int q = wq + 4 * qi;                   // this pass's rank quad
       // (a quad past the last rank has zero weights; it reads quad 0's rows, the
       // plane may end before its own, and writes zeros)
       const bool live = 4 * q < R;
-      const float* ab = As + (size_t)(live ? 4 * q : 0) * QA + h * RL;
+      const float* ab = As + (size_t)(live ? 4 * q : 0) * QA + tp.h * tp.RL;
       float o[4];
 #pragma unroll
       for (int r0 = 0; r0 < 4; r0 += RBT) {
@@ -709,7 +723,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #pragma unroll
           for (int ti = 0; ti < FS; ++ti)
 #pragma unroll
-            for (int j = 0; j < FS; ++j) av[rr][ti][j] = ab[(r0 + rr) * QA + ti * RL + off[j]];
+            for (int j = 0; j < FS; ++j) av[rr][ti][j] = ab[(r0 + rr) * QA + ti * tp.RL + tp.off[j]];
 #pragma unroll
         for (int rr = 0; rr < RBT; ++rr) {
           float s = 0.f;
@@ -717,12 +731,12 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           for (int ti = 0; ti < FS; ++ti) {
 #ifdef CP4_PIPE_TAPS2D
 #pragma unroll
-            for (int j = 0; j < FS; ++j) s += (in[j] ? w2[qi][r0 + rr][ti][j] : 0.f) * av[rr][ti][j];
+            for (int j = 0; j < FS; ++j) s += (tp.in[j] ? wa[r0 + rr][ti][j] : 0.f) * av[rr][ti][j];
 #else
             float hs = 0.f;
 #pragma unroll
-            for (int j = 0; j < FS; ++j) hs += (in[j] ? fw[qi][r0 + rr][j] : 0.f) * av[rr][ti][j];
-            s += fh[qi][r0 + rr][ti] * hs;
+            for (int j = 0; j < FS; ++j) hs += (tp.in[j] ? wb[r0 + rr][j] : 0.f) * av[rr][ti][j];
+            s += wa[r0 + rr][ti] * hs;
 #endif
           }
           o[r0 + rr] = live ? s : 0.f;
@@ -746,6 +760,26 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       *reinterpret_cast<u32x2*>(dst) = ph;
       *reinterpret_cast<u32x2*>(dst + 8 * 512) = pm;
       *reinterpret_cast<u32x2*>(dst + 16 * 512) = pl2;
+    };
+    auto await_blocks = [&](int i) {
+      const int need = need_of(i);
+      while (frontier <= need) {
+        wait_ge(&flags[frontier], NQ, backoff, wx, 2);
+        ++frontier;
+      }
+    };
+    auto taps = [&](int i, unsigned char* cb, auto ntq_c) {
+      const int g = rev ? ngroups - 1 - i : i;
+      await_blocks(i);
+      STAMPX(2 + 4 * i)
+      const TapPos tp = tap_pos(g);
+#pragma unroll
+      for (int qi = 0; qi < decltype(ntq_c)::value; ++qi) {
+#ifdef CP4_PIPE_TAPS2D
+        tap_quad(tp, wq + 4 * qi, w2[qi], w2[qi], cb);
+#else
+        tap_quad(tp, wq + 4 * qi, fh[qi], fw[qi], cb);
+#endif
       }
       STAMPX(3 + 4 * i)
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -888,6 +922,54 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     [[maybe_unused]] constexpr std::integral_constant<bool, true> yes{};
     constexpr std::integral_constant<bool, false> no{};
 #ifndef CP4_PIPE_TAPS2D
+    if constexpr (NQ == 1) {
+    if (own_groups) {
+      // Two waves share a 12 KB tile buffer: with one rank chunk a group's
+      // fragments fill only the chunk-0 planes of each part, and the chunk-1
+      // planes (4 * 512 bytes further) hold the other wave's.
+      unsigned char* cb = Cb + (wc >> 1) * kCcBuf + (wc & 1) * (4 * 512);
+      const int nq = (R + 3) >> 2;
+      load_fk(0, slot0);
+      if (nkb > 1) load_fk(1, slot1);
+      // the quads past the last rank: zeros, written once (the tile is never
+      // anyone else's)
+      for (int q = nq; q < 4; ++q) {
+        unsigned char* dst = cb + ((((q >> 1) & 1) * 2 + (lane & 1)) * 512) + (lane >> 1) * 16 + (q & 1) * 8;
+        const u32x2 zero = {0u, 0u};
+        *reinterpret_cast<u32x2*>(dst) = zero;
+        *reinterpret_cast<u32x2*>(dst + 8 * 512) = zero;
+        *reinterpret_cast<u32x2*>(dst + 16 * 512) = zero;
+      }
+      for (int i = wc; i < ngroups; i += kCons) {
+        const int g = rev ? ngroups - 1 - i : i;
+        await_blocks(i);
+        STAMPX(2 + 4 * (i >> 3))
+        const TapPos tp = tap_pos(g);
+        for (int q = 0; q < nq; ++q) {
+          float qh[4][FS], qw[4][FS];               // wave-uniform loads
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr)
+#pragma unroll
+            for (int j = 0; j < FS; ++j) {
+              const int tap = a.flip ? FS - 1 - j : j, r = 4 * q + rr;
+              qh[rr][j] = r < R ? a.FH[tap * ldf + r] : 0.f;
+              qw[rr][j] = r < R ? a.FW[tap * ldf + r] : 0.f;
+            }
+          tap_quad(tp, q, qh, qw, cb);
+        }
+        STAMPX(3 + 4 * (i >> 3))
+        // (the tile is this wave's own: its LDS writes and reads stay in order)
+        load_bias(0);
+        contract_block(cb, g, 0, one, false, i, slot0, yes);
+        if (nkb > 1) {
+          load_bias(1);
+          contract_block(cb, g, 1, one, false, i, slot1, yes);
+        }
+        STAMPX(5 + 4 * (i >> 3))
+      }
+      return;
+    }
+    }
     if (split_wide) {
       // As the narrow split below, with two rank quads per tap wave and up to two
       // channel blocks per contraction wave; the tile is free again once every
@@ -996,6 +1078,21 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 
 int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
+// Fragment tiles: three in rotation, or one per consumer wave (two to a buffer)
+// where the kernel may give every wave groups of its own.
+bool own_groups_wanted(const FwdArgs& a) {
+#ifdef CP4_PIPE_TAPS2D
+  return false;
+#else
+  const bool legal = a.R <= 16 && a.Cout <= 64 && a.Cin <= 64 && a.Y <= 5 && !a.accumulate;
+  // by default where one rank quad is the whole tap step (the other schedules
+  // would run three empty quads beside it); above that only when tuned so
+  // (tune_split2: 0 this rule, 1 no role split at all, 2 own groups)
+  return legal && (a.tune_split2 == 2 || (a.tune_split2 == 0 && a.R <= kOwnGroupsMaxRank));
+#endif
+}
+size_t cc_region_bytes(const FwdArgs& a) { return (size_t)(own_groups_wanted(a) ? 4 : 3) * kCcBuf; }
+
 // Rank rows of the A plane in LDS: the producers' 32 x 32 products carry 32, of
 // which the upper 16 are zero (and neither written nor read) up to 16 ranks.
 int plane_rows(const FwdArgs& a) { return a.R <= 16 ? 16 : kRP; }
@@ -1009,7 +1106,7 @@ int plane_rows(const FwdArgs& a) { return a.R <= 16 ? 16 : kRP; }
   const size_t a_bytes = (size_t)plane_rows(a) * QA * sizeof(float);
   // above 256 input channels: pre-split factor fragments, 192 B per (padded) channel
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
-  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 16) * sizeof(int);
+  const size_t bytes = a_bytes + fin_bytes + cc_region_bytes(a) + (kMaxBlk + 16) * sizeof(int);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
@@ -1019,7 +1116,7 @@ int plane_rows(const FwdArgs& a) { return a.R <= 16 ? 16 : kRP; }
   pl->QA = (int)QA;
   pl->fin_off = (int)a_bytes;
   pl->cc_off = (int)(a_bytes + fin_bytes);
-  pl->flag_off = (int)(a_bytes + fin_bytes + 3 * kCcBuf);
+  pl->flag_off = (int)(a_bytes + fin_bytes + cc_region_bytes(a));
   pl->lds_bytes = bytes;
   return true;
 }
@@ -1031,7 +1128,7 @@ bool layout_strided(const FwdArgs& a, int TH, PipePlan* pl) {
   const long QA = round_up((int)QLEN, 64) + 8;
   const size_t a_bytes = (size_t)plane_rows(a) * QA * sizeof(float);
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
-  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 16) * sizeof(int);
+  const size_t bytes = a_bytes + fin_bytes + cc_region_bytes(a) + (kMaxBlk + 16) * sizeof(int);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
@@ -1041,7 +1138,7 @@ bool layout_strided(const FwdArgs& a, int TH, PipePlan* pl) {
   pl->QA = (int)QA;
   pl->fin_off = (int)a_bytes;
   pl->cc_off = (int)(a_bytes + fin_bytes);
-  pl->flag_off = (int)(a_bytes + fin_bytes + 3 * kCcBuf);
+  pl->flag_off = (int)(a_bytes + fin_bytes + cc_region_bytes(a));
   pl->lds_bytes = bytes;
   return true;
 }
@@ -1073,7 +1170,7 @@ bool layout_tiled(const FwdArgs& a, int TH, int lgWt, PipePlan* pl) {
   const long QA = round_up((int)QLEN, 64) + 8;
   const size_t a_bytes = (size_t)plane_rows(a) * QA * sizeof(float);
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
-  const size_t bytes = a_bytes + fin_bytes + 3 * kCcBuf + (kMaxBlk + 16) * sizeof(int);
+  const size_t bytes = a_bytes + fin_bytes + cc_region_bytes(a) + (kMaxBlk + 16) * sizeof(int);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
@@ -1087,7 +1184,7 @@ bool layout_tiled(const FwdArgs& a, int TH, int lgWt, PipePlan* pl) {
   pl->QA = (int)QA;
   pl->fin_off = (int)a_bytes;
   pl->cc_off = (int)(a_bytes + fin_bytes);
-  pl->flag_off = (int)(a_bytes + fin_bytes + 3 * kCcBuf);
+  pl->flag_off = (int)(a_bytes + fin_bytes + cc_region_bytes(a));
   pl->lds_bytes = bytes;
   return true;
 }
@@ -1243,7 +1340,8 @@ bool fwd_pipe_supported(const FwdArgs& a) {
 hipError_t fwd_pipe_launch(const FwdArgs& a, hipStream_t st) {
   PipePlan pl;
   if (!plan(a, &pl)) return hipErrorInvalidValue;
-  pl.split2 = a.tune_split2 != 1;               // 0: the kernel's own rule, 1: off, 2: as 0
+  pl.split2 = a.tune_split2 != 1;               // 0: the kernel's own rule, 1: off
+  pl.own = own_groups_wanted(a);
   pl.spin_limit = a.spin_limit > 0 ? a.spin_limit : kSpinLimit;
 #ifdef CP4_DEBUG_PHASES
   pl.dbg = debug_stamp_buffer();

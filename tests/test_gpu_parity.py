@@ -402,6 +402,61 @@ def test_timed_launch_and_tuner(cp4):
     assert torch.equal(y3, y4)
 
 
+# N, C, H, W, T, Y, R: few ranks and channels, planes of many blocks (whole-block
+# producers; consumer waves that take whole pixel groups each)
+FEW_CHANNEL_CASES = [
+    (2, 64, 96, 96, 64, 3, 16),
+    (2, 32, 112, 112, 32, 3, 4),        # whole groups by the kernel's own rule
+    (1, 48, 224, 224, 40, 3, 9),        # ragged channels, three rank quads, wide plane (tiles)
+    (2, 20, 64, 80, 64, 5, 16),
+    (3, 16, 72, 72, 24, 3, 1),
+    (1, 64, 130, 70, 33, 1, 12),
+]
+
+
+@pytest.mark.parametrize("dims", FEW_CHANNEL_CASES, ids=lambda d: "x".join(map(str, d)))
+def test_consumer_schedules_at_few_channels(cp4, oracle, dims):
+    """Every consumer schedule (the kernel's rule, no role split, whole groups per
+    wave) of every producer / consumer variant that takes the shape, entered through
+    the tuner's table, against the oracle; forward and backward-data."""
+    N, C, H, W, T, Y, R = dims
+    rng = np.random.default_rng(sum(dims))
+    a = {"x": rng.standard_normal((N, C, H, W), dtype=np.float32),
+         "dy": rng.standard_normal((N, T, H, W), dtype=np.float32)}
+    for k, d in (("FK", T), ("FC", C), ("FH", Y), ("FW", Y)):
+        a[k] = rng.standard_normal((d, R), dtype=np.float32) * np.float32((R * C * Y * Y) ** -0.25)
+    fa = [a[k] for k in FACTORS]
+    f = [dev(a[k]) for k in FACTORS]
+    x, dy = dev(a["x"]), dev(a["dy"])
+    pad = (Y - 1) // 2
+    want_y = oracle.forward(a["x"], *fa, pad)
+    want_dx = oracle.backward_data(a["dy"], *fa, pad)
+    s = cp4.capi.shape_for(x.shape, *f, pad)
+    ran = 0
+    try:
+        for v, name, ok in cp4.forward_variants(s):
+            if not ok or "pipe" not in name:
+                continue
+            for schedule in (1, 0, 2):
+                for th in (0, 3):
+                    cols = 64 if (th and "tiled" in name) else 0
+                    for bwd in (False, True):
+                        try:
+                            cp4.set_tuned_choice(s, v, th, cols, schedule, backward_data=bwd)
+                        except cp4.Cp4Error as e:      # this tile does not fit this variant
+                            assert e.status == cp4.capi.ERR_UNSUPPORTED
+                            continue
+                        got = (cp4.conv2d_backward_data(dy, *f, pad=pad) if bwd
+                               else cp4.conv2d_forward(x, *f, pad=pad))
+                        assert_activation_close(host(got), want_dx if bwd else want_y,
+                                             f"{name} schedule {schedule} th {th} bwd {bwd}")
+                        ran += 1
+    finally:
+        cp4.tune_clear()
+    cp4.device_status()
+    assert ran >= 6
+
+
 # ------------------------------------------------ ranks beyond a kernel's tile ----
 @pytest.mark.parametrize("R", [33, 48, 64, 65, 96, 128, 200])
 def test_ranks_beyond_one_tile(cp4, oracle, R):
