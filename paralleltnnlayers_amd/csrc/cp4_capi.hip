@@ -942,9 +942,27 @@ cp4_status cp4_conv2d_backward_data_ex(const cp4_shape* shape, const cp4_geometr
   if (rc != CP4_OK) return rc;
   const cp4_shape& s = *shape;
   hipStream_t st = as_stream(stream);
-  // dx[h,w] = sum_{i,j} K[i,j] dyu[h + pad_top - i, w + pad_left - j] with dyu = dy spread
+  // In general: dx[h,w] = sum_{i,j} K[i,j] dyu[h + pad_top - i, w + pad_left - j] with dyu = dy spread
   // out with zeros: a stride-1 pass over dyu with the taps in reverse order, Y - 1 - pad_top
   // zeros before it and an H x W output.
+  if (g->stride_h > 1 || g->stride_w > 1) {
+    // The strided build's adjoint mode reads dy as it is: tap (i, j) of input pixel
+    // (h, w) takes dy at ((h + pad_top - i) / sh, (w + pad_left - j) / sw) where
+    // both divisions are exact.
+    cp4_shape sd = s;
+    sd.H = g->out_h; sd.W = g->out_w;
+    FwdArgs t = backward_data_args(sd, dy, FK, FC, FH, FW, dx);
+    t.flip = 0;
+    t.transposed = 1;
+    t.sh = (int)g->stride_h; t.sw = (int)g->stride_w;
+    t.pt = (int)g->pad_top; t.pl = (int)g->pad_left;
+    t.Ho = (int)s.H; t.Wo = (int)s.W;
+    if (cp4::fwd_pipe_strided_supported(t) && t.Cin + t.Cout >= kMatrixMinChannels) {
+      arm(t);
+      CP4_HIP(cp4::fwd_pipe_strided_launch(t, st));
+      return CP4_OK;
+    }
+  }
   const unsigned hu = g->stride_h * (g->out_h - 1) + 1, wu = g->stride_w * (g->out_w - 1) + 1;
   const float* src = dy;
   if (g->stride_h > 1 || g->stride_w > 1) {

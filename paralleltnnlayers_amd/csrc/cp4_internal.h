@@ -48,6 +48,13 @@ struct FwdArgs {
   // the output plane is Ho x Wo.  sh == 0: the reference's geometry, the other
   // fields unused.  Only kernels that say so take sh != 0.
   int sh, sw, pt, pl, Ho, Wo;
+  // Strided build of the producer / consumer kernel only: the adjoint of a strided
+  // layer (its backward-data pass).  The H x W input plane is then the strided
+  // layer's output gradient and the Ho x Wo output plane its input gradient:
+  // output pixel (h, w) sums tap (i, j) times input pixel ((h + pt - i) / sh,
+  // (w + pl - j) / sw) wherever both divisions are exact and land inside the plane
+  // (flip unused).
+  int transposed;
   // Recomposed-filter kernel only: the dense filter [Cout, Cin, Y, X] itself, taps in
   // the order the pass reads them; the four factors are unused then.
   const float* dense;

@@ -257,8 +257,12 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   const int QLEN = (pl.TH + FS - 1) * WL;
 #else
 #ifdef CP4_PIPE_STRIDED
-  const int qbase = (SH * h0 - PT) * W;          // global flat pixel of LDS column 0
-  const int QLEN = (SH * (pl.TH - 1) + FS) * W;
+  // adjoint of a strided layer: the plane holds the input rows trow0 ... that the
+  // strip's output rows h0 ... h0 + TH - 1 can draw on, (h + PT - i) / SH
+  const bool TR = a.transposed != 0;
+  const int trow0 = h0 + PT - (FS - 1) <= 0 ? 0 : (h0 + PT - (FS - 1) + SH - 1) / SH;
+  const int qbase = TR ? trow0 * W : (SH * h0 - PT) * W;   // global flat pixel of LDS column 0
+  const int QLEN = TR ? ((pl.TH + FS - 2) / SH + 1) * W : (SH * (pl.TH - 1) + FS) * W;
 #else
   const int qbase = (h0 - a.pad) * W;            // global flat pixel of LDS column 0
   const int QLEN = (pl.TH + FS - 1) * W;
@@ -635,6 +639,21 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       // read the plane rows SH*h ... SH*h + FS - 1 of its first to last output row h
       const int g = rev ? ngroups - 1 - i : i;
       const int pf = max(64 * g - gshift, 0), pz = min(64 * g - gshift + 63, nvalid - 1);
+      if (TR) {
+        // output rows hf ... hz draw on the input rows ceil((hf + PT - FS + 1) / SH)
+        // ... floor((hz + PT) / SH)
+        const int hf = h0 + pf / Wo, hz = h0 + pz / Wo;
+        if (rev) {
+          const int num = hf + PT - (FS - 1);
+          const int first = (num <= 0 ? 0 : (num + SH - 1) / SH) - trow0;   // >= 0
+          const int b = (first * W) >> 5;
+          return b > nblk - 1 ? 0 : nblk - 1 - b;
+        }
+        const int lastrow = min((hz + PT) / SH, H - 1) - trow0;
+        if (lastrow < 0) return 0;
+        const int last = ((lastrow + 1) * W - 1) >> 5;
+        return last > nblk - 1 ? nblk - 1 : last;
+      }
       if (rev) return nblk - 1 - ((SH * (pf / Wo) * W) >> 5);
       const int last = ((SH * (pz / Wo) + FS - 1) * W + W - 1) >> 5;
       return last > nblk - 1 ? nblk - 1 : last;
@@ -659,7 +678,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // lane's pixel, row length RL, and per tap column the (clamped) plane column
     // and whether it lies inside the image.
     struct TapPos {
-      int h, RL;
+      int roff[FS];                                // plane offset of tap row ti
+      bool rin[FS];                                // ... and whether that row exists
       int off[FS];
       bool in[FS];
     };
@@ -669,36 +689,59 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       // the plane carries the halo columns: tap (ti, j) of cell (h, w) is plane
       // cell (h + ti, w + j), no border cases
       const int p = 64 * g + lane;
-      const int w = p & (Wt - 1);
-      tp.h = p >> lgWt;
-      tp.RL = WL;                                  // row length of the plane
+      const int w = p & (Wt - 1), h = p >> lgWt;
 #pragma unroll
       for (int j = 0; j < FS; ++j) {
         tp.in[j] = true;
         tp.off[j] = w + j;
+        tp.rin[j] = true;
+        tp.roff[j] = (h + j) * WL;                 // WL: row length of the plane
       }
 #elif defined(CP4_PIPE_STRIDED)
-      tp.RL = W;
       // lanes before or past the strip's outputs: any valid pixel (not stored)
       const int p = min(max(64 * g - gshift + lane, 0), nvalid - 1);
       const int ho = p / Wo, wo = p - ho * Wo;
-      tp.h = SH * ho;                              // plane row of the first tap row
+      if (TR) {
+        // tap row ti: input row (h + PT - ti) / SH where that is exact and inside the
+        // plane; quotient and remainder step down with ti (one division per lane)
+        int qh = (h0 + ho + PT) / SH, rh = (h0 + ho + PT) - qh * SH;
+        int qw = (wo + PL) / SW, rw = (wo + PL) - qw * SW;
 #pragma unroll
-      for (int j = 0; j < FS; ++j) {
-        const int ww = SW * wo + j - PL;
-        tp.in[j] = ww >= 0 && ww < W;
-        tp.off[j] = ww < 0 ? 0 : (ww >= W ? W - 1 : ww);   // clamped: weight is 0 there
+        for (int j = 0; j < FS; ++j) {
+          tp.rin[j] = rh == 0 && qh >= 0 && qh < H;
+          tp.roff[j] = tp.rin[j] ? (qh - trow0) * W : 0;
+          tp.in[j] = rw == 0 && qw >= 0 && qw < W;
+          tp.off[j] = tp.in[j] ? qw : 0;
+          if (--rh < 0) {
+            rh += SH;
+            --qh;
+          }
+          if (--rw < 0) {
+            rw += SW;
+            --qw;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < FS; ++j) {
+          const int ww = SW * wo + j - PL;
+          tp.in[j] = ww >= 0 && ww < W;
+          tp.off[j] = ww < 0 ? 0 : (ww >= W ? W - 1 : ww);   // clamped: weight is 0 there
+          tp.rin[j] = true;
+          tp.roff[j] = (SH * ho + j) * W;          // plane row SH * ho is the first tap row
+        }
       }
 #else
-      tp.RL = W;
       const int p = max(64 * g - gshift + lane, 0);      // lanes before the strip: any valid column
-      tp.h = p / W;
-      const int w = p - tp.h * W;
+      const int h = p / W;
+      const int w = p - h * W;
 #pragma unroll
       for (int j = 0; j < FS; ++j) {
         const int ww = w + j - a.pad;
         tp.in[j] = ww >= 0 && ww < W;
         tp.off[j] = ww < 0 ? 0 : (ww >= W ? W - 1 : ww);   // clamped: weight is 0 there
+        tp.rin[j] = true;
+        tp.roff[j] = (h + j) * W;
       }
 #endif
       return tp;
@@ -713,7 +756,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       // (a quad past the last rank has zero weights; it reads quad 0's rows, the
       // plane may end before its own, and writes zeros)
       const bool live = 4 * q < R;
-      const float* ab = As + (size_t)(live ? 4 * q : 0) * QA + tp.h * tp.RL;
+      const float* ab = As + (size_t)(live ? 4 * q : 0) * QA;
       float o[4];
 #pragma unroll
       for (int r0 = 0; r0 < 4; r0 += RBT) {
@@ -723,7 +766,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #pragma unroll
           for (int ti = 0; ti < FS; ++ti)
 #pragma unroll
-            for (int j = 0; j < FS; ++j) av[rr][ti][j] = ab[(r0 + rr) * QA + ti * tp.RL + tp.off[j]];
+            for (int j = 0; j < FS; ++j) av[rr][ti][j] = ab[(r0 + rr) * QA + tp.roff[ti] + tp.off[j]];
 #pragma unroll
         for (int rr = 0; rr < RBT; ++rr) {
           float s = 0.f;
@@ -731,12 +774,13 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           for (int ti = 0; ti < FS; ++ti) {
 #ifdef CP4_PIPE_TAPS2D
 #pragma unroll
-            for (int j = 0; j < FS; ++j) s += (tp.in[j] ? wa[r0 + rr][ti][j] : 0.f) * av[rr][ti][j];
+            for (int j = 0; j < FS; ++j)
+              s += (tp.in[j] && tp.rin[ti] ? wa[r0 + rr][ti][j] : 0.f) * av[rr][ti][j];
 #else
             float hs = 0.f;
 #pragma unroll
             for (int j = 0; j < FS; ++j) hs += (tp.in[j] ? wb[r0 + rr][j] : 0.f) * av[rr][ti][j];
-            s += wa[r0 + rr][ti] * hs;
+            s += (tp.rin[ti] ? wa[r0 + rr][ti] : 0.f) * hs;
 #endif
           }
           o[r0 + rr] = live ? s : 0.f;
@@ -1124,7 +1168,8 @@ int plane_rows(const FwdArgs& a) { return a.R <= 16 ? 16 : kRP; }
 #ifdef CP4_PIPE_STRIDED
 // Strip of TH output rows: plane of the sh * (TH - 1) + Y input rows under them.
 bool layout_strided(const FwdArgs& a, int TH, PipePlan* pl) {
-  const long QLEN = ((long)a.sh * (TH - 1) + a.Y) * a.W;
+  const long QLEN = a.transposed ? ((long)(TH + a.Y - 2) / a.sh + 1) * a.W
+                                 : ((long)a.sh * (TH - 1) + a.Y) * a.W;
   const long QA = round_up((int)QLEN, 64) + 8;
   const size_t a_bytes = (size_t)plane_rows(a) * QA * sizeof(float);
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
@@ -1152,7 +1197,7 @@ bool plan(const FwdArgs& a, PipePlan* best) {
     if (!layout_strided(a, TH, &pl)) break;
     const double rounds = (pl.nWG + cus - 1) / cus;
     // cells read per channel and cells written per channel
-    const double cost = rounds * (((double)a.sh * (TH - 1) + a.Y) * a.W * a.Cin +
+    const double cost = rounds * ((double)pl.nblk * 32 * a.Cin +
                                   (double)TH * a.Wo * a.Cout + kTileStartCost);
     if (!found || cost <= best_cost) {
       best_cost = cost;

@@ -92,6 +92,9 @@ MATRIX_CASES = [
     (1, 32, 12, 12, 32, 3, 16, 1, 2),               # output larger than the input
     (1, 40, 33, 33, 72, 7, 16, 3, "same"),
     (2, 300, 14, 14, 64, 3, 16, 2, "same"),         # factor fragments in LDS
+    (1, 32, 31, 45, 48, 5, 16, (3, 2), 2),          # unequal strides, 5x5
+    (2, 32, 150, 40, 32, 3, 12, 2, "same"),         # many strips (both sweep directions)
+    (1, 64, 96, 96, 64, 3, 4, (1, 2), 1),           # stride across only; whole-group consumers
 ]
 
 
