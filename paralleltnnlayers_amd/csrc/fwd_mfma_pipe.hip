@@ -40,9 +40,9 @@
 // Cuda_kernels/cp4Conv2dForward.cu:84-133 (backward-data:
 // cp4Conv2dBackwardData.cu:57-108 through swapped factors and flipped taps).
 //
-// This file is compiled seven times: as is; with CP4_PIPE_EPILOGUE defined, which
-// adds y = act(conv + bias[k]) to the stores (the bias of the lane's sixteen
-// output rows rides in registers next to the output-factor fragment) and exports
+// This file is compiled nine times: as is; with CP4_PIPE_EPILOGUE defined, which
+// adds y = act(conv + bias[k]) to the stores (the bias, padded to whole channel
+// blocks, waits in LDS and is what the accumulators start from) and exports
 // the entry points under the names fwd_pipe_epi_*; and with CP4_PIPE_IO16, where
 // x and y are bfloat16 in memory (factors, bias and all arithmetic stay fp32):
 // a bf16 activation is its own high part, so the channel contraction needs
@@ -191,6 +191,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   // counters, then the 4 contraction counters of the split-role schedule, then
   // the abort word
   int* flags = reinterpret_cast<int*>(ldsb + pl.flag_off);
+#ifdef CP4_PIPE_EPILOGUE
+  float* biasL = reinterpret_cast<float*>(flags + kMaxBlk + 16);   // [32 * nkb], zero past Cout
+#endif
 
   const int per = (pl.nWG + 7) >> 3;
   const int t = (blockIdx.x & 7) * per + (blockIdx.x >> 3);         // XCD-contiguous tile order
@@ -278,6 +281,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   constexpr int NB = kProd / NQ;                   // blocks per producer round
   const int cpq = FLDS ? (Cin + 63) >> 6 : CPQ;    // 16-channel chunks per channel split
   if (tid < kMaxBlk + 16) flags[tid] = 0;
+#ifdef CP4_PIPE_EPILOGUE
+  for (int k = tid; k < 32 * nkb; k += kThreads) biasL[k] = (a.bias && k < Cout) ? a.bias[k] : 0.f;
+#endif
   if (FLDS) {
     for (int it = tid; it < 8 * cpq * 32; it += kThreads) {
       const int o = it >> 5, r = it & 31;          // channel octet (of the padded count), rank
@@ -503,18 +509,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // (slot 1: second block of a contraction wave in the wide split-role schedule)
     u32x4 fkh[2][2], fkm[2][2], fkl[2][2];
 #ifdef CP4_PIPE_EPILOGUE
-    float bs[16];                                  // bias of accumulator row v
     const bool relu = a.act != 0;
 #endif
-    [[maybe_unused]] auto load_bias = [&](int kb) {
-#ifdef CP4_PIPE_EPILOGUE
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int kk = 32 * kb + 8 * (v >> 2) + 4 * hi + (v & 3);
-        bs[v] = (a.bias && kk < Cout) ? a.bias[kk] : 0.f;
-      }
-#endif
-    };
     auto load_fk = [&](int kb, auto slot_c) {
       constexpr int slot = decltype(slot_c)::value;
       const int k = 32 * kb + l32;
@@ -553,9 +549,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     const bool own_groups = NQ == 1 && pl.own && ngroups >= 4;   // (the host checked ranks, blocks, filter)
 #endif
     const bool split_narrow = !own_groups && FS <= 5 && R <= 16 && nkb <= 4;  // (7x7: no registers to spare)
-#if defined(CP4_PIPE_TAPS2D) || defined(CP4_PIPE_EPILOGUE)
-    // (twice the 2-D weights would not fit; nor would the bias rows next to two
-    // output-factor fragments)
+#if defined(CP4_PIPE_TAPS2D)
+    // (twice the 2-D weights would not fit)
     const bool split_wide = false;
 #else
     // It pays with six or more channel blocks, or once the groups of a strip form a
@@ -570,7 +565,6 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     const int wq = split_roles ? (wc >= 4 ? wc - 4 : 0) : wc;     // (first) rank quad in the tap step
     if (!split_wide && fk_cached && wc < nkb) {
       load_fk(wc, slot0);
-      load_bias(wc);
     }
     // Tap weights of this wave's 4 ranks (wave-uniform values).
 #ifdef CP4_PIPE_TAPS2D
@@ -586,11 +580,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           w2[0][rr][ti][j] = r < R ? a.taps2d[(ty * FS + tx) * ldf + r] : 0.f;
         }
 #else
-#ifdef CP4_PIPE_EPILOGUE
-    constexpr int NTQ = 1;
-#else
     constexpr int NTQ = FS <= 3 ? 2 : 1;           // quads a tap wave may take (wide split)
-#endif
     float fh[NTQ][4][FS], fw[NTQ][4][FS];
     auto load_taps = [&](auto qi_c) {
       constexpr int qi = decltype(qi_c)::value;
@@ -836,7 +826,17 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     auto contract_block = [&](const unsigned char* cb, int g, int kb, auto nch, bool signal,
                               int step, auto slot_c, auto seq_c) {
       constexpr int slot = decltype(slot_c)::value;
+#ifdef CP4_PIPE_EPILOGUE
+      // the accumulators start at the bias of their rows (from LDS) instead of zero
+      const float* bkb = biasL + 32 * kb + 4 * hi;
+      f32x16 acc0 = {bkb[0],  bkb[1],  bkb[2],  bkb[3],  bkb[8],  bkb[9],  bkb[10], bkb[11],
+                     bkb[16], bkb[17], bkb[18], bkb[19], bkb[24], bkb[25], bkb[26], bkb[27]};
+      f32x16 acc1 = {bkb[0],  bkb[1],  bkb[2],  bkb[3],  bkb[8],  bkb[9],  bkb[10], bkb[11],
+                     bkb[16], bkb[17], bkb[18], bkb[19], bkb[24], bkb[25], bkb[26], bkb[27]};
+      __builtin_amdgcn_sched_barrier(0);
+#else
       f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
+#endif
 #pragma unroll
       for (int c = 0; c < decltype(nch)::value; ++c) {
         const unsigned char* bp = cb + ((c * 2 + hi) * 2) * 512 + l32 * 16;
@@ -875,17 +875,12 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           __hip_atomic_fetch_add(&cdone[step & 3], 1, __ATOMIC_RELEASE,
                                  __HIP_MEMORY_SCOPE_WORKGROUP);
       }
+      // The activation goes onto each value as it is stored (rewriting the
+      // accumulators in place costs the compiler some 150 spilled registers).
 #ifdef CP4_PIPE_EPILOGUE
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        float o0 = acc0[v] + bs[v], o1 = acc1[v] + bs[v];
-        if (relu) {
-          o0 = o0 < 0.f ? 0.f : o0;
-          o1 = o1 < 0.f ? 0.f : o1;
-        }
-        acc0[v] = o0;
-        acc1[v] = o1;
-      }
+#define EPI(val, v) (relu && (val) < 0.f ? 0.f : (val))          // (a NaN stays a NaN)
+#else
+#define EPI(val, v) (val)
 #endif
       // store rows: uniform row base + one 32-bit lane offset
       const int p = 64 * g - gshift + 2 * l32;       // lane's pixel pair p, p + 1
@@ -935,13 +930,13 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           if (32 * kb + 32 <= Cout) {
 #pragma unroll
             for (int v = 0; v < 16; ++v)
-              store_pair(rowbase + (size_t)(8 * (v >> 2) + (v & 3)) * HWo + lofs, acc0[v], acc1[v]);
+              store_pair(rowbase + (size_t)(8 * (v >> 2) + (v & 3)) * HWo + lofs, EPI(acc0[v], v), EPI(acc1[v], v));
           } else {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
               const int kk = 8 * (v >> 2) + (v & 3);         // + 4*hi is in lofs
               if (32 * kb + kk + 4 * hi < Cout)
-                store_pair(rowbase + (size_t)kk * HWo + lofs, acc0[v], acc1[v]);
+                store_pair(rowbase + (size_t)kk * HWo + lofs, EPI(acc0[v], v), EPI(acc1[v], v));
             }
           }
         }
@@ -954,8 +949,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           const int kk = 8 * (v >> 2) + (v & 3);
           if (32 * kb + kk + 4 * hi < Cout) {
             io_t* rp = rowbase + (size_t)kk * HWo + lofs;
-            if (in0) store_one(rp, acc0[v]);
-            if (in1) store_one(rp + 1, acc1[v]);
+            if (in0) store_one(rp, EPI(acc0[v], v));
+            if (in1) store_one(rp + 1, EPI(acc1[v], v));
           }
         }
       }
@@ -1003,10 +998,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         }
         STAMPX(3 + 4 * (i >> 3))
         // (the tile is this wave's own: its LDS writes and reads stay in order)
-        load_bias(0);
         contract_block(cb, g, 0, one, false, i, slot0, yes);
         if (nkb > 1) {
-          load_bias(1);
           contract_block(cb, g, 1, one, false, i, slot1, yes);
         }
         STAMPX(5 + 4 * (i >> 3))
@@ -1038,20 +1031,17 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         const bool second = wc + 4 < nkb;
         load_fk(wc, slot0);
         if (second) load_fk(wc + 4, slot1);
-        if (!second) load_bias(wc);
         for (int i = 0; i < ngroups; ++i) {
           const int g = rev ? ngroups - 1 - i : i;
           const unsigned char* cb = Cb + (i % 3) * kCcBuf;
           wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1), backoff, wx, 4);
           STAMPX(4 + 4 * i)
-          if (second) load_bias(wc);
           if (R <= 16) {
             contract_block(cb, g, wc, one, !second, i, slot0, yes);
           } else {
             contract_block(cb, g, wc, two, !second, i, slot0, yes);
           }
           if (second) {
-            load_bias(wc + 4);
             if (R <= 16) {
               contract_block(cb, g, wc + 4, one, true, i, slot1, yes);
             } else {
@@ -1106,7 +1096,6 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       for (int kb = wc; kb < nkb; kb += kCons) {
         if (!fk_cached) {
           load_fk(kb, slot0);
-          load_bias(kb);
         }
         contract_block(cb, g, kb, two, false, i, slot0, no);
       }
@@ -1121,6 +1110,16 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 }
 
 int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+// After the fragment tiles: the progress words and, in the builds with the bias /
+// activation epilogue, the bias padded to whole 32-channel blocks.
+size_t tail_bytes(const FwdArgs& a) {
+  size_t b = (kMaxBlk + 16) * sizeof(int);
+#ifdef CP4_PIPE_EPILOGUE
+  b += (size_t)((a.Cout + 31) & ~31) * sizeof(float);
+#endif
+  return b;
+}
 
 // Fragment tiles: three in rotation, or one per consumer wave (two to a buffer)
 // where the kernel may give every wave groups of its own.
@@ -1150,7 +1149,7 @@ int plane_rows(const FwdArgs& a) { return a.R <= 16 ? 16 : kRP; }
   const size_t a_bytes = (size_t)plane_rows(a) * QA * sizeof(float);
   // above 256 input channels: pre-split factor fragments, 192 B per (padded) channel
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
-  const size_t bytes = a_bytes + fin_bytes + cc_region_bytes(a) + (kMaxBlk + 16) * sizeof(int);
+  const size_t bytes = a_bytes + fin_bytes + cc_region_bytes(a) + tail_bytes(a);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
@@ -1173,7 +1172,7 @@ bool layout_strided(const FwdArgs& a, int TH, PipePlan* pl) {
   const long QA = round_up((int)QLEN, 64) + 8;
   const size_t a_bytes = (size_t)plane_rows(a) * QA * sizeof(float);
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
-  const size_t bytes = a_bytes + fin_bytes + cc_region_bytes(a) + (kMaxBlk + 16) * sizeof(int);
+  const size_t bytes = a_bytes + fin_bytes + cc_region_bytes(a) + tail_bytes(a);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
@@ -1215,7 +1214,7 @@ bool layout_tiled(const FwdArgs& a, int TH, int lgWt, PipePlan* pl) {
   const long QA = round_up((int)QLEN, 64) + 8;
   const size_t a_bytes = (size_t)plane_rows(a) * QA * sizeof(float);
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
-  const size_t bytes = a_bytes + fin_bytes + cc_region_bytes(a) + (kMaxBlk + 16) * sizeof(int);
+  const size_t bytes = a_bytes + fin_bytes + cc_region_bytes(a) + tail_bytes(a);
   if ((QLEN + 31) / 32 + 1 > kMaxBlk) return false;
   if (bytes > kLdsLimit) return false;
   pl->TH = TH;
