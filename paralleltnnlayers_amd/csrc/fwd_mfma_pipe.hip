@@ -1129,9 +1129,12 @@ bool own_groups_wanted(const FwdArgs& a) {
 #else
   const bool legal = a.R <= 16 && a.Cout <= 64 && a.Cin <= 64 && a.Y <= 5 && !a.accumulate;
   // by default where one rank quad is the whole tap step (the other schedules
-  // would run three empty quads beside it); above that only when tuned so
+  // would run three empty quads beside it), with 3x3 and smaller filters also for
+  // two quads (16 x 16 x 512 x 512 at rank 8: 212 against 276 us; 5x5: 28 against
+  // 22); above that only when tuned so
   // (tune_split2: 0 this rule, 1 no role split at all, 2 own groups)
-  return legal && (a.tune_split2 == 2 || (a.tune_split2 == 0 && a.R <= kOwnGroupsMaxRank));
+  const bool by_rule = a.R <= kOwnGroupsMaxRank || (a.R <= 2 * kOwnGroupsMaxRank && a.Y <= 3);
+  return legal && (a.tune_split2 == 2 || (a.tune_split2 == 0 && by_rule));
 #endif
 }
 size_t cc_region_bytes(const FwdArgs& a) { return (size_t)(own_groups_wanted(a) ? 4 : 3) * kCcBuf; }
