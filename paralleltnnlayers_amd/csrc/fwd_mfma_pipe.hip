@@ -112,6 +112,9 @@ constexpr int kOwnGroupsMaxRank = 4;         // ranks up to which consumer waves
 // fragments, the consumers' wait for the first rows: 7-8 us), in the planners'
 // unit of one channel of one cell read or written (7-11 thousand per us).
 constexpr double kTileStartCost = 50000.0;
+// C3 (56-pixel rows): 7-row strips, 256 workgroups, 39.6 us on one buffer set and
+// 61.6 us on rotating sets; 8-row strips, 224 workgroups, 38.1 and 56.0 us.
+constexpr double kUnalignedStripCost = 1.12;
 constexpr int kWholeBlockMin = CP4_WHOLE_BLOCK_MIN;   // blocks per plane from which 17-64 channels go unsplit
 constexpr int kSpinLimit = 1 << 19;      // default bound of a wait: about a quarter of a second at the longest nap
 constexpr int kMaxBlk = 64;                  // per-block progress words in LDS
@@ -1272,8 +1275,11 @@ bool plan(const FwdArgs& a, PipePlan* best) {
     PipePlan pl;
     if (!layout(a, TH, &pl)) break;
     const double rounds = (pl.nWG + cus - 1) / cus;
-    const double cost = rounds * ((double)(TH + a.Y - 1) * a.Cin + (double)TH * a.Cout +
-                                  kTileStartCost / a.W);
+    double cost = rounds * ((double)(TH + a.Y - 1) * a.Cin + (double)TH * a.Cout +
+                            kTileStartCost / a.W);
+    // Strips that do not end on a 128-byte line of y share that line with their
+    // neighbour (two partial writes) and start with a partly masked group.
+    if (((long)TH * a.W * kIoBytes) % 128 != 0 && TH < a.H) cost *= kUnalignedStripCost;
     // on equal cost (1x1 filters: no halo rows) the taller strip: fewer workgroups
     if (!found || cost <= best_cost) {
       best_cost = cost;
