@@ -45,7 +45,7 @@ FACTORS = ("FK", "FC", "FH", "FW")
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs, scaled by the plain copy kernel's reading (see
 # profiles/): {workload: bytes}.  None until measured for the current kernel.
-MEASURED_TRAFFIC = {"C3": 213.5e6}   # fwd_pipe_kernel<3,4,2,false,4>: 110.5 MB fetched + 103.1 MB written
+MEASURED_TRAFFIC = {"C3": 209.8e6}   # fwd_pipe_kernel<3,4,2,false,4>: 107.0 MB fetched + 102.8 MB written
 
 
 def main():
@@ -138,6 +138,9 @@ def main():
         f = [d[k] for k in FACTORS]
         xs = [d["x"]] + [d["x"].clone() for _ in range(args.cold_sets - 1)]
         ys = [torch.empty((w.N, w.T, w.H, w.W), device="cuda") for _ in xs]
+        t_settle = time.perf_counter()
+        while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+            cp4.time_forward_sets(xs, *f, ys, w.pad, 0, 200)
         cus = cp4.time_forward_sets(xs, *f, ys, w.pad, args.warmup, args.steps)
         print(json.dumps({"workload": w.name, "sets": len(xs), "us_per_launch": round(cus, 2),
                           "GB/s": round(nbytes / cus / 1e3, 1),
