@@ -244,11 +244,13 @@ cp4_status cp4_conv2d_forward_ex(const cp4_shape* shape, const cp4_geometry* g, 
                                  const float* FW, const float* bias, int activation, float* y,
                                  cp4_stream stream);
 /* The two gradients of that map: dx[N,C,H,W] (the exact adjoint, whatever the
- * padding) from dy[N,T,out_h,out_w], and the four factor gradients.  Both first
- * spread dy out with zeros to stride 1 in `workspace` (device memory of at least
- * cp4_conv2d_backward_ex_workspace_bytes, which also covers the factor pass's own
- * planes) and then run the stride-1 kernels, so their cost is that of the
- * stride-1 layer. */
+ * padding) from dy[N,T,out_h,out_w], and the four factor gradients.  With a
+ * stride both read dy as it is where the matrix-core kernels take the shape: the
+ * strided build's adjoint mode for dx, and for the factors a pass whose planes
+ * live on two grids (A, G1 on the input's, G3, Cc on the output's).  Otherwise dy
+ * is first spread out with zeros to stride 1 and the stride-1 kernels run.
+ * `workspace`: device memory of at least cp4_conv2d_backward_ex_workspace_bytes
+ * (sized for either route), 256-byte aligned. */
 size_t cp4_conv2d_backward_ex_workspace_bytes(const cp4_shape* shape, const cp4_geometry* g);
 cp4_status cp4_conv2d_backward_data_ex(const cp4_shape* shape, const cp4_geometry* g,
                                        const float* dy, const float* FK, const float* FC,

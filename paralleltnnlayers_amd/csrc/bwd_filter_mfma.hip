@@ -1357,4 +1357,412 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
   return hipGetLastError();
 }
 
+#ifndef CP4_BWF_IO16
+// ---- The same pass for a layer with a stride (and any zeros before the image) ----
+// y[ho, wo] reads x at (sh*ho + i - pt, sw*wo + j - pl), so the planes come in two
+// sizes: A = FC^T x and G1 (the adjoint taps of G3) on the input's H x W grid,
+// G3 = FK^T dy and Cc (the taps of A at the kept positions) on the output's
+// Ho x Wo grid.  The contraction and gradient-GEMM kernels above run once per
+// operand, each on its own plane size; only the tap step is new:
+//   Cc[ho,wo]  = sum_{i,j} FH[i] FW[j] A[sh*ho + i - pt, sw*wo + j - pl]
+//   G1[h,w]    = sum_{i,j} FH[i] FW[j] G3[(h + pt - i) / sh, (w + pl - j) / sw]   (exact divisions only)
+//   dFH[i]    += sum_{ho,wo} G3[ho,wo] sum_j FW[j] A[sh*ho + i - pt, sw*wo + j - pl]
+//   dFW[j]    += sum_{ho,wo} G3[ho,wo] sum_i FH[i] A[sh*ho + i - pt, sw*wo + j - pl]
+// (the reference's layers take strides, test/layers.py:264-279; its kernels do not).
+namespace {
+
+// One workgroup per (image, rank): both planes in LDS, tap-gradient partials
+// partH[n][i][r], partW[n][j][r] summed in a fixed order.
+__global__ __launch_bounds__(256) void taps_strided_plane_kernel(
+    const float* __restrict__ A, const float* __restrict__ G3, const float* __restrict__ FH,
+    const float* __restrict__ FW, float* __restrict__ Cc, float* __restrict__ G1,
+    float* __restrict__ partH, float* __restrict__ partW, int R, int H, int W, int Ho, int Wo,
+    int Y, int X, int sh, int sw, int pt, int pl_) {
+  extern __shared__ float pl[];
+  const int HW = H * W, HWo = Ho * Wo;
+  float *sA = pl, *sG = pl + HW;
+  float* red = sG + HWo;                          // [Y + X][4] wave partials
+  float* fh = red + 4 * (Y + X);                  // this rank's tap weights, read once
+  float* fw = fh + Y;
+  const int plane = blockIdx.x, r = plane % R, n = plane / R;
+  const size_t basef = (size_t)plane * HW, bases = (size_t)plane * HWo;
+  for (int p = threadIdx.x; p < HW; p += 256) sA[p] = A[basef + p];
+  for (int q = threadIdx.x; q < HWo; q += 256) sG[q] = G3[bases + q];
+  if ((int)threadIdx.x < Y) fh[threadIdx.x] = FH[threadIdx.x * R + r];
+  else if ((int)threadIdx.x < Y + X) fw[threadIdx.x - Y] = FW[(threadIdx.x - Y) * R + r];
+  __syncthreads();
+  // Cc on the output grid
+  for (int q = threadIdx.x; q < HWo; q += 256) {
+    const int ho = q / Wo, wo = q - ho * Wo;
+    float cc = 0.f;
+    for (int i = 0; i < Y; ++i) {
+      const int hh = sh * ho + i - pt;
+      if (hh < 0 || hh >= H) continue;
+      float row = 0.f;
+      for (int j = 0; j < X; ++j) {
+        const int ww = sw * wo + j - pl_;
+        if (ww >= 0 && ww < W) row += fw[j] * sA[hh * W + ww];
+      }
+      cc += fh[i] * row;
+    }
+    Cc[bases + q] = cc;
+  }
+  // G1 on the input grid: the adjoint taps of G3
+  for (int p = threadIdx.x; p < HW; p += 256) {
+    const int h = p / W, w = p - h * W;
+    float g1 = 0.f;
+    for (int i = 0; i < Y; ++i) {
+      const int num = h + pt - i;
+      if (num < 0) break;
+      const int ho = num / sh;
+      if (ho * sh != num || ho >= Ho) continue;
+      float row = 0.f;
+      for (int j = 0; j < X; ++j) {
+        const int numw = w + pl_ - j;
+        if (numw < 0) break;
+        const int wo = numw / sw;
+        if (wo * sw == numw && wo < Wo) row += fw[j] * sG[ho * Wo + wo];
+      }
+      g1 += fh[i] * row;
+    }
+    G1[basef + p] = g1;
+  }
+  // tap gradients of this plane: wave sums to LDS, one barrier, then a fixed-order
+  // sum of the four wave partials per tap
+  for (int t = 0; t < Y + X; ++t) {
+    const bool vertical = t < Y;
+    float acc = 0.f;
+    for (int q = threadIdx.x; q < HWo; q += 256) {
+      const int ho = q / Wo, wo = q - ho * Wo;
+      float inner = 0.f;
+      if (vertical) {
+        const int hh = sh * ho + t - pt;
+        if (hh >= 0 && hh < H)
+          for (int j = 0; j < X; ++j) {
+            const int ww = sw * wo + j - pl_;
+            if (ww >= 0 && ww < W) inner += fw[j] * sA[hh * W + ww];
+          }
+      } else {
+        const int ww = sw * wo + (t - Y) - pl_;
+        if (ww >= 0 && ww < W)
+          for (int i = 0; i < Y; ++i) {
+            const int hh = sh * ho + i - pt;
+            if (hh >= 0 && hh < H) inner += fh[i] * sA[hh * W + ww];
+          }
+      }
+      acc += sG[q] * inner;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off, 64);
+    if ((threadIdx.x & 63) == 0) red[t * 4 + (threadIdx.x >> 6)] = acc;
+  }
+  __syncthreads();
+  if ((int)threadIdx.x < Y + X) {
+    const int t = threadIdx.x;
+    const float tot = red[t * 4] + red[t * 4 + 1] + red[t * 4 + 2] + red[t * 4 + 3];
+    if (t < Y) partH[((size_t)n * Y + t) * R + r] = tot;
+    else partW[((size_t)n * X + (t - Y)) * R + r] = tot;
+  }
+}
+
+// The same for square filters of a compile-time size: the tap-gradient terms are
+// accumulated in registers while Cc is formed (one pass over the plane instead of
+// one per tap), and the adjoint taps are walked per block of sh x sw input pixels.
+template <int FS>
+__global__ __launch_bounds__(256) void taps_strided_fast_kernel(
+    const float* __restrict__ A, const float* __restrict__ G3, const float* __restrict__ FH,
+    const float* __restrict__ FW, float* __restrict__ Cc, float* __restrict__ G1,
+    float* __restrict__ partH, float* __restrict__ partW, int R, int H, int W, int Ho, int Wo,
+    int sh, int sw, int pt, int pl_) {
+  constexpr int Y = FS, X = FS;
+  extern __shared__ float pl[];
+  const int HW = H * W, HWo = Ho * Wo;
+  float *sA = pl, *sG = pl + HW;
+  float* red = sG + HWo;                          // [Y + X][4] wave partials
+  float* fh = red + 4 * (Y + X);                  // this rank's tap weights, read once
+  float* fw = fh + Y;
+  const int plane = blockIdx.x, r = plane % R, n = plane / R;
+  const size_t basef = (size_t)plane * HW, bases = (size_t)plane * HWo;
+  // planes into LDS, four pixels per load where the plane sizes allow (all of a
+  // thread's loads are then in flight together)
+  auto stage = [&](float* dst, const float* src, int n) {
+    if ((n & 3) == 0 && ((reinterpret_cast<uintptr_t>(src) | (uintptr_t)(dst - pl) * 4) & 15) == 0) {
+      const float4* s4 = reinterpret_cast<const float4*>(src);
+      float4* d4 = reinterpret_cast<float4*>(dst);
+#pragma unroll 4
+      for (int k = threadIdx.x; k < (n >> 2); k += 256) d4[k] = s4[k];
+    } else {
+      for (int k = threadIdx.x; k < n; k += 256) dst[k] = src[k];
+    }
+  };
+  stage(sA, A + basef, HW);
+  stage(sG, G3 + bases, HWo);
+  if ((int)threadIdx.x < Y) fh[threadIdx.x] = FH[threadIdx.x * R + r];
+  else if ((int)threadIdx.x < Y + X) fw[threadIdx.x - Y] = FW[(threadIdx.x - Y) * R + r];
+  __syncthreads();
+  // Cc on the output grid, and this thread's share of the tap gradients.  Reads
+  // outside the image go to a clamped cell and count zero: no branches, so the FS*FS
+  // LDS reads of a pixel are all in flight together.
+  float gh[FS], gw[FS];
+#pragma unroll
+  for (int t = 0; t < FS; ++t) gh[t] = gw[t] = 0.f;
+  for (int q = threadIdx.x; q < HWo; q += 256) {
+    const int ho = q / Wo, wo = q - ho * Wo;
+    const float gv = sG[q];
+    int ro[FS], co[FS];
+    bool rin[FS], cin[FS];
+#pragma unroll
+    for (int i = 0; i < FS; ++i) {
+      const int hh = sh * ho + i - pt, ww = sw * wo + i - pl_;
+      rin[i] = hh >= 0 && hh < H;
+      cin[i] = ww >= 0 && ww < W;
+      ro[i] = rin[i] ? hh * W : 0;
+      co[i] = cin[i] ? ww : 0;
+    }
+    float av[FS][FS];
+#pragma unroll
+    for (int i = 0; i < FS; ++i)
+#pragma unroll
+      for (int j = 0; j < FS; ++j) av[i][j] = sA[ro[i] + co[j]];
+    float cc = 0.f, col[FS];
+#pragma unroll
+    for (int j = 0; j < FS; ++j) col[j] = 0.f;
+#pragma unroll
+    for (int i = 0; i < FS; ++i) {
+      float row = 0.f;
+#pragma unroll
+      for (int j = 0; j < FS; ++j) {
+        const float v = (rin[i] && cin[j]) ? av[i][j] : 0.f;
+        row += fw[j] * v;
+        col[j] += fh[i] * v;
+      }
+      cc += fh[i] * row;
+      gh[i] += gv * row;
+    }
+#pragma unroll
+    for (int j = 0; j < FS; ++j) gw[j] += gv * col[j];
+    Cc[bases + q] = cc;
+  }
+  // G1 on the input grid: the adjoint taps of G3.  A thread takes a block of sh x sw
+  // input pixels (bh, bw): tap row i lands on the block's row ai[i] = (i - pt) mod sh
+  // and reads output row bh + dh[i] (both the same for every block), likewise for the
+  // columns - so a block costs FS*FS reads in all, whichever of its pixels they go to.
+  int ai[FS], dh[FS], bj[FS], dw[FS];
+#pragma unroll
+  for (int i = 0; i < FS; ++i) {
+    ai[i] = ((i - pt) % sh + sh) % sh;
+    dh[i] = (ai[i] + pt - i) / sh;               // exact
+    bj[i] = ((i - pl_) % sw + sw) % sw;
+    dw[i] = (bj[i] + pl_ - i) / sw;
+  }
+  const int nbw = (W + sw - 1) / sw, nbh = (H + sh - 1) / sh;
+  for (int blk = threadIdx.x; blk < nbh * nbw; blk += 256) {
+    const int bh = blk / nbw, bw = blk - bh * nbw;
+    for (int a = 0; a < sh; ++a) {
+      const int h = sh * bh + a;
+      if (h >= H) break;
+      for (int b = 0; b < sw; ++b) {
+        const int w = sw * bw + b;
+        if (w >= W) break;
+        float g1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < FS; ++i) {
+          if (ai[i] != a) continue;               // (the same for all threads)
+          const int ho = bh + dh[i];
+          const bool rok = ho >= 0 && ho < Ho;
+          float row = 0.f;
+#pragma unroll
+          for (int j = 0; j < FS; ++j) {
+            if (bj[j] != b) continue;
+            const int wo = bw + dw[j];
+            const bool ok = rok && wo >= 0 && wo < Wo;
+            const float v = sG[ok ? ho * Wo + wo : 0];
+            row += fw[j] * (ok ? v : 0.f);
+          }
+          g1 += fh[i] * row;
+        }
+        G1[basef + (size_t)h * W + w] = g1;
+      }
+    }
+  }
+  // wave sums of the tap gradients to LDS, one barrier, fixed-order sum of the four
+#pragma unroll
+  for (int t = 0; t < FS; ++t) {
+    float a = gh[t], b = gw[t];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      a += __shfl_down(a, off, 64);
+      b += __shfl_down(b, off, 64);
+    }
+    if ((threadIdx.x & 63) == 0) {
+      red[t * 4 + (threadIdx.x >> 6)] = a;
+      red[(Y + t) * 4 + (threadIdx.x >> 6)] = b;
+    }
+  }
+  __syncthreads();
+  if ((int)threadIdx.x < Y + X) {
+    const int t = threadIdx.x;
+    const float tot = red[t * 4] + red[t * 4 + 1] + red[t * 4 + 2] + red[t * 4 + 3];
+    if (t < Y) partH[((size_t)n * Y + t) * R + r] = tot;
+    else partW[((size_t)n * X + (t - Y)) * R + r] = tot;
+  }
+}
+
+size_t strided_taps_lds(int H, int W, int Ho, int Wo, int Y, int X) {
+  return ((size_t)H * W + (size_t)Ho * Wo + 5 * (size_t)(Y + X)) * sizeof(float);
+}
+
+// One channel -> rank contraction Z[n,r,p] = sum_c F[c,r] src[n,c,p] on planes of HW pixels.
+hipError_t contract_one(const float* src, const float* F, float* Z, int Cin, int N, int R, int RP,
+                        int HW, hipStream_t st) {
+  ContractArgs c{};
+  c.src[0] = src; c.F[0] = F; c.Z[0] = Z; c.Cin[0] = Cin;
+  c.N = N; c.R = R; c.RP = RP; c.HW = HW;
+  hipError_t e;
+  if ((Cin & 15) == 0 && (size_t)Cin * 192 <= 160 * 1024) {
+    c.npb = (HW + 31) / 32;
+    c.items = N * c.npb;
+    c.ks = 1;
+    while (c.ks < 4 && (long)c.items * (RP / 32) * c.ks < kKsWaves / 2 &&
+           ((Cin >> 4) % (2 * c.ks)) == 0 && (Cin >> 4) / (2 * c.ks) >= 2)
+      c.ks *= 2;
+    size_t smem = (size_t)Cin * 192;
+    if (c.ks > 1 && smem < (size_t)kSW * 16 * sizeof(float)) smem = (size_t)kSW * 16 * sizeof(float);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_split_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    const long slots = (long)c.items * c.ks;
+    contract_split_kernel<<<dim3((unsigned)((slots + kSW / 64 - 1) / (kSW / 64)), 1, RP / 32), kSW,
+                            smem, st>>>(c);
+  } else {
+    c.npb = (HW + 63) / 64;
+    c.items = N * c.npb;
+    const size_t smem = (size_t)Cin * 32 * sizeof(float);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_mfma_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    contract_mfma_kernel<<<dim3((c.items + kCW / 64 - 1) / (kCW / 64), 1, RP / 32), kCW, smem,
+                           st>>>(c);
+  }
+  return hipGetLastError();
+}
+
+// One gradient GEMM part[s][d][r] = sum_{p in split s} act[n,d,p] Z[n,r,p] on planes of HW pixels.
+hipError_t grad_one(const float* act, const float* Z, float* part, int D, int N, int R,
+                    const Plan& p, int HW, const void* ws, hipStream_t st) {
+  GradArgs g{};
+  g.act[0] = act; g.Z[0] = Z; g.part[0] = part; g.D[0] = D;
+  g.N = N; g.R = R; g.RP = p.RP; g.HW = HW; g.PS = p.PS; g.cps = p.cps;
+  const dim3 ggrid(p.S, (D + 127) / 128, 1);
+  const bool vec = (HW & 3) == 0 && (reinterpret_cast<uintptr_t>(ws) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(act) & 15) == 0;
+  if (vec) {
+    if (p.RP == 32) grad_split_kernel<1, true><<<ggrid, kCT, 0, st>>>(g);
+    else grad_split_kernel<2, true><<<ggrid, kCT, 0, st>>>(g);
+  } else if (HW & 1) {
+    if (p.RP == 32) grad_split_kernel<1, false><<<ggrid, kCT, 0, st>>>(g);
+    else grad_split_kernel<2, false><<<ggrid, kCT, 0, st>>>(g);
+  } else {
+    if (p.RP == 32) grad_gemm_kernel<1><<<ggrid, kCT, 0, st>>>(g);
+    else grad_gemm_kernel<2><<<ggrid, kCT, 0, st>>>(g);
+  }
+  return hipGetLastError();
+}
+
+struct StridedLayout {
+  Plan pf, ps;                                    // plans on the input's and on the output's grid
+  size_t A, G1, G3, Cc, pK, pC, pH, pW, total;    // float offsets into the workspace
+};
+StridedLayout strided_layout(const cp4_shape& s, const Geometry& g) {
+  StridedLayout l;
+  l.pf = make_plan(s.N, s.C, s.T, s.H, s.W, s.Y, s.X, s.Rank, 0);
+  l.ps = make_plan(s.N, s.C, s.T, g.Ho, g.Wo, s.Y, s.X, s.Rank, 0);
+  const size_t planef = (size_t)s.N * s.Rank * s.H * s.W, planes = (size_t)s.N * s.Rank * g.Ho * g.Wo;
+  auto al = [](size_t v) { return (v + 63) & ~(size_t)63; };   // 256-byte steps
+  size_t o = 0;
+  l.A = o; o += al(planef);
+  l.G1 = o; o += al(planef);
+  l.G3 = o; o += al(planes);
+  l.Cc = o; o += al(planes);
+  l.pK = o; o += al((size_t)l.ps.S * s.T * s.Rank);
+  l.pC = o; o += al((size_t)l.pf.S * s.C * s.Rank);
+  l.pH = o; o += al((size_t)s.N * s.Y * s.Rank);
+  l.pW = o; o += al((size_t)s.N * s.X * s.Rank);
+  l.total = o;
+  return l;
+}
+
+}  // namespace
+
+bool bwd_filter_mfma_strided_supported(const cp4_shape& s, const Geometry& g) {
+  cp4_shape so = s;
+  so.H = g.Ho; so.W = g.Wo;
+  return bwd_filter_mfma_supported(s) && bwd_filter_mfma_supported(so) && s.Y + s.X <= 256 &&
+         strided_taps_lds(s.H, s.W, g.Ho, g.Wo, s.Y, s.X) <= 150 * 1024;
+}
+
+size_t bwd_filter_mfma_strided_workspace_bytes(const cp4_shape& s, const Geometry& g) {
+  return strided_layout(s, g).total * sizeof(float);
+}
+
+hipError_t bwd_filter_mfma_strided_launch(const BwdFilterArgs& a, const Geometry& g,
+                                          hipStream_t st) {
+  cp4_shape s{};
+  s.N = a.N; s.C = a.C; s.T = a.T; s.H = a.H; s.W = a.W; s.pad = 0; s.Y = a.Y; s.X = a.X;
+  s.Rank = a.R;
+  const StridedLayout l = strided_layout(s, g);
+  float* ws = static_cast<float*>(a.workspace);
+  float *A = ws + l.A, *G1 = ws + l.G1, *G3 = ws + l.G3, *Cc = ws + l.Cc, *pK = ws + l.pK,
+        *pC = ws + l.pC, *pH = ws + l.pH, *pW = ws + l.pW;
+  const int N = a.N, R = a.R, HW = a.H * a.W, HWo = g.Ho * g.Wo;
+  hipError_t e = contract_one(a.x, a.FC, A, a.C, N, R, l.pf.RP, HW, st);
+  if (e != hipSuccess) return e;
+  e = contract_one(a.dy, a.FK, G3, a.T, N, R, l.ps.RP, HWo, st);
+  if (e != hipSuccess) return e;
+  const size_t tsm = strided_taps_lds(a.H, a.W, g.Ho, g.Wo, a.Y, a.X);
+  const bool fast = a.Y == a.X && (a.Y == 1 || a.Y == 3 || a.Y == 5 || a.Y == 7);
+#define CP4_STRIDED_TAPS(FS_)                                                                    \
+  {                                                                                              \
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(taps_strided_fast_kernel<FS_>),        \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)tsm);               \
+    if (e != hipSuccess) return e;                                                               \
+    taps_strided_fast_kernel<FS_><<<N * R, 256, tsm, st>>>(A, G3, a.FH, a.FW, Cc, G1, pH, pW, R, \
+                                                           a.H, a.W, g.Ho, g.Wo, g.sh, g.sw,     \
+                                                           g.pt, g.pl);                          \
+  }
+  if (fast) {
+    switch (a.Y) {
+      case 1: CP4_STRIDED_TAPS(1) break;
+      case 3: CP4_STRIDED_TAPS(3) break;
+      case 5: CP4_STRIDED_TAPS(5) break;
+      default: CP4_STRIDED_TAPS(7) break;
+    }
+  } else {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(taps_strided_plane_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)tsm);
+    if (e != hipSuccess) return e;
+    taps_strided_plane_kernel<<<N * R, 256, tsm, st>>>(A, G3, a.FH, a.FW, Cc, G1, pH, pW, R, a.H,
+                                                       a.W, g.Ho, g.Wo, a.Y, a.X, g.sh, g.sw, g.pt,
+                                                       g.pl);
+  }
+#undef CP4_STRIDED_TAPS
+  e = grad_one(a.dy, Cc, pK, a.T, N, R, l.ps, HWo, ws, st);
+  if (e != hipSuccess) return e;
+  e = grad_one(a.x, G1, pC, a.C, N, R, l.pf, HW, ws, st);
+  if (e != hipSuccess) return e;
+  ReduceArgs r{};
+  const float* parts[4] = {pK, pC, pH, pW};
+  float* outs[4] = {a.dFK, a.dFC, a.dFH, a.dFW};
+  const int counts[4] = {a.T * R, a.C * R, a.Y * R, a.X * R};
+  const int Ss[4] = {l.ps.S, l.pf.S, N, N};
+  int maxc = 0;
+  for (int i = 0; i < 4; ++i) {
+    r.part[i] = parts[i]; r.out[i] = outs[i]; r.count[i] = counts[i]; r.S[i] = Ss[i];
+    if (counts[i] > maxc) maxc = counts[i];
+  }
+  reduce4_kernel<<<dim3((maxc + 63) / 64, 4), 256, 0, st>>>(r);
+  return hipGetLastError();
+}
+#endif  // !CP4_BWF_IO16
+
 }  // namespace cp4

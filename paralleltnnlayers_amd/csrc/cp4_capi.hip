@@ -926,8 +926,15 @@ size_t cp4_conv2d_backward_ex_workspace_bytes(const cp4_shape* shape, const cp4_
   const size_t plane = (size_t)c.Hc * c.Wc * sizeof(float);
   // backward-filter: canvas x (unless in place), canvas dy, the stride-1 pass's workspace;
   // backward-data needs only dy spread out, which is no larger than canvas dy
-  return align256(c.x_in_place ? 0 : (size_t)shape->N * shape->C * plane) +
-         align256((size_t)shape->N * shape->T * plane) + filter_workspace(sc);
+  const size_t canvas = align256(c.x_in_place ? 0 : (size_t)shape->N * shape->C * plane) +
+                        align256((size_t)shape->N * shape->T * plane) + filter_workspace(sc);
+  // (the strided matrix-core pass needs far less; the maximum keeps either route open)
+  const cp4::Geometry gg{(int)g->stride_h, (int)g->stride_w, (int)g->pad_top, (int)g->pad_left,
+                         (int)g->out_h, (int)g->out_w};
+  const size_t strided = cp4::bwd_filter_mfma_strided_supported(*shape, gg)
+                             ? cp4::bwd_filter_mfma_strided_workspace_bytes(*shape, gg)
+                             : 0;
+  return canvas > strided ? canvas : strided;
 }
 
 cp4_status cp4_conv2d_backward_data_ex(const cp4_shape* shape, const cp4_geometry* g,
@@ -1004,9 +1011,27 @@ cp4_status cp4_conv2d_backward_filter_ex(const cp4_shape* shape, const cp4_geome
     return fail(CP4_ERR_WORKSPACE, "workspace smaller than cp4_conv2d_backward_ex_workspace_bytes");
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0)
     return fail(CP4_ERR_WORKSPACE, "workspace must be 256-byte aligned");
-  // The stride-1 layer on the canvas computes y1[sh*ho, sw*wo] = y[ho, wo]; with dy
-  // spread out with zeros the loss and so the factor gradients are the same.
   hipStream_t st = as_stream(stream);
+  if (g->stride_h > 1 || g->stride_w > 1) {
+    // With a stride: the matrix-core pass on planes of two sizes (A, G1 on the input's
+    // grid, G3, Cc on the output's), dy read as it is.
+    const cp4::Geometry gg{(int)g->stride_h, (int)g->stride_w, (int)g->pad_top, (int)g->pad_left,
+                           (int)g->out_h, (int)g->out_w};
+    if (cp4::bwd_filter_mfma_strided_supported(s, gg)) {
+      if (!FK || !FC || !FH || !FW || !dFK || !dFC || !dFH || !dFW)
+        return fail(CP4_ERR_NULL_POINTER, "a factor or gradient pointer is NULL");
+      cp4::BwdFilterArgs b{};
+      b.x = x; b.dy = dy; b.FK = FK; b.FC = FC; b.FH = FH; b.FW = FW;
+      b.dFK = dFK; b.dFC = dFC; b.dFH = dFH; b.dFW = dFW;
+      b.workspace = workspace;
+      b.N = (int)s.N; b.C = (int)s.C; b.T = (int)s.T; b.H = (int)s.H; b.W = (int)s.W; b.pad = 0;
+      b.Y = (int)s.Y; b.X = (int)s.X; b.R = (int)s.Rank;
+      CP4_HIP(cp4::bwd_filter_mfma_strided_launch(b, gg, st));
+      return CP4_OK;
+    }
+  }
+  // Otherwise the stride-1 layer on a canvas: it computes y1[sh*ho, sw*wo] = y[ho, wo]; with
+  // dy spread out with zeros the loss and so the factor gradients are the same.
   unsigned char* w = static_cast<unsigned char*>(workspace);
   const size_t plane = (size_t)c.Hc * c.Wc * sizeof(float);
   const float* xc = x;

@@ -138,6 +138,11 @@ bool bwd_filter_mfma_supported(const cp4_shape&);
 size_t bwd_filter_mfma_workspace_bytes(const cp4_shape&);
 bool bwd_filter_mfma_taps2d_supported(const cp4_shape&);   // with BwdFilterArgs::taps2d
 hipError_t bwd_filter_mfma_launch(const BwdFilterArgs&, hipStream_t);
+// A layer with a stride and zeros of its own before the image (BwdFilterArgs::H, W: the
+// input plane; pad unused; dy on the geometry's Ho x Wo grid).
+bool bwd_filter_mfma_strided_supported(const cp4_shape&, const Geometry&);
+size_t bwd_filter_mfma_strided_workspace_bytes(const cp4_shape&, const Geometry&);
+hipError_t bwd_filter_mfma_strided_launch(const BwdFilterArgs&, const Geometry&, hipStream_t);
 // The same with bfloat16 x and dy in memory (BwdFilterArgs::x / dy point at 16-bit
 // elements); split-bf16 kernels only: C and T multiples of 16.
 bool bwd_filter_mfma_io16_supported(const cp4_shape&);

@@ -104,7 +104,7 @@ constexpr int kProd = 8, kCons = 8;          // producer / consumer waves (4 per
 constexpr int kRP = 32;
 constexpr int kCcBuf = 24 * 512;             // bytes of one Cc fragment tile (64 pixels)
 constexpr size_t kLdsLimit = 160 * 1024;
-constexpr int kOwnGroupsMaxRank = 4;         // ranks up to which consumer waves take whole groups by default
+[[maybe_unused]] constexpr int kOwnGroupsMaxRank = 4;         // ranks up to which consumer waves take whole groups by default
 #ifndef CP4_WHOLE_BLOCK_MIN
 #define CP4_WHOLE_BLOCK_MIN 16
 #endif
@@ -114,7 +114,7 @@ constexpr int kOwnGroupsMaxRank = 4;         // ranks up to which consumer waves
 constexpr double kTileStartCost = 50000.0;
 // C3 (56-pixel rows): 7-row strips, 256 workgroups, 39.6 us on one buffer set and
 // 61.6 us on rotating sets; 8-row strips, 224 workgroups, 38.1 and 56.0 us.
-constexpr double kUnalignedStripCost = 1.12;
+[[maybe_unused]] constexpr double kUnalignedStripCost = 1.12;
 constexpr int kWholeBlockMin = CP4_WHOLE_BLOCK_MIN;   // blocks per plane from which 17-64 channels go unsplit
 constexpr int kSpinLimit = 1 << 19;      // default bound of a wait: about a quarter of a second at the longest nap
 constexpr int kMaxBlk = 64;                  // per-block progress words in LDS
