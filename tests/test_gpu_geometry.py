@@ -127,6 +127,36 @@ def test_geometry_matrix_core_shapes(cp4, oracle, dims):
     cp4.device_status()
 
 
+@pytest.mark.parametrize("dims", [(2, 32, 22, 26, 48, 3, 5, 12, (2, 3), (1, 2)),
+                                  (1, 16, 30, 30, 32, 9, 9, 8, (2, 2), (4, 4)),
+                                  (2, 48, 17, 19, 16, 2, 4, 40, (3, 2), (0, 1))],
+                         ids=lambda d: "x".join(map(str, d)))
+def test_strided_factor_gradients_other_filters(cp4, dims):
+    """Rectangular, even and 9x9 filters with a stride: the factor gradients run the
+    strided matrix-core pass with its general tap kernel; forward and input gradient
+    the general kernels.  Against float64 autograd of the dense strided convolution."""
+    N, C, H, W, T, Y, X, R, (sh, sw), (pt, pl) = dims
+    gen = torch.Generator(device="cuda").manual_seed(sum(map(ord, str(dims))))
+    x = torch.rand((N, C, H, W), device="cuda", generator=gen) * 2 - 1
+    fac = [torch.randn((d, R), device="cuda", generator=gen) * (R * C * Y * X) ** -0.25
+           for d in (T, C, Y, X)]
+    oh, ow = (H + 2 * pt - Y) // sh + 1, (W + 2 * pl - X) // sw + 1
+    geom = cp4.Geometry(sh, sw, pt, pl, oh, ow)
+    y = cp4.conv2d_forward_ex(x, *fac, geom)
+    dy = torch.randn(y.shape, device="cuda", generator=gen)
+    yd, dxd, gd = dense_reference(x, dy, fac, geom)
+    close_activation(y.cpu().numpy(), yd.astype(np.float32), "forward")
+    dx = cp4.conv2d_backward_data_ex(dy, (H, W), *fac, geom)
+    close_activation(dx.cpu().numpy(), dxd.astype(np.float32), "backward-data")
+    grads = cp4.conv2d_backward_filter_ex(x, dy, *fac, geom)
+    for got, wnt, k in zip(grads, gd, FACTORS):
+        close_gradient(got.cpu().numpy(), wnt.astype(np.float32), "d" + k)
+    again = cp4.conv2d_backward_filter_ex(x, dy, *fac, geom)
+    for a, b in zip(grads, again):
+        assert torch.equal(a, b)                    # fixed summation order
+    cp4.device_status()
+
+
 def test_stride_two_at_the_headline_shape(cp4, oracle):
     """C3's shape at stride 2: against the oracle, and against every second row and
     column of the stride-1 layer for the padding that makes the two coincide."""
