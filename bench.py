@@ -2,7 +2,7 @@
 """Benchmark of the fused CP4 Conv2d hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--no-cpu]
-                    [--settle-ms MS]
+                    [--settle-ms MS] [--shape PASS,N,C,H,W,pad,T,Y,R [--stride S]]
 
 A step is one launch of the workload's pass (default: the forward pass of the
 ResNet-stage workload N=32, C=K=256, 56x56, 3x3, R=32) on synthetic inputs that
@@ -57,6 +57,10 @@ def main():
     ap.add_argument("--shape", default=None, metavar="PASS,N,C,H,W,pad,T,Y,R",
                     help="time an ad-hoc shape instead of a named workload, e.g. "
                          "forward,8,64,224,224,1,64,3,16 (uniform inputs; no CPU leg, no table)")
+    ap.add_argument("--stride", type=int, default=0,
+                    help="with --shape: the same layer with this stride and the framework's "
+                         "\"same\" padding (out = ceil(in / stride)); times all three passes "
+                         "of the strided entry points and prints their figures")
     ap.add_argument("--settle-ms", type=float, default=150.0,
                     help="untimed back-to-back launches of the headline workload for this "
                          "long before the warm-up, so clocks are at their steady state")
@@ -122,6 +126,46 @@ def main():
         N, C, H, W_, pad, T, Y, R = (int(v) for v in f[1:])
         w = Workload("adhoc", f[0], N, C, H, W_, pad, T, Y, Y, R, "uniform")
         args.no_cpu = args.no_passes = True
+    if args.stride:
+        assert args.shape, "--stride goes with --shape"
+        gen = torch.Generator(device="cuda").manual_seed(0)
+        x = torch.rand((w.N, w.C, w.H, w.W), device="cuda", generator=gen)
+        f = [torch.randn((d, w.R), device="cuda", generator=gen) * (w.R * w.C) ** -0.5
+             for d in (w.T, w.C, w.Y, w.X)]
+        s = cp4.capi.shape_for(x.shape, *f, 0)
+        g = cp4.geometry(s, args.stride, "same")
+        y = torch.empty((w.N, w.T, g.out_h, g.out_w), device="cuda")
+        dy = torch.randn(y.shape, device="cuda", generator=gen)
+        dx = torch.empty_like(x)
+        ws = torch.empty(cp4.backward_ex_workspace_bytes(s, g) + 512, device="cuda",
+                         dtype=torch.uint8)
+        ws = ws[(-ws.data_ptr()) % 256:]
+        legs = {"forward": lambda: cp4.conv2d_forward_ex(x, *f, g, out=y),
+                "backward_data": lambda: cp4.conv2d_backward_data_ex(dy, (w.H, w.W), *f, g, out=dx,
+                                                                     workspace=ws),
+                "backward_filter": lambda: cp4.conv2d_backward_filter_ex(x, dy, *f, g, workspace=ws)}
+        nb = 4 * (x.numel() + y.numel())
+        res = {}
+        for name, fn in legs.items():
+            t0 = time.perf_counter()
+            while (time.perf_counter() - t0) * 1e3 < args.settle_ms:
+                fn()
+            for _ in range(args.warmup):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(args.steps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / args.steps
+            res[name] = {"us": round(us, 2), "GB/s": round(nb / us / 1e3, 1),
+                         "hbm_frac": round(nb / us / 1e3 / HBM_PEAK_GBS, 4)}
+        cp4.device_status()
+        print(json.dumps({"workload": "%s stride %d, out %dx%d" % (args.shape, args.stride, g.out_h,
+                                                                  g.out_w),
+                          "algorithmic_bytes": nb, "passes": res}))
+        return
     if args.calibrate_copy:
         n = w.N * w.C * w.H * w.W
         src = torch.randn(n, device="cuda")
