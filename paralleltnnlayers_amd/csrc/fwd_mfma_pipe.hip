@@ -183,7 +183,7 @@ __device__ __forceinline__ int wait_ge(int* word, int want, bool backoff, const 
 // NQ: channel splits of the producers (4: quarters, two blocks per round; 1: up to
 // 16 input channels, every producer wave takes a whole block of its own, eight
 // blocks per round and no partial sums to chain).
-template <int FS, int CPQ, int KR, bool PAD, int NQ = 4>
+template <int FS, int CPQ, int KR, int NQ = 4>
 __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan pl) {
   extern __shared__ float lds[];
   float* As = lds;                                                  // [32][QA] fp32
@@ -310,7 +310,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     const int bsel = wave % NB, cq = wave / NB;    // block within the round, channel split
     const int nrounds = (nblk + NB - 1) / NB;
     // lane's channel 16*(cpq*cq + chunk) + 8*hi + e
-    // (PAD: Cin is not a multiple of 64; channel groups past Cin count as zero)
+    // (channel groups past Cin count as zero: their factor rows are, and x reads there return 0)
     const int cg0 = 16 * cpq * cq + 8 * hi;        // lane's first channel of chunk 0
     // x is read through a buffer descriptor over this image: the address is
     // (descriptor base) + (32-bit lane offset) + (scalar offset), so the walk
@@ -326,15 +326,29 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     constexpr int NF = FLDS ? 1 : CPQ;
     u32x4 fh[NF], fm[NF], fl[NF];
     if (!FLDS) {
+      // (two copies of the loop on purpose: with whole chunks of channels the loads of
+      // a slice sit under one condition and go out together - the start of every
+      // workgroup waits for them; with a ragged channel count each has its own)
+      if ((Cin & (16 * NQ - 1)) == 0) {
 #pragma unroll
-      for (int c = 0; c < NF; ++c) {
-        float v[8];
+        for (int c = 0; c < NF; ++c) {
+          float v[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          v[e] = (l32 < R && (!PAD || cg0 + 16 * c + e < Cin))
-                     ? a.Fin[(size_t)(cg0 + 16 * c + e) * ldf + l32]
-                     : 0.f;
-        split8(v, fh[c], fm[c], fl[c]);
+          for (int e = 0; e < 8; ++e)
+            v[e] = l32 < R ? a.Fin[(size_t)(cg0 + 16 * c + e) * ldf + l32] : 0.f;
+          split8(v, fh[c], fm[c], fl[c]);
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < NF; ++c) {
+          float v[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            v[e] = (l32 < R && cg0 + 16 * c + e < Cin)
+                       ? a.Fin[(size_t)(cg0 + 16 * c + e) * ldf + l32]
+                       : 0.f;
+          split8(v, fh[c], fm[c], fl[c]);
+        }
       }
     }
     const u32x4* fbase =
@@ -1291,27 +1305,27 @@ bool plan(const FwdArgs& a, PipePlan* best) {
 }
 #endif
 
-template <int FS, int CPQ, int KR, bool PAD, int NQ = 4>
+template <int FS, int CPQ, int KR, int NQ = 4>
 hipError_t launch_as(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
-  const void* fn = reinterpret_cast<const void*>(fwd_pipe_kernel<FS, CPQ, KR, PAD, NQ>);
+  const void* fn = reinterpret_cast<const void*>(fwd_pipe_kernel<FS, CPQ, KR, NQ>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)pl.lds_bytes);
   if (e != hipSuccess) return e;
   const unsigned grid = 8u * ((pl.nWG + 7) / 8);
-  fwd_pipe_kernel<FS, CPQ, KR, PAD, NQ><<<grid, kThreads, pl.lds_bytes, st>>>(a, pl);
+  fwd_pipe_kernel<FS, CPQ, KR, NQ><<<grid, kThreads, pl.lds_bytes, st>>>(a, pl);
   return hipGetLastError();
 }
 
-template <int FS, bool PAD>
+template <int FS>
 hipError_t launch_cpq(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
   const int cpq = (a.Cin + 63) >> 6;             // 16-channel chunks per channel quarter
   switch (cpq) {
-    case 1: return launch_as<FS, 1, 1, PAD>(a, pl, st);
-    case 2: return launch_as<FS, 2, 2, PAD>(a, pl, st);
-    case 3: return launch_as<FS, 3, 1, PAD>(a, pl, st);
-    case 4: return launch_as<FS, 4, 2, PAD>(a, pl, st);
+    case 1: return launch_as<FS, 1, 1>(a, pl, st);
+    case 2: return launch_as<FS, 2, 2>(a, pl, st);
+    case 3: return launch_as<FS, 3, 1>(a, pl, st);
+    case 4: return launch_as<FS, 4, 2>(a, pl, st);
     default:                                      // factor fragments in LDS
-      return (cpq & 1) ? launch_as<FS, 0, 1, PAD>(a, pl, st) : launch_as<FS, 0, 2, PAD>(a, pl, st);
+      return (cpq & 1) ? launch_as<FS, 0, 1>(a, pl, st) : launch_as<FS, 0, 2>(a, pl, st);
   }
 }
 
@@ -1321,25 +1335,19 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
   // contracts a whole block of its own, eight blocks per round, nothing to chain.
   // (With 17-64 channels the four-way split is the faster one: C2 7.3 us against
   // 8.1 us; a wave would run its 2-4 chunks one after the other.)
-  if (a.Cin <= 16)
-    return (a.Cin & 15) ? launch_as<FS, 1, 1, true, 1>(a, pl, st)
-                        : launch_as<FS, 1, 1, false, 1>(a, pl, st);
+  if (a.Cin <= 16) return launch_as<FS, 1, 1, 1>(a, pl, st);
   // On planes of many blocks the waves' arithmetic bounds the sweep, not the
   // latency of one block, and the split's four chained LDS accumulations per block
   // are half of the producers' instructions at 17-64 channels: there, too, every
   // producer wave contracts whole blocks (N32 C32 112x112 R16: 63 -> 47 us).
   if (a.Cin <= 64 && pl.nblk >= kWholeBlockMin) {
-    const bool padc = (a.Cin & 15) != 0;
     switch ((a.Cin + 15) >> 4) {
-      case 2:
-        return padc ? launch_as<FS, 2, 2, true, 1>(a, pl, st) : launch_as<FS, 2, 2, false, 1>(a, pl, st);
-      case 3:
-        return padc ? launch_as<FS, 3, 1, true, 1>(a, pl, st) : launch_as<FS, 3, 1, false, 1>(a, pl, st);
-      default:
-        return padc ? launch_as<FS, 4, 2, true, 1>(a, pl, st) : launch_as<FS, 4, 2, false, 1>(a, pl, st);
+      case 2: return launch_as<FS, 2, 2, 1>(a, pl, st);
+      case 3: return launch_as<FS, 3, 1, 1>(a, pl, st);
+      default: return launch_as<FS, 4, 2, 1>(a, pl, st);
     }
   }
-  return (a.Cin & 63) ? launch_cpq<FS, true>(a, pl, st) : launch_cpq<FS, false>(a, pl, st);
+  return launch_cpq<FS>(a, pl, st);
 }
 
 }  // namespace
