@@ -836,16 +836,19 @@ cp4_status run_geometry(FwdArgs a, hipStream_t st) {
   return CP4_OK;
 }
 // Stride-1 canvas that carries the strided layer (backward-filter): pad P on every
-// side, x set in at (ot, ol), dy spread out with zeros from the origin.
+// side, x set in at (ot, ol), dy spread out with zeros from the origin.  The
+// stride-1 layer reads canvas row h + i - P = x row h + i - P - ot, which must be
+// x row h + i - pad_top: P is the smaller of the two pads and the side with more
+// zeros before the image gets the difference as rows (columns) of zeros in the canvas.
 struct Canvas {
   unsigned P, ot, ol, Hc, Wc;
   bool x_in_place, dy_in_place;
 };
 Canvas canvas_of(const cp4_shape& s, const cp4_geometry& g) {
   Canvas c;
-  c.P = g.pad_top > g.pad_left ? g.pad_top : g.pad_left;
-  c.ot = c.P - g.pad_top;
-  c.ol = c.P - g.pad_left;
+  c.P = g.pad_top < g.pad_left ? g.pad_top : g.pad_left;
+  c.ot = g.pad_top - c.P;
+  c.ol = g.pad_left - c.P;
   const unsigned hu = g.stride_h * (g.out_h - 1) + 1, wu = g.stride_w * (g.out_w - 1) + 1;
   c.Hc = c.ot + s.H > hu ? c.ot + s.H : hu;
   c.Wc = c.ol + s.W > wu ? c.ol + s.W : wu;

@@ -129,12 +129,19 @@ def test_geometry_matrix_core_shapes(cp4, oracle, dims):
 
 @pytest.mark.parametrize("dims", [(2, 32, 22, 26, 48, 3, 5, 12, (2, 3), (1, 2)),
                                   (1, 16, 30, 30, 32, 9, 9, 8, (2, 2), (4, 4)),
-                                  (2, 48, 17, 19, 16, 2, 4, 40, (3, 2), (0, 1))],
+                                  (2, 48, 17, 19, 16, 2, 4, 40, (3, 2), (0, 1)),
+                                  # unequal zeros before the image on the stride-1 canvas route
+                                  # (stride 1; an odd channel count; more than 64 ranks)
+                                  (2, 80, 22, 48, 4, 3, 3, 40, (1, 1), (1, 0)),
+                                  (3, 48, 17, 6, 33, 3, 3, 2, (2, 2), (2, 1)),
+                                  (1, 32, 30, 21, 32, 5, 5, 70, (2, 3), (0, 3))],
                          ids=lambda d: "x".join(map(str, d)))
 def test_strided_factor_gradients_other_filters(cp4, dims):
-    """Rectangular, even and 9x9 filters with a stride: the factor gradients run the
+    """Rectangular, even and 9x9 filters with a stride (the factor gradients run the
     strided matrix-core pass with its general tap kernel; forward and input gradient
-    the general kernels.  Against float64 autograd of the dense strided convolution."""
+    the general kernels), and layers with unequal zeros above and left of the image on
+    the route over a stride-1 canvas.  Against float64 autograd of the dense strided
+    convolution."""
     N, C, H, W, T, Y, X, R, (sh, sw), (pt, pl) = dims
     gen = torch.Generator(device="cuda").manual_seed(sum(map(ord, str(dims))))
     x = torch.rand((N, C, H, W), device="cuda", generator=gen) * 2 - 1
