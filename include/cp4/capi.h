@@ -350,6 +350,13 @@ cp4_status cp4_tuned_choice(const cp4_shape* shape, int backward_data, int* vari
  * CP4_ERR_UNSUPPORTED if the variant does not take the shape with that tile. */
 cp4_status cp4_set_tuned_choice(const cp4_shape* shape, int backward_data, int variant,
                                 int tile_rows, int tile_cols, int schedule);
+/* The table of cp4_tune_forward / cp4_tune_backward_data as a list, in
+ * cp4_tuned_choice's terms: a process can save it and a later one re-enter it
+ * with cp4_set_tuned_choice (variant numbers are those of this build of the
+ * library: keep cp4_forward_variant_name beside them). */
+int cp4_tuned_count(void);
+cp4_status cp4_tuned_entry(int index, cp4_shape* shape, int* backward_data, int* variant,
+                           int* tile_rows, int* tile_cols, int* schedule);
 void cp4_tune_clear(void);
 
 /* ---- device allocator / copy helpers (the reference's Tensor uses

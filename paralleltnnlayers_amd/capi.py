@@ -134,6 +134,8 @@ def lib():
                                                  ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
     L.cp4_tuned_choice.argtypes = [_S, ctypes.c_int] + [ctypes.POINTER(ctypes.c_int)] * 4
     L.cp4_set_tuned_choice.argtypes = [_S] + [ctypes.c_int] * 5
+    L.cp4_tuned_count.restype = ctypes.c_int
+    L.cp4_tuned_entry.argtypes = [ctypes.c_int, _S] + [ctypes.POINTER(ctypes.c_int)] * 5
     L.cp4_tune_clear.restype = None
     L.cp4_device_status.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
     L.cp4_set_spin_limit.argtypes = [ctypes.c_int]
@@ -587,6 +589,50 @@ def set_tuned_choice(s, variant, tile_rows=0, tile_cols=0, schedule=1, backward_
     kernel's rule, 0 = no role split, 2 = whole pixel groups per consumer wave)."""
     check(lib().cp4_set_tuned_choice(ctypes.byref(s), int(backward_data), int(variant),
                                      int(tile_rows), int(tile_cols), int(schedule)))
+
+
+def tuned_table():
+    """The forward / backward-data tuner table as a list of dicts (shape fields, pass,
+    variant name, tile, schedule)."""
+    L = lib()
+    names = {v: n for v, n, _ in forward_variants()}
+    out = []
+    for i in range(L.cp4_tuned_count()):
+        s = Shape()
+        v = [ctypes.c_int() for _ in range(5)]
+        check(L.cp4_tuned_entry(i, ctypes.byref(s), *[ctypes.byref(k) for k in v]))
+        out.append({"N": s.N, "H": s.H, "W": s.W, "pad": s.pad, "T": s.T, "C": s.C, "Y": s.Y,
+                    "X": s.X, "Rank": s.Rank, "backward_data": bool(v[0].value),
+                    "variant": names[v[1].value], "tile_rows": v[2].value,
+                    "tile_cols": v[3].value, "schedule": v[4].value})
+    return out
+
+
+def save_tuned(path):
+    """Writes the tuner table as JSON (variants by name, so that the file survives a
+    rebuild of the library)."""
+    import json
+    with open(path, "w") as f:
+        json.dump(tuned_table(), f, indent=1)
+
+
+def load_tuned(path):
+    """Re-enters a table written by save_tuned; entries this build does not take are
+    skipped.  Returns the number entered."""
+    import json
+    numbers = {n: v for v, n, _ in forward_variants()}
+    done = 0
+    for e in json.load(open(path)):
+        s = Shape(e["N"], e["H"], e["W"], e["pad"], e["T"], e["C"], e["Y"], e["X"], e["Rank"])
+        if e["variant"] not in numbers:
+            continue
+        try:
+            set_tuned_choice(s, numbers[e["variant"]], e["tile_rows"], e["tile_cols"],
+                             e["schedule"], backward_data=e["backward_data"])
+            done += 1
+        except Cp4Error:
+            pass
+    return done
 
 
 def tune_clear():

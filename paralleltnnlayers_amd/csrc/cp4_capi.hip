@@ -1273,6 +1273,38 @@ cp4_status cp4_set_tuned_choice(const cp4_shape* shape, int backward_data, int v
   return CP4_OK;
 }
 
+int cp4_tuned_count(void) {
+  std::lock_guard<std::mutex> lk(g_tune_mu);
+  return (int)g_tuned.size();
+}
+
+cp4_status cp4_tuned_entry(int index, cp4_shape* shape, int* backward_data, int* variant,
+                           int* tile_rows, int* tile_cols, int* schedule) {
+  if (!shape) return fail(CP4_ERR_NULL_POINTER, "shape is NULL");
+  std::lock_guard<std::mutex> lk(g_tune_mu);
+  if (index < 0 || index >= (int)g_tuned.size()) return fail(CP4_ERR_SHAPE, "index out of range");
+  auto it = g_tuned.begin();
+  std::advance(it, index);
+  const TuneKey& k = it->first;                    // N, Cin, Cout, H, W, pad, Y, X, R, flip
+  const bool bwd = std::get<9>(k) == 1;
+  shape->N = (unsigned)std::get<0>(k);
+  shape->C = (unsigned)(bwd ? std::get<2>(k) : std::get<1>(k));
+  shape->T = (unsigned)(bwd ? std::get<1>(k) : std::get<2>(k));
+  shape->H = (unsigned)std::get<3>(k);
+  shape->W = (unsigned)std::get<4>(k);
+  shape->pad = (unsigned)std::get<5>(k);
+  shape->Y = (unsigned)std::get<6>(k);
+  shape->X = (unsigned)std::get<7>(k);
+  shape->Rank = (unsigned)std::get<8>(k);
+  const Choice& c = it->second;
+  if (backward_data) *backward_data = bwd ? 1 : 0;
+  if (variant) *variant = c.variant;
+  if (tile_rows) *tile_rows = c.th;
+  if (tile_cols) *tile_cols = c.lgwt ? 1 << c.lgwt : 0;
+  if (schedule) *schedule = c.split2 == 1 ? 0 : (c.split2 == 2 ? 2 : 1);
+  return CP4_OK;
+}
+
 void cp4_tune_clear(void) {
   std::lock_guard<std::mutex> lk(g_tune_mu);
   g_tuned.clear();

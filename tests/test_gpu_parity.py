@@ -402,6 +402,34 @@ def test_timed_launch_and_tuner(cp4):
     assert torch.equal(y3, y4)
 
 
+def test_tuner_table_round_trip(cp4, tmp_path):
+    """The tuner's table written to a file and entered again (a later process): the
+    same choices come back, variants by name."""
+    w = WORKLOADS["C1"]
+    a = make_inputs(w)
+    f = [dev(a[k]) for k in FACTORS]
+    x = dev(a["x"])
+    s = cp4.capi.shape_for(x.shape, *f, w.pad)
+    names = [n for _, n, _ in cp4.forward_variants()]
+    try:
+        cp4.tune_clear()
+        cp4.set_tuned_choice(s, names.index("mfma_bf16x3_pipe"), 2, 0, 0)
+        cp4.set_tuned_choice(s, names.index("general_valu"), 0, 0, 1, backward_data=True)
+        table = cp4.tuned_table()
+        assert len(table) == 2 and {e["variant"] for e in table} == {"mfma_bf16x3_pipe", "general_valu"}
+        path = str(tmp_path / "tuned.json")
+        cp4.save_tuned(path)
+        cp4.tune_clear()
+        assert cp4.tuned_table() == []
+        assert cp4.load_tuned(path) == 2
+        assert cp4.tuned_table() == table
+        assert cp4.tuned_choice(s) == {"variant": names.index("mfma_bf16x3_pipe"), "tile_rows": 2,
+                                       "tile_cols": 0, "role_split": 0}
+        assert cp4.tuned_choice(s, backward_data=True)["variant"] == names.index("general_valu")
+    finally:
+        cp4.tune_clear()
+
+
 # N, C, H, W, T, Y, R: few ranks and channels, planes of many blocks (whole-block
 # producers; consumer waves that take whole pixel groups each)
 FEW_CHANNEL_CASES = [
