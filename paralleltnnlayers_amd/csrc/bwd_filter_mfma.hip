@@ -1558,28 +1558,37 @@ __global__ __launch_bounds__(256) void taps_strided_fast_kernel(
   const int nbw = (W + sw - 1) / sw, nbh = (H + sh - 1) / sh;
   for (int blk = threadIdx.x; blk < nbh * nbw; blk += 256) {
     const int bh = blk / nbw, bw = blk - bh * nbw;
+    // the FS*FS values of G3 the block's pixels draw on (0 outside the plane), once
+    float gv[FS][FS];
+#pragma unroll
+    for (int i = 0; i < FS; ++i) {
+      const int ho = bh + dh[i];
+      const bool rok = ho >= 0 && ho < Ho;
+#pragma unroll
+      for (int j = 0; j < FS; ++j) {
+        const int wo = bw + dw[j];
+        const bool ok = rok && wo >= 0 && wo < Wo;
+        const float v = sG[ok ? ho * Wo + wo : 0];
+        gv[i][j] = ok ? v : 0.f;
+      }
+    }
+    // pixel (a, b) of the block takes the taps that land on it: weights of the others 0
     for (int a = 0; a < sh; ++a) {
       const int h = sh * bh + a;
       if (h >= H) break;
+      float wr[FS];
+#pragma unroll
+      for (int i = 0; i < FS; ++i) wr[i] = ai[i] == a ? fh[i] : 0.f;
       for (int b = 0; b < sw; ++b) {
         const int w = sw * bw + b;
         if (w >= W) break;
         float g1 = 0.f;
 #pragma unroll
         for (int i = 0; i < FS; ++i) {
-          if (ai[i] != a) continue;               // (the same for all threads)
-          const int ho = bh + dh[i];
-          const bool rok = ho >= 0 && ho < Ho;
           float row = 0.f;
 #pragma unroll
-          for (int j = 0; j < FS; ++j) {
-            if (bj[j] != b) continue;
-            const int wo = bw + dw[j];
-            const bool ok = rok && wo >= 0 && wo < Wo;
-            const float v = sG[ok ? ho * Wo + wo : 0];
-            row += fw[j] * (ok ? v : 0.f);
-          }
-          g1 += fh[i] * row;
+          for (int j = 0; j < FS; ++j) row += (bj[j] == b ? fw[j] : 0.f) * gv[i][j];
+          g1 += wr[i] * row;
         }
         G1[basef + (size_t)h * W + w] = g1;
       }
