@@ -238,7 +238,8 @@ cp4_status cp4_geometry_symmetric(const cp4_shape* shape, unsigned stride_h, uns
 /* Forward x[N,C,H,W] -> y[N,T,out_h,out_w] = act(conv + bias) (bias [T] or NULL,
  * activation a cp4_activation).  Only the kept outputs are filtered, contracted
  * and stored: the producer / consumer kernel's strided build (square 1/3/5/7
- * filters, Rank <= 32), else the general kernel. */
+ * filters, Rank <= 32; bias and activation fused into its stores), else the
+ * general kernel followed by the in-place bias / activation kernel. */
 cp4_status cp4_conv2d_forward_ex(const cp4_shape* shape, const cp4_geometry* g, const float* x,
                                  const float* FK, const float* FC, const float* FH,
                                  const float* FW, const float* bias, int activation, float* y,

@@ -823,11 +823,15 @@ void set_geometry(FwdArgs& a, const cp4_geometry& g) {
 }
 // A launch with a geometry: the strided build of the producer / consumer kernel
 // where it applies and the matrix tiles are not mostly padding, else the general kernel.
-cp4_status run_geometry(FwdArgs a, hipStream_t st) {
+// (The strided build carries the bias / activation epilogue: a.bias / a.act are applied
+// there; *epilogue_done says whether they were.)
+cp4_status run_geometry(FwdArgs a, hipStream_t st, bool* epilogue_done = nullptr) {
+  if (epilogue_done) *epilogue_done = false;
   if (a.N == 0) return CP4_OK;
   arm(a);
   if (cp4::fwd_pipe_strided_supported(a) && a.Cin + a.Cout >= kMatrixMinChannels) {
     CP4_HIP(cp4::fwd_pipe_strided_launch(a, st));
+    if (epilogue_done) *epilogue_done = true;
     return CP4_OK;
   }
   if (!cp4::fwd_general_supported(a))
@@ -912,10 +916,13 @@ cp4_status cp4_conv2d_forward_ex(const cp4_shape* shape, const cp4_geometry* g, 
   if (rc != CP4_OK) return rc;
   FwdArgs a = forward_args(*shape, x, FK, FC, FH, FW, y);
   set_geometry(a, *g);
+  a.bias = bias;
+  a.act = activation;
   hipStream_t st = as_stream(stream);
-  rc = run_geometry(a, st);
+  bool fused = false;
+  rc = run_geometry(a, st, &fused);
   if (rc != CP4_OK) return rc;
-  if (bias || activation != CP4_ACT_NONE)
+  if (!fused && (bias || activation != CP4_ACT_NONE))
     CP4_HIP(cp4::bias_act_launch(y, bias, activation, shape->N, shape->T,
                                  (size_t)g->out_h * g->out_w, st));
   return CP4_OK;

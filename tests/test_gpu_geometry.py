@@ -122,8 +122,12 @@ def test_geometry_matrix_core_shapes(cp4, oracle, dims):
         close_gradient(got.cpu().numpy(), wnt.astype(np.float32), "d" + k)
     # bias and activation on the strided output
     bias = torch.randn(T, device="cuda", generator=gen) * 0.1
+    # (fused into the stores: the accumulators start at the bias, so the sum is
+    # rounded in another order than y + bias)
     yb = cp4.conv2d_forward_ex(x, *fac, geom, bias=bias, activation="relu")
-    assert torch.equal(yb, torch.relu(y + bias[None, :, None, None]))
+    wb = torch.relu(y + bias[None, :, None, None])
+    assert float((yb - wb).abs().max()) <= 1e-5 * float(wb.abs().max())
+    assert torch.equal(yb == 0, wb == 0) or float(wb[(yb == 0) != (wb == 0)].abs().max()) <= 1e-5
     cp4.device_status()
 
 
