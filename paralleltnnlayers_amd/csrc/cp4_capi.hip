@@ -495,6 +495,15 @@ cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
       return CP4_OK;
     }
   }
+  if (is_variant(c.variant, "mfma_bf16x3_pipe_tiled")) {
+    // (the tiled build carries the epilogue itself)
+    FwdArgs e = with_tile(a, c);
+    if (cp4::fwd_pipe_tiled_supported(e)) {
+      arm(e);
+      CP4_HIP(cp4::fwd_pipe_tiled_launch(e, st));
+      return CP4_OK;
+    }
+  }
   rc = run_choice(plain, c, st);
   if (rc != CP4_OK) return rc;
   CP4_HIP(cp4::bias_act_launch(y, bias, activation, shape->N, shape->T,

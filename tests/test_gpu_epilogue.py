@@ -37,6 +37,8 @@ SHAPES = [
     (1, 320, 14, 14, 1, 300, 3, 32),   # factor in LDS, more channel blocks than consumer waves
     (3, 5, 9, 9, 1, 7, 3, 3),          # general kernel + in-place epilogue
     (2, 64, 14, 14, 1, 64, 3, 48),     # rank above 32: strip kernel + in-place epilogue
+    (1, 24, 20, 224, 1, 40, 3, 16),    # wide plane: the tiled build, which carries the epilogue too
+    (2, 64, 30, 150, 1, 64, 3, 4),     # wide plane, whole pixel groups per consumer wave
 ]
 
 
