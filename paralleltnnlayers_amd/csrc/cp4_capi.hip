@@ -504,6 +504,10 @@ cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
       return CP4_OK;
     }
   }
+  if (is_variant(c.variant, "dense_small_valu") && cp4::fwd_dense_small_supported(a)) {
+    CP4_HIP(cp4::fwd_dense_small_launch(a, st));    // applies bias / activation in its stores
+    return CP4_OK;
+  }
   rc = run_choice(plain, c, st);
   if (rc != CP4_OK) return rc;
   CP4_HIP(cp4::bias_act_launch(y, bias, activation, shape->N, shape->T,

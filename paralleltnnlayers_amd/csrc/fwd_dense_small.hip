@@ -186,12 +186,20 @@ __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, De
       for (int k = 0; k < KO; ++k) {
         if (k < Cout) {
           float* dst = yp + (size_t)k * HW;
+          // y = act(conv + bias[k]) as the values are stored (FwdArgs::bias / act)
+          const float bk = a.bias ? a.bias[k0 + k] : 0.f;
+          float o[kPX];
+#pragma unroll
+          for (int p = 0; p < kPX; ++p) {
+            const float t = acc[k][p] + bk;
+            o[p] = (a.act != 0 && t < 0.f) ? 0.f : t;
+          }
           if (vec) {
-            *reinterpret_cast<float4*>(dst) = make_float4(acc[k][0], acc[k][1], acc[k][2], acc[k][3]);
+            *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
           } else {
 #pragma unroll
             for (int p = 0; p < kPX; ++p)
-              if (w + p < W) dst[p] = acc[k][p];
+              if (w + p < W) dst[p] = o[p];
           }
         }
       }

@@ -39,6 +39,8 @@ SHAPES = [
     (2, 64, 14, 14, 1, 64, 3, 48),     # rank above 32: strip kernel + in-place epilogue
     (1, 24, 20, 224, 1, 40, 3, 16),    # wide plane: the tiled build, which carries the epilogue too
     (2, 64, 30, 150, 1, 64, 3, 4),     # wide plane, whole pixel groups per consumer wave
+    (2, 3, 70, 130, 1, 1, 3, 16),      # three channels to one: the recomposed-filter kernel's own epilogue
+    (1, 4, 33, 47, 2, 12, 5, 8),       # ... with two groups of output channels, ragged tiles
 ]
 
 
