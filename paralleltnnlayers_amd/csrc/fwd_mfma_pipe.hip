@@ -580,8 +580,14 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #endif
     const bool split_roles = split_narrow || split_wide;
     const int wq = split_roles ? (wc >= 4 ? wc - 4 : 0) : wc;     // (first) rank quad in the tap step
-    if (!split_wide && fk_cached && wc < nkb) {
-      load_fk(wc, slot0);
+    // Narrow split with one or two channel blocks: the contraction waves left over
+    // take alternate groups (wave wc: block wc % nkb of the groups i = wc / nkb
+    // modulo crep), so two or four groups' contractions and stores are in flight.
+    // (From eight groups on; on shorter strips the extra waves' set-up costs more than
+    // they gain: C2 7.1 -> 7.3 us.)
+    const int crep = split_narrow && nkb <= 2 && ngroups >= 8 ? 4 / nkb : 1;
+    if (!split_wide && fk_cached && wc < nkb * crep) {
+      load_fk(wc % nkb, slot0);
     }
     // Tap weights of this wave's 4 ranks (wave-uniform values).
 #ifdef CP4_PIPE_TAPS2D
@@ -845,11 +851,14 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       constexpr int slot = decltype(slot_c)::value;
 #ifdef CP4_PIPE_EPILOGUE
       // the accumulators start at the bias of their rows (from LDS) instead of zero
-      const float* bkb = biasL + 32 * kb + 4 * hi;
-      f32x16 acc0 = {bkb[0],  bkb[1],  bkb[2],  bkb[3],  bkb[8],  bkb[9],  bkb[10], bkb[11],
-                     bkb[16], bkb[17], bkb[18], bkb[19], bkb[24], bkb[25], bkb[26], bkb[27]};
-      f32x16 acc1 = {bkb[0],  bkb[1],  bkb[2],  bkb[3],  bkb[8],  bkb[9],  bkb[10], bkb[11],
-                     bkb[16], bkb[17], bkb[18], bkb[19], bkb[24], bkb[25], bkb[26], bkb[27]};
+      f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
+      if (a.bias) {                                // (the same for all waves)
+        const float* bkb = biasL + 32 * kb + 4 * hi;
+        acc0 = f32x16{bkb[0],  bkb[1],  bkb[2],  bkb[3],  bkb[8],  bkb[9],  bkb[10], bkb[11],
+                      bkb[16], bkb[17], bkb[18], bkb[19], bkb[24], bkb[25], bkb[26], bkb[27]};
+        acc1 = f32x16{bkb[0],  bkb[1],  bkb[2],  bkb[3],  bkb[8],  bkb[9],  bkb[10], bkb[11],
+                      bkb[16], bkb[17], bkb[18], bkb[19], bkb[24], bkb[25], bkb[26], bkb[27]};
+      }
       __builtin_amdgcn_sched_barrier(0);
 #else
       f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
@@ -1082,11 +1091,14 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           if (i >= 3) wait_ge(&cdone[(i - 3) & 3], nkb * (((i - 3) >> 2) + 1), backoff, wx, 5);
           taps(i, Cb + (i % 3) * kCcBuf, one);
         }
-      } else if (wc < nkb) {
-        for (int i = 0; i < ngroups; ++i) {
+      } else if (wc < nkb * crep) {
+        // (a slot of cdone still gets its nkb signals per step, all from the same
+        // waves in step order)
+        const int kb = wc % nkb;
+        for (int i = wc / nkb; i < ngroups; i += crep) {
           const int g = rev ? ngroups - 1 - i : i;
           wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1), backoff, wx, 6);
-          contract_block(Cb + (i % 3) * kCcBuf, g, wc, one, true, i, slot0, no);
+          contract_block(Cb + (i % 3) * kCcBuf, g, kb, one, true, i, slot0, no);
         }
       }
       return;
