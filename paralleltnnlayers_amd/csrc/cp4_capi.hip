@@ -496,11 +496,11 @@ cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
     }
   }
   if (is_variant(c.variant, "mfma_bf16x3_pipe_tiled")) {
-    // (the tiled build carries the epilogue itself)
+    // (the tiled build's epilogue sibling)
     FwdArgs e = with_tile(a, c);
-    if (cp4::fwd_pipe_tiled_supported(e)) {
+    if (cp4::fwd_pipe_tiled_epi_supported(e)) {
       arm(e);
-      CP4_HIP(cp4::fwd_pipe_tiled_launch(e, st));
+      CP4_HIP(cp4::fwd_pipe_tiled_epi_launch(e, st));
       return CP4_OK;
     }
   }

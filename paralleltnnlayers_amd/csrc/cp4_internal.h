@@ -109,6 +109,8 @@ hipError_t fwd_pipe_rankpass_launch(const FwdArgs&, hipStream_t);
 // The same kernel on tiles of TH rows x Wt columns (wide planes).
 bool fwd_pipe_tiled_supported(const FwdArgs&);
 hipError_t fwd_pipe_tiled_launch(const FwdArgs&, hipStream_t);
+bool fwd_pipe_tiled_epi_supported(const FwdArgs&);          // ... with the bias / activation epilogue
+hipError_t fwd_pipe_tiled_epi_launch(const FwdArgs&, hipStream_t);
 // The same kernel for a stride or an output plane of its own (FwdArgs::sh ...
 // all filled in by the caller).
 bool fwd_pipe_strided_supported(const FwdArgs&);

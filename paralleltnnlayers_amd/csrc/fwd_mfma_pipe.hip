@@ -40,7 +40,7 @@
 // Cuda_kernels/cp4Conv2dForward.cu:84-133 (backward-data:
 // cp4Conv2dBackwardData.cu:57-108 through swapped factors and flipped taps).
 //
-// This file is compiled nine times: as is; with CP4_PIPE_EPILOGUE defined, which
+// This file is compiled ten times: as is; with CP4_PIPE_EPILOGUE defined, which
 // adds y = act(conv + bias[k]) to the stores (the bias, padded to whole channel
 // blocks, waits in LDS and is what the accumulators start from) and exports
 // the entry points under the names fwd_pipe_epi_*; and with CP4_PIPE_IO16, where
@@ -1370,6 +1370,9 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 #elif defined(CP4_PIPE_TAPS2D)
 #define fwd_pipe_supported fwd_pipe_taps2d_supported
 #define fwd_pipe_launch fwd_pipe_taps2d_launch
+#elif defined(CP4_PIPE_TILED) && defined(CP4_PIPE_EPILOGUE)
+#define fwd_pipe_supported fwd_pipe_tiled_epi_supported
+#define fwd_pipe_launch fwd_pipe_tiled_epi_launch
 #elif defined(CP4_PIPE_TILED)
 #define fwd_pipe_supported fwd_pipe_tiled_supported
 #define fwd_pipe_launch fwd_pipe_tiled_launch
