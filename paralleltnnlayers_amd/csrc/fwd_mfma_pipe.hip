@@ -1086,7 +1086,27 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       // contraction wave for the steps = s mod 4 (a single running total would
       // not do: a fast wave's later steps could stand in for a slow wave's
       // missing one); like the arrivals, a slot cannot run a whole cycle ahead.
+      // A tap wave whose rank quad lies past the last rank (up to 12 ranks) has
+      // nothing to compute: it zeroes its quad's entries in the three tiles once,
+      // arrives once (counted with step 0) and ends; the steps then count the
+      // live tap waves only.
+      const int nlive = min(4, (R + 3) >> 2), ndead = 4 - nlive;
       if (wc >= 4) {
+        if (4 * wq >= R) {
+          const u32x2 zero = {0u, 0u};
+#pragma unroll
+          for (int tb = 0; tb < 3; ++tb) {
+            unsigned char* dst = Cb + tb * kCcBuf + ((((wq >> 1) & 1) * 2 + (lane & 1)) * 512) +
+                                 (lane >> 1) * 16 + (wq & 1) * 8;
+            *reinterpret_cast<u32x2*>(dst) = zero;
+            *reinterpret_cast<u32x2*>(dst + 8 * 512) = zero;
+            *reinterpret_cast<u32x2*>(dst + 16 * 512) = zero;
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+          if (lane == 0)
+            __hip_atomic_fetch_add(&arrivals[0], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+          return;
+        }
         for (int i = 0; i < ngroups; ++i) {
           if (i >= 3) wait_ge(&cdone[(i - 3) & 3], nkb * (((i - 3) >> 2) + 1), backoff, wx, 5);
           taps(i, Cb + (i % 3) * kCcBuf, one);
@@ -1097,7 +1117,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         const int kb = wc % nkb;
         for (int i = wc / nkb; i < ngroups; i += crep) {
           const int g = rev ? ngroups - 1 - i : i;
-          wait_ge(&arrivals[i & 3], 4 * ((i >> 2) + 1), backoff, wx, 6);
+          wait_ge(&arrivals[i & 3], nlive * ((i >> 2) + 1) + ((i & 3) == 0 ? ndead : 0), backoff, wx,
+                  6);
           contract_block(Cb + (i % 3) * kCcBuf, g, kb, one, true, i, slot0, no);
         }
       }
