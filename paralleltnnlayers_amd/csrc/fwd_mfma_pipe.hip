@@ -1179,11 +1179,13 @@ bool own_groups_wanted(const FwdArgs& a) {
 #else
   const bool legal = a.R <= 16 && a.Cout <= 64 && a.Cin <= 64 && a.Y <= 5 && !a.accumulate;
   // by default where one rank quad is the whole tap step (the other schedules
-  // would run three empty quads beside it), with 3x3 and smaller filters also for
-  // two quads (16 x 16 x 512 x 512 at rank 8: 212 against 276 us; 5x5: 28 against
+  // would run three empty quads beside it), with 3x3 and smaller filters and at
+  // most 32 channels on one side also for two quads (16 x 16 x 512 x 512 at rank 8:
+  // 213 against 262 us; 64 -> 64 channels 224 x 224: 49 against 47; 5x5: 27 against
   // 22); above that only when tuned so
   // (tune_split2: 0 this rule, 1 no role split at all, 2 own groups)
-  const bool by_rule = a.R <= kOwnGroupsMaxRank || (a.R <= 2 * kOwnGroupsMaxRank && a.Y <= 3);
+  const bool by_rule = a.R <= kOwnGroupsMaxRank ||
+                       (a.R <= 2 * kOwnGroupsMaxRank && a.Y <= 3 && (a.Cin <= 32 || a.Cout <= 32));
   return legal && (a.tune_split2 == 2 || (a.tune_split2 == 0 && by_rule));
 #endif
 }
