@@ -122,7 +122,7 @@ constexpr int kMaxBlk = 64;                  // per-block progress words in LDS
 struct PipePlan {
   int TH, strips, nWG;
   int nblk;        // 32-pixel producer blocks of a workgroup's plane
-  int QA;          // LDS row stride of A (floats)
+  int QA;          // cells (of four ranks each) per rank quad of the A plane in LDS
   int fin_off;     // byte offsets inside LDS; factor fragments only above 256 input channels
   int cc_off;
   int flag_off;
@@ -186,7 +186,10 @@ __device__ __forceinline__ int wait_ge(int* word, int want, bool backoff, const 
 template <int FS, int CPQ, int KR, int NQ = 4>
 __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan pl) {
   extern __shared__ float lds[];
-  float* As = lds;                                                  // [32][QA] fp32
+  // A plane: [rank quad][QA cells] of four fp32 each (the quad's ranks side by side:
+  // one 16-byte LDS access moves a cell's four ranks)
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  f32x4* As4 = reinterpret_cast<f32x4*>(lds);
   unsigned char* ldsb = reinterpret_cast<unsigned char*>(lds);
   unsigned char* Fb = ldsb + pl.fin_off;     // Fin fragments [chunk][part][hi][r] x 16 B (CPQ == 0)
   unsigned char* Cb = ldsb + pl.cc_off;      // 3 x Cc fragment tiles
@@ -478,30 +481,30 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       if (j < nblk) {
         // add this quarter's partial sums after the lower quarters
         int* bf = &flags[j];
-        float* dst = &As[(4 * hi) * QA + qa];      // row 8*(v>>2) + (v&3) + 4*hi
+        // accumulator elements 4*g ... 4*g + 3 are ranks 8*g + 4*hi ...: rank quad 2*g + hi
+        f32x4* dst = As4 + (size_t)hi * QA + qa;
+        const int ng = low16 ? 2 : 4;              // the plane holds rank quads 0 ... 3 only
         if (cq == 0) {
 #pragma unroll
-          for (int v = 0; v < 8; ++v)
-            dst[(8 * (v >> 2) + (v & 3)) * QA] = valid ? acc[v] : 0.f;
-          if (!low16) {
-#pragma unroll
-            for (int v = 8; v < 16; ++v)
-              dst[(8 * (v >> 2) + (v & 3)) * QA] = valid ? acc[v] : 0.f;
-          }
+          for (int g = 0; g < 4; ++g)
+            if (g < ng)
+              dst[(2 * g) * QA] = valid ? f32x4{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]}
+                                        : f32x4{0.f, 0.f, 0.f, 0.f};
         } else {
           wait_ge(bf, cq, backoff, wx, 1);
-          // read all, then add, then write all: one LDS round trip per half, not
-          // one per element
+          // read, add, write two quads at a time: one LDS round trip per half
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
             if (half == 1 && low16) break;
-            float old[8];
+            f32x4 old[2];
 #pragma unroll
-            for (int v = 0; v < 8; ++v) old[v] = dst[(8 * ((8 * half + v) >> 2) + (v & 3)) * QA];
+            for (int g = 0; g < 2; ++g) old[g] = dst[(2 * (2 * half + g)) * QA];
 #pragma unroll
-            for (int v = 0; v < 8; ++v)
-              dst[(8 * ((8 * half + v) >> 2) + (v & 3)) * QA] =
-                  old[v] + (valid ? acc[8 * half + v] : 0.f);
+            for (int g = 0; g < 2; ++g) {
+              const int v = 4 * (2 * half + g);
+              dst[(2 * (2 * half + g)) * QA] =
+                  valid ? old[g] + f32x4{acc[v], acc[v + 1], acc[v + 2], acc[v + 3]} : old[g];
+            }
           }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -764,41 +767,61 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // else rows wa[rank][row] and columns wb[rank][col]).
     auto tap_quad = [&](const TapPos& tp, int q, const auto& wa, [[maybe_unused]] const auto& wb,
                         unsigned char* cb) {
-      // the LDS reads of RBT ranks go out together, then their arithmetic
-      constexpr int RBT = FS <= 3 ? 4 : (FS == 5 ? 2 : 1);
-      // (a quad past the last rank has zero weights; it reads quad 0's rows, the
+      // (a quad past the last rank has zero weights; it reads quad 0's cells, the
       // plane may end before its own, and writes zeros)
       const bool live = 4 * q < R;
-      const float* ab = As + (size_t)(live ? 4 * q : 0) * QA;
+      const f32x4* ab = As4 + (size_t)(live ? q : 0) * QA;
       float o[4];
+      // One 16-byte read per tap cell brings the quad's four ranks.  3x3 and
+      // smaller: all cells go out together, then the arithmetic; larger filters:
+      // tap row by tap row (registers).
+      if constexpr (FS <= 3) {
+        f32x4 av[FS][FS];
 #pragma unroll
-      for (int r0 = 0; r0 < 4; r0 += RBT) {
-        float av[RBT][FS][FS];
+        for (int ti = 0; ti < FS; ++ti)
 #pragma unroll
-        for (int rr = 0; rr < RBT; ++rr)
+          for (int j = 0; j < FS; ++j) av[ti][j] = ab[tp.roff[ti] + tp.off[j]];
 #pragma unroll
-          for (int ti = 0; ti < FS; ++ti)
-#pragma unroll
-            for (int j = 0; j < FS; ++j) av[rr][ti][j] = ab[(r0 + rr) * QA + tp.roff[ti] + tp.off[j]];
-#pragma unroll
-        for (int rr = 0; rr < RBT; ++rr) {
+        for (int rr = 0; rr < 4; ++rr) {
           float s = 0.f;
 #pragma unroll
           for (int ti = 0; ti < FS; ++ti) {
 #ifdef CP4_PIPE_TAPS2D
 #pragma unroll
             for (int j = 0; j < FS; ++j)
-              s += (tp.in[j] && tp.rin[ti] ? wa[r0 + rr][ti][j] : 0.f) * av[rr][ti][j];
+              s += (tp.in[j] && tp.rin[ti] ? wa[rr][ti][j] : 0.f) * av[ti][j][rr];
 #else
             float hs = 0.f;
 #pragma unroll
-            for (int j = 0; j < FS; ++j) hs += (tp.in[j] ? wb[r0 + rr][j] : 0.f) * av[rr][ti][j];
-            s += (tp.rin[ti] ? wa[r0 + rr][ti] : 0.f) * hs;
+            for (int j = 0; j < FS; ++j) hs += (tp.in[j] ? wb[rr][j] : 0.f) * av[ti][j][rr];
+            s += (tp.rin[ti] ? wa[rr][ti] : 0.f) * hs;
 #endif
           }
-          o[r0 + rr] = live ? s : 0.f;
+          o[rr] = live ? s : 0.f;
         }
-        if (RBT < 4) __builtin_amdgcn_sched_barrier(0);
+      } else {
+        float s[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ti = 0; ti < FS; ++ti) {
+          f32x4 av[FS];
+#pragma unroll
+          for (int j = 0; j < FS; ++j) av[j] = ab[tp.roff[ti] + tp.off[j]];
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+#ifdef CP4_PIPE_TAPS2D
+#pragma unroll
+            for (int j = 0; j < FS; ++j)
+              s[rr] += (tp.in[j] && tp.rin[ti] ? wa[rr][ti][j] : 0.f) * av[j][rr];
+#else
+            float hs = 0.f;
+#pragma unroll
+            for (int j = 0; j < FS; ++j) hs += (tp.in[j] ? wb[rr][j] : 0.f) * av[j][rr];
+            s[rr] += (tp.rin[ti] ? wa[rr][ti] : 0.f) * hs;
+#endif
+          }
+        }
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) o[rr] = live ? s[rr] : 0.f;
       }
       // exact split of the four values: two dwords per part
       u32x2 ph, pm, pl2;
