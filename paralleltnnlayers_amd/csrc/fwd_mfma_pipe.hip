@@ -183,7 +183,11 @@ __device__ __forceinline__ int wait_ge(int* word, int want, bool backoff, const 
 // NQ: channel splits of the producers (4: quarters, two blocks per round; 1: up to
 // 16 input channels, every producer wave takes a whole block of its own, eight
 // blocks per round and no partial sums to chain).
-template <int FS, int CPQ, int KR, int NQ = 4>
+// PAIR (16-bit activations, even row length): a producer lane loads two adjacent
+// pixels as one dword, a wave's block is 64 pixels (128-byte pieces of every
+// channel row instead of 64-byte ones) and holds two accumulators, one per pixel
+// parity; the progress words stay per 32 pixels.
+template <int FS, int CPQ, int KR, int NQ = 4, bool PAIR = false>
 __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan pl) {
   extern __shared__ float lds[];
   // A plane: [rank quad][QA cells] of four fp32 each (the quad's ranks side by side:
@@ -311,7 +315,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   if (wave < kProd) {
     // =========================== producers ==================================
     const int bsel = wave % NB, cq = wave / NB;    // block within the round, channel split
-    const int nrounds = (nblk + NB - 1) / NB;
+    const int nrounds = PAIR ? (((nblk + 1) >> 1) + NB - 1) / NB : (nblk + NB - 1) / NB;
     // lane's channel 16*(cpq*cq + chunk) + 8*hi + e
     // (channel groups past Cin count as zero: their factor rows are, and x reads there return 0)
     const int cg0 = 16 * cpq * cq + 8 * hi;        // lane's first channel of chunk 0
@@ -358,7 +362,20 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         reinterpret_cast<const u32x4*>(Fb + hi * 512 + l32 * 16) + (size_t)(cq * cpq) * (6 * 32);
     // Block of round r: sweep index j, LDS column qa of this lane, whether the
     // lane's pixel exists, and the lane's byte offset (clamped pixel, channel 8*hi).
-    auto geom = [&](int r, int& j, int& qa, bool& valid) -> unsigned {
+    auto geom = [&](int r, int& j, int& qa, bool& valid, [[maybe_unused]] bool& ex) -> unsigned {
+      if constexpr (PAIR) {
+        // span NB * r + bsel of the sweep: its 32-pixel blocks j and j + 1 (sweep
+        // order), 64 plane cells from s0 (-32 when the sweep runs backwards and
+        // the last span has one block only); the lane's pixels are cells qa, qa + 1
+        j = 2 * (NB * r + bsel);
+        const int s0 = rev ? 32 * (nblk - 2 - j) : 32 * j;
+        qa = s0 + 2 * l32;
+        const int q = qbase + qa;                  // even: W is
+        ex = j < nblk && qa >= 0 && qa < 32 * nblk;
+        valid = ex && q >= 0 && q < HW && qa < QLEN;
+        const int qc = q < 0 ? 0 : (q > HW - 2 ? HW - 2 : q);
+        return (unsigned)(8 * hi * HW + qc) * (unsigned)kIoBytes;
+      }
       j = NB * r + bsel;
       const int b = rev ? nblk - 1 - j : j;        // j == nblk happens when nblk is odd
       qa = 32 * b + l32;
@@ -381,9 +398,13 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     auto ld_chunk = [&](ring_t (&dst)[8], unsigned voff, int chunk) {   // chunk < cpq
       const unsigned soff = sbase + (unsigned)(16 * chunk) * (unsigned)HW * 2u;
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        dst[e] = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(
-            xrs, voff, soff + (unsigned)e * HW * 2u, 0);
+      for (int e = 0; e < 8; ++e) {
+        if constexpr (PAIR)
+          dst[e] = __builtin_amdgcn_raw_buffer_load_b32(xrs, voff, soff + (unsigned)e * HW * 2u, 0);
+        else
+          dst[e] = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(
+              xrs, voff, soff + (unsigned)e * HW * 2u, 0);
+      }
     };
 #else
     using ring_t = float;
@@ -397,19 +418,48 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #endif
     ring_t xb[KR][8];
     int j, qa;
-    bool valid;
-    unsigned xp = geom(0, j, qa, valid);
+    bool valid, ex = true;
+    unsigned xp = geom(0, j, qa, valid, ex);
 #pragma unroll
     for (int u = 0; u < KR; ++u) ld_chunk(xb[u], xp, u);
     for (int r = 0; r < nrounds; ++r) {
       int jn, qan;
-      bool validn;
-      const unsigned xpn = geom(r + 1 < nrounds ? r + 1 : r, jn, qan, validn);
+      bool validn, exn = true;
+      const unsigned xpn = geom(r + 1 < nrounds ? r + 1 : r, jn, qan, validn, exn);
       f32x16 acc = (f32x16)(0.f);
+      [[maybe_unused]] f32x16 acc2 = (f32x16)(0.f);      // PAIR: the odd pixels
       auto step = [&](int ch, int u) {
 #if CP4_PIPE_IO16 == 2
         // half-precision activations: 11 significand bits are two bfloat16 parts
         // (h + m exactly, l = 0), so five of the six partial products remain
+        if constexpr (PAIR) {
+          float xe[8], xo[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            xe[e] = (float)__builtin_bit_cast(_Float16, (unsigned short)xb[u][e]);
+            xo[e] = (float)__builtin_bit_cast(_Float16, (unsigned short)(xb[u][e] >> 16));
+          }
+          u32x4 eh, em, el, oh, om, ol;
+          split8(xe, eh, em, el);
+          split8(xo, oh, om, ol);
+          u32x4 tl, tm, th;
+          if (FLDS) {
+            const u32x4* fp = fbase + (size_t)(ch + u) * (6 * 32);
+            th = fp[0], tm = fp[64], tl = fp[128];
+          } else {
+            th = fh[FLDS ? 0 : ch + u], tm = fm[FLDS ? 0 : ch + u], tl = fl[FLDS ? 0 : ch + u];
+          }
+          acc = mfma16(tl, eh, acc);
+          acc = mfma16(tm, em, acc);
+          acc = mfma16(tm, eh, acc);
+          acc = mfma16(th, em, acc);
+          acc = mfma16(th, eh, acc);
+          acc2 = mfma16(tl, oh, acc2);
+          acc2 = mfma16(tm, om, acc2);
+          acc2 = mfma16(tm, oh, acc2);
+          acc2 = mfma16(th, om, acc2);
+          acc2 = mfma16(th, oh, acc2);
+        } else {
         float xv[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e)
@@ -430,21 +480,41 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           acc = mfma16(fh[FLDS ? 0 : ch + u], xm, acc);
           acc = mfma16(fh[FLDS ? 0 : ch + u], xh, acc);
         }
+        }
 #elif defined(CP4_PIPE_IO16)
         // the activations are bfloat16 already: pack pairs, multiply by the three
         // factor parts (smallest first)
         u32x4 xh;
+        [[maybe_unused]] u32x4 xo;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) xh[d] = xb[u][2 * d] | (xb[u][2 * d + 1] << 16);
+        for (int d = 0; d < 4; ++d) {
+          if constexpr (PAIR) {
+            // low halves: the even pixel of channels 2d, 2d + 1; high halves: the odd one
+            xh[d] = __builtin_amdgcn_perm(xb[u][2 * d + 1], xb[u][2 * d], 0x05040100u);
+            xo[d] = __builtin_amdgcn_perm(xb[u][2 * d + 1], xb[u][2 * d], 0x07060302u);
+          } else {
+            xh[d] = xb[u][2 * d] | (xb[u][2 * d + 1] << 16);
+          }
+        }
         if (FLDS) {
           const u32x4* fp = fbase + (size_t)(ch + u) * (6 * 32);
           acc = mfma16(fp[128], xh, acc);
           acc = mfma16(fp[64], xh, acc);
           acc = mfma16(fp[0], xh, acc);
+          if constexpr (PAIR) {
+            acc2 = mfma16(fp[128], xo, acc2);
+            acc2 = mfma16(fp[64], xo, acc2);
+            acc2 = mfma16(fp[0], xo, acc2);
+          }
         } else {
           acc = mfma16(fl[FLDS ? 0 : ch + u], xh, acc);
           acc = mfma16(fm[FLDS ? 0 : ch + u], xh, acc);
           acc = mfma16(fh[FLDS ? 0 : ch + u], xh, acc);
+          if constexpr (PAIR) {
+            acc2 = mfma16(fl[FLDS ? 0 : ch + u], xo, acc2);
+            acc2 = mfma16(fm[FLDS ? 0 : ch + u], xo, acc2);
+            acc2 = mfma16(fh[FLDS ? 0 : ch + u], xo, acc2);
+          }
         }
 #else
         u32x4 xh, xm, xl;
@@ -484,6 +554,42 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         // accumulator elements 4*g ... 4*g + 3 are ranks 8*g + 4*hi ...: rank quad 2*g + hi
         f32x4* dst = As4 + (size_t)hi * QA + qa;
         const int ng = low16 ? 2 : 4;              // the plane holds rank quads 0 ... 3 only
+        if constexpr (PAIR) {
+          // cells qa (even pixel) and qa + 1 (odd pixel); lanes whose half of the
+          // span has no block touch nothing
+          if (cq == 0) {
+            if (ex) {
+#pragma unroll
+              for (int g = 0; g < 4; ++g)
+                if (g < ng) {
+                  const int v = 4 * g;
+                  dst[(2 * g) * QA] = valid ? f32x4{acc[v], acc[v + 1], acc[v + 2], acc[v + 3]}
+                                            : f32x4{0.f, 0.f, 0.f, 0.f};
+                  dst[(2 * g) * QA + 1] =
+                      valid ? f32x4{acc2[v], acc2[v + 1], acc2[v + 2], acc2[v + 3]}
+                            : f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+          } else {
+            wait_ge(bf, cq, backoff, wx, 1);
+            if (ex && valid) {
+#pragma unroll
+              for (int g = 0; g < 4; ++g)
+                if (g < ng) {
+                  const int v = 4 * g;
+                  const f32x4 o0 = dst[(2 * g) * QA], o1 = dst[(2 * g) * QA + 1];
+                  dst[(2 * g) * QA] = o0 + f32x4{acc[v], acc[v + 1], acc[v + 2], acc[v + 3]};
+                  dst[(2 * g) * QA + 1] = o1 + f32x4{acc2[v], acc2[v + 1], acc2[v + 2], acc2[v + 3]};
+                }
+            }
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+          if (lane == 0) {
+            __hip_atomic_store(bf, cq + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (j + 1 < nblk)
+              __hip_atomic_store(bf + 1, cq + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+          }
+        } else {
         if (cq == 0) {
 #pragma unroll
           for (int g = 0; g < 4; ++g)
@@ -510,12 +616,14 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (lane == 0)
           __hip_atomic_store(bf, cq + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
       }
       STAMP(2 + r)
       xp = xpn;
       j = jn;
       qa = qan;
       valid = validn;
+      ex = exn;
     }
 #ifdef CP4_DEBUG_PHASES
     if (pl.dbg && lane == 0) pl.dbg[((size_t)t * 16 + wave) * 32 + 31] = clock64();
@@ -1365,6 +1473,18 @@ bool plan(const FwdArgs& a, PipePlan* best) {
 
 template <int FS, int CPQ, int KR, int NQ = 4>
 hipError_t launch_as(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
+#ifdef CP4_PIPE_IO16
+  // even rows, activations on a 4-byte boundary: the producers load pixel pairs
+  if ((a.W & 1) == 0 && (reinterpret_cast<uintptr_t>(a.x) & 3) == 0) {
+    const void* fp = reinterpret_cast<const void*>(fwd_pipe_kernel<FS, CPQ, KR, NQ, true>);
+    hipError_t ep = hipFuncSetAttribute(fp, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)pl.lds_bytes);
+    if (ep != hipSuccess) return ep;
+    fwd_pipe_kernel<FS, CPQ, KR, NQ, true>
+        <<<8u * ((pl.nWG + 7) / 8), kThreads, pl.lds_bytes, st>>>(a, pl);
+    return hipGetLastError();
+  }
+#endif
   const void* fn = reinterpret_cast<const void*>(fwd_pipe_kernel<FS, CPQ, KR, NQ>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)pl.lds_bytes);
