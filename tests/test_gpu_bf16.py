@@ -91,6 +91,47 @@ def test_bf16_matches_fp32_kernel_then_rounding(cp4):
     assert (a - b).abs().max().item() <= 2.0 ** -7 * b.abs().max().item()
 
 
+# even rows: producers load pixel pairs; plane lengths of an odd and an even number
+# of 32-pixel blocks, one strip and several (odd strips sweep backwards)
+PAIR_SHAPES = [
+    (2, 64, 40, 22, 1, 64, 3, 16),
+    (1, 128, 13, 30, 1, 96, 3, 32),
+    (3, 32, 9, 34, 2, 40, 5, 8),
+    (2, 16, 57, 12, 0, 16, 1, 4),
+    (1, 320, 21, 18, 1, 64, 3, 24),      # factor in LDS
+]
+
+
+@pytest.mark.parametrize("dims", PAIR_SHAPES, ids=lambda d: "x".join(map(str, d)))
+@pytest.mark.parametrize("half", [False, True], ids=["bf16", "f16"])
+def test_pixel_pair_producers_match_the_element_path(cp4, oracle, dims, half):
+    """With an even row length the producers of the 16-bit builds load two pixels
+    per lane.  An x that starts two bytes off a 4-byte boundary takes the
+    element-by-element path instead: same products in the same order, so the two
+    results are bit-identical, and both meet the oracle's bar."""
+    N, C, H, W, pad, T, Y, R = dims
+    rng = np.random.default_rng(sum(dims))
+    dt = torch.float16 if half else torch.bfloat16
+    x = torch.from_numpy(rng.standard_normal((N, C, H, W)).astype(np.float32)).to(dt)
+    fac = [(rng.standard_normal((d, R)) / np.sqrt(R)).astype(np.float32) for d in (T, C, Y, Y)]
+    f = [torch.from_numpy(v).cuda() for v in fac]
+    fwd = cp4.conv2d_forward_f16 if half else cp4.conv2d_forward_bf16
+    buf = torch.zeros(x.numel() + 2, dtype=dt, device="cuda")
+    aligned = buf[:x.numel()].view(x.shape)
+    shifted = buf[1:1 + x.numel()].view(x.shape)
+    assert aligned.data_ptr() % 4 == 0 and shifted.data_ptr() % 4 == 2
+    aligned.copy_(x)
+    ya = fwd(aligned, *f, pad=pad).clone()
+    shifted.copy_(x)
+    ys = fwd(shifted, *f, pad=pad)
+    assert torch.equal(ya, ys)
+    want = oracle.forward(x.float().numpy(), *fac, pad)
+    got = ya.float().cpu().numpy()
+    ulp = 2.0 ** -11 if half else 2.0 ** -8
+    scale = float(np.abs(want).max())
+    assert np.all(np.abs(got - want) <= ulp * 1.01 * np.abs(want) + 1e-4 * np.abs(want) + 1e-5 * scale)
+
+
 def test_bf16_unsupported_shapes_are_refused(cp4):
     x = torch.randn(1, 8, 6, 6, device="cuda").to(torch.bfloat16)
     fac = [torch.randn(d, 40, device="cuda") for d in (8, 8, 3, 3)]     # rank 40 > 32
