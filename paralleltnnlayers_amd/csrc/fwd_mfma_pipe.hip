@@ -363,6 +363,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // Block of round r: sweep index j, LDS column qa of this lane, whether the
     // lane's pixel exists, and the lane's byte offset (clamped pixel, channel 8*hi).
     auto geom = [&](int r, int& j, int& qa, bool& valid, [[maybe_unused]] bool& ex) -> unsigned {
+#ifdef CP4_PIPE_IO16
       if constexpr (PAIR) {
         // span NB * r + bsel of the sweep: its 32-pixel blocks j and j + 1 (sweep
         // order), 64 plane cells from s0 (-32 when the sweep runs backwards and
@@ -376,6 +377,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         const int qc = q < 0 ? 0 : (q > HW - 2 ? HW - 2 : q);
         return (unsigned)(8 * hi * HW + qc) * (unsigned)kIoBytes;
       }
+#endif
       j = NB * r + bsel;
       const int b = rev ? nblk - 1 - j : j;        // j == nblk happens when nblk is odd
       qa = 32 * b + l32;
@@ -1221,13 +1223,17 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       // nothing to compute: it zeroes its quad's entries in the three tiles once,
       // arrives once (counted with step 0) and ends; the steps then count the
       // live tap waves only.
+      // Up to 16 ranks a tile fills only the planes of its first rank chunk, so the
+      // first two of the three tiles share a buffer (the second in the planes of
+      // the unused chunk, 4 * 512 bytes further) and the plane gets the room.
+      auto tile3 = [&](int k) { return Cb + (k >> 1) * kCcBuf + (k & 1) * (4 * 512); };
       const int nlive = min(4, (R + 3) >> 2), ndead = 4 - nlive;
       if (wc >= 4) {
         if (4 * wq >= R) {
           const u32x2 zero = {0u, 0u};
 #pragma unroll
           for (int tb = 0; tb < 3; ++tb) {
-            unsigned char* dst = Cb + tb * kCcBuf + ((((wq >> 1) & 1) * 2 + (lane & 1)) * 512) +
+            unsigned char* dst = tile3(tb) + ((((wq >> 1) & 1) * 2 + (lane & 1)) * 512) +
                                  (lane >> 1) * 16 + (wq & 1) * 8;
             *reinterpret_cast<u32x2*>(dst) = zero;
             *reinterpret_cast<u32x2*>(dst + 8 * 512) = zero;
@@ -1240,7 +1246,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         }
         for (int i = 0; i < ngroups; ++i) {
           if (i >= 3) wait_ge(&cdone[(i - 3) & 3], nkb * (((i - 3) >> 2) + 1), backoff, wx, 5);
-          taps(i, Cb + (i % 3) * kCcBuf, one);
+          taps(i, tile3(i % 3), one);
         }
       } else if (wc < nkb * crep) {
         // (a slot of cdone still gets its nkb signals per step, all from the same
@@ -1250,7 +1256,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           const int g = rev ? ngroups - 1 - i : i;
           wait_ge(&arrivals[i & 3], nlive * ((i >> 2) + 1) + ((i & 3) == 0 ? ndead : 0), backoff, wx,
                   6);
-          contract_block(Cb + (i % 3) * kCcBuf, g, kb, one, true, i, slot0, no);
+          contract_block(tile3(i % 3), g, kb, one, true, i, slot0, no);
         }
       }
       return;
@@ -1320,7 +1326,13 @@ bool own_groups_wanted(const FwdArgs& a) {
   return legal && (a.tune_split2 == 2 || (a.tune_split2 == 0 && by_rule));
 #endif
 }
-size_t cc_region_bytes(const FwdArgs& a) { return (size_t)(own_groups_wanted(a) ? 4 : 3) * kCcBuf; }
+size_t cc_region_bytes(const FwdArgs& a) {
+  if (own_groups_wanted(a)) return (size_t)4 * kCcBuf;
+  // the narrow role split (the kernel's rule: up to 16 ranks, 4 channel blocks, 5x5)
+  // packs its first two tiles into one buffer; the third ends after 20 planes
+  if (a.R <= 16 && a.Cout <= 128 && a.Y <= 5) return (size_t)kCcBuf + 20 * 512;
+  return (size_t)3 * kCcBuf;
+}
 
 // Rank rows of the A plane in LDS: the producers' 32 x 32 products carry 32, of
 // which the upper 16 are zero (and neither written nor read) up to 16 ranks.
