@@ -312,6 +312,10 @@ int cp4_forward_variant_count(void);
 const char* cp4_forward_variant_name(int variant);
 /* CP4_OK if `variant` can run `shape`, else CP4_ERR_UNSUPPORTED. */
 cp4_status cp4_forward_variant_supported(const cp4_shape* shape, int variant);
+/* The variant the library's choice falls on for `shape` (forward, or the
+ * backward-data pass of that layer): the tuned entry if there is one, else the
+ * heuristic; -1 if the shape is invalid or no variant takes it. */
+int cp4_forward_default_variant(const cp4_shape* shape, int backward_data);
 cp4_status cp4_conv2d_forward_variant(const cp4_shape* shape, const float* x,
                                       const float* FK, const float* FC,
                                       const float* FH, const float* FW,

@@ -545,6 +545,15 @@ def forward_variants(s=None):
     return out
 
 
+def default_variant(s, backward_data=False):
+    """Name of the variant the library runs for shape s unless told otherwise
+    (None: no variant takes the shape)."""
+    L = lib()
+    L.cp4_forward_default_variant.restype = ctypes.c_int
+    v = L.cp4_forward_default_variant(ctypes.byref(s), int(backward_data))
+    return L.cp4_forward_variant_name(v).decode() if v >= 0 else None
+
+
 def tune_forward(x, FK, FC, FH, FW, y, pad, warmup=1, profcount=10, stream=None):
     s = shape_for(x.shape, FK, FC, FH, FW, pad)
     best, us = ctypes.c_int(-1), ctypes.c_float()

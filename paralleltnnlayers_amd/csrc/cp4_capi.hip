@@ -257,9 +257,29 @@ double general_estimate(const FwdArgs& a) {
   return 10.0 + 0.3 * a.R * (a.Cin + a.Cout + a.Y + a.X);
 }
 
-// Rows longer than this leave whole-row strips only a row or two (2 at W = 224):
-// tiles of TH x Wt pay less for their halo.
+// Rows longer than this may leave whole-row strips only a row or two (2 at
+// W = 224 and 32 ranks): tiles of TH x Wt then pay less for their halo.  Where the
+// strips still get a few rows (up to 16 ranks the LDS plane holds half the rank
+// rows) they win - long contiguous rows, no column halo: N8 C128 224x224 R16 96
+// against 112 us, N16 C256 160x160 R16 203 against 254 - unless too few of them
+// fill the chip or, with few channels, the halo rows cost more than they save
+// (N8 C32 150x300 R16: 45 against 30 us).
 constexpr int kWholeRowMaxWidth = 128;
+// What the halo rows add to a strip's traffic, (rows read x Cin + rows written x
+// Cout) over the same without halo: up to 1.35 with 128 input channels or more,
+// else up to 1.15 on strips of at least four rows that fill the chip.
+constexpr double kStripMaxTraffic = 1.15, kStripMaxTrafficManyChannels = 1.35;
+constexpr int kStripManyChannels = 128, kStripMinRows = 4;
+bool strips_on_wide_plane(const FwdArgs& a) {
+  int rows = 0, wgs = 0;
+  if (!cp4::fwd_pipe_strip_plan(a, &rows, &wgs)) return false;
+  const double traffic =
+      1.0 + (double)(a.Y - 1) * a.Cin / ((double)rows * (a.Cin + a.Cout));
+  if (a.Cin >= kStripManyChannels) return traffic <= kStripMaxTrafficManyChannels;
+  const bool fills = 4 * wgs >= 3 * cp4::num_compute_units();
+  return traffic <= kStripMaxTraffic && rows >= kStripMinRows && fills;
+}
+
 // Two rank passes read x twice and y once more; below this many activation
 // elements the fp32 matrix-core strip kernel is the faster one for ranks 33-64.
 constexpr long kTwoPassMinElements = 16l << 20;
@@ -284,7 +304,7 @@ int heuristic_variant(const FwdArgs& a) {
   if (pick >= 0 && !strncmp(kVariants[pick].name, "mfma_bf16x3_pipe", 16) &&
       a.Cin + a.Cout < kMatrixMinChannels && a.R <= kMatrixMinRank)
     prefer("general_valu");
-  if (is_variant(pick, "mfma_bf16x3_pipe") && a.W > kWholeRowMaxWidth)
+  if (is_variant(pick, "mfma_bf16x3_pipe") && a.W > kWholeRowMaxWidth && !strips_on_wide_plane(a))
     prefer("mfma_bf16x3_pipe_tiled");
   if (is_variant(pick, "mfma_bf16x3_pipe_rank_passes") && a.R <= 64 &&
       (long)a.N * a.H * a.W * (a.Cin + a.Cout) < kTwoPassMinElements)
@@ -1142,6 +1162,15 @@ cp4_status cp4_forward_variant_supported(const cp4_shape* shape, int variant) {
   return kVariants[variant].supported(a)
              ? CP4_OK
              : fail(CP4_ERR_UNSUPPORTED, "variant does not support this shape");
+}
+
+int cp4_forward_default_variant(const cp4_shape* shape, int backward_data) {
+  if (check_shape(shape) != CP4_OK) return -1;
+  const FwdArgs a =
+      backward_data
+          ? backward_data_args(*shape, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr)
+          : forward_args(*shape, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr);
+  return choose(a).variant;
 }
 
 namespace {

@@ -93,6 +93,8 @@ bool fwd_split_supported(const FwdArgs&);
 hipError_t fwd_split_launch(const FwdArgs&, hipStream_t);
 bool fwd_pipe_supported(const FwdArgs&);
 hipError_t fwd_pipe_launch(const FwdArgs&, hipStream_t);
+// Rows per strip and workgroups of the whole-row strip plan (false: no plan).
+bool fwd_pipe_strip_plan(const FwdArgs&, int* rows, int* workgroups);
 // The same kernel compiled with the bias / activation epilogue in its stores.
 bool fwd_pipe_epi_supported(const FwdArgs&);
 hipError_t fwd_pipe_epi_launch(const FwdArgs&, hipStream_t);

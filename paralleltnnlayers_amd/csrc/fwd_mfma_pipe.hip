@@ -1591,6 +1591,19 @@ bool fwd_pipe_supported(const FwdArgs& a) {
   return plan(a, &pl);
 }
 
+#if !defined(CP4_PIPE_STRIDED) && !defined(CP4_PIPE_TAPS2D) && !defined(CP4_PIPE_TILED) && \
+    !defined(CP4_PIPE_RANKPASS) && !defined(CP4_PIPE_IO16) && !defined(CP4_PIPE_EPILOGUE)
+// What the planner gives a shape as whole-row strips: rows per strip and
+// workgroups (the variant choice weighs them against tiles on wide planes).
+bool fwd_pipe_strip_plan(const FwdArgs& a, int* rows, int* workgroups) {
+  PipePlan pl;
+  if (!fwd_pipe_supported(a) || !plan(a, &pl)) return false;
+  *rows = pl.TH;
+  *workgroups = pl.nWG;
+  return true;
+}
+#endif
+
 hipError_t fwd_pipe_launch(const FwdArgs& a, hipStream_t st) {
   PipePlan pl;
   if (!plan(a, &pl)) return hipErrorInvalidValue;

@@ -99,6 +99,34 @@ def test_argument_errors_need_no_device(L):
                               ctypes.byref(us), None) == capi.ERR_SHAPE
 
 
+def test_default_variant_on_wide_planes(L):
+    """The variant choice needs no GPU (the planners assume 256 compute units when
+    no device is current).  Rows beyond 128 pixels: whole-row strips where their
+    plan keeps a few rows (up to 16 ranks the LDS plane holds half the rank rows),
+    tiles where strips would be a row or two; a tuned entry overrides both."""
+    from paralleltnnlayers_amd import capi
+
+    def shape(N, C, H, W, T, R, Y=3):
+        return capi.Shape(N=N, H=H, W=W, pad=Y // 2, T=T, C=C, Y=Y, X=Y, Rank=R)
+    capi.tune_clear()
+    assert capi.default_variant(shape(32, 256, 56, 56, 256, 32)) == "mfma_bf16x3_pipe"
+    assert capi.default_variant(shape(8, 64, 224, 224, 64, 16)) == "mfma_bf16x3_pipe"
+    assert capi.default_variant(shape(8, 64, 224, 224, 64, 32)) == "mfma_bf16x3_pipe_tiled"
+    assert capi.default_variant(shape(2, 64, 512, 512, 64, 16)) == "mfma_bf16x3_pipe_tiled"
+    assert capi.default_variant(shape(8, 32, 150, 300, 32, 16)) == "mfma_bf16x3_pipe_tiled"
+    assert capi.default_variant(shape(16, 256, 160, 160, 256, 16)) == "mfma_bf16x3_pipe"
+    assert capi.default_variant(shape(1, 3, 512, 512, 1, 16)) == "dense_small_valu"
+    assert capi.default_variant(shape(8, 64, 224, 224, 64, 16), backward_data=True) \
+        == "mfma_bf16x3_pipe"
+    s = shape(8, 64, 224, 224, 64, 16)
+    tiled = [v for v, n, _ in capi.forward_variants() if n == "mfma_bf16x3_pipe_tiled"][0]
+    capi.set_tuned_choice(s, tiled, 14, 64, 1)
+    assert capi.default_variant(s) == "mfma_bf16x3_pipe_tiled"
+    capi.tune_clear()
+    assert capi.default_variant(s) == "mfma_bf16x3_pipe"
+    assert capi.default_variant(capi.Shape(N=1, H=0, W=8, pad=1, T=4, C=4, Y=3, X=3, Rank=2)) is None
+
+
 def test_status_strings(L):
     seen = {L.cp4_status_string(i) for i in range(6)}
     assert len(seen) == 6 and b"ok" in seen
