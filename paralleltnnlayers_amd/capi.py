@@ -70,6 +70,8 @@ def lib():
     L.cp4_status_string.argtypes = [ctypes.c_int]
     L.cp4_last_error_message.restype = ctypes.c_char_p
     L.cp4_forward_variant_name.restype = ctypes.c_char_p
+    L.cp4_forward_default_variant.restype = ctypes.c_int
+    L.cp4_forward_default_variant.argtypes = [_S, ctypes.c_int]
     L.cp4_forward_variant_name.argtypes = [ctypes.c_int]
     L.cp4_conv2d_backward_filter_workspace_bytes.restype = ctypes.c_size_t
     L.cp4_conv2d_backward_filter_workspace_bytes.argtypes = [_S]
@@ -549,7 +551,6 @@ def default_variant(s, backward_data=False):
     """Name of the variant the library runs for shape s unless told otherwise
     (None: no variant takes the shape)."""
     L = lib()
-    L.cp4_forward_default_variant.restype = ctypes.c_int
     v = L.cp4_forward_default_variant(ctypes.byref(s), int(backward_data))
     return L.cp4_forward_variant_name(v).decode() if v >= 0 else None
 
