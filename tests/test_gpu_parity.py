@@ -280,6 +280,32 @@ def test_wide_role_split_at_scale(cp4, oracle):
                                 "backward-data")
 
 
+def test_whole_row_strips_on_a_wide_plane(cp4, oracle):
+    """Rows of 224 pixels, 16 ranks, 128 channels: the library's choice is the
+    whole-row strip variant (4-row strips, one round of workgroups; the LDS plane
+    has the room because up to 16 ranks it holds half the rank rows); with 32
+    ranks the same layer runs on tiles.  Forward, backward-data and the fused epilogue."""
+    N, C, H, W, pad, T, Y = 32, 128, 28, 224, 1, 128, 3     # (enough rows for several per strip)
+    rng = np.random.default_rng(224)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    dy = rng.standard_normal((N, T, H, W)).astype(np.float32)
+    for R, variant in ((16, "mfma_bf16x3_pipe"), (32, "mfma_bf16x3_pipe_tiled")):
+        fac = [(rng.standard_normal((d, R)) / np.sqrt(R)).astype(np.float32) for d in (T, C, Y, Y)]
+        f = [dev(v) for v in fac]
+        s = cp4.capi.shape_for(x.shape, *f, pad)
+        assert cp4.default_variant(s) == variant
+        assert cp4.default_variant(s, backward_data=True) == variant
+        want = oracle.forward(x, *fac, pad)
+        want_dx = oracle.backward_data(dy, *fac, pad)
+        bias = rng.standard_normal(T).astype(np.float32)
+        for _ in range(2):
+            assert_activation_close(host(cp4.conv2d_forward(dev(x), *f, pad=pad)), want, "forward")
+            assert_activation_close(host(cp4.conv2d_backward_data(dev(dy), *f, pad=pad)), want_dx,
+                                    "backward-data")
+        yb = host(cp4.conv2d_forward_bias_act(dev(x), *f, bias=dev(bias), activation="relu", pad=pad))
+        assert_activation_close(yb, np.maximum(want + bias[None, :, None, None], 0), "bias + relu")
+
+
 @pytest.mark.parametrize("dims", [(2, 64, 28, 28, 64, 3, 16), (2, 256, 28, 28, 256, 3, 32),
                                   (2, 128, 14, 14, 128, 5, 16), (3, 5, 9, 9, 7, 3, 3),
                                   (2, 48, 13, 13, 48, 3, 40)],
