@@ -266,16 +266,23 @@ double general_estimate(const FwdArgs& a) {
 // (N8 C32 150x300 R16: 45 against 30 us).
 constexpr int kWholeRowMaxWidth = 128;
 // What the halo rows add to a strip's traffic, (rows read x Cin + rows written x
-// Cout) over the same without halo: up to 1.35 with 128 input channels or more,
-// else up to 1.15 on strips of at least four rows that fill the chip.
+// Cout) over the same without halo: up to 1.35 with 128 input channels or more
+// (1.5 with 256 on rows up to 192 pixels), else up to 1.15 on strips of at least
+// four rows that fill the chip.
 constexpr double kStripMaxTraffic = 1.15, kStripMaxTrafficManyChannels = 1.35;
 constexpr int kStripManyChannels = 128, kStripMinRows = 4;
+// With 256 input channels even two-row strips (32 ranks) beat tiles up to this
+// width (N16 C256 160x160 R32: 225 against 265 us; 192 wide: 190 against 204;
+// 224 wide: 291 against 249).
+constexpr int kStripTwoRowMaxWidth = 192;
 bool strips_on_wide_plane(const FwdArgs& a) {
   int rows = 0, wgs = 0;
   if (!cp4::fwd_pipe_strip_plan(a, &rows, &wgs)) return false;
   const double traffic =
       1.0 + (double)(a.Y - 1) * a.Cin / ((double)rows * (a.Cin + a.Cout));
-  if (a.Cin >= kStripManyChannels) return traffic <= kStripMaxTrafficManyChannels;
+  if (a.Cin >= kStripManyChannels)
+    return traffic <= kStripMaxTrafficManyChannels ||
+           (a.Cin >= 2 * kStripManyChannels && a.W <= kStripTwoRowMaxWidth && traffic <= 1.5);
   const bool fills = 4 * wgs >= 3 * cp4::num_compute_units();
   return traffic <= kStripMaxTraffic && rows >= kStripMinRows && fills;
 }
