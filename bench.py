@@ -45,7 +45,7 @@ FACTORS = ("FK", "FC", "FH", "FW")
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs, scaled by the plain copy kernel's reading (see
 # profiles/): {workload: bytes}.  None until measured for the current kernel.
-MEASURED_TRAFFIC = {"C3": 209.8e6}   # fwd_pipe_kernel<3,4,2,4>: 107.0 MB fetched + 102.8 MB written
+MEASURED_TRAFFIC = {"C3": 209.9e6}   # fwd_pipe_kernel<3,4,2,4>: 107.1 MB fetched + 102.8 MB written
 
 
 def main():
