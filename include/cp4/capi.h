@@ -193,8 +193,11 @@ cp4_status cp4_conv2d_backward_filter_noalloc(const cp4_shape* shape, const floa
                                               float* dFH, float* dFW, cp4_stream stream);
 
 /* Same, with the kernel variant chosen by the caller: -1 library's choice,
- * 0 general (any shape), 1 matrix-core path (CP4_ERR_UNSUPPORTED if the shape
- * does not qualify). */
+ * 0 general (any shape), 1 matrix cores in four launches (contraction, taps,
+ * gradient GEMMs, sum), 2 matrix cores in three launches with the tap step inside
+ * the gradient GEMMs (square odd filters up to 5x5 with 2 * pad == Y - 1, channel
+ * counts multiples of 16, H * W a multiple of 4, W >= 8, 16-byte aligned x / dy /
+ * workspace); CP4_ERR_UNSUPPORTED if the shape does not qualify for 1 or 2. */
 cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const float* x,
                                               const float* dy, const float* FK,
                                               const float* FC, const float* FH,

@@ -385,9 +385,17 @@ size_t filter_workspace(const cp4_shape& s) {
     const size_t m = cp4::bwd_filter_mfma_workspace_bytes(s);
     if (m > b) b = m;
   }
+  if (cp4::bwd_filter_fused_supported(s)) {
+    const size_t m = cp4::bwd_filter_fused_workspace_bytes(s);
+    if (m > b) b = m;
+  }
   if (filter_rank_tiles_supported(s)) {
-    const size_t m = 2 * filter_rank_tile_floats(s) * sizeof(float) +
-                     cp4::bwd_filter_mfma_workspace_bytes(filter_rank_tile(s, 0));
+    size_t inner = cp4::bwd_filter_mfma_workspace_bytes(filter_rank_tile(s, 0));
+    if (cp4::bwd_filter_fused_supported(filter_rank_tile(s, 0))) {
+      const size_t f = cp4::bwd_filter_fused_workspace_bytes(filter_rank_tile(s, 0));
+      if (f > inner) inner = f;
+    }
+    const size_t m = 2 * filter_rank_tile_floats(s) * sizeof(float) + inner;
     if (m > b) b = m;
   }
   return b;
@@ -692,7 +700,14 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
   const bool tiles_ok = filter_rank_tiles_supported(s) && aligned &&
                         (reinterpret_cast<uintptr_t>(workspace) & 255) == 0;
   const bool mfma_ok = (cp4::bwd_filter_mfma_supported(s) && aligned) || tiles_ok;
-  if (variant > 1 || (variant == 1 && !mfma_ok))
+  const bool aligned16 = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) |
+                           reinterpret_cast<uintptr_t>(workspace)) & 15) == 0;
+  // more than 64 ranks: the fused variant runs per rank tile when every tile qualifies
+  const bool fused_tiles = tiles_ok && cp4::bwd_filter_fused_supported(filter_rank_tile(s, 0)) &&
+                           cp4::bwd_filter_fused_supported(filter_rank_tile(
+                               s, (s.Rank - 1) / kFilterRankTile * kFilterRankTile));
+  const bool fused_ok = aligned16 && (cp4::bwd_filter_fused_supported(s) || fused_tiles);
+  if (variant > 2 || (variant == 1 && !mfma_ok) || (variant == 2 && !fused_ok))
     return fail(CP4_ERR_UNSUPPORTED, "backward-filter variant cannot run this shape");
   cp4::BwdFilterArgs a{};
   a.x = x; a.dy = dy; a.FK = FK; a.FC = FC; a.FH = FH; a.FW = FW;
@@ -702,9 +717,17 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
   if (variant < 0) {
     std::lock_guard<std::mutex> lk(g_tune_mu);
     auto it = g_tuned_filter.find(key_of(s));
-    if (it != g_tuned_filter.end() && (it->second == 0 || mfma_ok)) variant = it->second;
+    if (it != g_tuned_filter.end() &&
+        (it->second == 0 || (it->second == 1 && mfma_ok) || (it->second == 2 && fused_ok)))
+      variant = it->second;
   }
-  if ((variant == 1 || (variant < 0 && mfma_ok)) && tiles_ok) {
+  if (variant < 0) {
+    const bool prefer_fused =
+        fused_ok && (cp4::bwd_filter_fused_preferred(s.Rank > kFilterRankTile ? filter_rank_tile(s, 0) : s) ||
+                     !mfma_ok);
+    variant = prefer_fused ? 2 : (mfma_ok ? 1 : 0);
+  }
+  if (variant >= 1 && tiles_ok) {
     float* cf = static_cast<float*>(workspace);                 // compact factors of a tile
     float* cg = cf + filter_rank_tile_floats(s);                // compact gradients
     void* inner = cg + filter_rank_tile_floats(s);
@@ -728,13 +751,15 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
       b.dFK = g[0]; b.dFC = g[1]; b.dFH = g[2]; b.dFW = g[3];
       b.R = rt;
       b.workspace = inner;
-      CP4_HIP(cp4::bwd_filter_mfma_launch(b, st));
+      if (variant == 2) CP4_HIP(cp4::bwd_filter_fused_launch(b, st));
+      else CP4_HIP(cp4::bwd_filter_mfma_launch(b, st));
       for (int i = 0; i < 4; ++i)
         CP4_HIP(cp4::copy_columns_launch(g[i], rt, grad[i] + r0, R, rows[i], rt, st));
     }
     return CP4_OK;
   }
-  if (variant == 1 || (variant < 0 && mfma_ok)) CP4_HIP(cp4::bwd_filter_mfma_launch(a, st));
+  if (variant == 2) CP4_HIP(cp4::bwd_filter_fused_launch(a, st));
+  else if (variant == 1) CP4_HIP(cp4::bwd_filter_mfma_launch(a, st));
   else CP4_HIP(cp4::bwd_filter_launch(a, st));
   return CP4_OK;
 }
@@ -1265,7 +1290,7 @@ cp4_status cp4_tune_backward_filter(const cp4_shape* shape, const float* x, cons
   if (shape->N == 0) return fail(CP4_ERR_SHAPE, "cannot tune an empty batch");
   int best = -1;
   float best_t = 0.f;
-  for (int v = 0; v < 2; ++v) {
+  for (int v = 0; v < 3; ++v) {
     float us = 0.f;
     rc = time_loop(
         [&] {

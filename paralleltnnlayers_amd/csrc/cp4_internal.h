@@ -142,6 +142,15 @@ bool bwd_filter_mfma_supported(const cp4_shape&);
 size_t bwd_filter_mfma_workspace_bytes(const cp4_shape&);
 bool bwd_filter_mfma_taps2d_supported(const cp4_shape&);   // with BwdFilterArgs::taps2d
 hipError_t bwd_filter_mfma_launch(const BwdFilterArgs&, hipStream_t);
+// Matrix-core variant with the tap step inside the gradient GEMMs (three launches;
+// square odd filters up to 5 with 2 * pad == Y - 1, channel counts multiples of 16,
+// H * W a multiple of 4, x / dy / workspace 16-byte aligned).
+bool bwd_filter_fused_supported(const cp4_shape&);
+// Where the three-launch variant is the faster one (small and medium problems, whose
+// time is launches and first-load latencies rather than bandwidth).
+bool bwd_filter_fused_preferred(const cp4_shape&);
+size_t bwd_filter_fused_workspace_bytes(const cp4_shape&);
+hipError_t bwd_filter_fused_launch(const BwdFilterArgs&, hipStream_t);
 // A layer with a stride and zeros of its own before the image (BwdFilterArgs::H, W: the
 // input plane; pad unused; dy on the geometry's Ho x Wo grid).
 bool bwd_filter_mfma_strided_supported(const cp4_shape&, const Geometry&);

@@ -2,6 +2,7 @@
 header declares, and rejects bad arguments before touching a device."""
 import ctypes
 import os
+import random
 import re
 
 import pytest
@@ -163,3 +164,21 @@ def test_geometry_helpers_need_no_device(L):
     assert L.cp4_conv2d_forward_ex(ctypes.byref(s), None, one, one, one, one, one, None, 0, one,
                                    None) == capi.ERR_NULL_POINTER
     assert capi.backward_ex_workspace_bytes(s, capi.geometry(s, 2, "same")) > 0
+
+
+def test_backward_filter_workspace_sizes_over_random_shapes():
+    """The workspace query plans every backward-filter variant on the host: it must
+    answer (a positive size, no crash) for any valid shape, also those none of the
+    matrix-core variants takes (tiny or odd planes, channel counts off the tiles,
+    more than 64 ranks, a padding that is not "same")."""
+    from paralleltnnlayers_amd import capi
+    L = capi.lib()
+    rng = random.Random(7)
+    for _ in range(4000):
+        fs = rng.choice((1, 2, 3, 5, 7, 9))
+        s = capi.Shape(N=rng.choice((1, 2, 3, 8, 64)), H=rng.randint(1, 70), W=rng.randint(1, 70),
+                       pad=rng.choice((0, 1, 2, 3, fs // 2)), T=rng.choice((1, 3, 16, 48, 96, 320)),
+                       C=rng.choice((1, 5, 16, 32, 64, 256, 528)), Y=fs, X=fs,
+                       Rank=rng.choice((1, 2, 7, 16, 32, 33, 64, 65, 130)))
+        need = L.cp4_conv2d_backward_filter_workspace_bytes(ctypes.byref(s))
+        assert need > 0, s

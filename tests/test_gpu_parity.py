@@ -69,13 +69,15 @@ def variants_for(cp4, x_shape, f, pad):
 
 def filter_variants(cp4, x, dy, f, pad):
     """Backward-filter variants that accept this shape: -1 (library's choice),
-    0 (general) and, where it qualifies, 1 (matrix cores)."""
+    0 (general) and, where they qualify, 1 (matrix cores, four launches) and
+    2 (matrix cores, tap step fused into the gradient GEMMs)."""
     out = [-1, 0]
-    try:
-        cp4.conv2d_backward_filter(x, dy, *f, pad=pad, variant=1)
-        out.append(1)
-    except cp4.Cp4Error as e:
-        assert e.status == cp4.capi.ERR_UNSUPPORTED
+    for v in (1, 2):
+        try:
+            cp4.conv2d_backward_filter(x, dy, *f, pad=pad, variant=v)
+            out.append(v)
+        except cp4.Cp4Error as e:
+            assert e.status == cp4.capi.ERR_UNSUPPORTED
     return out
 
 
@@ -132,10 +134,11 @@ def test_workload_backward_filter(cp4, oracle, workload):
                                          variant=variant)
         for g, wnt, k in zip(got, want, FACTORS):
             assert_gradient_close(host(g), wnt, f"{w.name} d{k} variant {variant}")
-    # bit-reproducible: no floating-point atomics anywhere in the reduction
-    again = cp4.conv2d_backward_filter(dev(a["x"]), dev(a["dy"]), *f, pad=w.pad)
-    for g1, g2 in zip(got, again):
-        assert torch.equal(g1, g2)
+        # bit-reproducible: no floating-point atomics anywhere in a variant's reductions
+        again = cp4.conv2d_backward_filter(dev(a["x"]), dev(a["dy"]), *f, pad=w.pad,
+                                           variant=variant)
+        for g1, g2 in zip(got, again):
+            assert torch.equal(g1, g2), f"{w.name} variant {variant} differs between two runs"
 
 
 def test_workload_properties(cp4, workload):
