@@ -309,15 +309,17 @@ cp4_status cp4_time_backward_filter(const cp4_shape* shape, const float* x,
  * forward / backward-data pass has several kernel variants; variant -1 means
  * "library's choice" (a tuned entry for this shape if cp4_tune_forward has
  * run, else a size heuristic; the environment variable
- * CP4_FORWARD_VARIANT=<variant name> overrides the heuristic for the shapes
- * that variant supports). */
+ * CP4_FORWARD_VARIANT=<variant name>, read once at the first launch of the
+ * process, overrides the heuristic for the shapes that variant supports). */
 int cp4_forward_variant_count(void);
 const char* cp4_forward_variant_name(int variant);
 /* CP4_OK if `variant` can run `shape`, else CP4_ERR_UNSUPPORTED. */
 cp4_status cp4_forward_variant_supported(const cp4_shape* shape, int variant);
 /* The variant the library's choice falls on for `shape` (forward, or the
  * backward-data pass of that layer): the tuned entry if there is one, else the
- * heuristic; -1 if the shape is invalid or no variant takes it. */
+ * heuristic - the CP4_FORWARD_VARIANT override included, so this names what a launch
+ * would run, not what the heuristic alone would pick; -1 if the shape is invalid or
+ * no variant takes it. */
 int cp4_forward_default_variant(const cp4_shape* shape, int backward_data);
 cp4_status cp4_conv2d_forward_variant(const cp4_shape* shape, const float* x,
                                       const float* FK, const float* FC,
@@ -331,7 +333,7 @@ cp4_status cp4_conv2d_forward_variant(const cp4_shape* shape, const float* x,
  * groups per wave) - remembers the fastest for this shape for the
  * rest of the process (a process-wide table behind a mutex; cp4_tune_clear
  * empties it) and reports it.  cp4_tune_backward_data does the same for that
- * pass, cp4_tune_backward_filter chooses between that pass's two variants.
+ * pass, cp4_tune_backward_filter chooses between that pass's three variants.
  * cp4_tuned_choice reports what a shape would run with now: the variant, the
  * tuned tile (rows, columns; 0 = the kernel's own planner) and the consumers'
  * schedule (1 = the kernel's rule, 0 = no role split, 2 = whole groups per wave). */
@@ -365,6 +367,13 @@ cp4_status cp4_set_tuned_choice(const cp4_shape* shape, int backward_data, int v
 int cp4_tuned_count(void);
 cp4_status cp4_tuned_entry(int index, cp4_shape* shape, int* backward_data, int* variant,
                            int* tile_rows, int* tile_cols, int* schedule);
+/* The backward-filter tuner's table (cp4_tune_backward_filter): enumeration, entry by
+ * hand and the names of that pass's variants (NULL past the last), so that a table can
+ * be carried from one process to the next like the forward one. */
+const char* cp4_backward_filter_variant_name(int variant);
+int cp4_tuned_filter_count(void);
+cp4_status cp4_tuned_filter_entry(int index, cp4_shape* shape, int* variant);
+cp4_status cp4_set_tuned_filter_choice(const cp4_shape* shape, int variant);
 void cp4_tune_clear(void);
 
 /* ---- device allocator / copy helpers (the reference's Tensor uses

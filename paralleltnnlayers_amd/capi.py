@@ -139,6 +139,11 @@ def lib():
     L.cp4_tuned_count.restype = ctypes.c_int
     L.cp4_tuned_entry.argtypes = [ctypes.c_int, _S] + [ctypes.POINTER(ctypes.c_int)] * 5
     L.cp4_tune_clear.restype = None
+    L.cp4_backward_filter_variant_name.restype = ctypes.c_char_p
+    L.cp4_backward_filter_variant_name.argtypes = [ctypes.c_int]
+    L.cp4_tuned_filter_count.restype = ctypes.c_int
+    L.cp4_tuned_filter_entry.argtypes = [ctypes.c_int, _S, ctypes.POINTER(ctypes.c_int)]
+    L.cp4_set_tuned_filter_choice.argtypes = [_S, ctypes.c_int]
     L.cp4_device_status.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
     L.cp4_set_spin_limit.argtypes = [ctypes.c_int]
     L.cp4_set_spin_limit.restype = None
@@ -575,7 +580,8 @@ def tune_backward_data(dy, FK, FC, FH, FW, dx, pad, warmup=1, profcount=10, stre
 
 def tune_backward_filter(x, dy, FK, FC, FH, FW, pad, warmup=1, profcount=10, workspace=None,
                          stream=None):
-    """(best variant: 0 general / 1 matrix-core, its mean us)."""
+    """(best variant: 0 general / 1 matrix cores in four launches / 2 with the tap step
+    inside the gradient GEMMs, its mean us)."""
     s = shape_for(x.shape, FK, FC, FH, FW, pad)
     outs = [torch.empty_like(f) for f in (FK, FC, FH, FW)]
     ws, ws_bytes = _workspace(s, x.device, workspace)
@@ -618,12 +624,39 @@ def tuned_table():
     return out
 
 
+def backward_filter_variants():
+    """Names of the backward-filter variants, by number."""
+    L = lib()
+    out = []
+    while L.cp4_backward_filter_variant_name(len(out)) is not None:
+        out.append(L.cp4_backward_filter_variant_name(len(out)).decode())
+    return out
+
+
+def tuned_filter_table():
+    """The backward-filter tuner table as a list of dicts (shape fields, variant name)."""
+    L = lib()
+    names = backward_filter_variants()
+    out = []
+    for i in range(L.cp4_tuned_filter_count()):
+        s, v = Shape(), ctypes.c_int()
+        check(L.cp4_tuned_filter_entry(i, ctypes.byref(s), ctypes.byref(v)))
+        out.append({"N": s.N, "H": s.H, "W": s.W, "pad": s.pad, "T": s.T, "C": s.C, "Y": s.Y,
+                    "X": s.X, "Rank": s.Rank, "pass": "backward_filter",
+                    "variant": names[v.value]})
+    return out
+
+
+def set_tuned_filter_choice(s, variant):
+    check(lib().cp4_set_tuned_filter_choice(ctypes.byref(s), int(variant)))
+
+
 def save_tuned(path):
-    """Writes the tuner table as JSON (variants by name, so that the file survives a
-    rebuild of the library)."""
+    """Writes the tuner tables of all three passes as JSON (variants by name, so that
+    the file survives a rebuild of the library)."""
     import json
     with open(path, "w") as f:
-        json.dump(tuned_table(), f, indent=1)
+        json.dump(tuned_table() + tuned_filter_table(), f, indent=1)
 
 
 def load_tuned(path):
@@ -631,9 +664,17 @@ def load_tuned(path):
     skipped.  Returns the number entered."""
     import json
     numbers = {n: v for v, n, _ in forward_variants()}
+    filter_numbers = {n: v for v, n in enumerate(backward_filter_variants())}
     done = 0
-    for e in json.load(open(path)):
+    with open(path) as f:
+        entries = json.load(f)
+    for e in entries:
         s = Shape(e["N"], e["H"], e["W"], e["pad"], e["T"], e["C"], e["Y"], e["X"], e["Rank"])
+        if e.get("pass") == "backward_filter":
+            if e["variant"] in filter_numbers:
+                set_tuned_filter_choice(s, filter_numbers[e["variant"]])
+                done += 1
+            continue
         if e["variant"] not in numbers:
             continue
         try:

@@ -1,18 +1,26 @@
-// Backward-filter on the fp32 matrix cores (ranks up to 64, even H*W, even
-// channel counts).  Same reassociation of the reference's 8-deep sums
+// Backward-filter on the matrix cores in four launches (ranks up to 64 per pass,
+// even channel counts).  Same reassociation of the reference's 8-deep sums
 // (Cuda_kernels/cp4Conv2dBackwardFilter.cu:64-257) as the general path:
 //   A = FC^T x,  B = FH *v A,  Cc = FW *h B,  G3 = FK^T dy,  G2, G1 = adjoint taps
 //   dFK = dy . Cc^T   dFC = x . G1^T   dFW[j] = <G3, shift_j B>   dFH[i] = <G2, shift_i A>
-// in four launches:
-//   1. contract: both channel->rank contractions, one wave per (image, 64-pixel
-//      block, 32-rank tile), x / dy streamed as float2 straight into the MFMA B
-//      operand, the factor from an LDS copy;
-//   2. taps: B, Cc, G2, G1 elementwise from A and G3 (L2-resident);
-//   3. gradient GEMMs: dF[d,r] = sum_{n,p} act[n,d,p] Z[n,r,p], split over
-//      images (and pixel ranges) across workgroups, 32 channel rows per wave,
-//      operands staged through LDS so that global reads stay row-contiguous;
-//      plus the small tap gradients;
-//   4. fixed-order sum of the per-workgroup partials (bit-reproducible).
+//   1. contract_split_kernel: both channel -> rank contractions as exact fp32
+//      products on the bf16 matrix cores (three-way split of both operands, six
+//      MFMAs per 16-channel chunk); a wave owns one (image, 32-pixel block, 32-rank
+//      tile) and streams x / dy through a register ring, the factor tile sits
+//      pre-split in LDS.  contract_mfma_kernel (plain fp32 MFMA) takes the channel
+//      counts that are not multiples of 16.
+//   2. taps: B, Cc, G2, G1 and the tap-gradient partials, one wave per (image, rank)
+//      plane - taps_wave_kernel (planes up to 256 pixels, wave-private LDS) or
+//      taps_column_kernel (lane = column, rows in registers); B and G2 never leave
+//      the compute unit.  taps_plane_kernel / taps_kernel for the other filter shapes.
+//   3. grad_split_kernel: dF[d,r] = sum_{n,p} act[n,d,p] Z[n,r,p] as split products,
+//      split over images (and pixel ranges) across workgroups, the Z tile split once
+//      per 32-pixel chunk into double-buffered B fragments in LDS.  grad_gemm_kernel
+//      (fp32 MFMA) where rows cannot move as 16-byte vectors.
+//   4. reduce4_kernel: fixed-order sum of the per-workgroup partials (bit-reproducible).
+// The library's choice for large problems and for shapes the three-launch variant
+// (bwd_filter_fused.hip) does not take; also the strided layer's pass and the
+// 3-factor op's (depthwise-filter tap step).
 #include <cstdint>
 #include <cstdlib>
 

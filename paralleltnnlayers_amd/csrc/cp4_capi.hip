@@ -50,8 +50,7 @@ cp4_status hip_fail(hipError_t e, const char* where) {
 
 hipStream_t as_stream(cp4_stream s) { return static_cast<hipStream_t>(s); }
 
-// Address of this device's fault record (null if the runtime cannot say; the
-// kernels then run without one).
+// Address of this device's fault record (null if the runtime cannot say).
 int* fault_of_current_device() {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
@@ -88,11 +87,20 @@ cp4_status scratch_of_current_device(void** out) {
   return CP4_OK;
 }
 
-// The launch context every producer / consumer launch carries.
-void arm(FwdArgs& a) {
+// The launch context every producer / consumer launch carries.  A launch without a
+// fault record could give up a wait unseen, so an unresolved record is an error.
+cp4_status arm(FwdArgs& a) {
   a.fault = fault_of_current_device();
+  if (!a.fault)
+    return fail(CP4_ERR_HIP, "the device's fault record could not be resolved (hipGetSymbolAddress)");
   a.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
+  return CP4_OK;
 }
+#define CP4_ARM(a)                     \
+  do {                                 \
+    const cp4_status rc_ = arm(a);     \
+    if (rc_ != CP4_OK) return rc_;     \
+  } while (0)
 
 // Synchronise `st`, read and clear the device's fault record.
 cp4_status device_status(hipStream_t st, int* detail) {
@@ -291,13 +299,20 @@ bool strips_on_wide_plane(const FwdArgs& a) {
 // elements the fp32 matrix-core strip kernel is the faster one for ranks 33-64.
 constexpr long kTwoPassMinElements = 16l << 20;
 
+// CP4_FORWARD_VARIANT=<name> overrides the heuristic where that variant can run the
+// shape (profiling and A/B runs of unmodified callers).  Read once, at the first launch:
+// the process's environment is not consulted per call.
+int forced_variant() {
+  static const int forced = [] {
+    const char* want = getenv("CP4_FORWARD_VARIANT");
+    return want ? variant_named(want) : -1;
+  }();
+  return forced;
+}
+
 int heuristic_variant(const FwdArgs& a) {
-  // CP4_FORWARD_VARIANT=<name> overrides the heuristic where that variant can
-  // run the shape (profiling and A/B runs of unmodified callers).
-  if (const char* want = getenv("CP4_FORWARD_VARIANT")) {
-    const int v = variant_named(want);
-    if (v >= 0 && kVariants[v].supported(a)) return v;
-  }
+  const int forced = forced_variant();
+  if (forced >= 0 && kVariants[forced].supported(a)) return forced;
   int pick = -1;
   for (int v = kNumVariants - 1; v >= 0 && pick < 0; --v)
     if (kVariants[v].supported(a) && !is_variant(v, "dense_small_valu")) pick = v;
@@ -349,7 +364,7 @@ cp4_status run_choice(const FwdArgs& a0, const Choice& c, hipStream_t st) {
   FwdArgs a = with_tile(a0, c);
   if (!kVariants[c.variant].supported(a))
     return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape");
-  arm(a);
+  CP4_ARM(a);
   CP4_HIP(kVariants[c.variant].launch(a, st));
   return CP4_OK;
 }
@@ -525,7 +540,7 @@ cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
   if (is_variant(c.variant, "mfma_bf16x3_pipe")) {
     FwdArgs e = with_tile(a, c);
     if (cp4::fwd_pipe_epi_supported(e)) {
-      arm(e);
+      CP4_ARM(e);
       CP4_HIP(cp4::fwd_pipe_epi_launch(e, st));
       return CP4_OK;
     }
@@ -534,7 +549,7 @@ cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
     // (the tiled build's epilogue sibling)
     FwdArgs e = with_tile(a, c);
     if (cp4::fwd_pipe_tiled_epi_supported(e)) {
-      arm(e);
+      CP4_ARM(e);
       CP4_HIP(cp4::fwd_pipe_tiled_epi_launch(e, st));
       return CP4_OK;
     }
@@ -593,7 +608,7 @@ cp4_status cp4_conv2d_forward_bf16(const cp4_shape* shape, const void* x_bf16,
                            static_cast<float*>(y_bf16));
   a.bias = bias;
   a.act = activation;
-  arm(a);
+  CP4_ARM(a);
   if (!cp4::fwd_pipe_io16_supported(a))
     return fail(CP4_ERR_UNSUPPORTED, "bfloat16 I/O: shape not taken by the producer/consumer kernel");
   CP4_HIP(cp4::fwd_pipe_io16_launch(a, as_stream(stream)));
@@ -611,7 +626,7 @@ cp4_status cp4_conv2d_backward_data_bf16(const cp4_shape* shape, const void* dy_
   if (rc != CP4_OK) return rc;
   FwdArgs a = backward_data_args(*shape, static_cast<const float*>(dy_bf16), FK, FC, FH, FW,
                                  static_cast<float*>(dx_bf16));
-  arm(a);
+  CP4_ARM(a);
   if (!cp4::fwd_pipe_io16_supported(a))
     return fail(CP4_ERR_UNSUPPORTED, "bfloat16 I/O: shape not taken by the producer/consumer kernel");
   CP4_HIP(cp4::fwd_pipe_io16_launch(a, as_stream(stream)));
@@ -635,7 +650,7 @@ cp4_status cp4_conv2d_forward_f16(const cp4_shape* shape, const void* x_f16,
                            static_cast<float*>(y_f16));
   a.bias = bias;
   a.act = activation;
-  arm(a);
+  CP4_ARM(a);
   if (!cp4::fwd_pipe_iof16_supported(a))
     return fail(CP4_ERR_UNSUPPORTED, "half-precision I/O: shape not taken by the producer/consumer kernel");
   CP4_HIP(cp4::fwd_pipe_iof16_launch(a, as_stream(stream)));
@@ -653,7 +668,7 @@ cp4_status cp4_conv2d_backward_data_f16(const cp4_shape* shape, const void* dy_f
   if (rc != CP4_OK) return rc;
   FwdArgs a = backward_data_args(*shape, static_cast<const float*>(dy_f16), FK, FC, FH, FW,
                                  static_cast<float*>(dx_f16));
-  arm(a);
+  CP4_ARM(a);
   if (!cp4::fwd_pipe_iof16_supported(a))
     return fail(CP4_ERR_UNSUPPORTED, "half-precision I/O: shape not taken by the producer/consumer kernel");
   CP4_HIP(cp4::fwd_pipe_iof16_launch(a, as_stream(stream)));
@@ -893,16 +908,24 @@ void set_geometry(FwdArgs& a, const cp4_geometry& g) {
 cp4_status run_geometry(FwdArgs a, hipStream_t st, bool* epilogue_done = nullptr) {
   if (epilogue_done) *epilogue_done = false;
   if (a.N == 0) return CP4_OK;
-  arm(a);
+  CP4_ARM(a);
   if (cp4::fwd_pipe_strided_supported(a) && a.Cin + a.Cout >= kMatrixMinChannels) {
     CP4_HIP(cp4::fwd_pipe_strided_launch(a, st));
     if (epilogue_done) *epilogue_done = true;
     return CP4_OK;
   }
-  if (!cp4::fwd_general_supported(a))
-    return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape and geometry");
-  CP4_HIP(cp4::fwd_general_launch(a, st));
-  return CP4_OK;
+  if (cp4::fwd_general_supported(a)) {
+    CP4_HIP(cp4::fwd_general_launch(a, st));
+    return CP4_OK;
+  }
+  // few channels on a geometry whose rows do not fit the general kernel's LDS tile:
+  // the matrix-core build takes it after all, below the channel count it pays from
+  if (cp4::fwd_pipe_strided_supported(a)) {
+    CP4_HIP(cp4::fwd_pipe_strided_launch(a, st));
+    if (epilogue_done) *epilogue_done = true;
+    return CP4_OK;
+  }
+  return fail(CP4_ERR_UNSUPPORTED, "no kernel variant supports this shape and geometry");
 }
 // Stride-1 canvas that carries the strided layer (backward-filter): pad P on every
 // side, x set in at (ot, ol), dy spread out with zeros from the origin.  The
@@ -959,6 +982,11 @@ cp4_status cp4_geometry_symmetric(const cp4_shape* s, unsigned sh, unsigned sw, 
   if (!sh || !sw) return fail(CP4_ERR_SHAPE, "strides must be >= 1");
   if (s->H + 2 * ph < s->Y || s->W + 2 * pw < s->X)
     return fail(CP4_ERR_SHAPE, "the filter is larger than the padded image");
+  // the layer entry points take at most Y - 1 / X - 1 zeros before the image (a window
+  // that lies wholly in the padding would produce outputs of zero): say so here, not
+  // at the first launch
+  if (ph > s->Y - 1 || pw > s->X - 1)
+    return fail(CP4_ERR_SHAPE, "padding must be <= Y - 1 rows and <= X - 1 columns");
   *g = cp4_geometry{sh, sw, ph, pw, (s->H + 2 * ph - s->Y) / sh + 1, (s->W + 2 * pw - s->X) / sw + 1};
   return CP4_OK;
 }
@@ -1040,7 +1068,7 @@ cp4_status cp4_conv2d_backward_data_ex(const cp4_shape* shape, const cp4_geometr
     t.pt = (int)g->pad_top; t.pl = (int)g->pad_left;
     t.Ho = (int)s.H; t.Wo = (int)s.W;
     if (cp4::fwd_pipe_strided_supported(t) && t.Cin + t.Cout >= kMatrixMinChannels) {
-      arm(t);
+      CP4_ARM(t);
       CP4_HIP(cp4::fwd_pipe_strided_launch(t, st));
       return CP4_OK;
     }
@@ -1386,6 +1414,48 @@ cp4_status cp4_tuned_entry(int index, cp4_shape* shape, int* backward_data, int*
   return CP4_OK;
 }
 
+const char* cp4_backward_filter_variant_name(int variant) {
+  static const char* const names[3] = {"general_valu", "mfma_four_launches", "mfma_fused_taps"};
+  return variant >= 0 && variant < 3 ? names[variant] : nullptr;
+}
+
+int cp4_tuned_filter_count(void) {
+  std::lock_guard<std::mutex> lk(g_tune_mu);
+  return (int)g_tuned_filter.size();
+}
+
+cp4_status cp4_tuned_filter_entry(int index, cp4_shape* shape, int* variant) {
+  if (!shape) return fail(CP4_ERR_NULL_POINTER, "shape is NULL");
+  std::lock_guard<std::mutex> lk(g_tune_mu);
+  if (index < 0 || index >= (int)g_tuned_filter.size())
+    return fail(CP4_ERR_SHAPE, "index out of range");
+  auto it = g_tuned_filter.begin();
+  std::advance(it, index);
+  const TuneKey& k = it->first;                    // N, C, T, H, W, pad, Y, X, Rank, 2
+  shape->N = (unsigned)std::get<0>(k);
+  shape->C = (unsigned)std::get<1>(k);
+  shape->T = (unsigned)std::get<2>(k);
+  shape->H = (unsigned)std::get<3>(k);
+  shape->W = (unsigned)std::get<4>(k);
+  shape->pad = (unsigned)std::get<5>(k);
+  shape->Y = (unsigned)std::get<6>(k);
+  shape->X = (unsigned)std::get<7>(k);
+  shape->Rank = (unsigned)std::get<8>(k);
+  if (variant) *variant = it->second;
+  return CP4_OK;
+}
+
+cp4_status cp4_set_tuned_filter_choice(const cp4_shape* shape, int variant) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (variant < 0 || variant > 2)
+    return fail(CP4_ERR_UNSUPPORTED, "backward-filter variants are numbered 0, 1 and 2");
+  // (a choice the shape or the caller's alignment does not allow is ignored at launch)
+  std::lock_guard<std::mutex> lk(g_tune_mu);
+  g_tuned_filter[key_of(*shape)] = variant;
+  return CP4_OK;
+}
+
 void cp4_tune_clear(void) {
   std::lock_guard<std::mutex> lk(g_tune_mu);
   g_tuned.clear();
@@ -1552,7 +1622,7 @@ cp4_status cp3_run(const cp4_shape* shape, const float* in, const float* K0, con
   FwdArgs a = backward ? backward_data_args(*shape, in, FK, K0, nullptr, nullptr, out)
                        : forward_args(*shape, in, FK, K0, nullptr, nullptr, out);
   a.taps2d = K1;
-  arm(a);
+  CP4_ARM(a);
   const size_t pixels = (size_t)a.N * a.H * a.W;
   if (cp4::fwd_pipe_taps2d_supported(a) && a.W <= 128 && a.Cin + a.Cout >= 24 &&
       !(a.Cin > 256 && pixels > 8192)) {

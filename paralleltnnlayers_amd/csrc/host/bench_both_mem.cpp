@@ -24,7 +24,10 @@ int main(int argc, char** argv) {
   }
   std::ostream results(buf);
   results << std::showpoint << std::setw(5);
-  results << "N C H W pad T Y X, dense, Rank 1, Rank 2, Rank 4, Rank 8, Rank 16" << std::endl;
+  // the reference's header, column names included (BenchBothTime.cu:49, BenchBothMem.cu:49):
+  // scripts keyed on it read both files; the "cuDNN" column is the vendor library's dense
+  // convolution, MIOpen here
+  results << "N C H W pad T Y X, cuDNN, Rank 1, Rank 2, Rank 4, Rank 8, Rank 16" << std::endl;
   std::vector<tensor_shape> shapes;
   if (!read_shapes(argv[1], &shapes)) return 1;
   if (cp4_set_device(device) != CP4_OK) {

@@ -107,5 +107,7 @@ void Tensor::upload() const {
 void Tensor::download() {
   if (!size()) return;
   check(cp4_memcpy_d2h(m_data, device(), size() * sizeof(float), nullptr), "download");
-  check(cp4_stream_synchronize(nullptr), "download sync");
+  // synchronises, and reports a kernel that gave up a wait between its waves: what
+  // was copied is incomplete then
+  check(cp4_device_status(nullptr, nullptr), "download");
 }

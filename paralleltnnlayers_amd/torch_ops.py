@@ -13,10 +13,40 @@ run as they are; that is the only case in which its backward-data formula
 (flipped taps at offset +y-pad, Cuda_kernels/cp4Conv2dBackwardData.cu:79-87) is
 the adjoint of its forward.  Strides and every other padding go through the
 library's geometry entry points (cp4_conv2d_forward_ex and its exact gradients).
+
+Launches are asynchronous.  A producer / consumer kernel whose wait between waves
+runs out ends early and leaves its output incomplete; the library records that per
+device and reports it from ``cp4_device_status``, which synchronises the stream.
+``check_device()`` is that call: use it wherever the training loop synchronises
+anyway (reading the loss, a checkpoint).  ``set_device_checks(True)`` - or the
+environment variable ``CP4_CHECK_DEVICE=1`` - makes every backward pass of the
+Functions below end with it, at the price of one synchronisation per layer and step.
 """
+import os
+
 import torch
 
 from . import capi
+
+_check_every_backward = os.environ.get("CP4_CHECK_DEVICE", "0") not in ("", "0")
+
+
+def set_device_checks(on):
+    """Check the device's fault record at the end of every backward pass (synchronises)."""
+    global _check_every_backward
+    _check_every_backward = bool(on)
+
+
+def check_device(stream=None):
+    """Synchronises ``stream`` and raises ``capi.Cp4Error`` (ERR_DEVICE) if a kernel of
+    the library gave up a wait since the last check: outputs computed since then are
+    incomplete.  The record is cleared."""
+    capi.device_status(stream)
+
+
+def _after_backward():
+    if _check_every_backward:
+        capi.device_status()
 
 
 class CP4Conv2dFunction(torch.autograd.Function):
@@ -87,6 +117,7 @@ class CP4Conv2dFunction(torch.autograd.Function):
                                                     pad=ctx.pad)
                 grads = tuple(g if need else None
                               for g, need in zip(grads, ctx.needs_input_grad[1:5]))
+            _after_backward()
             return (dx,) + grads + (None, dbias, None)
         if ctx.needs_input_grad[0]:
             if dy16 and capi.bf16_supported(s, backward_data=True):
@@ -104,6 +135,7 @@ class CP4Conv2dFunction(torch.autograd.Function):
                                                     pad=ctx.pad)
             grads = tuple(g if need else None
                           for g, need in zip(grads, ctx.needs_input_grad[1:5]))
+        _after_backward()
         return (dx,) + grads + (None, dbias, None)
 
 
@@ -137,6 +169,7 @@ class CP4Conv2dGeometryFunction(torch.autograd.Function):
             grads = capi.conv2d_backward_filter_ex(x, dy, FK, FC, FH, FW, ctx.geom)
             grads = tuple(g if need else None
                           for g, need in zip(grads, ctx.needs_input_grad[1:5]))
+        _after_backward()
         return (dx,) + grads + (None, dbias, None)
 
 
@@ -194,6 +227,11 @@ class CP4Conv2d(torch.nn.Module):
         return cp4_conv2d(x, self.FK, self.FC, self.FH, self.FW, self.pad, self.bias,
                           self.activation, self.stride, self.padding)
 
+    @staticmethod
+    def check_device(stream=None):
+        """See ``check_device``: call where the loop synchronises anyway."""
+        check_device(stream)
+
     def dense_filter(self):
         """The recomposed [T,C,Y,X] filter (on the device, through cp4_recompose)."""
         return capi.recompose(self.FK.detach(), self.FC.detach(), self.FH.detach(),
@@ -232,6 +270,7 @@ class CP3Conv2dFunction(torch.autograd.Function):
         if any(ctx.needs_input_grad[1:4]):
             grads = capi.cp3_conv2d_backward_filter(x, dy, K0, K1, K2, pad=ctx.pad)
             grads = tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad[1:4]))
+        _after_backward()
         return (dx,) + grads + (None,)
 
 
@@ -294,6 +333,7 @@ class RCPConv2dFunction(torch.autograd.Function):
         if any(ctx.needs_input_grad[1:4]):
             grads = capi.rcp_conv2d_backward_filter(x, dy, K0, K1, KC, pad=ctx.pad)
             grads = tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad[1:4]))
+        _after_backward()
         return (dx,) + grads + (None,)
 
 

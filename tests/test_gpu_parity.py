@@ -444,14 +444,21 @@ def test_tuner_table_round_trip(cp4, tmp_path):
         cp4.tune_clear()
         cp4.set_tuned_choice(s, names.index("mfma_bf16x3_pipe"), 2, 0, 0)
         cp4.set_tuned_choice(s, names.index("general_valu"), 0, 0, 1, backward_data=True)
+        # the backward-filter tuner's own table travels in the same file
+        best, _ = cp4.tune_backward_filter(x, dev(a["dy"]), *f, w.pad, warmup=1, profcount=3)
+        fnames = cp4.backward_filter_variants()
+        assert fnames == ["general_valu", "mfma_four_launches", "mfma_fused_taps"]
+        ftable = cp4.tuned_filter_table()
+        assert len(ftable) == 1 and ftable[0]["variant"] == fnames[best]
         table = cp4.tuned_table()
         assert len(table) == 2 and {e["variant"] for e in table} == {"mfma_bf16x3_pipe", "general_valu"}
         path = str(tmp_path / "tuned.json")
         cp4.save_tuned(path)
         cp4.tune_clear()
-        assert cp4.tuned_table() == []
-        assert cp4.load_tuned(path) == 2
+        assert cp4.tuned_table() == [] and cp4.tuned_filter_table() == []
+        assert cp4.load_tuned(path) == 3
         assert cp4.tuned_table() == table
+        assert cp4.tuned_filter_table() == ftable
         assert cp4.tuned_choice(s) == {"variant": names.index("mfma_bf16x3_pipe"), "tile_rows": 2,
                                        "tile_cols": 0, "role_split": 0}
         assert cp4.tuned_choice(s, backward_data=True)["variant"] == names.index("general_valu")

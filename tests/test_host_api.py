@@ -68,7 +68,7 @@ def test_bench_driver_csv(tmp_path):
                        text=True, timeout=100)
     assert r.returncode == 0, r.stderr
     lines = r.stdout.strip().splitlines()
-    assert lines[0] == "N C H W pad T Y X, dense, Rank 1, Rank 2, Rank 4, Rank 8, Rank 16"
+    assert lines[0] == "N C H W pad T Y X, cuDNN, Rank 1, Rank 2, Rank 4, Rank 8, Rank 16"
     assert len(lines) == 3 and lines[1].startswith("1 192 13 13 1 256 3 3, ")
     assert float(lines[1].split(",")[1]) > 0          # the vendor library's dense time
     assert all(float(v) > 0 for v in lines[2].split(", ")[2:])

@@ -61,6 +61,34 @@ def test_noalloc_backward_filter_matches_workspace_entry_twice(cp4, oracle):
                 assert err <= 1e-3, f"{w.name} d{k}: {err:.2e} against the oracle"
 
 
+def test_noalloc_leaves_device_memory_untouched(cp4, oracle):
+    """The property that names the entry point: after a first call (which loads the
+    code object and looks the scratch array up) a call allocates and frees nothing -
+    neither through the runtime (free device memory unchanged) nor through torch's
+    caching allocator.  Checked on a shape of each route: general kernels, matrix
+    cores, and more than 64 ranks (rank tiles on compact factor copies in the scratch)."""
+    shapes = [Workload("general", "backward_filter", 3, 20, 9, 11, 1, 12, 3, 3, 5, "uniform"),
+              Workload("matrix", "backward_filter", 8, 64, 14, 14, 1, 32, 3, 3, 16, "uniform"),
+              Workload("tiles", "backward_filter", 4, 32, 12, 12, 1, 48, 3, 3, 80, "uniform")]
+    for w in shapes:
+        a = make_inputs(w, seed=4)
+        f = [dev(a[k]) for k in FACTORS]
+        x, dy = dev(a["x"]), dev(a["dy"])
+        outs = [torch.empty_like(t) for t in f]
+        cp4.conv2d_backward_filter_noalloc(x, dy, *f, outs, pad=w.pad)      # warm-up
+        torch.cuda.synchronize()
+        free0, torch0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
+        reserved0 = torch.cuda.memory_reserved()
+        cp4.conv2d_backward_filter_noalloc(x, dy, *f, outs, pad=w.pad)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free0, f"{w.name}: device memory changed"
+        assert torch.cuda.memory_allocated() == torch0 and torch.cuda.memory_reserved() == reserved0
+        ref = oracle.backward_filter(a["x"], a["dy"], a["FK"], a["FC"], a["FH"], a["FW"], w.pad)
+        for g, r, k in zip(outs, ref, FACTORS):
+            err = np.abs(g.cpu().numpy() - r).max() / np.abs(r).max()
+            assert err <= 1e-3, f"{w.name} d{k}: {err:.2e} against the oracle"
+
+
 def test_noalloc_rejects_shapes_beyond_its_scratch(cp4):
     L = cp4.lib()
     s = cp4.capi.Shape(N=32, H=56, W=56, pad=1, T=256, C=256, Y=3, X=3, Rank=32)
