@@ -125,8 +125,7 @@ cp4_status cp4_conv2d_backward_data_bf16(const cp4_shape* shape, const void* dy_
  * half is exactly two bfloat16 parts, so the products with the fp32 factors are
  * still exact; y / dx are rounded once, to nearest-even (values beyond 65504
  * become infinities, as in any fp16 store).  Same shape limits as the bfloat16
- * entry points (cp4_bf16_supported answers for both).  There is no fp16
- * backward-filter entry: widen x and dy and use the fp32 one. */
+ * entry points (cp4_bf16_supported answers for both). */
 cp4_status cp4_conv2d_forward_f16(const cp4_shape* shape, const void* x_f16,
                                   const float* FK, const float* FC,
                                   const float* FH, const float* FW,
@@ -136,10 +135,12 @@ cp4_status cp4_conv2d_backward_data_f16(const cp4_shape* shape, const void* dy_f
                                         const float* FK, const float* FC,
                                         const float* FH, const float* FW,
                                         void* dx_f16, cp4_stream stream);
-/* Backward-filter with bfloat16 x and dy in memory; factors, gradients, the
- * workspace (cp4_conv2d_backward_filter_workspace_bytes) and all arithmetic stay
- * fp32.  Matrix-core path only: Rank <= 64, C and T multiples of 16
- * (cp4_bf16_backward_filter_supported); CP4_ERR_UNSUPPORTED otherwise. */
+/* Backward-filter with bfloat16 (_bf16) or IEEE half (_f16) x and dy in memory;
+ * factors, gradients, the workspace (cp4_conv2d_backward_filter_workspace_bytes)
+ * and all arithmetic stay fp32: a bfloat16 value is one bf16 part, a half value two,
+ * so the products are exact as in the fp32 pass.  Matrix-core path only: Rank <= 64,
+ * C and T multiples of 16 (cp4_bf16_backward_filter_supported answers for both);
+ * CP4_ERR_UNSUPPORTED otherwise. */
 int cp4_bf16_backward_filter_supported(const cp4_shape* shape);
 cp4_status cp4_conv2d_backward_filter_bf16(const cp4_shape* shape, const void* x_bf16,
                                            const void* dy_bf16, const float* FK,
@@ -147,6 +148,12 @@ cp4_status cp4_conv2d_backward_filter_bf16(const cp4_shape* shape, const void* x
                                            const float* FW, float* dFK, float* dFC,
                                            float* dFH, float* dFW, void* workspace,
                                            size_t workspace_bytes, cp4_stream stream);
+cp4_status cp4_conv2d_backward_filter_f16(const cp4_shape* shape, const void* x_f16,
+                                          const void* dy_f16, const float* FK,
+                                          const float* FC, const float* FH,
+                                          const float* FW, float* dFK, float* dFC,
+                                          float* dFH, float* dFW, void* workspace,
+                                          size_t workspace_bytes, cp4_stream stream);
 
 /* Replaces cp4_conv2d_backward_data_gpu
  * (Cuda_kernels/cp4Conv2dBackwardData.cuh:7-14, .cu:112-282):

@@ -9,7 +9,7 @@ layer under ``csrc/host``.  There is no CPU or PyTorch fallback: importing
 from .capi import (Shape, Geometry, geometry, conv2d_forward_ex, conv2d_backward_data_ex,
                    conv2d_backward_filter_ex, backward_ex_workspace_bytes, Cp4Error, lib, library_path, conv2d_forward, conv2d_forward_bias_act, conv2d_forward_bf16,
                    conv2d_backward_data_bf16, conv2d_backward_filter_bf16, bf16_supported,
-                   conv2d_forward_f16, conv2d_backward_data_f16, rcp_conv2d_forward,
+                   conv2d_forward_f16, conv2d_backward_data_f16, conv2d_backward_filter_f16, rcp_conv2d_forward,
                    rcp_conv2d_backward_data, rcp_conv2d_backward_filter,
                    conv2d_backward_data, conv2d_backward_filter, conv2d_backward_filter_noalloc,
                    conv2d_backward_filter_full, backward_filter_workspace_bytes,

@@ -113,6 +113,7 @@ def lib():
     L.cp4_conv2d_backward_filter_bf16.argtypes = (
         [_S, ctypes.c_void_p, ctypes.c_void_p] + [_F] * 8 +
         [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p])
+    L.cp4_conv2d_backward_filter_f16.argtypes = L.cp4_conv2d_backward_filter_bf16.argtypes
     bwf = [_S] + [_F] * 10 + [ctypes.c_void_p, ctypes.c_size_t]
     L.cp4_conv2d_backward_filter.argtypes = bwf + [ctypes.c_void_p]
     L.cp4_conv2d_backward_filter_variant.argtypes = bwf + [ctypes.c_int, ctypes.c_void_p]
@@ -432,6 +433,19 @@ def conv2d_backward_filter_bf16(x, dy, FK, FC, FH, FW, pad=1, workspace=None, st
     check(lib().cp4_conv2d_backward_filter_bf16(
         ctypes.byref(s), _ptr16(x), _ptr16(dy), _ptr(FK), _ptr(FC), _ptr(FH), _ptr(FW),
         *[_ptr(o) for o in outs], ctypes.c_void_p(ws.data_ptr()), ws_bytes, _stream(stream)))
+    return tuple(outs)
+
+
+def conv2d_backward_filter_f16(x, dy, FK, FC, FH, FW, pad=1, workspace=None, stream=None):
+    """float16 x, dy -> fp32 (dFK, dFC, dFH, dFW); fp32 factors and arithmetic."""
+    s = shape_for(x.shape, FK, FC, FH, FW, pad)
+    assert tuple(dy.shape) == (s.N, s.T, s.H, s.W) and x.shape[1] == s.C
+    outs = [torch.empty_like(f) for f in (FK, FC, FH, FW)]
+    ws, ws_bytes = _workspace(s, x.device, workspace)
+    check(lib().cp4_conv2d_backward_filter_f16(
+        ctypes.byref(s), _ptr16(x, torch.float16), _ptr16(dy, torch.float16), _ptr(FK), _ptr(FC),
+        _ptr(FH), _ptr(FW), *[_ptr(o) for o in outs], ctypes.c_void_p(ws.data_ptr()), ws_bytes,
+        _stream(stream)))
     return tuple(outs)
 
 

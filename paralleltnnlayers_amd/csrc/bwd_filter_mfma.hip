@@ -30,13 +30,19 @@
 #endif
 #include "split_bf16.h"
 
-// Compiled a second time with CP4_BWF_IO16: x and dy are then bfloat16 in memory
-// (factors, intermediates and gradients stay fp32).  Only the split-bf16 kernels
-// exist in that build (contract_split_kernel, grad_split_kernel): a bf16
-// activation is its own high part, so neither splits its activations and both
-// run three MFMAs per product instead of six; the entry points are exported as
-// bwd_filter_mfma_io16_*.
-#ifdef CP4_BWF_IO16
+// Compiled twice more with CP4_BWF_IO16: x and dy are then 16-bit in memory (factors,
+// intermediates and gradients stay fp32).  Only the split-bf16 kernels exist in
+// those builds (contract_split_kernel, grad_split_kernel).  CP4_BWF_IO16 == 1,
+// bfloat16: an activation is its own high part, so neither kernel splits its
+// activations and both run three MFMAs per product instead of six; entry points
+// bwd_filter_mfma_io16_*.  CP4_BWF_IO16 == 2, IEEE half: 11 significand bits are two
+// bf16 parts (8 + 3), five MFMAs per product; entry points bwd_filter_mfma_iof16_*.
+#if defined(CP4_BWF_IO16) && CP4_BWF_IO16 == 2
+#define bwd_filter_mfma_supported bwd_filter_mfma_iof16_supported
+#define bwd_filter_mfma_workspace_bytes bwd_filter_mfma_iof16_workspace_bytes
+#define bwd_filter_mfma_launch bwd_filter_mfma_iof16_launch
+#define CP4_BWF_HALF 1
+#elif defined(CP4_BWF_IO16)
 #define bwd_filter_mfma_supported bwd_filter_mfma_io16_supported
 #define bwd_filter_mfma_workspace_bytes bwd_filter_mfma_io16_workspace_bytes
 #define bwd_filter_mfma_launch bwd_filter_mfma_io16_launch
@@ -45,7 +51,22 @@
 namespace cp4 {
 namespace {
 
-#ifdef CP4_BWF_IO16
+#ifdef CP4_BWF_HALF
+using act_t = unsigned short;      // IEEE half bits
+[[maybe_unused]] __device__ __forceinline__ float act_to_f32(act_t v) {
+  return (float)__builtin_bit_cast(_Float16, v);
+}
+// Exact split of 8 half-precision values (widened to fp32) into two bf16 parts.
+[[maybe_unused]] __device__ __forceinline__ void split8_half(const float (&v)[8], split::u32x4& h,
+                                                             split::u32x4& m) {
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const float a = v[2 * d], b = v[2 * d + 1];
+    h[d] = split::pack_hi16(a, b);
+    m[d] = split::pack_hi16(a - split::trunc_bf16(a), b - split::trunc_bf16(b));
+  }
+}
+#elif defined(CP4_BWF_IO16)
 using act_t = unsigned short;      // bfloat16 bits
 [[maybe_unused]] __device__ __forceinline__ float act_to_f32(act_t v) {
   return __uint_as_float((unsigned)v << 16);
@@ -201,7 +222,7 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
   const int nch = (Cin >> 4) / ks, c0 = part * nch;     // this wave's chunks c0 .. c0 + nch - 1
   const act_t* xp = a.src[which] + ((size_t)n * Cin + 16 * c0 + 8 * hi) * HW + pc;
 #ifdef CP4_BWF_IO16
-  using ring_t = unsigned;     // raw bfloat16 bits, zero-extended
+  using ring_t = unsigned;     // raw 16-bit values, zero-extended
 #else
   using ring_t = float;
 #endif
@@ -248,13 +269,23 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
   // they do not wait for each other), the vector ALU splits chunk c+1.
   f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
   u32x4 xh, xm, xl;
-#ifdef CP4_BWF_IO16
+#ifdef CP4_BWF_HALF
+  // half-precision activations: widened, then two bf16 parts
+  auto pack8 = [](const ring_t (&v)[8], u32x4& h, u32x4& m) {
+    float w[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) w[e] = act_to_f32((act_t)v[e]);
+    split8_half(w, h, m);
+  };
+  pack8(xb[0], xh, xm);
+  xl = xh;                      // unused
+#elif defined(CP4_BWF_IO16)
   // bfloat16 activations: the chunk's B operand is the packed bits themselves
-  auto pack8 = [](const ring_t (&v)[8], u32x4& h) {
+  auto pack8 = [](const ring_t (&v)[8], u32x4& h, u32x4&) {
 #pragma unroll
     for (int d = 0; d < 4; ++d) h[d] = v[2 * d] | (v[2 * d + 1] << 16);
   };
-  pack8(xb[0], xh);
+  pack8(xb[0], xh, xm);
   xm = xl = xh;                 // unused
 #else
   split8(xb[0], xh, xm, xl);
@@ -271,11 +302,19 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
         const u32x4 fh = fp[0], fm = fp[64], fl = fp[128];
         // one MFMA, then a quarter of the next chunk's split, pinned in this order
         ring_t (&nx)[8] = xb[(u + 1) % kSplitRing];
-#ifdef CP4_BWF_IO16
+#ifdef CP4_BWF_HALF
+        acc0 = mfma16(fl, xh, acc0);
+        acc1 = mfma16(fm, xm, acc1);
+        acc0 = mfma16(fm, xh, acc0);
+        acc1 = mfma16(fh, xm, acc1);
+        acc0 = mfma16(fh, xh, acc0);
+        pack8(nx, nh, nm);
+        ld_chunk(nx, c + 1 + kSplitRing);             // refill the slot just split
+#elif defined(CP4_BWF_IO16)
         acc0 = mfma16(fl, xh, acc0);
         acc1 = mfma16(fm, xh, acc1);
         acc0 = mfma16(fh, xh, acc0);
-        pack8(nx, nh);
+        pack8(nx, nh, nm);
         ld_chunk(nx, c + 1 + kSplitRing);             // refill the slot just packed
 #else
         auto piece = [&](int d) {
@@ -967,16 +1006,23 @@ __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
   const bool zmine = zr < 32 * RB;
   float4 av[4], zv[2];
 #ifdef CP4_BWF_IO16
-  // four bfloat16 activations (one 8-byte load when VEC) widened to fp32
+  // four 16-bit activations (one 8-byte load when VEC) widened to fp32
   auto load4_act = [&](const act_t* row, int p) {
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (VEC) {
       if (p < HW) {
         const uint2 b = *reinterpret_cast<const uint2*>(row + p);
+#ifdef CP4_BWF_HALF
+        v.x = act_to_f32((act_t)(b.x & 0xffffu));
+        v.y = act_to_f32((act_t)(b.x >> 16));
+        v.z = act_to_f32((act_t)(b.y & 0xffffu));
+        v.w = act_to_f32((act_t)(b.y >> 16));
+#else
         v.x = __uint_as_float(b.x << 16);
         v.y = __uint_as_float(b.x & 0xffff0000u);
         v.z = __uint_as_float(b.y << 16);
         v.w = __uint_as_float(b.y & 0xffff0000u);
+#endif
       }
     } else {
       if (p < HW) v.x = act_to_f32(row[p]);
@@ -1049,7 +1095,20 @@ __global__ __launch_bounds__(kCT) void grad_split_kernel(GradArgs a) {
       const float4 a0 = *reinterpret_cast<const float4*>(ap);
       const float4 a1 = *reinterpret_cast<const float4*>(ap + 4);
       const float v[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-#ifdef CP4_BWF_IO16
+#ifdef CP4_BWF_HALF
+      // the activations are half-precision values: two bf16 parts
+      u32x4 ah, am;
+      split8_half(v, ah, am);
+#pragma unroll
+      for (int mb = 0; mb < RB; ++mb) {
+        const u32x4* zp = &Zf[buf][((mb * 2 + st) * 3 * 2 + hi) * 32 + l32];
+        acc[mb] = mfma16(ah, zp[128], acc[mb]);
+        acc[mb] = mfma16(am, zp[64], acc[mb]);
+        acc[mb] = mfma16(ah, zp[64], acc[mb]);
+        acc[mb] = mfma16(am, zp[0], acc[mb]);
+        acc[mb] = mfma16(ah, zp[0], acc[mb]);
+      }
+#elif defined(CP4_BWF_IO16)
       // the activations are bfloat16 values: their high part is all of them
       u32x4 ah;
 #pragma unroll

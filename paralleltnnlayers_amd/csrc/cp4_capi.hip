@@ -810,12 +810,12 @@ int cp4_bf16_backward_filter_supported(const cp4_shape* shape) {
   return check_shape(shape) == CP4_OK && cp4::bwd_filter_mfma_io16_supported(*shape) ? 1 : 0;
 }
 
-cp4_status cp4_conv2d_backward_filter_bf16(const cp4_shape* shape, const void* x_bf16,
-                                           const void* dy_bf16, const float* FK,
-                                           const float* FC, const float* FH,
-                                           const float* FW, float* dFK, float* dFC,
-                                           float* dFH, float* dFW, void* workspace,
-                                           size_t workspace_bytes, cp4_stream stream) {
+namespace {
+// The two 16-bit backward-filter entry points: same checks, the build for the element type.
+cp4_status backward_filter_16(const cp4_shape* shape, const void* x16, const void* dy16,
+                              const float* FK, const float* FC, const float* FH, const float* FW,
+                              float* dFK, float* dFC, float* dFH, float* dFW, void* workspace,
+                              size_t workspace_bytes, bool half, cp4_stream stream) {
   cp4_status rc = check_shape(shape);
   if (rc != CP4_OK) return rc;
   if (!FK || !FC || !FH || !FW || !dFK || !dFC || !dFH || !dFW)
@@ -829,25 +829,47 @@ cp4_status cp4_conv2d_backward_filter_bf16(const cp4_shape* shape, const void* x
     CP4_HIP(cp4::zero_f32_launch(dFW, (size_t)s.X * s.Rank, st));
     return CP4_OK;
   }
-  if (!x_bf16 || !dy_bf16) return fail(CP4_ERR_NULL_POINTER, "x or dy is NULL");
+  if (!x16 || !dy16) return fail(CP4_ERR_NULL_POINTER, "x or dy is NULL");
   if (!cp4::bwd_filter_mfma_io16_supported(s))
     return fail(CP4_ERR_UNSUPPORTED,
-                "bfloat16 backward-filter needs Rank <= 64 and C, T multiples of 16");
+                "16-bit backward-filter needs Rank <= 64 and C, T multiples of 16");
   if (!workspace || workspace_bytes < cp4::bwd_filter_mfma_io16_workspace_bytes(s))
     return fail(CP4_ERR_WORKSPACE,
                 "workspace smaller than cp4_conv2d_backward_filter_workspace_bytes");
   if ((reinterpret_cast<uintptr_t>(workspace) & 7) != 0)
     return fail(CP4_ERR_WORKSPACE, "workspace must be 8-byte aligned");
   cp4::BwdFilterArgs a{};
-  // the bfloat16 kernels read BwdFilterArgs::x / dy as 16-bit elements
-  a.x = static_cast<const float*>(x_bf16);
-  a.dy = static_cast<const float*>(dy_bf16);
+  // the 16-bit kernels read BwdFilterArgs::x / dy as 16-bit elements
+  a.x = static_cast<const float*>(x16);
+  a.dy = static_cast<const float*>(dy16);
   a.FK = FK; a.FC = FC; a.FH = FH; a.FW = FW;
   a.dFK = dFK; a.dFC = dFC; a.dFH = dFH; a.dFW = dFW; a.workspace = workspace;
   a.N = s.N; a.C = s.C; a.T = s.T; a.H = s.H; a.W = s.W; a.pad = s.pad;
   a.Y = s.Y; a.X = s.X; a.R = s.Rank;
-  CP4_HIP(cp4::bwd_filter_mfma_io16_launch(a, st));
+  if (half) CP4_HIP(cp4::bwd_filter_mfma_iof16_launch(a, st));
+  else CP4_HIP(cp4::bwd_filter_mfma_io16_launch(a, st));
   return CP4_OK;
+}
+}  // namespace
+
+cp4_status cp4_conv2d_backward_filter_bf16(const cp4_shape* shape, const void* x_bf16,
+                                           const void* dy_bf16, const float* FK,
+                                           const float* FC, const float* FH,
+                                           const float* FW, float* dFK, float* dFC,
+                                           float* dFH, float* dFW, void* workspace,
+                                           size_t workspace_bytes, cp4_stream stream) {
+  return backward_filter_16(shape, x_bf16, dy_bf16, FK, FC, FH, FW, dFK, dFC, dFH, dFW, workspace,
+                            workspace_bytes, false, stream);
+}
+
+cp4_status cp4_conv2d_backward_filter_f16(const cp4_shape* shape, const void* x_f16,
+                                          const void* dy_f16, const float* FK,
+                                          const float* FC, const float* FH,
+                                          const float* FW, float* dFK, float* dFC,
+                                          float* dFH, float* dFW, void* workspace,
+                                          size_t workspace_bytes, cp4_stream stream) {
+  return backward_filter_16(shape, x_f16, dy_f16, FK, FC, FH, FW, dFK, dFC, dFH, dFW, workspace,
+                            workspace_bytes, true, stream);
 }
 
 cp4_status cp4_conv2d_backward_filter_full(const cp4_shape* shape,

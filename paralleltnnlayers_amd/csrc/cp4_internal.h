@@ -161,6 +161,10 @@ hipError_t bwd_filter_mfma_strided_launch(const BwdFilterArgs&, const Geometry&,
 bool bwd_filter_mfma_io16_supported(const cp4_shape&);
 size_t bwd_filter_mfma_io16_workspace_bytes(const cp4_shape&);
 hipError_t bwd_filter_mfma_io16_launch(const BwdFilterArgs&, hipStream_t);
+// The same with IEEE half-precision x and dy in memory.
+bool bwd_filter_mfma_iof16_supported(const cp4_shape&);
+size_t bwd_filter_mfma_iof16_workspace_bytes(const cp4_shape&);
+hipError_t bwd_filter_mfma_iof16_launch(const BwdFilterArgs&, hipStream_t);
 hipError_t bwd_filter_full_launch(const cp4_shape&, const float* x,
                                   const float* dy, float* dK, int accumulate,
                                   hipStream_t);

@@ -68,8 +68,8 @@ class CP4Conv2dFunction(torch.autograd.Function):
         s = capi.shape_for(x.shape, FK, FC, FH, FW, pad)
         ctx.half = x.dtype == torch.float16
         if ctx.half:
-            # half-precision activations: forward and input gradient on the library's
-            # float16 entry points, the factor gradients on widened copies
+            # half-precision activations: all three passes on the library's float16 entry
+            # points where they take the shape, else on widened copies
             x = x.contiguous()
             ctx.pad, ctx.bf16, ctx.shape = pad, False, s
             ctx.relu = capi.ACTIVATIONS[activation] == 1
@@ -113,8 +113,11 @@ class CP4Conv2dFunction(torch.autograd.Function):
                     dx = capi.conv2d_backward_data(dy.float(), FK, FC, FH, FW, pad=ctx.pad).half()
             grads = (None, None, None, None)
             if any(ctx.needs_input_grad[1:5]):
-                grads = capi.conv2d_backward_filter(x.float(), dy.float(), FK, FC, FH, FW,
-                                                    pad=ctx.pad)
+                if dy.dtype == torch.float16 and capi.bf16_backward_filter_supported(s):
+                    grads = capi.conv2d_backward_filter_f16(x, dy, FK, FC, FH, FW, pad=ctx.pad)
+                else:
+                    grads = capi.conv2d_backward_filter(x.float(), dy.float(), FK, FC, FH, FW,
+                                                        pad=ctx.pad)
                 grads = tuple(g if need else None
                               for g, need in zip(grads, ctx.needs_input_grad[1:5]))
             _after_backward()

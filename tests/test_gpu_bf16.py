@@ -184,6 +184,28 @@ def test_backward_filter_bf16(cp4, oracle, dims):
         assert (g - r).abs().max().item() <= 1e-5 * r.abs().max().item()
 
 
+@pytest.mark.parametrize("dims", FILTER_SHAPES, ids=lambda d: "x".join(map(str, d)))
+def test_backward_filter_f16(cp4, oracle, dims):
+    """x and dy IEEE half in memory, gradients fp32: a half value is two bf16 parts, so
+    the products stay exact and the bar is the fp32 pass's."""
+    N, C, H, W, pad, T, Y, R = dims
+    rng = np.random.default_rng(sum(dims) + 2)
+    x = torch.from_numpy(rng.standard_normal((N, C, H, W)).astype(np.float32)).half()
+    dy = torch.from_numpy(rng.standard_normal((N, T, H, W)).astype(np.float32)).half()
+    x[0, 0, 0, 0] = 6.1e-5          # a value near the bottom of the normal range, and a subnormal
+    dy[0, 0, 0, 1] = 3.0e-7
+    fac = [(rng.standard_normal((d, R)) / np.sqrt(R)).astype(np.float32) for d in (T, C, Y, Y)]
+    f = [torch.from_numpy(v).cuda() for v in fac]
+    got = cp4.conv2d_backward_filter_f16(x.cuda(), dy.cuda(), *f, pad=pad)
+    want = oracle.backward_filter(x.float().numpy(), dy.float().numpy(), *fac, pad)
+    for g, wnt, name in zip(got, want, ("dFK", "dFC", "dFH", "dFW")):
+        assert g.dtype == torch.float32
+        assert_gradient_close(g.cpu().numpy(), wnt, name)
+    ref = cp4.conv2d_backward_filter(x.float().cuda(), dy.float().cuda(), *f, pad=pad)
+    for g, r in zip(got, ref):
+        assert (g - r).abs().max().item() <= 1e-5 * r.abs().max().item()
+
+
 def test_backward_filter_bf16_unsupported(cp4):
     x = torch.randn(1, 24, 6, 6, device="cuda").to(torch.bfloat16)      # 24 channels: not a multiple of 16
     dy = torch.randn(1, 16, 6, 6, device="cuda").to(torch.bfloat16)
