@@ -463,8 +463,9 @@ cp4_status cp3_conv2d_backward_filter(const cp4_shape* shape, const float* x, co
  * [N,Rank,H,W] intermediate to pass through as in the CP ops; for the channel
  * counts the op is meant for (16 in the reference) the cheaper order is the dense
  * filter, recomposed on the device, in a direct convolution (the recomposed-filter
- * kernel of the CP4 passes).  Square odd filters up to 17x17, pad <= Y - 1,
- * 8*C*Y*X <= 8192; CP4_ERR_UNSUPPORTED beyond.  shape->C and shape->T must equal
+ * kernel of the CP4 passes; with more than 8192 / (8*Y*X) input channels - 113 at
+ * 3x3 - the filter's weights stream through LDS by channel chunk).  Square odd
+ * filters up to 17x17, pad <= Y - 1; CP4_ERR_UNSUPPORTED beyond.  shape->C and shape->T must equal
  * S0*S1 and T0*T1.  `workspace`: device memory of rcp_conv2d_workspace_bytes (the
  * dense filter and, for the factor gradients, its gradient).  The input gradient
  * follows the reference's backward-data convention (reversed taps at offset

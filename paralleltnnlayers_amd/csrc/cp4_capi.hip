@@ -1799,7 +1799,7 @@ cp4_status rcp_dense_pass(const cp4_shape& s, const float* in, float* out, const
   a.H = s.H; a.W = s.W; a.pad = s.pad; a.Y = s.Y; a.X = s.X; a.R = s.Rank;
   if (!cp4::fwd_dense_small_supported(a))
     return fail(CP4_ERR_UNSUPPORTED,
-                "reshaped-CP op: square odd filters up to 17x17, pad <= Y-1, 8*C*Y*X <= 8192");
+                "reshaped-CP op: square odd filters up to 17x17 with pad <= Y-1");
   CP4_HIP(cp4::fwd_dense_small_launch(a, st));
   return CP4_OK;
 }

@@ -13,7 +13,9 @@
 // One workgroup (256 threads) owns `tpw` vertically adjacent tiles of 16 rows x
 // 64 columns of one image and up to eight output channels (more output channels:
 // more workgroups).  With FwdArgs::dense the filter K is given instead of the
-// factors (the reshaped-CP sibling op recomposes its own):
+// factors (the reshaped-CP sibling op recomposes its own); a given filter of any
+// number of input channels is taken - beyond 8192 weights per workgroup only the
+// current channel chunk's weights are in LDS, reloaded with every chunk:
 //   prologue  the four factors go to LDS, then every workgroup recomposes K into
 //             LDS itself (Cout*Cin*Y*X*R multiply-adds: a few thousand, no scratch
 //             memory, no extra launch; the tiles of a workgroup share it)
@@ -41,6 +43,8 @@ struct DensePlan {
   int tile_w;    // LDS row length of the tile (floats, odd: conflict-free segment reads)
   int tpw;       // tiles per workgroup, down the image
   int wfloats;   // LDS floats set aside for a workgroup's filter (a multiple of 4)
+  int stream_w;  // the filter does not fit: only the current channel chunk's weights are
+                 // in LDS, reloaded with every chunk of the tile (given filters only)
   int cols, rowgroups, ntiles;   // tile columns, groups of tpw tile rows, workgroups with work
   size_t lds_bytes;
 };
@@ -70,8 +74,10 @@ __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, De
 
   if (a.dense) {
     // the filter is given: [Cout][Cin][FS][FS], taps in the order this pass reads them
-    const float* src = a.dense + (size_t)k0 * Cin * FS * FS;
-    for (int q = tid; q < nw; q += kThreads) wts[q] = src[q];
+    if (!pl.stream_w) {
+      const float* src = a.dense + (size_t)k0 * Cin * FS * FS;
+      for (int q = tid; q < nw; q += kThreads) wts[q] = src[q];
+    }
   } else {
     // the factors once through LDS (they alias the tile, which is loaded later) ...
     float* fo = tile;                                 // Fout [Cout][R]
@@ -118,6 +124,14 @@ __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, De
       const int cn = min(pl.cc, Cin - c0);
       __syncthreads();                                // weights written / previous tile read
       const int nrows = cn * HT;                      // (channel, tile row) pairs
+      if (pl.stream_w) {
+        // this chunk's weights: [Cout][cn][FS][FS] out of the filter's [Cout][Cin][FS][FS]
+        const int per = cn * FS * FS;
+        for (int q = tid; q < Cout * per; q += kThreads) {
+          const int k = q / per, e = q - k * per;
+          wts[q] = a.dense[((size_t)(k0 + k) * Cin + c0) * FS * FS + e];
+        }
+      }
       if (vec_in) {
         // the 64 inner columns of a row: sixteen float4
         for (int q = tid; q < nrows * 16; q += kThreads) {
@@ -165,7 +179,8 @@ __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, De
 #pragma unroll
           for (int k = 0; k < KO; ++k) {
             if (k < Cout) {
-              const float* wr = wts + ((k * Cin + c0 + c) * FS + i) * FS;
+              const float* wr = pl.stream_w ? wts + ((k * cn + c) * FS + i) * FS
+                                            : wts + ((k * Cin + c0 + c) * FS + i) * FS;
 #pragma unroll
               for (int j = 0; j < FS; ++j) {
                 const float wv = wr[j];
@@ -212,8 +227,9 @@ bool plan(const FwdArgs& a, DensePlan* pl) {
   if (a.ldf || a.accumulate || a.sh) return false;
   const int kgrp = a.Cout < 8 ? a.Cout : 8;           // output channels of a workgroup
   const long ngrp = (a.Cout + 7) / 8;
-  const long nw = (long)kgrp * a.Cin * a.Y * a.X;
-  if (nw > kMaxWeights) return false;
+  long nw = (long)kgrp * a.Cin * a.Y * a.X;
+  const bool stream_w = nw > kMaxWeights;
+  if (stream_w && (!a.dense || (long)kgrp * a.Y * a.X > kMaxWeights)) return false;
   const long nf = a.dense ? 0 : (long)a.R * (kgrp + a.Cin + a.Y + a.X);
   if (nf > kMaxFactorFloats) return false;
 
@@ -224,6 +240,11 @@ bool plan(const FwdArgs& a, DensePlan* pl) {
   int cc = (int)(kTileBudget / per_channel);
   if (cc < 1) return false;
   if (cc > a.Cin) cc = a.Cin;
+  if (stream_w) {
+    const int wcc = (int)(kMaxWeights / ((long)kgrp * a.Y * a.X));   // channels whose weights fit
+    if (cc > wcc) cc = wcc;
+    nw = (long)kgrp * cc * a.Y * a.X;
+  }
   size_t tile_bytes = cc * per_channel;
   if (tile_bytes < (size_t)nf * sizeof(float)) tile_bytes = (size_t)nf * sizeof(float);
   // enough workgroups to fill the device sixteen times over, each amortising its
@@ -244,6 +265,7 @@ bool plan(const FwdArgs& a, DensePlan* pl) {
   pl->tile_w = tile_w;
   pl->tpw = (int)tpw;
   pl->wfloats = (int)((nw + 3) & ~3l);
+  pl->stream_w = stream_w ? 1 : 0;
   pl->lds_bytes = (size_t)pl->wfloats * sizeof(float) + tile_bytes;
   return true;
 }

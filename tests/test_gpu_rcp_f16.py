@@ -34,6 +34,10 @@ RCP_CASES = [
     (2, 2, 3, 3, 2, 9, 11, 3, 4),
     (3, 4, 8, 2, 5, 14, 14, 5, 6),        # 32 -> 10 channels, 5x5
     (1, 3, 3, 5, 5, 20, 24, 1, 7),        # 1x1 filter, 25 output channels (four groups of 8)
+    (2, 12, 12, 6, 4, 14, 18, 3, 5),      # 144 -> 24 channels at 3x3: the filter's weights stream
+                                          # through LDS by channel chunk (forward)
+    (1, 4, 5, 16, 10, 12, 12, 3, 4),      # 20 -> 160 channels: the same for the input gradient
+    (1, 8, 8, 8, 8, 10, 10, 5, 3),        # 64 -> 64 at 5x5: both
 ]
 
 
