@@ -752,12 +752,19 @@ __global__ __launch_bounds__(256) void taps_column_kernel(
     const float* __restrict__ A, const float* __restrict__ G3, const float* __restrict__ FH,
     const float* __restrict__ FW, float* __restrict__ Cc, float* __restrict__ G1,
     float* __restrict__ partH, float* __restrict__ partW, int R, int H, int W, int P,
-    int nplanes, int segs, int Q) {
+    int nplanes, int segs, int Q, int rsegs, int RH) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int unit = blockIdx.x * 4 + wave;        // (plane, column segment)
-  if (unit >= nplanes * segs) return;
-  const int plane = unit / segs, seg = unit - plane * segs;
+  const int unit = blockIdx.x * 4 + wave;        // (plane, column segment, row segment)
+  if (unit >= nplanes * segs * rsegs) return;
+  const int pseg = unit / rsegs, rseg = unit - pseg * rsegs;
+  const int plane = pseg / segs, seg = pseg - plane * segs;
+  // Rows r0 .. r1-1 are this wave's: it stores and sums those only.  Its walk starts Q
+  // rows above (the windows of its first outputs hold rows from r0 - Q on; what the
+  // windows hold from further up is not used by any row it stores) and ends as the
+  // whole-plane walk does.
+  const int r0 = rseg * RH, r1 = min(H, r0 + RH);
+  const int tstart = max(0, r0 - Q);
   const int r = plane % R, n = plane / R;
   const size_t base = (size_t)plane * H * W;
   // lane's image column; one segment: lane = column, no halo
@@ -797,13 +804,13 @@ __global__ __launch_bounds__(256) void taps_column_kernel(
     gr[slot] = G3[base + (size_t)rc * W + wc];
   };
 #pragma unroll
-  for (int u = 0; u < kRowsAhead; ++u) request(u, u);
+  for (int u = 0; u < kRowsAhead; ++u) request(u, tstart + u);
   const int tail = (FS - 1 - P) > P ? (FS - 1 - P) : P;
-  for (int t0 = 0; t0 < H + tail; t0 += kRowsAhead) {
+  for (int t0 = tstart; t0 < r1 + tail; t0 += kRowsAhead) {
 #pragma unroll
     for (int u = 0; u < kRowsAhead; ++u) {
       const int t = t0 + u;
-      if (t < H + tail) {
+      if (t < r1 + tail) {
         const bool live = col && t < H;
         const float a_t = live ? ar[u] : 0.f, g_t = live ? gr[u] : 0.f;
         request(u, t + kRowsAhead);
@@ -825,7 +832,7 @@ __global__ __launch_bounds__(256) void taps_column_kernel(
         g2w[FS - 1] = g2_t;
         // B, Cc and the tap-gradient terms of row hb
         const int hb = t - (FS - 1 - P);
-        if (hb >= 0 && hb < H) {
+        if (hb >= r0 && hb < r1) {
           float b = 0.f;
 #pragma unroll
           for (int i = 0; i < FS; ++i) b += fh[i] * aw[i];
@@ -844,7 +851,7 @@ __global__ __launch_bounds__(256) void taps_column_kernel(
         }
         // G1 row hg: vertical adjoint taps of the G2 window
         const int hg = t - P;
-        if (hg >= 0 && hg < H) {
+        if (hg >= r0 && hg < r1) {
           float g1 = 0.f;
 #pragma unroll
           for (int i = 0; i < FS; ++i) g1 += fh[i] * g2w[FS - 1 - i];
@@ -864,8 +871,8 @@ __global__ __launch_bounds__(256) void taps_column_kernel(
   if (lane == 0) {
 #pragma unroll
     for (int i = 0; i < FS; ++i) {
-      partH[(((size_t)n * segs + seg) * FS + i) * R + r] = accH[i];
-      partW[(((size_t)n * segs + seg) * FS + i) * R + r] = accW[i];
+      partH[((((size_t)n * segs + seg) * rsegs + rseg) * FS + i) * R + r] = accH[i];
+      partW[((((size_t)n * segs + seg) * rsegs + rseg) * FS + i) * R + r] = accW[i];
     }
   }
 }
@@ -875,15 +882,31 @@ int column_segments(int W, int FS, int P) {
   const int Q = P > FS - 1 - P ? P : FS - 1 - P;
   return W <= 64 ? 1 : (W + (64 - 2 * Q) - 1) / (64 - 2 * Q);
 }
+// Rows per row segment: a wave walks its rows one after the other, so tall planes are
+// cut until there are about 4096 waves, but not below 8 rows a segment (each walk
+// starts with Q rows of the segment above).
+int column_row_height(int N, int R, int H, int W, int FS, int P) {
+  const long units = (long)N * R * column_segments(W, FS, P);
+  long rsegs = (4096 + units - 1) / units;
+  if (rsegs > H / 8) rsegs = H / 8;
+  if (rsegs < 1) rsegs = 1;
+  return (int)((H + rsegs - 1) / rsegs);
+}
+int column_row_segments(int N, int R, int H, int W, int FS, int P) {
+  const int RH = column_row_height(N, R, H, W, FS, P);
+  return (H + RH - 1) / RH;
+}
 
 template <int FS>
 hipError_t launch_taps_column(const float* A, const float* G3, const BwdFilterArgs& a, float* Cc,
                               float* G1, float* pH, float* pW, hipStream_t st) {
   const int nplanes = a.N * a.R, segs = column_segments(a.W, FS, a.pad);
   const int Q = a.pad > FS - 1 - a.pad ? a.pad : FS - 1 - a.pad;
-  const long units = (long)nplanes * segs;
+  const int RH = column_row_height(a.N, a.R, a.H, a.W, FS, a.pad);
+  const int rsegs = (a.H + RH - 1) / RH;
+  const long units = (long)nplanes * segs * rsegs;
   taps_column_kernel<FS><<<(unsigned)((units + 3) / 4), 256, 0, st>>>(
-      A, G3, a.FH, a.FW, Cc, G1, pH, pW, a.R, a.H, a.W, a.pad, nplanes, segs, Q);
+      A, G3, a.FH, a.FW, Cc, G1, pH, pW, a.R, a.H, a.W, a.pad, nplanes, segs, Q, rsegs, RH);
   return hipGetLastError();
 }
 
@@ -1240,7 +1263,7 @@ Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R, int pad) 
                 wave_tap_layout(H, W, Y, pad).smem <= 64 * 1024;
   // one wave per plane (or per column segment of a wide plane), in registers
   p.column_taps = !p.wave_taps && odd_square && pad <= Y - 1;
-  p.St = p.column_taps ? N * column_segments(W, Y, pad)
+  p.St = p.column_taps ? N * column_segments(W, Y, pad) * column_row_segments(N, R, H, W, Y, pad)
                        : (p.plane_taps ? N : (N < 8 ? N : 8));
   p.plane = (size_t)N * R * HW;
   // (tap partials: Y + X per plane, Y * X with the 3-factor op's depthwise filter)
