@@ -43,9 +43,13 @@ HBM_PEAK_GBS = 8000.0
 FACTORS = ("FK", "FC", "FH", "FW")
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs, scaled by the plain copy kernel's reading (see
-# profiles/): {workload: bytes}.  None until measured for the current kernel.
-MEASURED_TRAFFIC = {"C3": 209.9e6}   # fwd_pipe_kernel<3,4,2,4>: 107.1 MB fetched + 102.8 MB written
+# WRITE_SIZE runs, scaled by the plain copy kernel's reading (profiles/), keyed by the
+# workload AND the plan the counters were taken on (variant, strip rows, workgroups): a
+# launch that runs another plan reports null rather than another kernel's bytes.
+MEASURED_TRAFFIC = {
+    # fwd_pipe_kernel<3,4,2,4>: 107.1 MB fetched + 102.8 MB written
+    ("C3", "mfma_bf16x3_pipe", 8, 224): 209.9e6,
+}
 
 
 def main():
@@ -190,6 +194,8 @@ def main():
                           "GB/s": round(nbytes / cus / 1e3, 1),
                           "hbm_frac": round(nbytes / cus / 1e3 / HBM_PEAK_GBS, 4)}))
         return
+    plan = cp4.plan_query(cp4.capi.shape_for((w.N, w.C, w.H, w.W), *[d[k] for k in FACTORS],
+                                             w.pad), w.pass_)
     us, wall = timed(w, d, args.warmup, args.steps, args.settle_ms)
     value = nbytes * args.steps / wall / 1e9
     achieved = nbytes / us / 1e3
@@ -214,10 +220,11 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s %s fp32 NCHW N=%d C=%d K=%d H=W=%d %dx%d pad=%d R=%d"
                                % (w.name, w.pass_, w.N, w.C, w.T, w.H, w.Y, w.X, w.pad, w.R),
-                   "algorithmic_bytes": nbytes, "us_per_launch": round(us, 2)},
+                   "algorithmic_bytes": nbytes, "us_per_launch": round(us, 2), "plan": plan},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC.get(w.name),
+                     "traffic": MEASURED_TRAFFIC.get((w.name, plan["variant"], plan["strip_rows"],
+                                                      plan["workgroups"])),
                      "regime": "one buffer set re-launched (%.0f MB working set; the part's "
                                "memory-side cache holds 256 MB)" % (nbytes / 1e6),
                      "cold": cold},

@@ -362,6 +362,15 @@ cp4_status cp4_tune_backward_filter(const cp4_shape* shape, const float* x, cons
                                     float* best_us, cp4_stream stream);
 cp4_status cp4_tuned_choice(const cp4_shape* shape, int backward_data, int* variant,
                             int* tile_rows, int* tile_cols, int* role_split);
+/* What a launch of `shape` would run with now, for reports and benchmarks: pass 0 =
+ * forward, 1 = backward-data, 2 = backward-filter.  `variant` indexes
+ * cp4_forward_variant_name (passes 0, 1) or cp4_backward_filter_variant_name (pass 2,
+ * for operands and a workspace aligned to 16 bytes); for the whole-row strip kernel
+ * `strip_rows` and `workgroups` are the planner's strip height and grid, else 0.
+ * No counterpart in the reference, whose kernel has one fixed tile
+ * (reference/kernels/cp4Conv2dForward.cu:183-198). */
+cp4_status cp4_plan_query(const cp4_shape* shape, int pass, int* variant, int* strip_rows,
+                          int* workgroups);
 /* Enters a choice into the table as cp4_tune_forward / cp4_tune_backward_data
  * would (one saved from an earlier process, say), in cp4_tuned_choice's terms.
  * CP4_ERR_UNSUPPORTED if the variant does not take the shape with that tile. */

@@ -14,7 +14,7 @@ from .capi import (Shape, Geometry, geometry, conv2d_forward_ex, conv2d_backward
                    conv2d_backward_data, conv2d_backward_filter, conv2d_backward_filter_noalloc,
                    conv2d_backward_filter_full, backward_filter_workspace_bytes,
                    time_forward, time_forward_sets, time_backward_data, time_backward_filter,
-                   tune_forward, tune_backward_data, tune_backward_filter, tuned_choice,
+                   tune_forward, tune_backward_data, tune_backward_filter, tuned_choice, plan_query,
                    set_tuned_choice, tuned_table, tuned_filter_table, set_tuned_filter_choice,
                    backward_filter_variants, save_tuned, load_tuned, tune_clear, device_status, device_status_detail, set_spin_limit,
                    forward_variants, default_variant, recompose, count_exceeding,

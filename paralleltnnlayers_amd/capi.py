@@ -136,6 +136,7 @@ def lib():
                                                  ctypes.POINTER(ctypes.c_int),
                                                  ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
     L.cp4_tuned_choice.argtypes = [_S, ctypes.c_int] + [ctypes.POINTER(ctypes.c_int)] * 4
+    L.cp4_plan_query.argtypes = [_S, ctypes.c_int] + [ctypes.POINTER(ctypes.c_int)] * 3
     L.cp4_set_tuned_choice.argtypes = [_S] + [ctypes.c_int] * 5
     L.cp4_tuned_count.restype = ctypes.c_int
     L.cp4_tuned_entry.argtypes = [ctypes.c_int, _S] + [ctypes.POINTER(ctypes.c_int)] * 5
@@ -612,6 +613,20 @@ def tuned_choice(s, backward_data=False):
     v = [ctypes.c_int() for _ in range(4)]
     check(lib().cp4_tuned_choice(ctypes.byref(s), int(backward_data), *[ctypes.byref(i) for i in v]))
     return dict(zip(("variant", "tile_rows", "tile_cols", "role_split"), (i.value for i in v)))
+
+
+def plan_query(s, pass_="forward"):
+    """{'variant' (its name), 'strip_rows', 'workgroups'} a launch of this pass would run with
+    now; rows and workgroups are 0 unless the whole-row strip kernel takes the shape."""
+    idx = ("forward", "backward_data", "backward_filter").index(pass_)
+    v = [ctypes.c_int() for _ in range(3)]
+    check(lib().cp4_plan_query(ctypes.byref(s), idx, *[ctypes.byref(i) for i in v]))
+    if idx == 2:
+        names = dict(enumerate(backward_filter_variants()))
+    else:
+        names = {i: n for i, n, _ in forward_variants()}
+    return {"variant": names.get(v[0].value, str(v[0].value)), "strip_rows": v[1].value,
+            "workgroups": v[2].value}
 
 
 def set_tuned_choice(s, variant, tile_rows=0, tile_cols=0, schedule=1, backward_data=False):

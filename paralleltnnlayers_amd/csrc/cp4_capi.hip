@@ -1378,6 +1378,53 @@ cp4_status cp4_tuned_choice(const cp4_shape* shape, int backward_data, int* vari
   return CP4_OK;
 }
 
+cp4_status cp4_plan_query(const cp4_shape* shape, int pass, int* variant, int* strip_rows,
+                          int* workgroups) {
+  cp4_status rc = check_shape(shape);
+  if (rc != CP4_OK) return rc;
+  if (pass < 0 || pass > 2) return fail(CP4_ERR_SHAPE, "pass must be 0, 1 or 2");
+  int v = -1, rows = 0, wgs = 0;
+  if (pass == 2) {
+    // the choice for operands aligned as every allocator returns them
+    const cp4_shape& s = *shape;
+    const bool tiles_ok = filter_rank_tiles_supported(s);
+    const bool mfma_ok = cp4::bwd_filter_mfma_supported(s) || tiles_ok;
+    const bool fused_ok =
+        cp4::bwd_filter_fused_supported(s) ||
+        (tiles_ok && cp4::bwd_filter_fused_supported(filter_rank_tile(s, 0)) &&
+         cp4::bwd_filter_fused_supported(
+             filter_rank_tile(s, (s.Rank - 1) / kFilterRankTile * kFilterRankTile)));
+    {
+      std::lock_guard<std::mutex> lk(g_tune_mu);
+      auto it = g_tuned_filter.find(key_of(s));
+      if (it != g_tuned_filter.end() &&
+          (it->second == 0 || (it->second == 1 && mfma_ok) || (it->second == 2 && fused_ok)))
+        v = it->second;
+    }
+    if (v < 0) {
+      const bool prefer_fused =
+          fused_ok && (cp4::bwd_filter_fused_preferred(
+                           s.Rank > kFilterRankTile ? filter_rank_tile(s, 0) : s) ||
+                       !mfma_ok);
+      v = prefer_fused ? 2 : (mfma_ok ? 1 : 0);
+    }
+  } else {
+    FwdArgs a = pass == 1
+        ? backward_data_args(*shape, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr)
+        : forward_args(*shape, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr);
+    const Choice c = choose(a);
+    v = c.variant;
+    if (is_variant(v, "mfma_bf16x3_pipe")) {
+      a.tune_th = c.th;
+      if (!cp4::fwd_pipe_strip_plan(a, &rows, &wgs)) rows = wgs = 0;
+    }
+  }
+  if (variant) *variant = v;
+  if (strip_rows) *strip_rows = rows;
+  if (workgroups) *workgroups = wgs;
+  return CP4_OK;
+}
+
 cp4_status cp4_set_tuned_choice(const cp4_shape* shape, int backward_data, int variant,
                                 int tile_rows, int tile_cols, int schedule) {
   cp4_status rc = check_shape(shape);

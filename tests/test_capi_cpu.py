@@ -128,6 +128,27 @@ def test_default_variant_on_wide_planes(L):
     assert capi.default_variant(capi.Shape(N=1, H=0, W=8, pad=1, T=4, C=4, Y=3, X=3, Rank=2)) is None
 
 
+def test_plan_query_names_what_a_launch_runs(L):
+    """The plan report needs no GPU: the headline forward runs eight-row strips, 224 workgroups in one
+    wave, its backward-filter takes the four-launch variant, a small layer's the
+    three-launch one; an invalid pass is a shape error."""
+    from paralleltnnlayers_amd import capi
+    capi.tune_clear()
+    s = capi.Shape(N=32, H=56, W=56, pad=1, T=256, C=256, Y=3, X=3, Rank=32)
+    p = capi.plan_query(s, "forward")
+    assert p == {"variant": "mfma_bf16x3_pipe", "strip_rows": 8, "workgroups": 224}
+    assert capi.plan_query(s, "backward_data")["variant"] == "mfma_bf16x3_pipe"
+    names = capi.backward_filter_variants()
+    assert capi.plan_query(s, "backward_filter")["variant"] == names[1]
+    small = capi.Shape(N=8, H=28, W=28, pad=1, T=64, C=64, Y=3, X=3, Rank=16)
+    assert capi.plan_query(small, "backward_filter")["variant"] == names[2]
+    capi.set_tuned_filter_choice(small, 1)
+    assert capi.plan_query(small, "backward_filter")["variant"] == names[1]
+    capi.tune_clear()
+    v = ctypes.c_int()
+    assert L.cp4_plan_query(ctypes.byref(s), 3, ctypes.byref(v), None, None) == capi.ERR_SHAPE
+
+
 def test_status_strings(L):
     seen = {L.cp4_status_string(i) for i in range(6)}
     assert len(seen) == 6 and b"ok" in seen
