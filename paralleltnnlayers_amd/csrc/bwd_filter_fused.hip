@@ -384,7 +384,7 @@ __global__ __launch_bounds__(512) void grad_fused_kernel(FusedArgs a) {
         const int i = lane + 64 * (kb * KM + kk);
         const int row = (int)__umulhi((unsigned)i, a.wmagic);
         cellk[kk] = i < run ? cbase + i + row * 2 * Q : dummy;
-        const unsigned vo = (unsigned)min(i, run - 1) * 4u;   // (the scalar offset is not range-checked)
+        const unsigned vo = (unsigned)min(i, run - 1) * 4u;   // (lanes past the run: a valid cell, for the dummy)
         if (kb * KM + kk < per) {                      // wave-uniform
 #pragma unroll
           for (int jj = 0; jj < JM; ++jj) {

@@ -200,6 +200,7 @@ const Variant kVariants[] = {
     {"dense_small_valu", cp4::fwd_dense_small_supported, cp4::fwd_dense_small_launch},
     {"mfma_f32_strip", cp4::fwd_mfma_supported, cp4::fwd_mfma_launch},
     {"mfma_bf16x3_strip", cp4::fwd_split_supported, cp4::fwd_split_launch},
+    {"mfma_bf16x3_light", cp4::fwd_light_supported, cp4::fwd_light_launch},
     {"mfma_bf16x3_pipe_tiled", cp4::fwd_pipe_tiled_supported, cp4::fwd_pipe_tiled_launch},
     {"mfma_bf16x3_pipe", cp4::fwd_pipe_supported, cp4::fwd_pipe_launch},
     {"mfma_bf16x3_pipe_rank_passes", fwd_pipe2_supported, fwd_pipe2_launch},
@@ -299,6 +300,16 @@ bool strips_on_wide_plane(const FwdArgs& a) {
 // elements the fp32 matrix-core strip kernel is the faster one for ranks 33-64.
 constexpr long kTwoPassMinElements = 16l << 20;
 
+// Where the light kernel beats the producer / consumer kernel (and, below a few
+// tens of thousands of pixels, the recomposed-filter kernel, whose threads each run
+// Cout x Cin x Y x X multiply-adds per pixel quad in series): measured over 90 shapes
+// it takes 0.61-0.97 of the other's time inside these bounds - N8 C16 56x56 R16 9.3 ->
+// 5.7 us, N4 C32 112x112 R16 11.1 -> 9.1, N16 C8 32x32 R16 29.9 -> 5.6 - and more
+// outside them: 1.0-1.1 with 48-64 input channels or 32 ranks, 1.2-2.3 from 100,000
+// pixels on (its grid then needs several rounds of workgroups of 200 registers a lane).
+constexpr long kLightMaxPixels = 50176;      // 4 x 112 x 112
+constexpr int kLightMaxCin = 32, kLightMaxCout = 64, kLightMaxRank = 16;
+
 // CP4_FORWARD_VARIANT=<name> overrides the heuristic where that variant can run the
 // shape (profiling and A/B runs of unmodified callers).  Read once, at the first launch:
 // the process's environment is not consulted per call.
@@ -338,6 +349,10 @@ int heuristic_variant(const FwdArgs& a) {
     if (dense_small_estimate(a) <= (matrix ? kMatrixSmallChannelEstimate : general_estimate(a)))
       prefer("dense_small_valu");
   }
+  // Small problems with few channels: the light kernel's three short phases.
+  if ((long)a.N * a.H * a.W <= kLightMaxPixels && a.Cin <= kLightMaxCin &&
+      a.Cout <= kLightMaxCout && a.R <= kLightMaxRank)
+    prefer("mfma_bf16x3_light");
   return pick;
 }
 
@@ -557,6 +572,13 @@ cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
   if (is_variant(c.variant, "dense_small_valu") && cp4::fwd_dense_small_supported(a)) {
     CP4_HIP(cp4::fwd_dense_small_launch(a, st));    // applies bias / activation in its stores
     return CP4_OK;
+  }
+  if (is_variant(c.variant, "mfma_bf16x3_light")) {
+    FwdArgs e = with_tile(a, c);
+    if (cp4::fwd_light_supported(e)) {
+      CP4_HIP(cp4::fwd_light_launch(e, st));        // the same
+      return CP4_OK;
+    }
   }
   rc = run_choice(plain, c, st);
   if (rc != CP4_OK) return rc;

@@ -91,6 +91,9 @@ bool fwd_mfma_supported(const FwdArgs&);
 hipError_t fwd_mfma_launch(const FwdArgs&, hipStream_t);
 bool fwd_split_supported(const FwdArgs&);
 hipError_t fwd_split_launch(const FwdArgs&, hipStream_t);
+// Few short phases in small workgroups, for small problems (ranks up to 32).
+bool fwd_light_supported(const FwdArgs&);
+hipError_t fwd_light_launch(const FwdArgs&, hipStream_t);
 bool fwd_pipe_supported(const FwdArgs&);
 hipError_t fwd_pipe_launch(const FwdArgs&, hipStream_t);
 // Rows per strip and workgroups of the whole-row strip plan (false: no plan).

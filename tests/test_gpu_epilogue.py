@@ -41,6 +41,8 @@ SHAPES = [
     (2, 64, 30, 150, 1, 64, 3, 4),     # wide plane, whole pixel groups per consumer wave
     (2, 3, 70, 130, 1, 1, 3, 16),      # three channels to one: the recomposed-filter kernel's own epilogue
     (1, 4, 33, 47, 2, 12, 5, 8),       # ... with two groups of output channels, ragged tiles
+    (2, 16, 28, 28, 1, 40, 3, 8),      # small layer: the light kernel's own epilogue
+    (1, 32, 20, 30, 2, 64, 5, 16),     # ... 5x5, two blocks of output channels
 ]
 
 
