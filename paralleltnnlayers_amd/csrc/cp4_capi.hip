@@ -262,6 +262,38 @@ double dense_small_estimate(const FwdArgs& a) {
          0.0025 * a.Cout * a.Cin * a.Y * a.X;
 }
 constexpr double kMatrixSmallChannelEstimate = 26.0;
+// Below about a million pixels the recomposed-filter kernel is bound not by that rate
+// but by the time of one workgroup: each thread runs the multiply-adds of its four
+// pixels in series, Cin filter rows' segment reads and Cin x min(Cout, 8) filter rows
+// of multiply-adds, with one wave per vector unit to hide the LDS latency behind
+// (measured on 16 x 64 tiles, 3x3, any size from a thousand pixels up: 3 -> 1 channels
+// 7.4 us, 4 -> 4 12.8, 3 -> 16 15.7, 16 -> 1 23, 8 -> 8 31, 16 -> 3 34), times the
+// rounds of workgroups the grid needs at six tenths of the occupancy its LDS allows
+// (co-resident workgroups share the vector units).  The matrix-core kernels take
+// 6 us + 16.5 us per 2^18 pixels there (few channels, rank 16: 12 us at 100,000
+// pixels, 18 at 200,000, 56 at 800,000).
+constexpr long kDenseSmallRateFromPixels = 1l << 20;
+double dense_small_floor(const FwdArgs& a) {
+  const double ko = a.Cout < 8 ? a.Cout : 8;
+  // rows of whole 64-column tiles are loaded sixteen bytes a lane: the per-channel part
+  // shrinks (N1 512x512, 16 -> 1: 15.4 us, 8 -> 1: 8.1, 3 -> 8: 13.8)
+  const double v = a.W % 64 == 0 ? 0.65 : 1.0;
+  return 3.8 * v + a.Cin * (a.Y / 3.0) * (1.2 * v + 0.34 * (ko - 1));   // (5x5, 3 -> 16: 24 us)
+}
+bool dense_small_loses_to_matrix(const FwdArgs& a) {
+  const long pixels = (long)a.N * a.H * a.W;
+  if (pixels > kDenseSmallRateFromPixels) return false;
+  long tiles = 0;
+  size_t lds = 0;
+  if (!cp4::fwd_dense_small_plan_info(a, &tiles, &lds)) return false;
+  long occ = (long)(160 * 1024 / (lds ? lds : 1));
+  occ = occ < 1 ? 1 : (occ > 8 ? 8 : occ);
+  const double rounds = (double)tiles / (0.6 * occ * cp4::num_compute_units());
+  const double dense = dense_small_floor(a) * (rounds > 1.0 ? rounds : 1.0);
+  // (the matrix-core kernels' tap step grows with the filter: 28 us per 2^18 pixels at
+  // 5x5, 52 at 7x7)
+  return dense > 6.0 + 16.5 * (a.Y * a.X + 9) / 18.0 * pixels / 262144.0;
+}
 double general_estimate(const FwdArgs& a) {
   return 10.0 + 0.3 * a.R * (a.Cin + a.Cout + a.Y + a.X);
 }
@@ -309,6 +341,7 @@ constexpr long kTwoPassMinElements = 16l << 20;
 // pixels on (its grid then needs several rounds of workgroups of 200 registers a lane).
 constexpr long kLightMaxPixels = 50176;      // 4 x 112 x 112
 constexpr int kLightMaxCin = 32, kLightMaxCout = 64, kLightMaxRank = 16;
+constexpr double kLightMinDenseFloor = 6.0;  // us
 
 // CP4_FORWARD_VARIANT=<name> overrides the heuristic where that variant can run the
 // shape (profiling and A/B runs of unmodified callers).  Read once, at the first launch:
@@ -346,12 +379,16 @@ int heuristic_variant(const FwdArgs& a) {
   // multiply-adds per pixel than the factor-by-factor order.
   if (cp4::fwd_dense_small_supported(a)) {
     const bool matrix = pick >= 0 && !strncmp(kVariants[pick].name, "mfma_", 5);
-    if (dense_small_estimate(a) <= (matrix ? kMatrixSmallChannelEstimate : general_estimate(a)))
+    if (dense_small_estimate(a) <= (matrix ? kMatrixSmallChannelEstimate : general_estimate(a)) &&
+        !(matrix && dense_small_loses_to_matrix(a)))
       prefer("dense_small_valu");
   }
   // Small problems with few channels: the light kernel's three short phases.
+  // (not where the recomposed-filter kernel was picked and is as quick: 3 -> 1 channels on
+  // whole tiles, 4.8 us)
   if ((long)a.N * a.H * a.W <= kLightMaxPixels && a.Cin <= kLightMaxCin &&
-      a.Cout <= kLightMaxCout && a.R <= kLightMaxRank)
+      a.Cout <= kLightMaxCout && a.R <= kLightMaxRank &&
+      !(is_variant(pick, "dense_small_valu") && dense_small_floor(a) <= kLightMinDenseFloor))
     prefer("mfma_bf16x3_light");
   return pick;
 }

@@ -87,6 +87,8 @@ hipError_t fwd_general_launch(const FwdArgs&, hipStream_t);
 // Recomposed-filter direct convolution for very few channels on both sides.
 bool fwd_dense_small_supported(const FwdArgs&);
 hipError_t fwd_dense_small_launch(const FwdArgs&, hipStream_t);
+// Its plan for a shape: 16 x 64 tiles in all and LDS bytes per workgroup (false: no plan).
+bool fwd_dense_small_plan_info(const FwdArgs&, long* tiles, size_t* lds_bytes);
 bool fwd_mfma_supported(const FwdArgs&);
 hipError_t fwd_mfma_launch(const FwdArgs&, hipStream_t);
 bool fwd_split_supported(const FwdArgs&);

@@ -49,7 +49,8 @@ struct DensePlan {
   size_t lds_bytes;
 };
 
-template <int FS, int KO>
+// SW: the filter does not fit LDS and streams by channel chunk (DensePlan::stream_w).
+template <int FS, int KO, bool SW>
 __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, DensePlan pl) {
   extern __shared__ float lds[];
   const int Cin = a.Cin, R = a.R, H = a.H, W = a.W;
@@ -74,7 +75,7 @@ __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, De
 
   if (a.dense) {
     // the filter is given: [Cout][Cin][FS][FS], taps in the order this pass reads them
-    if (!pl.stream_w) {
+    if (!SW) {
       const float* src = a.dense + (size_t)k0 * Cin * FS * FS;
       for (int q = tid; q < nw; q += kThreads) wts[q] = src[q];
     }
@@ -124,7 +125,7 @@ __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, De
       const int cn = min(pl.cc, Cin - c0);
       __syncthreads();                                // weights written / previous tile read
       const int nrows = cn * HT;                      // (channel, tile row) pairs
-      if (pl.stream_w) {
+      if (SW) {
         // this chunk's weights: [Cout][cn][FS][FS] out of the filter's [Cout][Cin][FS][FS]
         const int per = cn * FS * FS;
         for (int q = tid; q < Cout * per; q += kThreads) {
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(kThreads) void fwd_dense_small_kernel(FwdArgs a, De
 #pragma unroll
           for (int k = 0; k < KO; ++k) {
             if (k < Cout) {
-              const float* wr = pl.stream_w ? wts + ((k * cn + c) * FS + i) * FS
+              const float* wr = SW ? wts + ((k * cn + c) * FS + i) * FS
                                             : wts + ((k * Cin + c0 + c) * FS + i) * FS;
 #pragma unroll
               for (int j = 0; j < FS; ++j) {
@@ -270,14 +271,18 @@ bool plan(const FwdArgs& a, DensePlan* pl) {
   return true;
 }
 
-template <int FS, int KO>
-hipError_t launch_as(const FwdArgs& a, const DensePlan& pl, hipStream_t st) {
-  const void* fn = reinterpret_cast<const void*>(fwd_dense_small_kernel<FS, KO>);
+template <int FS, int KO, bool SW>
+hipError_t launch_sw(const FwdArgs& a, const DensePlan& pl, hipStream_t st) {
+  const void* fn = reinterpret_cast<const void*>(fwd_dense_small_kernel<FS, KO, SW>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds_bytes);
   if (e != hipSuccess) return e;
   const unsigned grid = 8u * ((pl.ntiles + 7) / 8);
-  fwd_dense_small_kernel<FS, KO><<<grid, kThreads, pl.lds_bytes, st>>>(a, pl);
+  fwd_dense_small_kernel<FS, KO, SW><<<grid, kThreads, pl.lds_bytes, st>>>(a, pl);
   return hipGetLastError();
+}
+template <int FS, int KO>
+hipError_t launch_as(const FwdArgs& a, const DensePlan& pl, hipStream_t st) {
+  return pl.stream_w ? launch_sw<FS, KO, true>(a, pl, st) : launch_sw<FS, KO, false>(a, pl, st);
 }
 
 template <int FS>
@@ -293,6 +298,14 @@ hipError_t launch_ko(const FwdArgs& a, const DensePlan& pl, hipStream_t st) {
 bool fwd_dense_small_supported(const FwdArgs& a) {
   DensePlan pl;
   return plan(a, &pl);
+}
+
+bool fwd_dense_small_plan_info(const FwdArgs& a, long* tiles, size_t* lds_bytes) {
+  DensePlan pl;
+  if (!plan(a, &pl)) return false;
+  *tiles = (long)pl.ntiles * pl.tpw;
+  *lds_bytes = pl.lds_bytes;
+  return true;
 }
 
 hipError_t fwd_dense_small_launch(const FwdArgs& a, hipStream_t st) {
