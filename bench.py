@@ -3,6 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--no-cpu]
                     [--settle-ms MS] [--shape PASS,N,C,H,W,pad,T,Y,R [--stride S]]
+                    [--filter-variant V]
 
 A step is one launch of the workload's pass (default: the forward pass of the
 ResNet-stage workload N=32, C=K=256, 56x56, 3x3, R=32) on synthetic inputs that
@@ -74,6 +75,9 @@ def main():
     ap.add_argument("--cold-only", action="store_true",
                     help="run only the rotating leg (profiling: every launch of the process "
                          "then streams from and to HBM); prints that leg's figures")
+    ap.add_argument("--filter-variant", type=int, default=-1,
+                    help="backward-filter workloads: run this variant (0 general, 1 four launches, "
+                         "2 three launches) instead of the library's choice")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-passes", action="store_true", help="skip the five-workload table")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -194,8 +198,11 @@ def main():
                           "GB/s": round(nbytes / cus / 1e3, 1),
                           "hbm_frac": round(nbytes / cus / 1e3 / HBM_PEAK_GBS, 4)}))
         return
-    plan = cp4.plan_query(cp4.capi.shape_for((w.N, w.C, w.H, w.W), *[d[k] for k in FACTORS],
-                                             w.pad), w.pass_)
+    shape = cp4.capi.shape_for((w.N, w.C, w.H, w.W), *[d[k] for k in FACTORS], w.pad)
+    if args.filter_variant >= 0:
+        assert w.pass_ == "backward_filter", "--filter-variant goes with a backward-filter workload"
+        cp4.set_tuned_filter_choice(shape, args.filter_variant)
+    plan = cp4.plan_query(shape, w.pass_)
     us, wall = timed(w, d, args.warmup, args.steps, args.settle_ms)
     value = nbytes * args.steps / wall / 1e9
     achieved = nbytes / us / 1e3
