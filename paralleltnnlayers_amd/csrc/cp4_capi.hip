@@ -734,6 +734,43 @@ cp4_status cp4_conv2d_backward_data_f16(const cp4_shape* shape, const void* dy_f
   return CP4_OK;
 }
 
+namespace {
+// Which backward-filter variants can run a shape whose operands and workspace are aligned to
+// `align` bytes (variant 1 and the rank-tile route need 8, variant 2 needs 16, the rank-tile
+// route a workspace on a 256-byte boundary as well), and the one a launch picks: the tuned
+// entry if it can run, else the three-launch variant where it is preferred or the only
+// matrix-core one, else four launches, else the general kernel.
+struct FilterRoutes {
+  bool tiles_ok, mfma_ok, fused_ok;
+};
+FilterRoutes filter_routes(const cp4_shape& s, bool aligned8, bool aligned16, bool ws256) {
+  FilterRoutes r;
+  r.tiles_ok = filter_rank_tiles_supported(s) && aligned8 && ws256;
+  r.mfma_ok = (cp4::bwd_filter_mfma_supported(s) && aligned8) || r.tiles_ok;
+  // more than 64 ranks: the fused variant runs per rank tile when every tile qualifies
+  const bool fused_tiles =
+      r.tiles_ok && cp4::bwd_filter_fused_supported(filter_rank_tile(s, 0)) &&
+      cp4::bwd_filter_fused_supported(
+          filter_rank_tile(s, (s.Rank - 1) / kFilterRankTile * kFilterRankTile));
+  r.fused_ok = aligned16 && (cp4::bwd_filter_fused_supported(s) || fused_tiles);
+  return r;
+}
+int default_filter_variant(const cp4_shape& s, const FilterRoutes& r) {
+  {
+    std::lock_guard<std::mutex> lk(g_tune_mu);
+    auto it = g_tuned_filter.find(key_of(s));
+    if (it != g_tuned_filter.end() &&
+        (it->second == 0 || (it->second == 1 && r.mfma_ok) || (it->second == 2 && r.fused_ok)))
+      return it->second;
+  }
+  const bool prefer_fused =
+      r.fused_ok && (cp4::bwd_filter_fused_preferred(
+                         s.Rank > kFilterRankTile ? filter_rank_tile(s, 0) : s) ||
+                     !r.mfma_ok);
+  return prefer_fused ? 2 : (r.mfma_ok ? 1 : 0);
+}
+}  // namespace
+
 cp4_status cp4_conv2d_backward_filter(const cp4_shape* shape, const float* x,
                                       const float* dy, const float* FK,
                                       const float* FC, const float* FH,
@@ -769,38 +806,19 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
   if (!workspace || workspace_bytes < filter_workspace(s))
     return fail(CP4_ERR_WORKSPACE,
                 "workspace smaller than cp4_conv2d_backward_filter_workspace_bytes");
-  const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) |
-                         reinterpret_cast<uintptr_t>(workspace)) & 7) == 0;
-  const bool tiles_ok = filter_rank_tiles_supported(s) && aligned &&
-                        (reinterpret_cast<uintptr_t>(workspace) & 255) == 0;
-  const bool mfma_ok = (cp4::bwd_filter_mfma_supported(s) && aligned) || tiles_ok;
-  const bool aligned16 = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) |
-                           reinterpret_cast<uintptr_t>(workspace)) & 15) == 0;
-  // more than 64 ranks: the fused variant runs per rank tile when every tile qualifies
-  const bool fused_tiles = tiles_ok && cp4::bwd_filter_fused_supported(filter_rank_tile(s, 0)) &&
-                           cp4::bwd_filter_fused_supported(filter_rank_tile(
-                               s, (s.Rank - 1) / kFilterRankTile * kFilterRankTile));
-  const bool fused_ok = aligned16 && (cp4::bwd_filter_fused_supported(s) || fused_tiles);
-  if (variant > 2 || (variant == 1 && !mfma_ok) || (variant == 2 && !fused_ok))
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) |
+                         reinterpret_cast<uintptr_t>(workspace);
+  const FilterRoutes routes = filter_routes(s, (bits & 7) == 0, (bits & 15) == 0,
+                                            (reinterpret_cast<uintptr_t>(workspace) & 255) == 0);
+  const bool tiles_ok = routes.tiles_ok;
+  if (variant > 2 || (variant == 1 && !routes.mfma_ok) || (variant == 2 && !routes.fused_ok))
     return fail(CP4_ERR_UNSUPPORTED, "backward-filter variant cannot run this shape");
   cp4::BwdFilterArgs a{};
   a.x = x; a.dy = dy; a.FK = FK; a.FC = FC; a.FH = FH; a.FW = FW;
   a.dFK = dFK; a.dFC = dFC; a.dFH = dFH; a.dFW = dFW; a.workspace = workspace;
   a.N = s.N; a.C = s.C; a.T = s.T; a.H = s.H; a.W = s.W; a.pad = s.pad;
   a.Y = s.Y; a.X = s.X; a.R = s.Rank;
-  if (variant < 0) {
-    std::lock_guard<std::mutex> lk(g_tune_mu);
-    auto it = g_tuned_filter.find(key_of(s));
-    if (it != g_tuned_filter.end() &&
-        (it->second == 0 || (it->second == 1 && mfma_ok) || (it->second == 2 && fused_ok)))
-      variant = it->second;
-  }
-  if (variant < 0) {
-    const bool prefer_fused =
-        fused_ok && (cp4::bwd_filter_fused_preferred(s.Rank > kFilterRankTile ? filter_rank_tile(s, 0) : s) ||
-                     !mfma_ok);
-    variant = prefer_fused ? 2 : (mfma_ok ? 1 : 0);
-  }
+  if (variant < 0) variant = default_filter_variant(s, routes);
   if (variant >= 1 && tiles_ok) {
     float* cf = static_cast<float*>(workspace);                 // compact factors of a tile
     float* cg = cf + filter_rank_tile_floats(s);                // compact gradients
@@ -1445,28 +1463,7 @@ cp4_status cp4_plan_query(const cp4_shape* shape, int pass, int* variant, int* s
   int v = -1, rows = 0, wgs = 0;
   if (pass == 2) {
     // the choice for operands aligned as every allocator returns them
-    const cp4_shape& s = *shape;
-    const bool tiles_ok = filter_rank_tiles_supported(s);
-    const bool mfma_ok = cp4::bwd_filter_mfma_supported(s) || tiles_ok;
-    const bool fused_ok =
-        cp4::bwd_filter_fused_supported(s) ||
-        (tiles_ok && cp4::bwd_filter_fused_supported(filter_rank_tile(s, 0)) &&
-         cp4::bwd_filter_fused_supported(
-             filter_rank_tile(s, (s.Rank - 1) / kFilterRankTile * kFilterRankTile)));
-    {
-      std::lock_guard<std::mutex> lk(g_tune_mu);
-      auto it = g_tuned_filter.find(key_of(s));
-      if (it != g_tuned_filter.end() &&
-          (it->second == 0 || (it->second == 1 && mfma_ok) || (it->second == 2 && fused_ok)))
-        v = it->second;
-    }
-    if (v < 0) {
-      const bool prefer_fused =
-          fused_ok && (cp4::bwd_filter_fused_preferred(
-                           s.Rank > kFilterRankTile ? filter_rank_tile(s, 0) : s) ||
-                       !mfma_ok);
-      v = prefer_fused ? 2 : (mfma_ok ? 1 : 0);
-    }
+    v = default_filter_variant(*shape, filter_routes(*shape, true, true, true));
   } else {
     FwdArgs a = pass == 1
         ? backward_data_args(*shape, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr)
