@@ -169,7 +169,12 @@ cp4_status cp4_conv2d_backward_data(const cp4_shape* shape, const float* dy,
  * OVERWRITTEN (the reference's per-factor functions accumulate; the C++
  * wrappers of the same names keep that).  `workspace` must hold at least
  * cp4_conv2d_backward_filter_workspace_bytes(shape) bytes of device memory;
- * its contents are scratch.  Deterministic: no floating-point atomics. */
+ * its contents are scratch.  Deterministic: no floating-point atomics.
+ * The matrix-core variants want x, dy and the workspace on 16-byte boundaries, and
+ * the routes that run them on copies - rank tiles beyond 64 ranks; zero channels
+ * appended where a channel count is odd (on planes of an odd number of pixels: not a
+ * multiple of 16), a first layer's three input channels say - the workspace on a
+ * 256-byte one; operands aligned to less run the general kernel, same results. */
 size_t cp4_conv2d_backward_filter_workspace_bytes(const cp4_shape* shape);
 cp4_status cp4_conv2d_backward_filter(const cp4_shape* shape, const float* x,
                                       const float* dy, const float* FK,

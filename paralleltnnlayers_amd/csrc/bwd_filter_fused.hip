@@ -740,18 +740,22 @@ bool bwd_filter_fused_supported(const cp4_shape& s) {
   return make_fused_plan(s).ok;
 }
 
-// Measured on one MI355X against the four-launch variant over 60 shapes: up to about
-// 40 MB of activations the three-launch variant is ahead (20-27 us against 27-37 us
-// up to 13 MB, 26.6 against 33.6 us at N32 C128 28x28 R16); beyond that its tap step
-// and GEMM no longer overlap the loads of the other workgroups and the four-launch
-// variant streams better (C64 56x56 N32 R16: 65 against 61 us).  On planes of up to
-// 256 pixels with more than 32 ranks the crossing is at about 10 MB (N64 C256 14x14
-// R64: 36.6 against 34.5 us).
+// Measured on one MI355X against the four-launch variant over 150 shapes (the library's
+// own timed loop): the three-launch variant is ahead wherever the batch holds up to
+// 25,000 pixels or so (17-20 us against 21-25 on the smallest layers, N16 C128 28x28
+// R16 19.9 against 26.6, N8 C256 56x56 R32 36.3 against 38.5), and on planes of up to
+// 32 x 32 pixels up to 65,000 (N64 C256 28x28 R64: 93.7 against 105.9 us).  Beyond
+// that, and from 50,000 pixels on planes of 56 x 56 and more, its plane copy, tap step
+// and GEMM - one after the other in a workgroup that has the compute unit to itself -
+// cost more than the launch and the planes they save (N16 C64 56x56 R16: 37.3 against
+// 32.7 us, N8 C32 112x112: 63.9 against 44.9).  On planes of up to 256 pixels with more
+// than 32 ranks one partial set per image outweighs the planes from about 10 MB of
+// activations on (N64 C256 14x14 R64: 36.3 against 34.0 us).
 bool bwd_filter_fused_preferred(const cp4_shape& s) {
   if (!bwd_filter_fused_supported(s)) return false;
-  const double mb = 4e-6 * s.N * ((double)s.C + s.T) * s.H * s.W;
-  if (s.H * s.W <= 256 && s.Rank > 32) return mb <= 10.;
-  return mb <= 40.;
+  const long plane = (long)s.H * s.W, pixels = plane * s.N;
+  if (plane <= 256 && s.Rank > 32) return 4e-6 * s.N * ((double)s.C + s.T) * plane <= 10.;
+  return pixels <= 25088 || (plane <= 1024 && pixels <= 65536);
 }
 
 size_t bwd_filter_fused_workspace_bytes(const cp4_shape& s) {

@@ -445,8 +445,58 @@ size_t filter_rank_tile_floats(const cp4_shape& s) {   // compact factors or gra
   return align256((size_t)(s.T + s.C + s.Y + s.X) * kFilterRankTile * sizeof(float)) / sizeof(float);
 }
 
+// Channel counts the matrix-core backward-filter kernels do not take - odd ones, and on
+// planes of an odd number of pixels anything but multiples of 16 (a first layer's three
+// input channels, a single output channel) - run them all the same on copies of x and dy
+// with zero channels appended and factors with zero rows appended: the appended channels
+// add nothing to A, G3 or the tap gradients, and their own gradient rows are dropped.
+// The copies cost a pass over x and dy; the general kernel such a layer would otherwise
+// run takes 50 to 1000 times the forward pass (N8 C3 K1 512x512 R16: 14.5 ms).
+cp4_shape filter_padded_shape(const cp4_shape& s) {
+  const unsigned m = ((size_t)s.H * s.W) & 1 ? 16 : 2;
+  cp4_shape t = s;
+  t.C = (s.C + m - 1) / m * m;
+  t.T = (s.T + m - 1) / m * m;
+  return t;
+}
+// (Also on the smallest layers: N2 C3 K5 8x8 R4 24.8 against 42.3 us.)
+bool filter_pad_route(const cp4_shape& s) {
+  if (cp4::bwd_filter_mfma_supported(s) || filter_rank_tiles_supported(s)) return false;
+  const cp4_shape t = filter_padded_shape(s);
+  if (t.C == s.C && t.T == s.T) return false;
+  if (t.C > 65535 || t.T > 65535) return false;
+  return cp4::bwd_filter_mfma_supported(t) || filter_rank_tiles_supported(t);
+}
+// Floats at the head of the workspace: padded x, dy (only where a channel is appended),
+// factors FC, FK and gradients dFC, dFK, each on a 256-byte boundary.
+struct FilterPadLayout {
+  size_t x, dy, fc, fk, gfc, gfk, head;   // offsets in floats; head = floats before the inner workspace
+};
+FilterPadLayout filter_pad_layout(const cp4_shape& s, const cp4_shape& t) {
+  FilterPadLayout l{};
+  const size_t hw = (size_t)s.H * s.W;
+  auto take = [&](size_t floats) {
+    const size_t at = l.head;
+    l.head += align256(floats * sizeof(float)) / sizeof(float);
+    return at;
+  };
+  l.x = take(t.C != s.C ? (size_t)s.N * t.C * hw : 0);
+  l.dy = take(t.T != s.T ? (size_t)s.N * t.T * hw : 0);
+  l.fc = take((size_t)t.C * s.Rank);
+  l.fk = take((size_t)t.T * s.Rank);
+  l.gfc = take((size_t)t.C * s.Rank);
+  l.gfk = take((size_t)t.T * s.Rank);
+  return l;
+}
+
 // One workspace size serves every backward-filter variant.
 size_t filter_workspace(const cp4_shape& s) {
+  if (filter_pad_route(s)) {
+    const cp4_shape t = filter_padded_shape(s);
+    const size_t general = cp4::bwd_filter_workspace_bytes(s);
+    const size_t padded = filter_pad_layout(s, t).head * sizeof(float) + filter_workspace(t);
+    return padded > general ? padded : general;
+  }
   size_t b = cp4::bwd_filter_workspace_bytes(s);
   if (cp4::bwd_filter_mfma_supported(s)) {
     const size_t m = cp4::bwd_filter_mfma_workspace_bytes(s);
@@ -818,6 +868,40 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
   a.dFK = dFK; a.dFC = dFC; a.dFH = dFH; a.dFW = dFW; a.workspace = workspace;
   a.N = s.N; a.C = s.C; a.T = s.T; a.H = s.H; a.W = s.W; a.pad = s.pad;
   a.Y = s.Y; a.X = s.X; a.R = s.Rank;
+  if (variant < 0 && filter_pad_route(s) && (bits & 15) == 0 &&
+      (reinterpret_cast<uintptr_t>(workspace) & 255) == 0) {
+    bool tuned_general = false;
+    {
+      std::lock_guard<std::mutex> lk(g_tune_mu);
+      auto it = g_tuned_filter.find(key_of(s));
+      tuned_general = it != g_tuned_filter.end() && it->second == 0;
+    }
+    if (!tuned_general) {
+      // zero channels appended: the matrix-core variants on copies (see filter_padded_shape)
+      const cp4_shape t = filter_padded_shape(s);
+      const FilterPadLayout l = filter_pad_layout(s, t);
+      float* w = static_cast<float*>(workspace);
+      const size_t hw = (size_t)s.H * s.W;
+      const float *xp = x, *dyp = dy;
+      if (t.C != s.C) {
+        CP4_HIP(cp4::pad_rows_launch(x, w + l.x, s.N, s.C, t.C, hw, st));
+        xp = w + l.x;
+      }
+      if (t.T != s.T) {
+        CP4_HIP(cp4::pad_rows_launch(dy, w + l.dy, s.N, s.T, t.T, hw, st));
+        dyp = w + l.dy;
+      }
+      CP4_HIP(cp4::pad_rows_launch(FC, w + l.fc, 1, s.C, t.C, s.Rank, st));
+      CP4_HIP(cp4::pad_rows_launch(FK, w + l.fk, 1, s.T, t.T, s.Rank, st));
+      rc = cp4_conv2d_backward_filter_variant(&t, xp, dyp, w + l.fk, w + l.fc, FH, FW, w + l.gfk,
+                                              w + l.gfc, dFH, dFW, w + l.head,
+                                              workspace_bytes - l.head * sizeof(float), -1, stream);
+      if (rc != CP4_OK) return rc;
+      CP4_HIP(cp4::copy_f32_launch(dFC, w + l.gfc, (size_t)s.C * s.Rank, st));
+      CP4_HIP(cp4::copy_f32_launch(dFK, w + l.gfk, (size_t)s.T * s.Rank, st));
+      return CP4_OK;
+    }
+  }
   if (variant < 0) variant = default_filter_variant(s, routes);
   if (variant >= 1 && tiles_ok) {
     float* cf = static_cast<float*>(workspace);                 // compact factors of a tile
@@ -1464,6 +1548,10 @@ cp4_status cp4_plan_query(const cp4_shape* shape, int pass, int* variant, int* s
   if (pass == 2) {
     // the choice for operands aligned as every allocator returns them
     v = default_filter_variant(*shape, filter_routes(*shape, true, true, true));
+    if (v == 0 && filter_pad_route(*shape)) {   // runs on copies with zero channels appended
+      const cp4_shape t = filter_padded_shape(*shape);
+      v = default_filter_variant(t, filter_routes(t, true, true, true));
+    }
   } else {
     FwdArgs a = pass == 1
         ? backward_data_args(*shape, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr)

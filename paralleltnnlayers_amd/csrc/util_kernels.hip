@@ -65,6 +65,23 @@ __global__ __launch_bounds__(256) void copy_f32x4_kernel(
        i += (size_t)gridDim.x * 256)
     dst[i] = src[i];
 }
+// dst[g][r][e] = r < rows ? src[g][r][e] : 0 for r < rows_padded: matrices or image
+// stacks with zero rows (channels) appended.  V = float4 when rows are whole quads.
+template <class V>
+__global__ __launch_bounds__(256) void pad_rows_kernel(V* __restrict__ dst,
+                                                       const V* __restrict__ src, size_t groups,
+                                                       size_t rows, size_t rows_padded,
+                                                       size_t row_elems) {
+  const size_t total = groups * rows_padded * row_elems;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (size_t)gridDim.x * 256) {
+    const size_t e = i % row_elems, gr = i / row_elems;
+    const size_t r = gr % rows_padded, g = gr / rows_padded;
+    V v{};
+    if (r < rows) v = src[(g * rows + r) * row_elems + e];
+    dst[i] = v;
+  }
+}
 __global__ __launch_bounds__(256) void copy_f32_kernel(
     float* __restrict__ dst, const float* __restrict__ src, size_t lo, size_t n) {
   const size_t i = lo + (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -364,6 +381,20 @@ hipError_t cp3_fold_launch(const cp4_shape& s, const float* dFK, const float* dF
 hipError_t transpose_f32_launch(const float* src, float* dst, int rows, int cols,
                                 hipStream_t st) {
   transpose_f32_kernel<<<grid_for((size_t)rows * cols, 4096), 256, 0, st>>>(src, dst, rows, cols);
+  return hipGetLastError();
+}
+
+hipError_t pad_rows_launch(const float* src, float* dst, size_t groups, size_t rows,
+                           size_t rows_padded, size_t row_elems, hipStream_t st) {
+  const size_t total = groups * rows_padded * row_elems;
+  if (total == 0) return hipSuccess;
+  if ((row_elems & 3) == 0 && (((uintptr_t)dst | (uintptr_t)src) & 15) == 0)
+    pad_rows_kernel<float4><<<grid_for(total / 4, 2048), 256, 0, st>>>(
+        reinterpret_cast<float4*>(dst), reinterpret_cast<const float4*>(src), groups, rows,
+        rows_padded, row_elems / 4);
+  else
+    pad_rows_kernel<float><<<grid_for(total, 2048), 256, 0, st>>>(dst, src, groups, rows,
+                                                                  rows_padded, row_elems);
   return hipGetLastError();
 }
 

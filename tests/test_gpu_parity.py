@@ -248,6 +248,47 @@ def test_edge_shapes(cp4, oracle, dims):
             assert_gradient_close(host(g), wnt, f"d{k} variant {variant}")
 
 
+# (N, C, H, W, pad, T, Y, R): channel counts the matrix-core backward-filter kernels do not
+# take as they are
+PADDED = [
+    (2, 3, 12, 16, 1, 5, 3, 4),      # odd C and T on an even plane: one zero channel appended to each
+    (3, 5, 9, 7, 1, 7, 3, 6),        # odd plane: padded to 16 channels
+    (2, 3, 10, 10, 1, 1, 3, 70),     # three channels to one, more than 64 ranks: padding, then rank tiles
+    (1, 3, 24, 40, 2, 16, 5, 16),    # only x is copied (T is even)
+    (4, 16, 15, 15, 1, 20, 3, 8),    # odd plane, only dy is copied
+]
+
+
+@pytest.mark.parametrize("dims", PADDED, ids=lambda d: "x".join(map(str, d)))
+def test_backward_filter_with_padded_channels(cp4, oracle, dims):
+    """The library's choice runs these layers on the matrix cores, on copies of x / dy with
+    zero channels appended (the general kernel takes 50 to 1000 times the forward pass on a
+    first layer); a workspace off the 256-byte boundary falls back to the general kernel.
+    Both against the oracle."""
+    N, C, H, W, pad, T, Y, R = dims
+    rng = np.random.default_rng(sum(dims))
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    dy = rng.standard_normal((N, T, H, W)).astype(np.float32)
+    fac = [rng.standard_normal((d, R)).astype(np.float32) / np.sqrt(R) for d in (T, C, Y, Y)]
+    f = [dev(v) for v in fac]
+    want = oracle.backward_filter(x, dy, *fac, pad)
+    s = cp4.capi.shape_for(x.shape, *f, pad)
+    cp4.tune_clear()
+    assert cp4.plan_query(s, "backward_filter")["variant"] != cp4.backward_filter_variants()[0]
+    nbytes = cp4.backward_filter_workspace_bytes(s)
+    buf = torch.empty(nbytes + 512, dtype=torch.uint8, device="cuda")
+    off = (-buf.data_ptr()) % 256
+    for shift, label in ((0, "padded route"), (16, "workspace off the boundary")):
+        ws = buf[off + shift:off + shift + nbytes].view(torch.float32)
+        got = cp4.conv2d_backward_filter(dev(x), dev(dy), *f, pad=pad, workspace=ws)
+        for g, wnt, k in zip(got, want, FACTORS):
+            assert_gradient_close(host(g), wnt, f"d{k} {label}")
+    again = cp4.conv2d_backward_filter(dev(x), dev(dy), *f, pad=pad)
+    for g1, g2 in zip(got, again):
+        assert g1.shape == g2.shape
+    cp4.device_status()
+
+
 def test_split_role_schedule_at_scale(cp4, oracle):
     """Twice as many workgroups as compute units, five 64-pixel groups per strip,
     at most 16 ranks and 4 channel blocks: tap waves and contraction waves of a
