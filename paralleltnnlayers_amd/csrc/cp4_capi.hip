@@ -164,33 +164,53 @@ struct Variant {
   bool (*supported)(const FwdArgs&);
   hipError_t (*launch)(const FwdArgs&, hipStream_t);
 };
-// More than 32 ranks on the producer / consumer kernel (which holds 32): the sum
-// over ranks splits, so the kernel runs on ranks [0, 32), then on [32, 64) with
-// y +=, and so on - the factor pointers moved 32 columns in per pass, the row
-// stride unchanged.  Every pass reads x again (and y, after the first).
-constexpr int kMaxRankPasses = 8;     // ranks up to 256
+// More than 32 ranks or more than 768 input channels on the producer / consumer kernel
+// (which holds 32 and 768): the sum over ranks splits, and so does the sum over input
+// channels, so the kernel runs on ranks [0, 32) of the first channels, then with y += on
+// the next 32 ranks, and so on through every (channel slice, rank tile) pair - the factor
+// pointers moved 32 columns in per rank tile (row stride unchanged) and a slice's rows
+// down, x moved a slice's planes in (image stride unchanged).  Every pass reads its slice
+// of x again (and y, after the first).  Without the channel slices a layer with 1024
+// input channels - or the backward-data pass of one with 1000 outputs - ran the general
+// VALU kernel (N4 C512 K1000 32x32 R64 backward-data: 3.3 ms).
+constexpr int kMaxPasses = 16;        // rank tiles x channel slices
+constexpr int kPassMaxChannels = 768;   // one pass up to here ...
+constexpr int kSliceMaxChannels = 512;  // ... slices no wider than this (98 KB of factor fragments in LDS)
 int rank_passes(const FwdArgs& a) { return (a.R + 31) / 32; }
-FwdArgs rank_pass(const FwdArgs& a, int pass) {
+int channel_slices(const FwdArgs& a) {
+  return a.Cin <= kPassMaxChannels ? 1 : (a.Cin + kSliceMaxChannels - 1) / kSliceMaxChannels;
+}
+int slice_channels(const FwdArgs& a) {          // channels per slice, a multiple of 16
+  const int n = channel_slices(a);
+  return ((a.Cin + n - 1) / n + 15) / 16 * 16;
+}
+FwdArgs pass_args(const FwdArgs& a, int slice, int tile) {
   FwdArgs b = a;
   b.ldf = a.R;
-  const int r0 = 32 * pass;
+  const int r0 = 32 * tile, c0 = slice_channels(a) * slice;
   b.R = a.R - r0 < 32 ? a.R - r0 : 32;
-  b.Fin += r0; b.Fout += r0; b.FH += r0; b.FW += r0;
-  b.accumulate = pass > 0;
+  b.Cin = a.Cin - c0 < slice_channels(a) ? a.Cin - c0 : slice_channels(a);
+  b.ldx = (size_t)a.Cin * a.H * a.W;
+  b.x = a.x + (size_t)c0 * a.H * a.W;
+  b.Fin += (size_t)c0 * a.R + r0; b.Fout += r0; b.FH += r0; b.FW += r0;
+  b.accumulate = slice > 0 || tile > 0;
   return b;
 }
 bool fwd_pipe2_supported(const FwdArgs& a) {
-  if (a.R <= 32 || rank_passes(a) > kMaxRankPasses || a.ldf || a.accumulate || a.bias || a.act)
+  if ((a.R <= 32 && a.Cin <= kPassMaxChannels) || rank_passes(a) * channel_slices(a) > kMaxPasses ||
+      a.ldf || a.ldx || a.accumulate || a.bias || a.act)
     return false;
-  // (the passes differ in their rank count only: the first and the last decide)
-  return cp4::fwd_pipe_rankpass_supported(rank_pass(a, 0)) &&
-         cp4::fwd_pipe_rankpass_supported(rank_pass(a, rank_passes(a) - 1));
+  // (the passes differ in their rank and channel counts only: the first and the last decide)
+  return cp4::fwd_pipe_rankpass_supported(pass_args(a, 0, 0)) &&
+         cp4::fwd_pipe_rankpass_supported(
+             pass_args(a, channel_slices(a) - 1, rank_passes(a) - 1));
 }
 hipError_t fwd_pipe2_launch(const FwdArgs& a, hipStream_t st) {
-  for (int p = 0; p < rank_passes(a); ++p) {
-    const hipError_t e = cp4::fwd_pipe_rankpass_launch(rank_pass(a, p), st);
-    if (e != hipSuccess) return e;
-  }
+  for (int t = 0; t < rank_passes(a); ++t)
+    for (int c = 0; c < channel_slices(a); ++c) {
+      const hipError_t e = cp4::fwd_pipe_rankpass_launch(pass_args(a, c, t), st);
+      if (e != hipSuccess) return e;
+    }
   return hipSuccess;
 }
 

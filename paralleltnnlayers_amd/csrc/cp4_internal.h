@@ -27,10 +27,13 @@ struct FwdArgs {
   // (the caller runs bias_act_launch after the others).
   const float* bias;  // [Cout] or null
   int act;            // 0: none, 1: max(., 0)
-  // Rank passes (rank-pass build of the producer / consumer kernel only): the factor pointers may address
-  // a column block of wider matrices - ldf is their row stride in floats (0: R) -
-  // and accumulate != 0 adds to y instead of overwriting it.
+  // Rank and channel passes (rank-pass build of the producer / consumer kernel only): the
+  // factor pointers may address a column block of wider matrices - ldf is their row
+  // stride in floats (0: R) -, x a slice of Cin channels out of wider images - ldx is
+  // the distance between images in elements (0: Cin * H * W) - and accumulate != 0 adds
+  // to y instead of overwriting it.
   int ldf;
+  size_t ldx;
   int accumulate;
   // 2-D-tap build of the producer / consumer kernel only: depthwise filter
   // [Y, X, R] used instead of the outer product FH x FW (FH, FW unused then).

@@ -324,7 +324,13 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // over channels runs on the scalar unit and no 64-bit vector adds sit between
     // the MFMAs; reads past the last channel (padded channel groups) return 0.
     const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
+#ifdef CP4_PIPE_RANKPASS
+        // (channel passes: this launch's Cin channels are a slice of wider images)
+        const_cast<io_t*>(reinterpret_cast<const io_t*>(a.x) +
+                          (size_t)n * (a.ldx ? (size_t)a.ldx : (size_t)Cin * HW)), 0,
+#else
         const_cast<io_t*>(reinterpret_cast<const io_t*>(a.x) + (size_t)n * Cin * HW), 0,
+#endif
         Cin * HW * kIoBytes, 0x00020000);
     const unsigned sbase =
         (unsigned)(16 * cpq * cq) * (unsigned)HW * (unsigned)kIoBytes;   // uniform byte offset
@@ -1571,7 +1577,7 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 bool fwd_pipe_supported(const FwdArgs& a) {
   if (a.R > kRP || a.Cin > 768) return false;
 #ifndef CP4_PIPE_RANKPASS
-  if (a.accumulate || a.ldf) return false;       // only the rank-pass build has these
+  if (a.accumulate || a.ldf || a.ldx) return false;   // only the rank-pass build has these
 #endif
   if (!fits_int_indexing(a.N, a.H, a.W)) return false;
 #ifdef CP4_PIPE_STRIDED

@@ -594,3 +594,40 @@ def test_ranks_beyond_one_tile(cp4, oracle, R):
         for g, wnt, k in zip(grads, wants, FACTORS):
             assert_gradient_close(host(g), wnt, f"R={R} d{k} variant {variant}")
     cp4.device_status()
+
+
+# (N, C, H, W, pad, T, Y, R): more than 768 channels on the side a pass contracts first
+WIDE_CHANNELS = [
+    (2, 1024, 14, 14, 1, 96, 3, 16),     # forward: two slices of 512 input channels
+    (1, 800, 9, 12, 0, 64, 1, 8),        # 1x1, slices of 400 channels; backward-data is a single pass
+    (2, 64, 10, 10, 1, 1000, 3, 24),     # backward-data: 1000 output channels are its input side
+    (1, 1600, 7, 8, 1, 32, 3, 40),       # three slices x two rank tiles
+]
+
+
+@pytest.mark.parametrize("dims", WIDE_CHANNELS, ids=lambda d: "x".join(map(str, d)))
+def test_channels_beyond_one_slice(cp4, oracle, dims):
+    """The producer / consumer kernel holds 768 input channels: wider layers run it once per
+    channel slice (and rank tile) with y +=, forward and backward-data, instead of the
+    general kernel.  Against the oracle; the library's choice must not be the general kernel."""
+    N, C, H, W, pad, T, Y, R = dims
+    rng = np.random.default_rng(sum(dims))
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    dy = rng.standard_normal((N, T, H, W)).astype(np.float32)
+    fac = [rng.standard_normal((d, R)).astype(np.float32) * np.float32((R * max(C, T)) ** -0.25)
+           for d in (T, C, Y, Y)]
+    f = [dev(v) for v in fac]
+    s = cp4.capi.shape_for(x.shape, *f, pad)
+    cp4.tune_clear()
+    assert cp4.default_variant(s) != "general_valu"
+    assert cp4.default_variant(s, backward_data=True) != "general_valu"
+    want = oracle.forward(x, *fac, pad)
+    assert_activation_close(host(cp4.conv2d_forward(dev(x), *f, pad=pad)), want, "forward")
+    if C > 768:     # the variant by number as well (a small layer's default may be another)
+        v = {n: i for i, n, _ in cp4.forward_variants()}["mfma_bf16x3_pipe_rank_passes"]
+        assert_activation_close(host(cp4.conv2d_forward(dev(x), *f, pad=pad, variant=v)), want,
+                                "forward, channel passes")
+    assert_activation_close(host(cp4.conv2d_backward_data(dev(dy), *f, pad=pad)),
+                            oracle.backward_data(dy, *fac, pad), "backward-data")
+    cp4.device_status()
+
