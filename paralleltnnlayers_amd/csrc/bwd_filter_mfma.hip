@@ -93,6 +93,8 @@ using split::f32x16;
 constexpr int kCT = 256;   // gradient-GEMM workgroup: 4 waves
 [[maybe_unused]] constexpr int kCW = 256;   // contraction workgroup: 4 waves (one per SIMD) sharing one 32-rank factor tile
 [[maybe_unused]] constexpr int kPF = 8;     // channel pairs per prefetch chunk in the contraction
+[[maybe_unused]] constexpr int kSplitSlice = 768;   // channels per launch of the split contraction beyond its fragment tile
+[[maybe_unused]] constexpr int kContractSlice = 1024;   // channels of the fp32 contraction's factor tile in LDS at a time
 
 // ---- 1. Z[n,r,p] = sum_c F[c,r] src[n,c,p] ---------------------------------
 struct ContractArgs {
@@ -100,6 +102,7 @@ struct ContractArgs {
   const float* F[2];     // FC, FK
   float* Z[2];           // A, G3
   int Cin[2];
+  int ldc[2];            // split kernel: channels of an image in memory when Cin is a slice of them (0: Cin)
   int N, R, RP, HW, npb, items;   // items per contraction and rank tile = N * npb
   int ks;   // split kernel: waves per item, each contracting 1/ks of the channels (1, 2 or 4)
   long long* dbg;
@@ -107,63 +110,69 @@ struct ContractArgs {
 
 #ifndef CP4_BWF_IO16
 __global__ __launch_bounds__(kCW) void contract_mfma_kernel(ContractArgs a) {
-  extern __shared__ float Fs[];   // [Cin][32]: the 32-rank tile mb of F, zero-padded
+  extern __shared__ float Fs[];   // [slice of Cin][32]: the 32-rank tile mb of F, zero-padded
   const int which = blockIdx.y, mb = blockIdx.z;
   const int Cin = a.Cin[which], R = a.R, HW = a.HW;
   constexpr int RP = 32;
   const float* F = a.F[which];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hi = lane >> 5;
-  for (int i0 = tid; i0 < Cin * 32; i0 += kCW * 16) {
-    float v[16];
-#pragma unroll
-    for (int u = 0; u < 16; ++u) {
-      const int i = i0 + u * kCW, c = i >> 5, r = 32 * mb + (i & 31);
-      v[u] = (i < Cin * 32 && r < R) ? F[(size_t)c * R + r] : 0.f;
-    }
-#pragma unroll
-    for (int u = 0; u < 16; ++u)
-      if (i0 + u * kCW < Cin * 32) Fs[i0 + u * kCW] = v[u];
-  }
-  __syncthreads();
   const int item = blockIdx.x * (kCW / 64) + wave;   // (image, 64-pixel block)
-  if (item >= a.items) return;
-  const int pb = item % a.npb, n = item / a.npb;
+  const bool active = item < a.items;                 // (idle waves still meet the barriers)
+  const int pb = active ? item % a.npb : 0, n = active ? item / a.npb : 0;
   const int p = pb * 64 + 2 * l32;
-  const bool valid = p < HW;
+  const bool valid = active && p < HW;
   const int pc = valid ? p : HW - 2;
-  const float* xp = a.src[which] + ((size_t)n * Cin + hi) * HW + pc;
   const float* fp = Fs + hi * RP + l32;
   f32x16 acc0 = (f32x16)(0.f), acc1 = (f32x16)(0.f);
-  const int nsteps = Cin >> 1, nchunks = nsteps / kPF;
-  float2 xb0[kPF], xb1[kPF];
-  auto load = [&](float2 (&xb)[kPF], int ch) {
+  // the factor tile goes through LDS a slice of kContractSlice channels at a time
+  for (int c0 = 0; c0 < Cin; c0 += kContractSlice) {
+    const int cs = Cin - c0 < kContractSlice ? Cin - c0 : kContractSlice;
+    if (c0) __syncthreads();                          // every wave is done with the last slice
+    for (int i0 = tid; i0 < cs * 32; i0 += kCW * 16) {
+      float v[16];
 #pragma unroll
-    for (int s = 0; s < kPF; ++s)
-      xb[s] = *reinterpret_cast<const float2*>(xp + (size_t)(2 * (ch * kPF + s)) * HW);
-  };
-  auto compute = [&](const float2 (&xb)[kPF], int ch) {
+      for (int u = 0; u < 16; ++u) {
+        const int i = i0 + u * kCW, c = c0 + (i >> 5), r = 32 * mb + (i & 31);
+        v[u] = (i < cs * 32 && r < R) ? F[(size_t)c * R + r] : 0.f;
+      }
 #pragma unroll
-    for (int s = 0; s < kPF; ++s) {
-      const float f = fp[(ch * kPF + s) * 2 * RP];
-      acc0 = mfma32(f, xb[s].x, acc0);
-      acc1 = mfma32(f, xb[s].y, acc1);
+      for (int u = 0; u < 16; ++u)
+        if (i0 + u * kCW < cs * 32) Fs[i0 + u * kCW] = v[u];
     }
-  };
-  if (nchunks > 0) load(xb0, 0);
-  for (int ch = 0; ch < nchunks; ch += 2) {
-    if (ch + 1 < nchunks) load(xb1, ch + 1);
-    compute(xb0, ch);
-    if (ch + 1 < nchunks) {
-      if (ch + 2 < nchunks) load(xb0, ch + 2);
-      compute(xb1, ch + 1);
+    __syncthreads();
+    if (!active) continue;
+    const float* xp = a.src[which] + ((size_t)n * Cin + c0 + hi) * HW + pc;
+    const int nsteps = cs >> 1, nchunks = nsteps / kPF;
+    float2 xb0[kPF], xb1[kPF];
+    auto load = [&](float2 (&xb)[kPF], int ch) {
+#pragma unroll
+      for (int s = 0; s < kPF; ++s)
+        xb[s] = *reinterpret_cast<const float2*>(xp + (size_t)(2 * (ch * kPF + s)) * HW);
+    };
+    auto compute = [&](const float2 (&xb)[kPF], int ch) {
+#pragma unroll
+      for (int s = 0; s < kPF; ++s) {
+        const float f = fp[(ch * kPF + s) * 2 * RP];
+        acc0 = mfma32(f, xb[s].x, acc0);
+        acc1 = mfma32(f, xb[s].y, acc1);
+      }
+    };
+    if (nchunks > 0) load(xb0, 0);
+    for (int ch = 0; ch < nchunks; ch += 2) {
+      if (ch + 1 < nchunks) load(xb1, ch + 1);
+      compute(xb0, ch);
+      if (ch + 1 < nchunks) {
+        if (ch + 2 < nchunks) load(xb0, ch + 2);
+        compute(xb1, ch + 1);
+      }
     }
-  }
-  for (int st = nchunks * kPF; st < nsteps; ++st) {
-    const float2 xv = *reinterpret_cast<const float2*>(xp + (size_t)(2 * st) * HW);
-    const float f = fp[st * 2 * RP];
-    acc0 = mfma32(f, xv.x, acc0);
-    acc1 = mfma32(f, xv.y, acc1);
+    for (int st = nchunks * kPF; st < nsteps; ++st) {
+      const float2 xv = *reinterpret_cast<const float2*>(xp + (size_t)(2 * st) * HW);
+      const float f = fp[st * 2 * RP];
+      acc0 = mfma32(f, xv.x, acc0);
+      acc1 = mfma32(f, xv.y, acc1);
+    }
   }
   if (valid) {
     float* zn = a.Z[which] + (size_t)n * R * HW + p;
@@ -220,7 +229,8 @@ __global__ __launch_bounds__(kSW) void contract_split_kernel(ContractArgs a) {
   const int pc = p < HW ? p : HW - 1;
   // lane's channel 16*chunk + 8*hi + e
   const int nch = (Cin >> 4) / ks, c0 = part * nch;     // this wave's chunks c0 .. c0 + nch - 1
-  const act_t* xp = a.src[which] + ((size_t)n * Cin + 16 * c0 + 8 * hi) * HW + pc;
+  const act_t* xp = a.src[which] +
+                    ((size_t)n * (a.ldc[which] ? a.ldc[which] : Cin) + 16 * c0 + 8 * hi) * HW + pc;
 #ifdef CP4_BWF_IO16
   using ring_t = unsigned;     // raw 16-bit values, zero-extended
 #else
@@ -1277,16 +1287,17 @@ Plan make_plan(int N, int C, int T, int H, int W, int Y, int X, int R, int pad) 
 
 bool bwd_filter_mfma_supported(const cp4_shape& s) {
   // odd planes need the split contraction (scalar loads): channel counts multiples of 16
+#ifdef CP4_BWF_IO16
+  // the 16-bit builds have the split kernels only, one fragment tile of channels
   const bool odd_plane_ok = (s.C & 15) == 0 && (s.T & 15) == 0 &&
                             (size_t)(s.C > s.T ? s.C : s.T) * 192 <= 160 * 1024;
-#ifdef CP4_BWF_IO16
-  if (!odd_plane_ok) return false;      // the bfloat16 build has the split kernels only
+  if (!odd_plane_ok) return false;
+#else
+  const bool odd_plane_ok = (s.C & 15) == 0 && (s.T & 15) == 0;   // (more channels: in slices)
 #endif
   return s.Rank <= 64 && fits_int_indexing((int)s.N, (int)s.H, (int)s.W) &&
          (((s.H * s.W) & 1) == 0 || odd_plane_ok) && (s.C & 1) == 0 &&
-         (s.T & 1) == 0 &&
-         (size_t)(s.C > s.T ? s.C : s.T) * (s.Rank <= 32 ? 32 : 64) * 4 <= 160 * 1024 &&
-         s.Y + s.X <= 65535;
+         (s.T & 1) == 0 && s.Y + s.X <= 65535;   // (any channel count: the factor tile is sliced)
 }
 
 #ifndef CP4_BWF_IO16
@@ -1347,11 +1358,49 @@ hipError_t bwd_filter_mfma_launch(const BwdFilterArgs& a, hipStream_t st) {
     const long slots = (long)c.items * c.ks;
     contract_split_kernel<<<dim3((unsigned)((slots + kSW / 64 - 1) / (kSW / 64)), 2, p.RP / 32),
                             kSW, smem, st>>>(c);
+#ifndef CP4_BWF_IO16
+  } else if ((a.C & 15) == 0 && (a.T & 15) == 0 && (HW & 1)) {
+    // an odd plane (no float2 rows for the fp32 kernel below) with more channels than
+    // the split kernel's fragment tile holds (853): the sum over channels runs a slice
+    // of up to 768 at a time, each slice's contraction into the idle B plane and added
+    // to its plane in slice order (the planes have R rows against hundreds of channels,
+    // so the extra pass over them is cheap; N8 C2048 K512 7x7: 90 us, general kernel
+    // 1085).  Even planes: one launch of the fp32 kernel, which slices its own factor
+    // tile, is the quicker (N4 C1024 K2048 14x14 R48: 108 against 121 us).
+    c.npb = (HW + 31) / 32;
+    c.items = N * c.npb;
+    c.ks = 1;
+    for (int which = 0; which < 2; ++which) {
+      const int Cin = which ? a.T : a.C;
+      const int nsl = (Cin + kSplitSlice - 1) / kSplitSlice;
+      const int cs = ((Cin + nsl - 1) / nsl + 15) / 16 * 16;
+      float* Z = which ? G3 : A;
+      for (int c0 = 0; c0 < Cin; c0 += cs) {
+        ContractArgs d = c;
+        d.src[0] = (which ? ady : ax) + (size_t)c0 * HW;
+        d.F[0] = (which ? a.FK : a.FC) + (size_t)c0 * R;
+        d.Z[0] = c0 ? B : Z;
+        d.Cin[0] = Cin - c0 < cs ? Cin - c0 : cs;
+        d.ldc[0] = Cin;
+        const size_t smem = (size_t)d.Cin[0] * 192;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_split_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return e;
+        contract_split_kernel<<<dim3((unsigned)((c.items + kSW / 64 - 1) / (kSW / 64)), 1,
+                                     p.RP / 32),
+                                kSW, smem, st>>>(d);
+        if (c0) {
+          e = add_f32_launch(Z, B, (size_t)N * R * HW, st);
+          if (e != hipSuccess) return e;
+        }
+      }
+    }
+#endif
   } else {
 #ifdef CP4_BWF_IO16
     return hipErrorInvalidValue;      // excluded by bwd_filter_mfma_io16_supported
 #else
-    const size_t smem = (size_t)cmax * 32 * sizeof(float);
+    const size_t smem = (size_t)(cmax < kContractSlice ? cmax : kContractSlice) * 32 * sizeof(float);
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_mfma_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
@@ -1736,7 +1785,7 @@ hipError_t contract_one(const float* src, const float* F, float* Z, int Cin, int
   } else {
     c.npb = (HW + 63) / 64;
     c.items = N * c.npb;
-    const size_t smem = (size_t)Cin * 32 * sizeof(float);
+    const size_t smem = (size_t)(Cin < kContractSlice ? Cin : kContractSlice) * 32 * sizeof(float);
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(contract_mfma_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;

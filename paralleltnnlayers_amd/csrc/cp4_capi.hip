@@ -451,15 +451,24 @@ cp4_status run_forward_like(const FwdArgs& a, int variant, hipStream_t st) {
 // so the pass runs once per tile of 64 ranks on compact copies of the factor
 // columns and its gradients are copied back into their columns.
 constexpr unsigned kFilterRankTile = 64;
+// (tiles of 32 ranks where the contraction's 64-rank factor tile of the wider channel
+// side would not fit LDS: more than 640 channels)
+unsigned filter_tile_ranks(const cp4_shape& s) {
+  cp4_shape t = s;
+  t.Rank = kFilterRankTile;
+  return cp4::bwd_filter_mfma_supported(t) ? kFilterRankTile : 32;
+}
 cp4_shape filter_rank_tile(const cp4_shape& s, unsigned r0) {
   cp4_shape t = s;
-  t.Rank = s.Rank - r0 < kFilterRankTile ? s.Rank - r0 : kFilterRankTile;
+  const unsigned tile = filter_tile_ranks(s);
+  t.Rank = s.Rank - r0 < tile ? s.Rank - r0 : tile;
   return t;
 }
 size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
 bool filter_rank_tiles_supported(const cp4_shape& s) {
-  return s.Rank > kFilterRankTile && cp4::bwd_filter_mfma_supported(filter_rank_tile(s, 0)) &&
-         cp4::bwd_filter_mfma_supported(filter_rank_tile(s, (s.Rank - 1) / kFilterRankTile * kFilterRankTile));
+  const unsigned tile = filter_tile_ranks(s);
+  return s.Rank > tile && cp4::bwd_filter_mfma_supported(filter_rank_tile(s, 0)) &&
+         cp4::bwd_filter_mfma_supported(filter_rank_tile(s, (s.Rank - 1) / tile * tile));
 }
 size_t filter_rank_tile_floats(const cp4_shape& s) {   // compact factors or gradients of a tile
   return align256((size_t)(s.T + s.C + s.Y + s.X) * kFilterRankTile * sizeof(float)) / sizeof(float);
@@ -821,7 +830,7 @@ FilterRoutes filter_routes(const cp4_shape& s, bool aligned8, bool aligned16, bo
   const bool fused_tiles =
       r.tiles_ok && cp4::bwd_filter_fused_supported(filter_rank_tile(s, 0)) &&
       cp4::bwd_filter_fused_supported(
-          filter_rank_tile(s, (s.Rank - 1) / kFilterRankTile * kFilterRankTile));
+          filter_rank_tile(s, (s.Rank - 1) / filter_tile_ranks(s) * filter_tile_ranks(s)));
   r.fused_ok = aligned16 && (cp4::bwd_filter_fused_supported(s) || fused_tiles);
   return r;
 }
@@ -835,7 +844,7 @@ int default_filter_variant(const cp4_shape& s, const FilterRoutes& r) {
   }
   const bool prefer_fused =
       r.fused_ok && (cp4::bwd_filter_fused_preferred(
-                         s.Rank > kFilterRankTile ? filter_rank_tile(s, 0) : s) ||
+                         s.Rank > filter_tile_ranks(s) ? filter_rank_tile(s, 0) : s) ||
                      !r.mfma_ok);
   return prefer_fused ? 2 : (r.mfma_ok ? 1 : 0);
 }
@@ -931,7 +940,7 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
     const float* fac[4] = {FK, FC, FH, FW};
     float* grad[4] = {dFK, dFC, dFH, dFW};
     const int rows[4] = {(int)s.T, (int)s.C, (int)s.Y, (int)s.X};
-    for (unsigned r0 = 0; r0 < s.Rank; r0 += kFilterRankTile) {
+    for (unsigned r0 = 0; r0 < s.Rank; r0 += filter_tile_ranks(s)) {
       const cp4_shape t = filter_rank_tile(s, r0);
       const int rt = (int)t.Rank;
       float *f[4], *g[4];

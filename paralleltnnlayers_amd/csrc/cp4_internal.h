@@ -212,6 +212,7 @@ hipError_t rcp_fold_launch(const float* dK, const float* K0, const float* K1, co
 // dst [cols, rows] = transpose of src [rows, cols]
 hipError_t transpose_f32_launch(const float* src, float* dst, int rows, int cols, hipStream_t);
 hipError_t copy_f32_launch(float* dst, const float* src, size_t n, hipStream_t);
+hipError_t add_f32_launch(float* dst, const float* src, size_t n, hipStream_t);   // dst += src
 // dst [groups][rows_padded][row_elems] = src [groups][rows][row_elems] with zero rows appended
 hipError_t pad_rows_launch(const float* src, float* dst, size_t groups, size_t rows,
                            size_t rows_padded, size_t row_elems, hipStream_t);

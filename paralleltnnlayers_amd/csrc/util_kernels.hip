@@ -82,6 +82,11 @@ __global__ __launch_bounds__(256) void pad_rows_kernel(V* __restrict__ dst,
     dst[i] = v;
   }
 }
+__global__ __launch_bounds__(256) void add_f32_kernel(float* __restrict__ dst,
+                                                      const float* __restrict__ src, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+    dst[i] += src[i];
+}
 __global__ __launch_bounds__(256) void copy_f32_kernel(
     float* __restrict__ dst, const float* __restrict__ src, size_t lo, size_t n) {
   const size_t i = lo + (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -395,6 +400,12 @@ hipError_t pad_rows_launch(const float* src, float* dst, size_t groups, size_t r
   else
     pad_rows_kernel<float><<<grid_for(total, 2048), 256, 0, st>>>(dst, src, groups, rows,
                                                                   rows_padded, row_elems);
+  return hipGetLastError();
+}
+
+hipError_t add_f32_launch(float* dst, const float* src, size_t n, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  add_f32_kernel<<<grid_for(n, 2048), 256, 0, st>>>(dst, src, n);
   return hipGetLastError();
 }
 

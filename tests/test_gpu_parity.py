@@ -602,6 +602,7 @@ WIDE_CHANNELS = [
     (1, 800, 9, 12, 0, 64, 1, 8),        # 1x1, slices of 400 channels; backward-data is a single pass
     (2, 64, 10, 10, 1, 1000, 3, 24),     # backward-data: 1000 output channels are its input side
     (1, 1600, 7, 8, 1, 32, 3, 40),       # three slices x two rank tiles
+    (2, 1024, 7, 7, 1, 1360, 3, 24),     # odd plane: backward-filter contracts slice by slice
 ]
 
 
@@ -629,5 +630,11 @@ def test_channels_beyond_one_slice(cp4, oracle, dims):
                                 "forward, channel passes")
     assert_activation_close(host(cp4.conv2d_backward_data(dev(dy), *f, pad=pad)),
                             oracle.backward_data(dy, *fac, pad), "backward-data")
+    # backward-filter: the contraction's factor tile in slices (even planes: inside the fp32
+    # kernel; odd planes with channel counts that are multiples of 16: one launch per slice)
+    assert cp4.plan_query(s, "backward_filter")["variant"] != cp4.backward_filter_variants()[0]
+    grads = cp4.conv2d_backward_filter(dev(x), dev(dy), *f, pad=pad)
+    for g, wnt, k in zip(grads, oracle.backward_filter(x, dy, *fac, pad), FACTORS):
+        assert_gradient_close(host(g), wnt, f"d{k}")
     cp4.device_status()
 
