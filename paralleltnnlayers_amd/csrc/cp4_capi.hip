@@ -1117,6 +1117,32 @@ void set_geometry(FwdArgs& a, const cp4_geometry& g) {
 // where it applies and the matrix tiles are not mostly padding, else the general kernel.
 // (The strided build carries the bias / activation epilogue: a.bias / a.act are applied
 // there; *epilogue_done says whether they were.)
+// The strided build in passes over rank tiles and channel slices (more than 32 ranks or
+// 768 input channels; a downsampling 1x1 layer with 1024 inputs, its backward-data pass
+// with 2048): as fwd_pipe2_* for the reference's geometry, without the epilogue.
+FwdArgs strided_pass_args(const FwdArgs& a, int slice, int tile) {
+  FwdArgs b = pass_args(a, slice, tile);
+  b.bias = nullptr;
+  b.act = 0;
+  return b;
+}
+bool strided_passes_supported(const FwdArgs& a) {
+  if ((a.R <= 32 && a.Cin <= kPassMaxChannels) || rank_passes(a) * channel_slices(a) > kMaxPasses ||
+      a.ldf || a.ldx || a.accumulate)
+    return false;
+  return cp4::fwd_pipe_strided_supported(strided_pass_args(a, 0, 0)) &&
+         cp4::fwd_pipe_strided_supported(
+             strided_pass_args(a, channel_slices(a) - 1, rank_passes(a) - 1));
+}
+hipError_t strided_passes_launch(const FwdArgs& a, hipStream_t st) {
+  for (int t = 0; t < rank_passes(a); ++t)
+    for (int c = 0; c < channel_slices(a); ++c) {
+      const hipError_t e = cp4::fwd_pipe_strided_launch(strided_pass_args(a, c, t), st);
+      if (e != hipSuccess) return e;
+    }
+  return hipSuccess;
+}
+
 cp4_status run_geometry(FwdArgs a, hipStream_t st, bool* epilogue_done = nullptr) {
   if (epilogue_done) *epilogue_done = false;
   if (a.N == 0) return CP4_OK;
@@ -1124,6 +1150,10 @@ cp4_status run_geometry(FwdArgs a, hipStream_t st, bool* epilogue_done = nullptr
   if (cp4::fwd_pipe_strided_supported(a) && a.Cin + a.Cout >= kMatrixMinChannels) {
     CP4_HIP(cp4::fwd_pipe_strided_launch(a, st));
     if (epilogue_done) *epilogue_done = true;
+    return CP4_OK;
+  }
+  if (strided_passes_supported(a)) {
+    CP4_HIP(strided_passes_launch(a, st));
     return CP4_OK;
   }
   if (cp4::fwd_general_supported(a)) {
@@ -1264,6 +1294,12 @@ cp4_status cp4_conv2d_backward_data_ex(const cp4_shape* shape, const cp4_geometr
   if (rc != CP4_OK) return rc;
   const cp4_shape& s = *shape;
   hipStream_t st = as_stream(stream);
+  if (is_reference_geometry(s, *g) && 2 * g->pad_top == s.Y - 1 && 2 * g->pad_left == s.X - 1) {
+    // the reference's own layer: its backward-data pass is this adjoint, and has every variant
+    cp4_shape r = s;
+    r.pad = g->pad_top;
+    return cp4_conv2d_backward_data(&r, dy, FK, FC, FH, FW, dx, stream);
+  }
   // In general: dx[h,w] = sum_{i,j} K[i,j] dyu[h + pad_top - i, w + pad_left - j] with dyu = dy spread
   // out with zeros: a stride-1 pass over dyu with the taps in reverse order, Y - 1 - pad_top
   // zeros before it and an H x W output.
@@ -1282,6 +1318,11 @@ cp4_status cp4_conv2d_backward_data_ex(const cp4_shape* shape, const cp4_geometr
     if (cp4::fwd_pipe_strided_supported(t) && t.Cin + t.Cout >= kMatrixMinChannels) {
       CP4_ARM(t);
       CP4_HIP(cp4::fwd_pipe_strided_launch(t, st));
+      return CP4_OK;
+    }
+    if (strided_passes_supported(t)) {
+      CP4_ARM(t);
+      CP4_HIP(strided_passes_launch(t, st));
       return CP4_OK;
     }
   }

@@ -80,6 +80,12 @@
 #define CP4_PIPE_EPILOGUE 1
 #endif
 
+// Passes over rank tiles and channel slices (FwdArgs::ldf, ldx, accumulate): the rank-pass
+// build and the strided build honour them.
+#if defined(CP4_PIPE_RANKPASS) || defined(CP4_PIPE_STRIDED)
+#define CP4_PIPE_PASSES 1
+#endif
+
 namespace cp4 {
 namespace {
 
@@ -245,7 +251,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   [[maybe_unused]] const int Ho = H, Wo = W, HWo = HW;
 #endif
   const int QA = pl.QA;
-#ifdef CP4_PIPE_RANKPASS
+#ifdef CP4_PIPE_PASSES
   const int ldf = a.ldf ? a.ldf : R;             // row stride of the factor matrices
 #else
   const int ldf = R;
@@ -324,7 +330,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     // over channels runs on the scalar unit and no 64-bit vector adds sit between
     // the MFMAs; reads past the last channel (padded channel groups) return 0.
     const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
-#ifdef CP4_PIPE_RANKPASS
+#ifdef CP4_PIPE_PASSES
         // (channel passes: this launch's Cin channels are a slice of wider images)
         const_cast<io_t*>(reinterpret_cast<const io_t*>(a.x) +
                           (size_t)n * (a.ldx ? (size_t)a.ldx : (size_t)Cin * HW)), 0,
@@ -1067,7 +1073,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         float2 o;
         o.x = v0;
         o.y = v1;
-#ifdef CP4_PIPE_RANKPASS
+#ifdef CP4_PIPE_PASSES
         if (accumulate) {                        // second rank pass: y += (wave-uniform)
           const float2 old = *reinterpret_cast<const float2*>(dst);
           o.x += old.x;
@@ -1081,7 +1087,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #ifdef CP4_PIPE_IO16
         *dst = to_io(v);
 #else
-#ifdef CP4_PIPE_RANKPASS
+#ifdef CP4_PIPE_PASSES
         *dst = accumulate ? *dst + v : v;
 #else
         *dst = v;
@@ -1576,8 +1582,8 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 
 bool fwd_pipe_supported(const FwdArgs& a) {
   if (a.R > kRP || a.Cin > 768) return false;
-#ifndef CP4_PIPE_RANKPASS
-  if (a.accumulate || a.ldf || a.ldx) return false;   // only the rank-pass build has these
+#ifndef CP4_PIPE_PASSES
+  if (a.accumulate || a.ldf || a.ldx) return false;   // only the rank-pass and strided builds have these
 #endif
   if (!fits_int_indexing(a.N, a.H, a.W)) return false;
 #ifdef CP4_PIPE_STRIDED

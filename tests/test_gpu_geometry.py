@@ -95,6 +95,11 @@ MATRIX_CASES = [
     (1, 32, 31, 45, 48, 5, 16, (3, 2), 2),          # unequal strides, 5x5
     (2, 32, 150, 40, 32, 3, 12, 2, "same"),         # many strips (both sweep directions)
     (1, 64, 96, 96, 64, 3, 4, (1, 2), 1),           # stride across only; whole-group consumers
+    # passes of the strided build over channel slices and rank tiles
+    (2, 1024, 14, 14, 96, 1, 16, 2, "same"),        # downsampling 1x1 layer, two slices of 512 channels
+    (2, 64, 14, 14, 1000, 1, 24, 2, "same"),        # its adjoint contracts the 1000 output channels
+    (2, 32, 20, 20, 48, 3, 48, 2, "same"),          # 48 ranks: two rank tiles, forward and adjoint
+    (2, 48, 13, 13, 64, 3, 40, 1, "same"),          # stride 1, the reference's own layer: the plain passes
 ]
 
 
