@@ -1913,6 +1913,25 @@ cp4_status cp3_run(const cp4_shape* shape, const float* in, const float* K0, con
     CP4_HIP(cp4::fwd_pipe_taps2d_launch(a, st));
     return CP4_OK;
   }
+  // more than 32 ranks (or 768 input channels): the same build in passes with y +=, R ranks
+  // in tiles of 32 instead of Y * R expanded ones (N32 C256 K256 56x56 3x3 R48: two passes
+  // against five)
+  auto tap_pass = [&](int slice, int tile) {
+    FwdArgs b = pass_args(a, slice, tile);
+    b.FH = b.FW = nullptr;
+    b.taps2d = a.taps2d + 32 * tile;
+    return b;
+  };
+  if ((a.R > 32 || a.Cin > kPassMaxChannels) && a.W <= 128 && a.Cin + a.Cout >= 24 &&
+      rank_passes(a) * channel_slices(a) <= kMaxPasses &&
+      cp4::fwd_pipe_taps2d_supported(tap_pass(0, 0)) &&
+      cp4::fwd_pipe_taps2d_supported(tap_pass(channel_slices(a) - 1, rank_passes(a) - 1))) {
+    CP4_HIP(cp4::transpose_f32_launch(K2, FK, (int)shape->Rank, (int)shape->T, st));
+    for (int t = 0; t < rank_passes(a); ++t)
+      for (int c = 0; c < channel_slices(a); ++c)
+        CP4_HIP(cp4::fwd_pipe_taps2d_launch(tap_pass(c, t), st));
+    return CP4_OK;
+  }
 
   float* FC = FK + cp3_align(shape->T * Q);
   float* FH = FC + cp3_align(shape->C * Q);

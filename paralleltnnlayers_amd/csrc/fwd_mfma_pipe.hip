@@ -81,8 +81,8 @@
 #endif
 
 // Passes over rank tiles and channel slices (FwdArgs::ldf, ldx, accumulate): the rank-pass
-// build and the strided build honour them.
-#if defined(CP4_PIPE_RANKPASS) || defined(CP4_PIPE_STRIDED)
+// build, the strided build and the 2-D-tap build honour them.
+#if defined(CP4_PIPE_RANKPASS) || defined(CP4_PIPE_STRIDED) || defined(CP4_PIPE_TAPS2D)
 #define CP4_PIPE_PASSES 1
 #endif
 
@@ -1583,7 +1583,7 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 bool fwd_pipe_supported(const FwdArgs& a) {
   if (a.R > kRP || a.Cin > 768) return false;
 #ifndef CP4_PIPE_PASSES
-  if (a.accumulate || a.ldf || a.ldx) return false;   // only the rank-pass and strided builds have these
+  if (a.accumulate || a.ldf || a.ldx) return false;   // only the rank-pass, strided and 2-D-tap builds have these
 #endif
   if (!fits_int_indexing(a.N, a.H, a.W)) return false;
 #ifdef CP4_PIPE_STRIDED

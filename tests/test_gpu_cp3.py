@@ -70,6 +70,8 @@ NATIVE = [
     (3, 40, 13, 13, 3, 21, 72),    # odd plane, ragged channels and ranks
     (1, 320, 14, 14, 3, 12, 300),  # factor fragments in LDS
     (2, 16, 20, 20, 1, 8, 24),     # 1x1, one-chunk producers
+    (2, 64, 20, 20, 3, 40, 48),    # 40 ranks: two passes of the 2-D-tap build with y +=
+    (1, 1024, 10, 10, 3, 12, 32),  # 1024 input channels: two channel slices
 ]
 
 
