@@ -196,22 +196,32 @@ FwdArgs pass_args(const FwdArgs& a, int slice, int tile) {
   b.accumulate = slice > 0 || tile > 0;
   return b;
 }
-bool fwd_pipe2_supported(const FwdArgs& a) {
+// A build of the kernel that honours the pass arguments, run over every (channel slice,
+// rank tile) pair of a layer it cannot take in one launch.
+struct PassBuild {
+  bool (*supported)(const FwdArgs&);
+  hipError_t (*launch)(const FwdArgs&, hipStream_t);
+};
+bool passes_supported(const FwdArgs& a, const PassBuild& b) {
   if ((a.R <= 32 && a.Cin <= kPassMaxChannels) || rank_passes(a) * channel_slices(a) > kMaxPasses ||
       a.ldf || a.ldx || a.accumulate || a.bias || a.act)
     return false;
   // (the passes differ in their rank and channel counts only: the first and the last decide)
-  return cp4::fwd_pipe_rankpass_supported(pass_args(a, 0, 0)) &&
-         cp4::fwd_pipe_rankpass_supported(
-             pass_args(a, channel_slices(a) - 1, rank_passes(a) - 1));
+  return b.supported(pass_args(a, 0, 0)) &&
+         b.supported(pass_args(a, channel_slices(a) - 1, rank_passes(a) - 1));
 }
-hipError_t fwd_pipe2_launch(const FwdArgs& a, hipStream_t st) {
+hipError_t passes_launch(const FwdArgs& a, const PassBuild& b, hipStream_t st) {
   for (int t = 0; t < rank_passes(a); ++t)
     for (int c = 0; c < channel_slices(a); ++c) {
-      const hipError_t e = cp4::fwd_pipe_rankpass_launch(pass_args(a, c, t), st);
+      const hipError_t e = b.launch(pass_args(a, c, t), st);
       if (e != hipSuccess) return e;
     }
   return hipSuccess;
+}
+constexpr PassBuild kRankPassBuild{cp4::fwd_pipe_rankpass_supported, cp4::fwd_pipe_rankpass_launch};
+bool fwd_pipe2_supported(const FwdArgs& a) { return passes_supported(a, kRankPassBuild); }
+hipError_t fwd_pipe2_launch(const FwdArgs& a, hipStream_t st) {
+  return passes_launch(a, kRankPassBuild, st);
 }
 
 // Order = preference of the untuned heuristic, last to first.
@@ -1113,36 +1123,28 @@ void set_geometry(FwdArgs& a, const cp4_geometry& g) {
   a.sh = (int)g.stride_h; a.sw = (int)g.stride_w; a.pt = (int)g.pad_top; a.pl = (int)g.pad_left;
   a.Ho = (int)g.out_h; a.Wo = (int)g.out_w;
 }
-// A launch with a geometry: the strided build of the producer / consumer kernel
-// where it applies and the matrix tiles are not mostly padding, else the general kernel.
-// (The strided build carries the bias / activation epilogue: a.bias / a.act are applied
-// there; *epilogue_done says whether they were.)
 // The strided build in passes over rank tiles and channel slices (more than 32 ranks or
 // 768 input channels; a downsampling 1x1 layer with 1024 inputs, its backward-data pass
 // with 2048): as fwd_pipe2_* for the reference's geometry, without the epilogue.
-FwdArgs strided_pass_args(const FwdArgs& a, int slice, int tile) {
-  FwdArgs b = pass_args(a, slice, tile);
-  b.bias = nullptr;
-  b.act = 0;
-  return b;
+constexpr PassBuild kStridedPassBuild{cp4::fwd_pipe_strided_supported,
+                                      cp4::fwd_pipe_strided_launch};
+FwdArgs without_epilogue(FwdArgs a) {
+  a.bias = nullptr;
+  a.act = 0;
+  return a;
 }
 bool strided_passes_supported(const FwdArgs& a) {
-  if ((a.R <= 32 && a.Cin <= kPassMaxChannels) || rank_passes(a) * channel_slices(a) > kMaxPasses ||
-      a.ldf || a.ldx || a.accumulate)
-    return false;
-  return cp4::fwd_pipe_strided_supported(strided_pass_args(a, 0, 0)) &&
-         cp4::fwd_pipe_strided_supported(
-             strided_pass_args(a, channel_slices(a) - 1, rank_passes(a) - 1));
+  return passes_supported(without_epilogue(a), kStridedPassBuild);
 }
 hipError_t strided_passes_launch(const FwdArgs& a, hipStream_t st) {
-  for (int t = 0; t < rank_passes(a); ++t)
-    for (int c = 0; c < channel_slices(a); ++c) {
-      const hipError_t e = cp4::fwd_pipe_strided_launch(strided_pass_args(a, c, t), st);
-      if (e != hipSuccess) return e;
-    }
-  return hipSuccess;
+  return passes_launch(without_epilogue(a), kStridedPassBuild, st);
 }
 
+// A launch with a geometry: the strided build of the producer / consumer kernel
+// where it applies and the matrix tiles are not mostly padding (in passes where one launch
+// does not hold the layer), else the general kernel.
+// (The strided build carries the bias / activation epilogue: a.bias / a.act are applied
+// there in a single launch; *epilogue_done says whether they were.)
 cp4_status run_geometry(FwdArgs a, hipStream_t st, bool* epilogue_done = nullptr) {
   if (epilogue_done) *epilogue_done = false;
   if (a.N == 0) return CP4_OK;
