@@ -369,6 +369,8 @@ constexpr long kTwoPassMinElements = 16l << 20;
 // 5.7 us, N4 C32 112x112 R16 11.1 -> 9.1, N16 C8 32x32 R16 29.9 -> 5.6 - and more
 // outside them: 1.0-1.1 with 48-64 input channels or 32 ranks, 1.2-2.3 from 100,000
 // pixels on (its grid then needs several rounds of workgroups of 200 registers a lane).
+// (whole rows: on rows beyond 128 pixels the tiled kernel stays ahead, N1 C3 K64 224x224
+// 9.4 against 10.1 us)
 constexpr long kLightMaxPixels = 50176;      // 4 x 112 x 112
 constexpr int kLightMaxCin = 32, kLightMaxCout = 64, kLightMaxRank = 16;
 constexpr double kLightMinDenseFloor = 6.0;  // us
@@ -416,8 +418,8 @@ int heuristic_variant(const FwdArgs& a) {
   // Small problems with few channels: the light kernel's three short phases.
   // (not where the recomposed-filter kernel was picked and is as quick: 3 -> 1 channels on
   // whole tiles, 4.8 us)
-  if ((long)a.N * a.H * a.W <= kLightMaxPixels && a.Cin <= kLightMaxCin &&
-      a.Cout <= kLightMaxCout && a.R <= kLightMaxRank &&
+  if ((long)a.N * a.H * a.W <= kLightMaxPixels && a.W <= kWholeRowMaxWidth &&
+      a.Cin <= kLightMaxCin && a.Cout <= kLightMaxCout && a.R <= kLightMaxRank &&
       !(is_variant(pick, "dense_small_valu") && dense_small_floor(a) <= kLightMinDenseFloor))
     prefer("mfma_bf16x3_light");
   return pick;
