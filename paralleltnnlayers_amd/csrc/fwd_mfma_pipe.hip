@@ -138,6 +138,11 @@ struct PipePlan {
   int split2;               // consumer waves split roles also above 16 ranks / 4 channel blocks
   int own;                  // consumer waves take whole groups each (few ranks and channel blocks)
   int spin_limit;           // polls before a wait between waves gives up
+  // Few strips (one image, small planes) leave compute units idle: the output channels are
+  // then cut into kparts slices of kslice channels (a multiple of 32), one workgroup per
+  // (strip, slice) - blockIdx.y is the slice; every slice's workgroup contracts the strip's
+  // A plane again and writes its own channels.  1: no slices.
+  int kparts = 1, kslice = 0;
 #ifdef CP4_DEBUG_PHASES
   long long* dbg;
 #endif
@@ -243,7 +248,11 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   if (pl.dbg && lane == 0) pl.dbg[((size_t)t * 16 + wave) * 32 + 30] = clock64();
 #endif
   const int l32 = lane & 31, hi = lane >> 5;
-  const int H = a.H, W = a.W, HW = H * W, R = a.R, Cin = a.Cin, Cout = a.Cout;
+  const int H = a.H, W = a.W, HW = H * W, R = a.R, Cin = a.Cin;
+  // this workgroup's output channels [k0, k0 + Cout) of the layer's CoutAll
+  const int CoutAll = a.Cout;
+  const int k0 = pl.kparts > 1 ? (int)blockIdx.y * pl.kslice : 0;
+  const int Cout = pl.kparts > 1 ? min(pl.kslice, CoutAll - k0) : CoutAll;
 #ifdef CP4_PIPE_STRIDED
   // output plane, stride, zeros before the image; h0 counts output rows
   const int Ho = a.Ho, Wo = a.Wo, HWo = Ho * Wo, SH = a.sh, SW = a.sw, PT = a.pt, PL = a.pl;
@@ -298,7 +307,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   const int cpq = FLDS ? (Cin + 63) >> 6 : CPQ;    // 16-channel chunks per channel split
   if (tid < kMaxBlk + 16) flags[tid] = 0;
 #ifdef CP4_PIPE_EPILOGUE
-  for (int k = tid; k < 32 * nkb; k += kThreads) biasL[k] = (a.bias && k < Cout) ? a.bias[k] : 0.f;
+  for (int k = tid; k < 32 * nkb; k += kThreads) biasL[k] = (a.bias && k < Cout) ? a.bias[k0 + k] : 0.f;
 #endif
   if (FLDS) {
     for (int it = tid; it < 8 * cpq * 32; it += kThreads) {
@@ -662,7 +671,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int r = 16 * c + 8 * hi + e;
-          v[e] = (k < Cout && r < R) ? a.Fout[(size_t)k * ldf + r] : 0.f;
+          v[e] = (k < Cout && r < R) ? a.Fout[(size_t)(k0 + k) * ldf + r] : 0.f;
         }
         split8(v, fkh[slot][c], fkm[slot][c], fkl[slot][c]);
       }
@@ -744,9 +753,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
     load_taps(std::integral_constant<int, 0>{});
 #endif
 #ifdef CP4_PIPE_TILED
-    io_t* yn = reinterpret_cast<io_t*>(a.y) + (size_t)n * Cout * HW + (size_t)h0 * W + w0;
+    io_t* yn = reinterpret_cast<io_t*>(a.y) + ((size_t)n * CoutAll + k0) * HW + (size_t)h0 * W + w0;
 #else
-    io_t* yn = reinterpret_cast<io_t*>(a.y) + (size_t)n * Cout * HWo + (size_t)h0 * Wo;
+    io_t* yn = reinterpret_cast<io_t*>(a.y) + ((size_t)n * CoutAll + k0) * HWo + (size_t)h0 * Wo;
 #endif
     [[maybe_unused]] const bool accumulate = a.accumulate != 0;
     const bool pair_stores =                       // one store per pixel pair is legal
@@ -1469,6 +1478,19 @@ bool plan(const FwdArgs& a, PipePlan* best) {
 }
 #endif
 #if !defined(CP4_PIPE_TILED) && !defined(CP4_PIPE_STRIDED)
+// Strips that fill at most half the chip, four or more blocks of 32 output channels: as
+// many slices of at least two blocks as bring the grid up to the compute units
+// (N1 C512 K512 28x28: 28 strips, 16 blocks -> 8 slices of two).
+void choose_output_slices(const FwdArgs& a, int cus, PipePlan* pl) {
+  const int nkb = (a.Cout + 31) / 32;
+  if (a.tune_th > 0 || 2 * pl->nWG > cus || nkb < 4) return;
+  int parts = cus / pl->nWG;
+  if (parts > nkb / 2) parts = nkb / 2;
+  if (parts < 2) return;
+  const int blocks = (nkb + parts - 1) / parts;     // blocks per slice
+  pl->kslice = 32 * blocks;
+  pl->kparts = (nkb + blocks - 1) / blocks;
+}
 bool plan(const FwdArgs& a, PipePlan* best) {
   double best_cost = 0;
   bool found = false;
@@ -1491,6 +1513,7 @@ bool plan(const FwdArgs& a, PipePlan* best) {
       found = true;
     }
   }
+  if (found) choose_output_slices(a, cus, best);
   return found;
 }
 #endif
@@ -1505,7 +1528,7 @@ hipError_t launch_as(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
                                         (int)pl.lds_bytes);
     if (ep != hipSuccess) return ep;
     fwd_pipe_kernel<FS, CPQ, KR, NQ, true>
-        <<<8u * ((pl.nWG + 7) / 8), kThreads, pl.lds_bytes, st>>>(a, pl);
+        <<<dim3(8u * ((pl.nWG + 7) / 8), pl.kparts), kThreads, pl.lds_bytes, st>>>(a, pl);
     return hipGetLastError();
   }
 #endif
@@ -1513,7 +1536,7 @@ hipError_t launch_as(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)pl.lds_bytes);
   if (e != hipSuccess) return e;
-  const unsigned grid = 8u * ((pl.nWG + 7) / 8);
+  const dim3 grid(8u * ((pl.nWG + 7) / 8), pl.kparts);
   fwd_pipe_kernel<FS, CPQ, KR, NQ><<<grid, kThreads, pl.lds_bytes, st>>>(a, pl);
   return hipGetLastError();
 }
@@ -1611,7 +1634,7 @@ bool fwd_pipe_strip_plan(const FwdArgs& a, int* rows, int* workgroups) {
   PipePlan pl;
   if (!fwd_pipe_supported(a) || !plan(a, &pl)) return false;
   *rows = pl.TH;
-  *workgroups = pl.nWG;
+  *workgroups = pl.nWG * pl.kparts;
   return true;
 }
 #endif

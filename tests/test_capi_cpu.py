@@ -142,6 +142,10 @@ def test_plan_query_names_what_a_launch_runs(L):
     p = capi.plan_query(s, "forward")
     assert p == {"variant": "mfma_bf16x3_pipe", "strip_rows": 8, "workgroups": 224}
     assert capi.plan_query(s, "backward_data")["variant"] == "mfma_bf16x3_pipe"
+    # one image leaves 28 strips: the 16 blocks of output channels are cut into 8 slices
+    one = capi.Shape(N=1, H=28, W=28, pad=1, T=512, C=512, Y=3, X=3, Rank=16)
+    assert capi.plan_query(one, "forward") == {"variant": "mfma_bf16x3_pipe", "strip_rows": 1,
+                                               "workgroups": 224}
     names = capi.backward_filter_variants()
     assert capi.plan_query(s, "backward_filter")["variant"] == names[1]
     small = capi.Shape(N=8, H=28, W=28, pad=1, T=64, C=64, Y=3, X=3, Rank=16)

@@ -223,6 +223,9 @@ EDGE = [
     (64, 32, 8, 8, 1, 48, 3, 3, 20),
     (70, 16, 6, 10, 2, 16, 5, 5, 40),     # two rank tiles, the second partly filled
     (64, 16, 14, 14, 0, 32, 1, 1, 8),     # 1x1 filter, no padding
+    # few strips, many output channels: slices of output channels per strip
+    (1, 96, 12, 12, 1, 200, 3, 3, 16),    # seven blocks in four slices, the last one of one ragged block
+    (2, 320, 9, 10, 0, 130, 1, 1, 24),    # 1x1, factor fragments in LDS, five blocks in two slices
 ]
 
 
