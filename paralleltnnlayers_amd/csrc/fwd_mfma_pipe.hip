@@ -1383,6 +1383,19 @@ int plane_rows(const FwdArgs& a) { return a.R <= 16 ? 16 : kRP; }
   return true;
 }
 
+// Strips (tiles) that fill at most half the chip, four or more blocks of 32 output channels: as
+// many slices of at least two blocks as bring the grid up to the compute units
+// (N1 C512 K512 28x28: 28 strips, 16 blocks -> 8 slices of two).
+void choose_output_slices(const FwdArgs& a, int cus, PipePlan* pl) {
+  const int nkb = (a.Cout + 31) / 32;
+  if (a.tune_th > 0 || 2 * pl->nWG > cus || nkb < 4) return;
+  int parts = cus / pl->nWG;
+  if (parts > nkb / 2) parts = nkb / 2;
+  if (parts < 2) return;
+  const int blocks = (nkb + parts - 1) / parts;     // blocks per slice
+  pl->kslice = 32 * blocks;
+  pl->kparts = (nkb + blocks - 1) / blocks;
+}
 #ifdef CP4_PIPE_STRIDED
 // Strip of TH output rows: plane of the sh * (TH - 1) + Y input rows under them.
 bool layout_strided(const FwdArgs& a, int TH, PipePlan* pl) {
@@ -1423,6 +1436,7 @@ bool plan(const FwdArgs& a, PipePlan* best) {
       found = true;
     }
   }
+  if (found) choose_output_slices(a, cus, best);
   return found;
 }
 #elif defined(CP4_PIPE_TILED)
@@ -1474,23 +1488,11 @@ bool plan(const FwdArgs& a, PipePlan* best) {
         found = true;
       }
     }
+  if (found) choose_output_slices(a, cus, best);
   return found;
 }
 #endif
 #if !defined(CP4_PIPE_TILED) && !defined(CP4_PIPE_STRIDED)
-// Strips that fill at most half the chip, four or more blocks of 32 output channels: as
-// many slices of at least two blocks as bring the grid up to the compute units
-// (N1 C512 K512 28x28: 28 strips, 16 blocks -> 8 slices of two).
-void choose_output_slices(const FwdArgs& a, int cus, PipePlan* pl) {
-  const int nkb = (a.Cout + 31) / 32;
-  if (a.tune_th > 0 || 2 * pl->nWG > cus || nkb < 4) return;
-  int parts = cus / pl->nWG;
-  if (parts > nkb / 2) parts = nkb / 2;
-  if (parts < 2) return;
-  const int blocks = (nkb + parts - 1) / parts;     // blocks per slice
-  pl->kslice = 32 * blocks;
-  pl->kparts = (nkb + blocks - 1) / blocks;
-}
 bool plan(const FwdArgs& a, PipePlan* best) {
   double best_cost = 0;
   bool found = false;
