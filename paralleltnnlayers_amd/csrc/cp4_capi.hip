@@ -224,12 +224,55 @@ hipError_t fwd_pipe2_launch(const FwdArgs& a, hipStream_t st) {
   return passes_launch(a, kRankPassBuild, st);
 }
 
+// The strided build in passes over rank tiles and channel slices (more than 32 ranks or
+// 768 input channels; a downsampling 1x1 layer with 1024 inputs, its backward-data pass
+// with 2048): as fwd_pipe2_* for the reference's geometry, without the epilogue.
+constexpr PassBuild kStridedPassBuild{cp4::fwd_pipe_strided_supported,
+                                      cp4::fwd_pipe_strided_launch};
+FwdArgs without_epilogue(FwdArgs a) {
+  a.bias = nullptr;
+  a.act = 0;
+  return a;
+}
+bool strided_passes_supported(const FwdArgs& a) {
+  return passes_supported(without_epilogue(a), kStridedPassBuild);
+}
+hipError_t strided_passes_launch(const FwdArgs& a, hipStream_t st) {
+  return passes_launch(without_epilogue(a), kStridedPassBuild, st);
+}
+
+// Even and rectangular filters of up to 7 taps a side (2x2, 4x4, 1x7, 7x1 ...) on the matrix
+// cores: the strided build runs them as the next odd square window around the filter, here
+// on the reference's geometry (stride 1, `pad` zeros before the image, an H x W output), in
+// passes where one launch does not hold the layer.  (Such layers ran the fp32 strip kernel
+// where its LDS plan fits - N32 C256 K256 56x56 2x2 R32: 68 us, here 46 - and the general
+// kernel elsewhere: N16 C192 K192 17x17 1x7 R32 400 us, here 16.)
+FwdArgs on_reference_geometry(FwdArgs a) {
+  a.sh = a.sw = 1;
+  a.pt = a.pl = a.pad;
+  a.Ho = a.H;
+  a.Wo = a.W;
+  return a;
+}
+bool fwd_window_supported(const FwdArgs& a) {
+  if (a.sh || a.dense || a.taps2d || a.bias || a.act || a.accumulate || a.ldf || a.ldx) return false;
+  if ((a.Y == a.X && (a.Y & 1)) || a.Y > 7 || a.X > 7) return false;   // square odd filters: the other builds
+  const FwdArgs g = on_reference_geometry(a);
+  return cp4::fwd_pipe_strided_supported(g) || strided_passes_supported(g);
+}
+hipError_t fwd_window_launch(const FwdArgs& a, hipStream_t st) {
+  const FwdArgs g = on_reference_geometry(a);
+  if (cp4::fwd_pipe_strided_supported(g)) return cp4::fwd_pipe_strided_launch(g, st);
+  return strided_passes_launch(g, st);
+}
+
 // Order = preference of the untuned heuristic, last to first.
 const Variant kVariants[] = {
     {"general_valu", cp4::fwd_general_supported, cp4::fwd_general_launch},
     {"dense_small_valu", cp4::fwd_dense_small_supported, cp4::fwd_dense_small_launch},
     {"mfma_f32_strip", cp4::fwd_mfma_supported, cp4::fwd_mfma_launch},
     {"mfma_bf16x3_strip", cp4::fwd_split_supported, cp4::fwd_split_launch},
+    {"mfma_bf16x3_pipe_window", fwd_window_supported, fwd_window_launch},
     {"mfma_bf16x3_light", cp4::fwd_light_supported, cp4::fwd_light_launch},
     {"mfma_bf16x3_pipe_tiled", cp4::fwd_pipe_tiled_supported, cp4::fwd_pipe_tiled_launch},
     {"mfma_bf16x3_pipe", cp4::fwd_pipe_supported, cp4::fwd_pipe_launch},
@@ -1124,22 +1167,6 @@ bool is_reference_geometry(const cp4_shape& s, const cp4_geometry& g) {
 void set_geometry(FwdArgs& a, const cp4_geometry& g) {
   a.sh = (int)g.stride_h; a.sw = (int)g.stride_w; a.pt = (int)g.pad_top; a.pl = (int)g.pad_left;
   a.Ho = (int)g.out_h; a.Wo = (int)g.out_w;
-}
-// The strided build in passes over rank tiles and channel slices (more than 32 ranks or
-// 768 input channels; a downsampling 1x1 layer with 1024 inputs, its backward-data pass
-// with 2048): as fwd_pipe2_* for the reference's geometry, without the epilogue.
-constexpr PassBuild kStridedPassBuild{cp4::fwd_pipe_strided_supported,
-                                      cp4::fwd_pipe_strided_launch};
-FwdArgs without_epilogue(FwdArgs a) {
-  a.bias = nullptr;
-  a.act = 0;
-  return a;
-}
-bool strided_passes_supported(const FwdArgs& a) {
-  return passes_supported(without_epilogue(a), kStridedPassBuild);
-}
-hipError_t strided_passes_launch(const FwdArgs& a, hipStream_t st) {
-  return passes_launch(without_epilogue(a), kStridedPassBuild, st);
 }
 
 // A launch with a geometry: the strided build of the producer / consumer kernel

@@ -58,6 +58,9 @@ struct FwdArgs {
   // (w + pl - j) / sw) wherever both divisions are exact and land inside the plane
   // (flip unused).
   int transposed;
+  // Strided build only, set by its own entry points: a filter of ty x tx taps that runs as
+  // the square window of Y = X taps around it (even and rectangular filters); 0: Y, X.
+  int ty, tx;
   // Recomposed-filter kernel only: the dense filter [Cout, Cin, Y, X] itself, taps in
   // the order the pass reads them; the four factors are unused then.
   const float* dense;

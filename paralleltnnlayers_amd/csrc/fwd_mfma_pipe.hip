@@ -256,6 +256,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
 #ifdef CP4_PIPE_STRIDED
   // output plane, stride, zeros before the image; h0 counts output rows
   const int Ho = a.Ho, Wo = a.Wo, HWo = Ho * Wo, SH = a.sh, SW = a.sw, PT = a.pt, PL = a.pl;
+  // a filter of FY x FX taps set into the FS x FS window (even or rectangular filters):
+  // the plane holds the rows FY taps reach, taps past FY / FX weigh nothing
+  const int FY = a.ty ? a.ty : FS, FX = a.tx ? a.tx : FS;
 #else
   [[maybe_unused]] const int Ho = H, Wo = W, HWo = HW;
 #endif
@@ -288,9 +291,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
   // adjoint of a strided layer: the plane holds the input rows trow0 ... that the
   // strip's output rows h0 ... h0 + TH - 1 can draw on, (h + PT - i) / SH
   const bool TR = a.transposed != 0;
-  const int trow0 = h0 + PT - (FS - 1) <= 0 ? 0 : (h0 + PT - (FS - 1) + SH - 1) / SH;
+  const int trow0 = h0 + PT - (FY - 1) <= 0 ? 0 : (h0 + PT - (FY - 1) + SH - 1) / SH;
   const int qbase = TR ? trow0 * W : (SH * h0 - PT) * W;   // global flat pixel of LDS column 0
-  const int QLEN = TR ? ((pl.TH + FS - 2) / SH + 1) * W : (SH * (pl.TH - 1) + FS) * W;
+  const int QLEN = TR ? ((pl.TH + FY - 2) / SH + 1) * W : (SH * (pl.TH - 1) + FY) * W;
 #else
   const int qbase = (h0 - a.pad) * W;            // global flat pixel of LDS column 0
   const int QLEN = (pl.TH + FS - 1) * W;
@@ -745,9 +748,16 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
       for (int rr = 0; rr < 4; ++rr)
 #pragma unroll
         for (int j = 0; j < FS; ++j) {
+#ifdef CP4_PIPE_STRIDED
+          const int r = 4 * (wq + 4 * qi) + rr;
+          const int tap = a.flip ? FY - 1 - j : j, tapw = a.flip ? FX - 1 - j : j;
+          fh[qi][rr][j] = r < R && j < FY ? a.FH[tap * ldf + r] : 0.f;
+          fw[qi][rr][j] = r < R && j < FX ? a.FW[tapw * ldf + r] : 0.f;
+#else
           const int tap = a.flip ? FS - 1 - j : j, r = 4 * (wq + 4 * qi) + rr;
           fh[qi][rr][j] = r < R ? a.FH[tap * ldf + r] : 0.f;
           fw[qi][rr][j] = r < R ? a.FW[tap * ldf + r] : 0.f;
+#endif
         }
     };
     load_taps(std::integral_constant<int, 0>{});
@@ -791,7 +801,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         // ... floor((hz + PT) / SH)
         const int hf = h0 + pf / Wo, hz = h0 + pz / Wo;
         if (rev) {
-          const int num = hf + PT - (FS - 1);
+          const int num = hf + PT - (FY - 1);
           const int first = (num <= 0 ? 0 : (num + SH - 1) / SH) - trow0;   // >= 0
           const int b = (first * W) >> 5;
           return b > nblk - 1 ? 0 : nblk - 1 - b;
@@ -802,7 +812,7 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         return last > nblk - 1 ? nblk - 1 : last;
       }
       if (rev) return nblk - 1 - ((SH * (pf / Wo) * W) >> 5);
-      const int last = ((SH * (pz / Wo) + FS - 1) * W + W - 1) >> 5;
+      const int last = ((SH * (pz / Wo) + FY - 1) * W + W - 1) >> 5;
       return last > nblk - 1 ? nblk - 1 : last;
 #else
       const int g = rev ? ngroups - 1 - i : i;
@@ -855,9 +865,9 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
         int qw = (wo + PL) / SW, rw = (wo + PL) - qw * SW;
 #pragma unroll
         for (int j = 0; j < FS; ++j) {
-          tp.rin[j] = rh == 0 && qh >= 0 && qh < H;
+          tp.rin[j] = rh == 0 && qh >= 0 && qh < H && j < FY;
           tp.roff[j] = tp.rin[j] ? (qh - trow0) * W : 0;
-          tp.in[j] = rw == 0 && qw >= 0 && qw < W;
+          tp.in[j] = rw == 0 && qw >= 0 && qw < W && j < FX;
           tp.off[j] = tp.in[j] ? qw : 0;
           if (--rh < 0) {
             rh += SH;
@@ -874,8 +884,8 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           const int ww = SW * wo + j - PL;
           tp.in[j] = ww >= 0 && ww < W;
           tp.off[j] = ww < 0 ? 0 : (ww >= W ? W - 1 : ww);   // clamped: weight is 0 there
-          tp.rin[j] = true;
-          tp.roff[j] = (SH * ho + j) * W;          // plane row SH * ho is the first tap row
+          tp.rin[j] = j < FY;                      // (rows past the filter's own: not in the plane)
+          tp.roff[j] = j < FY ? (SH * ho + j) * W : 0;   // plane row SH * ho is the first tap row
         }
       }
 #else
@@ -1170,9 +1180,16 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe_kernel(FwdArgs a, PipePlan 
           for (int rr = 0; rr < 4; ++rr)
 #pragma unroll
             for (int j = 0; j < FS; ++j) {
+#ifdef CP4_PIPE_STRIDED
+              const int r = 4 * q + rr;
+              const int tap = a.flip ? FY - 1 - j : j, tapw = a.flip ? FX - 1 - j : j;
+              qh[rr][j] = r < R && j < FY ? a.FH[tap * ldf + r] : 0.f;
+              qw[rr][j] = r < R && j < FX ? a.FW[tapw * ldf + r] : 0.f;
+#else
               const int tap = a.flip ? FS - 1 - j : j, r = 4 * q + rr;
               qh[rr][j] = r < R ? a.FH[tap * ldf + r] : 0.f;
               qw[rr][j] = r < R ? a.FW[tap * ldf + r] : 0.f;
+#endif
             }
           tap_quad(tp, q, qh, qw, cb);
         }
@@ -1399,8 +1416,9 @@ void choose_output_slices(const FwdArgs& a, int cus, PipePlan* pl) {
 #ifdef CP4_PIPE_STRIDED
 // Strip of TH output rows: plane of the sh * (TH - 1) + Y input rows under them.
 bool layout_strided(const FwdArgs& a, int TH, PipePlan* pl) {
-  const long QLEN = a.transposed ? ((long)(TH + a.Y - 2) / a.sh + 1) * a.W
-                                 : ((long)a.sh * (TH - 1) + a.Y) * a.W;
+  const int FY = a.ty ? a.ty : a.Y;              // the filter's own rows (window: a.Y)
+  const long QLEN = a.transposed ? ((long)(TH + FY - 2) / a.sh + 1) * a.W
+                                 : ((long)a.sh * (TH - 1) + FY) * a.W;
   const long QA = round_up((int)QLEN, 64) + 8;
   const size_t a_bytes = (size_t)plane_rows(a) * QA * sizeof(float);
   const size_t fin_bytes = a.Cin > 256 ? (size_t)((a.Cin + 63) & ~63) * 192 : 0;
@@ -1605,7 +1623,29 @@ hipError_t launch_fs(const FwdArgs& a, const PipePlan& pl, hipStream_t st) {
 #define fwd_pipe_launch fwd_pipe_epi_launch
 #endif
 
-bool fwd_pipe_supported(const FwdArgs& a) {
+#ifdef CP4_PIPE_STRIDED
+// Even and rectangular filters up to 7 taps a side run as the square window of the next odd
+// size: FwdArgs::ty / tx keep the filter's own rows and columns (the plane holds the rows
+// ty taps reach; the taps past ty / tx weigh nothing), Y = X the window.
+FwdArgs in_window(const FwdArgs& a) {
+  FwdArgs b = a;
+  if (a.ty || a.tx) return b;
+  const int m = a.Y > a.X ? a.Y : a.X;
+  if (m > 7 || (a.Y == a.X && (a.Y & 1))) return b;
+  b.ty = a.Y;
+  b.tx = a.X;
+  b.Y = b.X = m | 1;
+  return b;
+}
+#endif
+
+bool fwd_pipe_supported(const FwdArgs& a_in) {
+#ifdef CP4_PIPE_STRIDED
+  const FwdArgs a = in_window(a_in);
+  if (a.ty > a.Y || a.tx > a.X || a.ty < 0 || a.tx < 0) return false;
+#else
+  const FwdArgs& a = a_in;
+#endif
   if (a.R > kRP || a.Cin > 768) return false;
 #ifndef CP4_PIPE_PASSES
   if (a.accumulate || a.ldf || a.ldx) return false;   // only the rank-pass, strided and 2-D-tap builds have these
@@ -1641,7 +1681,12 @@ bool fwd_pipe_strip_plan(const FwdArgs& a, int* rows, int* workgroups) {
 }
 #endif
 
-hipError_t fwd_pipe_launch(const FwdArgs& a, hipStream_t st) {
+hipError_t fwd_pipe_launch(const FwdArgs& a_in, hipStream_t st) {
+#ifdef CP4_PIPE_STRIDED
+  const FwdArgs a = in_window(a_in);
+#else
+  const FwdArgs& a = a_in;
+#endif
   PipePlan pl;
   if (!plan(a, &pl)) return hipErrorInvalidValue;
   pl.split2 = a.tune_split2 != 1;               // 0: the kernel's own rule, 1: off

@@ -251,6 +251,44 @@ def test_edge_shapes(cp4, oracle, dims):
             assert_gradient_close(host(g), wnt, f"d{k} variant {variant}")
 
 
+# (N, C, H, W, pad, T, Y, X, R): even and rectangular filters of up to 7 taps a side - the
+# strided build of the producer / consumer kernel takes them as the next odd square window
+WINDOWED = [
+    (2, 32, 20, 24, 0, 48, 2, 2, 16),     # 2x2 in a 3x3 window, no zeros before the image
+    (2, 32, 20, 24, 1, 48, 2, 2, 16),
+    (1, 64, 17, 17, 1, 64, 4, 4, 32),     # 4x4 in 5x5, odd plane
+    (2, 48, 14, 30, 3, 32, 1, 7, 16),     # 1x7: a one-row plane per output row
+    (2, 48, 30, 14, 0, 32, 7, 1, 16),     # 7x1
+    (1, 32, 28, 28, 1, 64, 3, 5, 24),     # 3x5
+    (1, 32, 28, 28, 2, 64, 6, 6, 8),      # 6x6 in 7x7
+    (2, 40, 13, 13, 1, 24, 3, 1, 48),     # two rank tiles: in passes
+    (1, 900, 10, 10, 1, 32, 1, 3, 16),    # two channel slices
+    (1, 16, 33, 35, 2, 16, 5, 2, 4),      # whole-group consumers
+    (2, 32, 150, 12, 1, 32, 2, 4, 12),    # many strips, both sweep directions
+]
+
+
+@pytest.mark.parametrize("dims", WINDOWED, ids=lambda d: "x".join(map(str, d)))
+def test_even_and_rectangular_filters(cp4, oracle, dims):
+    N, C, H, W, pad, T, Y, X, R = dims
+    rng = np.random.default_rng(sum(dims))
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    dy = rng.standard_normal((N, T, H, W)).astype(np.float32)
+    fac = [rng.standard_normal((d, R)).astype(np.float32) / np.sqrt(R) for d in (T, C, Y, X)]
+    f = [dev(v) for v in fac]
+    s = cp4.capi.shape_for(x.shape, *f, pad)
+    assert cp4.default_variant(s) == "mfma_bf16x3_pipe_window"
+    assert cp4.default_variant(s, backward_data=True) == "mfma_bf16x3_pipe_window"
+    y = host(cp4.conv2d_forward(dev(x), *f, pad=pad))
+    assert_activation_close(y, oracle.forward(x, *fac, pad), "forward")
+    dx = host(cp4.conv2d_backward_data(dev(dy), *f, pad=pad))
+    assert_activation_close(dx, oracle.backward_data(dy, *fac, pad), "backward-data")
+    bias = rng.standard_normal(T).astype(np.float32)
+    yb = host(cp4.conv2d_forward_bias_act(dev(x), *f, dev(bias), "relu", pad=pad))
+    assert_activation_close(yb, np.maximum(y + bias[None, :, None, None], 0), "bias + relu")
+    cp4.device_status()
+
+
 # (N, C, H, W, pad, T, Y, R): channel counts the matrix-core backward-filter kernels do not
 # take as they are
 PADDED = [
