@@ -277,6 +277,7 @@ const Variant kVariants[] = {
     {"mfma_bf16x3_pipe_tiled", cp4::fwd_pipe_tiled_supported, cp4::fwd_pipe_tiled_launch},
     {"mfma_bf16x3_pipe", cp4::fwd_pipe_supported, cp4::fwd_pipe_launch},
     {"mfma_bf16x3_pipe_rank_passes", fwd_pipe2_supported, fwd_pipe2_launch},
+    {"mfma_bf16x3_pipe64", cp4::fwd_pipe64_supported, cp4::fwd_pipe64_launch},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -447,7 +448,7 @@ int heuristic_variant(const FwdArgs& a) {
     prefer("general_valu");
   if (is_variant(pick, "mfma_bf16x3_pipe") && a.W > kWholeRowMaxWidth && !strips_on_wide_plane(a))
     prefer("mfma_bf16x3_pipe_tiled");
-  if (is_variant(pick, "mfma_bf16x3_pipe_rank_passes") && a.R <= 64 &&
+  if ((is_variant(pick, "mfma_bf16x3_pipe_rank_passes") || is_variant(pick, "mfma_bf16x3_pipe64")) && a.R <= 64 &&
       (long)a.N * a.H * a.W * (a.Cin + a.Cout) < kTwoPassMinElements)
     prefer("mfma_f32_strip");
   // A handful of channels on both sides: the recomposed filter costs fewer
@@ -1662,6 +1663,10 @@ cp4_status cp4_plan_query(const cp4_shape* shape, int pass, int* variant, int* s
     if (is_variant(v, "mfma_bf16x3_pipe")) {
       a.tune_th = c.th;
       if (!cp4::fwd_pipe_strip_plan(a, &rows, &wgs)) rows = wgs = 0;
+    }
+    if (is_variant(v, "mfma_bf16x3_pipe64")) {
+      a.tune_th = c.th;
+      if (!cp4::fwd_pipe64_plan(a, &rows, &wgs)) rows = wgs = 0;
     }
   }
   if (variant) *variant = v;

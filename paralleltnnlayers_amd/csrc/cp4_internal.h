@@ -106,6 +106,11 @@ bool fwd_pipe_supported(const FwdArgs&);
 hipError_t fwd_pipe_launch(const FwdArgs&, hipStream_t);
 // Rows per strip and workgroups of the whole-row strip plan (false: no plan).
 bool fwd_pipe_strip_plan(const FwdArgs&, int* rows, int* workgroups);
+// Producer / consumer kernel with a 64-rank plane: ranks 33 - 64 in one pass (1x1 and 3x3
+// filters, up to 256 input channels); honours FwdArgs::ldf, ldx and accumulate.
+bool fwd_pipe64_supported(const FwdArgs&);
+hipError_t fwd_pipe64_launch(const FwdArgs&, hipStream_t);
+bool fwd_pipe64_plan(const FwdArgs&, int* rows, int* workgroups);
 // The same kernel compiled with the bias / activation epilogue in its stores.
 bool fwd_pipe_epi_supported(const FwdArgs&);
 hipError_t fwd_pipe_epi_launch(const FwdArgs&, hipStream_t);
