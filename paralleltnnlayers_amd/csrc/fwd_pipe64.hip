@@ -114,7 +114,10 @@ __global__ __launch_bounds__(kThreads) void fwd_pipe64_kernel(FwdArgs a, Plan64 
   const int ngroups = (nvalid + gshift + 63) >> 6;
   const int nkb = (Cout + 31) >> 5;
   const int qbase = (h0 - a.pad) * W;            // global flat pixel of LDS column 0
-  const int QLEN = (pl.TH + FS - 1) * W;
+  // The plane covers the strip's own rows (the image's last strip may have fewer than
+  // TH): every block of the sweep is then read by some tap step, which the ring's
+  // producer-side wait relies on.
+  const int QLEN = (rows + FS - 1) * W;
   const int nblk = (QLEN + 31) >> 5;             // 32-pixel producer blocks
   const bool backoff = nblk >= 4;                // growing naps in the spin waits
   const int L = pl.L, NBL = L >> 5;              // the plane's ring: cells, blocks
