@@ -224,6 +224,78 @@ hipError_t fwd_pipe2_launch(const FwdArgs& a, hipStream_t st) {
   return passes_launch(a, kRankPassBuild, st);
 }
 
+// Passes with tiles of 64 ranks: the 64-rank single-pass kernel (which holds 33 - 64 ranks
+// and 256 input channels) once per (tile of 64 ranks, slice of up to 256 channels), and the
+// 32-rank build above for a last tile of up to 32 ranks.  Against passes of 32 ranks x is
+// read once per 64 ranks instead of once per 32, and a layer with 33 - 64 ranks and more
+// than 256 input channels reads x once in all.
+constexpr int kWideTileRanks = 64, kWideSliceChannels = 256;
+struct WidePass {
+  int r0, rn, c0, cn;
+  bool wide;            // the 64-rank kernel; else the 32-rank build
+};
+// The passes of a layer in launch order; 0 if there would be more than kMaxPasses.
+int wide_passes(const FwdArgs& a, WidePass* out) {
+  int n = 0;
+  for (int r0 = 0; r0 < a.R; r0 += kWideTileRanks) {
+    const int rn = a.R - r0 < kWideTileRanks ? a.R - r0 : kWideTileRanks;
+    const bool wide = rn > 32;
+    const int cap = wide ? kWideSliceChannels : kPassMaxChannels;
+    const int most = wide ? kWideSliceChannels : kSliceMaxChannels;
+    const int slices = a.Cin <= cap ? 1 : (a.Cin + most - 1) / most;
+    const int per = ((a.Cin + slices - 1) / slices + 15) / 16 * 16;
+    for (int c0 = 0; c0 < a.Cin; c0 += per) {
+      if (n == kMaxPasses) return 0;
+      out[n++] = WidePass{r0, rn, c0, a.Cin - c0 < per ? a.Cin - c0 : per, wide};
+    }
+  }
+  return n;
+}
+FwdArgs wide_pass_args(const FwdArgs& a, const WidePass& p, bool first) {
+  FwdArgs b = a;
+  b.ldf = a.R;
+  b.R = p.rn;
+  b.Cin = p.cn;
+  b.ldx = (size_t)a.Cin * a.H * a.W;
+  b.x = a.x + (size_t)p.c0 * a.H * a.W;
+  b.Fin += (size_t)p.c0 * a.R + p.r0; b.Fout += p.r0; b.FH += p.r0; b.FW += p.r0;
+  b.accumulate = !first;
+  return b;
+}
+bool fwd_pipe64_passes_supported(const FwdArgs& a) {
+  if (a.R <= 32 || (a.R <= kWideTileRanks && a.Cin <= kWideSliceChannels) || a.ldf || a.ldx ||
+      a.accumulate || a.bias || a.act)
+    return false;
+  WidePass ps[kMaxPasses];
+  const int n = wide_passes(a, ps);
+  for (int i = 0; i < n; ++i) {
+    const FwdArgs b = wide_pass_args(a, ps[i], i == 0);
+    if (!(ps[i].wide ? cp4::fwd_pipe64_supported(b) : cp4::fwd_pipe_rankpass_supported(b)))
+      return false;
+  }
+  return n > 0;
+}
+hipError_t fwd_pipe64_passes_launch(const FwdArgs& a, hipStream_t st) {
+  WidePass ps[kMaxPasses];
+  const int n = wide_passes(a, ps);
+  for (int i = 0; i < n; ++i) {
+    const FwdArgs b = wide_pass_args(a, ps[i], i == 0);
+    const hipError_t e = ps[i].wide ? cp4::fwd_pipe64_launch(b, st) : cp4::fwd_pipe_rankpass_launch(b, st);
+    if (e != hipSuccess) return e;
+  }
+  return n > 0 ? hipSuccess : hipErrorInvalidValue;
+}
+// Channel planes moved per pixel by the passes of either kind: x once per rank tile, y
+// written by every pass and read back by all but the first.
+long pass_traffic(const FwdArgs& a, bool wide) {
+  if (wide) {
+    WidePass ps[kMaxPasses];
+    const int n = wide_passes(a, ps);
+    return (long)((a.R + kWideTileRanks - 1) / kWideTileRanks) * a.Cin + (long)(2 * n - 1) * a.Cout;
+  }
+  return (long)rank_passes(a) * a.Cin + (long)(2 * rank_passes(a) * channel_slices(a) - 1) * a.Cout;
+}
+
 // The strided build in passes over rank tiles and channel slices (more than 32 ranks or
 // 768 input channels; a downsampling 1x1 layer with 1024 inputs, its backward-data pass
 // with 2048): as fwd_pipe2_* for the reference's geometry, without the epilogue.
@@ -278,6 +350,7 @@ const Variant kVariants[] = {
     {"mfma_bf16x3_pipe", cp4::fwd_pipe_supported, cp4::fwd_pipe_launch},
     {"mfma_bf16x3_pipe_rank_passes", fwd_pipe2_supported, fwd_pipe2_launch},
     {"mfma_bf16x3_pipe64", cp4::fwd_pipe64_supported, cp4::fwd_pipe64_launch},
+    {"mfma_bf16x3_pipe64_passes", fwd_pipe64_passes_supported, fwd_pipe64_passes_launch},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -406,6 +479,37 @@ bool strips_on_wide_plane(const FwdArgs& a) {
 // elements the fp32 matrix-core strip kernel is the faster one for ranks 33-64.
 constexpr long kTwoPassMinElements = 16l << 20;
 
+// Ranks 33-64 in one pass (the 64-rank kernel) against the fp32 strip kernel, over 248
+// layers with C = K in {32 ... 256}, planes of 7 - 56 pixels a side, 1 - 64 images, 40 and 64
+// ranks: the fp32 kernel is the faster one (by 1.05 - 1.9) with a 3x3 filter and up to 64
+// channels below 8 M activation elements, with up to 128 channels on batches of 8 - 32
+// thousand pixels (1.1 - 1.25); with a 1x1 filter and everywhere else the 64-rank kernel
+// is (within 1.0 - 1.2 at 32 channels, by up to 5x at 256).
+constexpr int kF32StripFewChannels = 64, kF32StripMidChannels = 128;
+constexpr long kF32StripFewMaxElements = 8l << 20;
+constexpr long kF32StripMidMinPixels = 8192, kF32StripMidMaxPixels = 32768;
+bool f32_strip_beats_pipe64(const FwdArgs& a) {
+  const long px = (long)a.N * a.H * a.W;
+  const int ch = (a.Cin + a.Cout + 1) / 2;
+  if (a.Y == 1) return false;
+  if (ch <= kF32StripFewChannels) return px * (a.Cin + a.Cout) < kF32StripFewMaxElements;
+  return ch <= kF32StripMidChannels && px >= kF32StripMidMinPixels && px < kF32StripMidMaxPixels;
+}
+
+// Passes with tiles of 64 ranks against passes of 32 ranks.  Without channel slices (up to
+// 256 input channels) the 64-rank tiles read x half as often and win throughout (N32 C256
+// 56x56 R96: 150 against 182 us, R128 162 / 248, R200 314 / 461; N32 C128 28x28 R128 53 /
+// 66).  With more than 256 input channels they run more, shorter passes, each adding y
+// once more: they win on large batches where they move a tenth less (N32 C512 K512 28x28
+// R64: 132 against 157 us) and lose on small ones (N32 C1024 K256 14x14 1x1 R64: 81 / 62;
+// N8 C384 K384 28x28 R96 83 / 64; N4 C512 K1000 32x32 R64 71 / 51).
+constexpr long kWideSlicesMinPixels = 16384;
+bool wide_passes_preferred(const FwdArgs& a) {
+  if (a.Cin <= kWideSliceChannels) return true;
+  return (long)a.N * a.H * a.W >= kWideSlicesMinPixels &&
+         10 * pass_traffic(a, true) <= 9 * pass_traffic(a, false);
+}
+
 // Where the light kernel beats the producer / consumer kernel (and, below a few
 // tens of thousands of pixels, the recomposed-filter kernel, whose threads each run
 // Cout x Cin x Y x X multiply-adds per pixel quad in series): measured over 90 shapes
@@ -448,9 +552,16 @@ int heuristic_variant(const FwdArgs& a) {
     prefer("general_valu");
   if (is_variant(pick, "mfma_bf16x3_pipe") && a.W > kWholeRowMaxWidth && !strips_on_wide_plane(a))
     prefer("mfma_bf16x3_pipe_tiled");
-  if ((is_variant(pick, "mfma_bf16x3_pipe_rank_passes") || is_variant(pick, "mfma_bf16x3_pipe64")) && a.R <= 64 &&
-      (long)a.N * a.H * a.W * (a.Cin + a.Cout) < kTwoPassMinElements)
+  if (is_variant(pick, "mfma_bf16x3_pipe64_passes") && fwd_pipe2_supported(a) &&
+      !wide_passes_preferred(a))
+    prefer("mfma_bf16x3_pipe_rank_passes");
+  if (is_variant(pick, "mfma_bf16x3_pipe64")) {
+    if (f32_strip_beats_pipe64(a)) prefer("mfma_f32_strip");
+  } else if ((is_variant(pick, "mfma_bf16x3_pipe_rank_passes") ||
+              is_variant(pick, "mfma_bf16x3_pipe64_passes")) && a.R <= 64 &&
+             (long)a.N * a.H * a.W * (a.Cin + a.Cout) < kTwoPassMinElements) {
     prefer("mfma_f32_strip");
+  }
   // A handful of channels on both sides: the recomposed filter costs fewer
   // multiply-adds per pixel than the factor-by-factor order.
   if (cp4::fwd_dense_small_supported(a)) {

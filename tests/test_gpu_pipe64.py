@@ -122,6 +122,39 @@ def test_pipe64_strip_heights_on_a_ring(cp4, oracle, R):
     assert ran >= 20
 
 
+# More than 64 ranks or 256 input channels: the kernel once per (tile of 64 ranks, slice of up
+# to 256 channels) with y += after the first pass, the 32-rank build for a last tile of up to 32.
+PASSES = [
+    (2, 320, 20, 20, 1, 64, 3, 64),      # two channel slices of one rank tile
+    (2, 64, 28, 28, 1, 96, 3, 96),       # 64 ranks, then 32 on the 32-rank build
+    (1, 600, 12, 12, 1, 48, 3, 100),     # tiles of 64 and 36 ranks x three slices of 208 channels
+    (1, 1024, 7, 7, 0, 32, 1, 129),      # 1x1: two tiles x four slices, a last rank in two slices of 512
+    (2, 128, 56, 56, 1, 128, 3, 128),    # two tiles on a wrapped ring
+]
+
+
+@pytest.mark.parametrize("dims", PASSES, ids=lambda d: "x".join(map(str, d)))
+def test_pipe64_in_passes(cp4, oracle, dims):
+    N, C, H, W, pad, T, Y, R = dims
+    x, dy, fac = layer(dims)
+    f = [dev(v) for v in fac]
+    v = {n: i for i, n, _ in cp4.forward_variants()}[NAME + "_passes"]
+    y = cp4.conv2d_forward(dev(x), *f, pad=pad, variant=v)
+    close(host(y), oracle.forward(x, *fac, pad), "forward")
+    s = cp4.capi.shape_for(x.shape, *f, pad)
+    cp4.tune_clear()
+    try:
+        try:
+            cp4.set_tuned_choice(s, v, backward_data=True)
+        except cp4.Cp4Error as e:       # up to 64 ranks and 256 output channels: a single pass
+            assert e.status == cp4.capi.ERR_UNSUPPORTED and R <= 64 and T <= 256
+        dx = cp4.conv2d_backward_data(dev(dy), *f, pad=pad)
+    finally:
+        cp4.tune_clear()
+    close(host(dx), oracle.backward_data(dy, *fac, pad), "backward-data")
+    cp4.device_status()
+
+
 def test_pipe64_is_the_default_for_33_to_64_ranks(cp4):
     def shape(N, C, H, W, T, R, Y=3):
         return cp4.capi.Shape(N=N, H=H, W=W, pad=Y // 2, T=T, C=C, Y=Y, X=Y, Rank=R)
@@ -134,6 +167,9 @@ def test_pipe64_is_the_default_for_33_to_64_ranks(cp4):
     assert cp4.default_variant(shape(32, 256, 56, 56, 256, 32)) == "mfma_bf16x3_pipe"
     # 5x5 filters: passes of 32 ranks
     assert cp4.default_variant(shape(32, 256, 56, 56, 256, 64, Y=5)) == "mfma_bf16x3_pipe_rank_passes"
+    # tiles of 64 ranks beyond 64 ranks, slices of 256 channels beyond 256 channels
+    assert cp4.default_variant(shape(32, 256, 56, 56, 256, 128)) == NAME + "_passes"
+    assert cp4.default_variant(shape(32, 512, 28, 28, 512, 64)) == NAME + "_passes"
     q = cp4.plan_query(shape(32, 256, 56, 56, 256, 64), "forward")
     assert q["variant"] == NAME and q["strip_rows"] >= 1 and q["workgroups"] >= 200
 
