@@ -345,6 +345,7 @@ const Variant kVariants[] = {
     {"mfma_f32_strip", cp4::fwd_mfma_supported, cp4::fwd_mfma_launch},
     {"mfma_bf16x3_strip", cp4::fwd_split_supported, cp4::fwd_split_launch},
     {"mfma_bf16x3_pipe_window", fwd_window_supported, fwd_window_launch},
+    {"mfma_bf16x3_few", cp4::fwd_few_supported, cp4::fwd_few_launch},
     {"mfma_bf16x3_light", cp4::fwd_light_supported, cp4::fwd_light_launch},
     {"mfma_bf16x3_pipe_tiled", cp4::fwd_pipe_tiled_supported, cp4::fwd_pipe_tiled_launch},
     {"mfma_bf16x3_pipe", cp4::fwd_pipe_supported, cp4::fwd_pipe_launch},
@@ -440,6 +441,42 @@ bool dense_small_loses_to_matrix(const FwdArgs& a) {
   // (the matrix-core kernels' tap step grows with the filter: 28 us per 2^18 pixels at
   // 5x5, 52 at 7x7)
   return dense > 6.0 + 16.5 * (a.Y * a.X + 9) / 18.0 * pixels / 262144.0;
+}
+// The few-channel tiled kernel (persistent small workgroups, taps and output contraction in
+// registers) against the other kernels, over 1620 layers (3 - 64 channels in, 1 - 128 out,
+// 1x1 / 3x3 / 5x5, ranks 4 and 16, a thousand to a million pixels): with up to 32 input and
+// 64 output channels it is the faster one from about 60,000 pixels on - by 1.05 - 1.3 at 64
+// output channels, 1.3 - 2.7 below (N16 C16 K16 512x512 R16: 271 -> 160 us, N32 C16 K16 56x56
+// 13.1 -> 7.5, N16 C8 K32 256x256 84 -> 35) - and with a 1x1 filter and up to 32 output
+// channels at any size (1.05 - 1.35); below that size the others are within 0.93 - 1.08 and
+// stay.  Against the recomposed-filter kernel it is weighed by time: its own 5 us + a rate
+// per 2^18 pixels (6.5 - 9 with up to 16 input channels, 11 - 17 with 32; 3x3) against the
+// larger of that kernel's workgroup floor times its rounds and its rate (measured at a million
+// pixels: 3 -> 1 channels 1.9 us per 2^18 pixels, 3 -> 16 7.9, 8 -> 8 8.5, 16 -> 1 8.4).
+constexpr long kFewMinPixels = 60000;
+constexpr int kFewMaxCin = 32, kFewMaxCout = 64, kFewPointwiseMaxCout = 32;
+double few_time(const FwdArgs& a) {
+  const double rate = a.Cin <= 16 ? 6.5 + 0.07 * a.Cout : 11.0 + 0.19 * a.Cout;
+  return 5.0 + rate * (0.7 + 0.3 * a.Y * a.X / 9.0) * (double)a.N * a.H * a.W / 262144.0;
+}
+double dense_small_time(const FwdArgs& a) {
+  long tiles = 0;
+  size_t lds = 0;
+  if (!cp4::fwd_dense_small_plan_info(a, &tiles, &lds)) return 1e30;
+  long occ = (long)(160 * 1024 / (lds ? lds : 1));
+  occ = occ < 1 ? 1 : (occ > 8 ? 8 : occ);
+  const double rounds = (double)tiles / (0.6 * occ * cp4::num_compute_units());
+  const double floor_time = dense_small_floor(a) * (rounds > 1.0 ? rounds : 1.0);
+  const int groups = (a.Cout + 7) / 8;
+  const double rate = 1.0 + 0.1 * a.Cin * groups * a.Y + 0.0012 * a.Cout * a.Cin * a.Y * a.X;
+  const double rate_time = rate * (double)a.N * a.H * a.W / 262144.0;
+  return floor_time > rate_time ? floor_time : rate_time;
+}
+bool few_preferred(const FwdArgs& a, bool over_dense_small) {
+  if (a.Cin > kFewMaxCin || a.Cout > kFewMaxCout) return false;
+  const long pixels = (long)a.N * a.H * a.W;
+  if (pixels < kFewMinPixels && !(a.Y == 1 && a.Cout <= kFewPointwiseMaxCout)) return false;
+  return !over_dense_small || few_time(a) < dense_small_time(a);
 }
 double general_estimate(const FwdArgs& a) {
   return 10.0 + 0.3 * a.R * (a.Cin + a.Cout + a.Y + a.X);
@@ -577,6 +614,10 @@ int heuristic_variant(const FwdArgs& a) {
       a.Cin <= kLightMaxCin && a.Cout <= kLightMaxCout && a.R <= kLightMaxRank &&
       !(is_variant(pick, "dense_small_valu") && dense_small_floor(a) <= kLightMinDenseFloor))
     prefer("mfma_bf16x3_light");
+  // Few channels from a few tens of thousands of pixels on: the tiled few-channel kernel.
+  if (pick >= 0 && !is_variant(pick, "general_valu") && cp4::fwd_few_supported(a) &&
+      few_preferred(a, is_variant(pick, "dense_small_valu")))
+    prefer("mfma_bf16x3_few");
   return pick;
 }
 
@@ -860,6 +901,13 @@ cp4_status cp4_conv2d_forward_bias_act(const cp4_shape* shape, const float* x,
     FwdArgs e = with_tile(a, c);
     if (cp4::fwd_light_supported(e)) {
       CP4_HIP(cp4::fwd_light_launch(e, st));        // the same
+      return CP4_OK;
+    }
+  }
+  if (is_variant(c.variant, "mfma_bf16x3_few")) {
+    FwdArgs e = with_tile(a, c);
+    if (cp4::fwd_few_supported(e)) {
+      CP4_HIP(cp4::fwd_few_launch(e, st));          // the same
       return CP4_OK;
     }
   }
@@ -1655,9 +1703,10 @@ cp4_status tune_forward_like(const FwdArgs& a, unsigned warmup, unsigned profcou
     if (rc != CP4_OK) return rc;
     const bool strips = is_variant(v, "mfma_bf16x3_pipe") || is_variant(v, "mfma_bf16x3_pipe_rank_passes");
     const bool tiles = is_variant(v, "mfma_bf16x3_pipe_tiled");
-    if (!strips && !tiles) continue;
+    const bool few = is_variant(v, "mfma_bf16x3_few");      // tiles of 32, 64 or 128 columns
+    if (!strips && !tiles && !few) continue;
     const int max_th = a.H < 16 ? a.H : 16;
-    for (int lgwt = tiles ? 6 : 0; lgwt <= (tiles ? 8 : 0); ++lgwt)
+    for (int lgwt = tiles ? 6 : (few ? 5 : 0); lgwt <= (tiles ? 8 : (few ? 7 : 0)); ++lgwt)
       for (int th = 1; th <= max_th; ++th)
         for (int split2 = 0; split2 <= 2; ++split2) {   // 2: consumer waves with groups of their own
           rc = consider(Choice{v, th, lgwt, split2});
@@ -1779,6 +1828,13 @@ cp4_status cp4_plan_query(const cp4_shape* shape, int pass, int* variant, int* s
       a.tune_th = c.th;
       if (!cp4::fwd_pipe64_plan(a, &rows, &wgs)) rows = wgs = 0;
     }
+    if (is_variant(v, "mfma_bf16x3_few")) {       // (tile rows; its persistent workgroups)
+      int cols = 0;
+      a.tune_th = c.th;
+      a.tune_lgwt = c.lgwt;
+      a.tune_split2 = c.split2;
+      if (!cp4::fwd_few_plan(a, &rows, &cols, &wgs)) rows = wgs = 0;
+    }
   }
   if (variant) *variant = v;
   if (strip_rows) *strip_rows = rows;
@@ -1794,8 +1850,8 @@ cp4_status cp4_set_tuned_choice(const cp4_shape* shape, int backward_data, int v
   int lgwt = 0;
   if (tile_cols) {
     while ((1 << lgwt) < tile_cols) ++lgwt;
-    if ((1 << lgwt) != tile_cols || lgwt < 6 || lgwt > 8)
-      return fail(CP4_ERR_SHAPE, "tile_cols must be 0, 64, 128 or 256");
+    if ((1 << lgwt) != tile_cols || lgwt < 5 || lgwt > 8)
+      return fail(CP4_ERR_SHAPE, "tile_cols must be 0, 32, 64, 128 or 256");
   }
   if (tile_rows < 0 || schedule < 0 || schedule > 2)
     return fail(CP4_ERR_SHAPE, "tile_rows >= 0 and schedule 0, 1 or 2 expected");

@@ -102,6 +102,11 @@ hipError_t fwd_split_launch(const FwdArgs&, hipStream_t);
 // Few short phases in small workgroups, for small problems (ranks up to 32).
 bool fwd_light_supported(const FwdArgs&);
 hipError_t fwd_light_launch(const FwdArgs&, hipStream_t);
+// Persistent small workgroups over 2-D tiles, taps and output contraction in registers:
+// few channels (up to 64 in), up to 16 ranks, planes of any width.
+bool fwd_few_supported(const FwdArgs&);
+hipError_t fwd_few_launch(const FwdArgs&, hipStream_t);
+bool fwd_few_plan(const FwdArgs&, int* rows, int* cols, int* workgroups);
 bool fwd_pipe_supported(const FwdArgs&);
 hipError_t fwd_pipe_launch(const FwdArgs&, hipStream_t);
 // Rows per strip and workgroups of the whole-row strip plan (false: no plan).

@@ -114,13 +114,16 @@ def test_default_variant_on_wide_planes(L):
     assert capi.default_variant(shape(8, 64, 224, 224, 64, 16)) == "mfma_bf16x3_pipe"
     assert capi.default_variant(shape(8, 64, 224, 224, 64, 32)) == "mfma_bf16x3_pipe_tiled"
     assert capi.default_variant(shape(2, 64, 512, 512, 64, 16)) == "mfma_bf16x3_pipe_tiled"
-    assert capi.default_variant(shape(8, 32, 150, 300, 32, 16)) == "mfma_bf16x3_pipe_tiled"
+    assert capi.default_variant(shape(8, 48, 150, 300, 48, 16)) == "mfma_bf16x3_pipe_tiled"
+    # up to 32 input and 64 output channels, 16 ranks, from 60,000 pixels on: the few-channel kernel
+    assert capi.default_variant(shape(8, 32, 150, 300, 32, 16)) == "mfma_bf16x3_few"
+    assert capi.default_variant(shape(16, 16, 512, 512, 16, 16)) == "mfma_bf16x3_few"
     assert capi.default_variant(shape(16, 256, 160, 160, 256, 16)) == "mfma_bf16x3_pipe"
     assert capi.default_variant(shape(1, 3, 512, 512, 1, 16)) == "dense_small_valu"
     # small layers with few channels: the light kernel (workload C1), not beyond its bounds
     assert capi.default_variant(shape(1, 16, 32, 32, 16, 8)) == "mfma_bf16x3_light"
     assert capi.default_variant(shape(16, 64, 32, 32, 64, 16)) == "mfma_bf16x3_pipe"
-    assert capi.default_variant(shape(32, 16, 56, 56, 16, 16)) == "mfma_bf16x3_pipe"
+    assert capi.default_variant(shape(32, 16, 56, 56, 16, 16)) == "mfma_bf16x3_few"
     assert capi.default_variant(shape(8, 64, 224, 224, 64, 16), backward_data=True) \
         == "mfma_bf16x3_pipe"
     s = shape(8, 64, 224, 224, 64, 16)

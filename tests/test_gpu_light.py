@@ -104,7 +104,7 @@ def test_light_is_the_default_for_small_layers_only(cp4):
     assert cp4.default_variant(shape(8, 16, 56, 56, 16, 16)) == NAME
     assert cp4.default_variant(shape(16, 8, 32, 32, 8, 16)) == NAME            # not the recomposed filter
     assert cp4.default_variant(shape(16, 64, 32, 32, 64, 16)) == "mfma_bf16x3_pipe"   # workload C2
-    assert cp4.default_variant(shape(32, 16, 56, 56, 16, 16)) == "mfma_bf16x3_pipe"   # 100,000 pixels
+    assert cp4.default_variant(shape(32, 16, 56, 56, 16, 16)) == "mfma_bf16x3_few"    # 100,000 pixels
     assert cp4.default_variant(shape(8, 16, 56, 56, 16, 32)) == "mfma_bf16x3_pipe"    # 32 ranks
 
 
