@@ -449,15 +449,16 @@ bool dense_small_loses_to_matrix(const FwdArgs& a) {
 // output channels, 1.3 - 2.7 below (N16 C16 K16 512x512 R16: 271 -> 160 us, N32 C16 K16 56x56
 // 13.1 -> 7.5, N16 C8 K32 256x256 84 -> 35) - and with a 1x1 filter and up to 32 output
 // channels at any size (1.05 - 1.35); below that size the others are within 0.93 - 1.08 and
-// stay.  Against the recomposed-filter kernel it is weighed by time: its own 5 us + a rate
-// per 2^18 pixels (6.5 - 9 with up to 16 input channels, 11 - 17 with 32; 3x3) against the
+// stay.  Against the recomposed-filter kernel it is weighed by time: its own 4.2 us + a rate
+// per 2^18 pixels (6 - 9 with up to 16 input channels, 10 - 16 with 32; 3x3; two thirds of
+// that at 1x1, 1.35 times at 5x5) against the
 // larger of that kernel's workgroup floor times its rounds and its rate (measured at a million
 // pixels: 3 -> 1 channels 1.9 us per 2^18 pixels, 3 -> 16 7.9, 8 -> 8 8.5, 16 -> 1 8.4).
 constexpr long kFewMinPixels = 60000;
 constexpr int kFewMaxCin = 32, kFewMaxCout = 64, kFewPointwiseMaxCout = 32;
 double few_time(const FwdArgs& a) {
-  const double rate = a.Cin <= 16 ? 6.5 + 0.07 * a.Cout : 11.0 + 0.19 * a.Cout;
-  return 5.0 + rate * (0.7 + 0.3 * a.Y * a.X / 9.0) * (double)a.N * a.H * a.W / 262144.0;
+  const double rate = a.Cin <= 16 ? 5.8 + 0.1 * a.Cout : 10.0 + 0.2 * a.Cout;
+  return 4.2 + rate * (0.49 + 0.17 * a.Y) * (double)a.N * a.H * a.W / 262144.0;
 }
 double dense_small_time(const FwdArgs& a) {
   long tiles = 0;
@@ -468,7 +469,7 @@ double dense_small_time(const FwdArgs& a) {
   const double rounds = (double)tiles / (0.6 * occ * cp4::num_compute_units());
   const double floor_time = dense_small_floor(a) * (rounds > 1.0 ? rounds : 1.0);
   const int groups = (a.Cout + 7) / 8;
-  const double rate = 1.0 + 0.1 * a.Cin * groups * a.Y + 0.0012 * a.Cout * a.Cin * a.Y * a.X;
+  const double rate = 1.0 + 0.1 * a.Cin * groups * a.Y + 0.011 * a.Cout * a.Cin * a.Y * a.X;
   const double rate_time = rate * (double)a.N * a.H * a.W / 262144.0;
   return floor_time > rate_time ? floor_time : rate_time;
 }
@@ -621,13 +622,26 @@ int heuristic_variant(const FwdArgs& a) {
   return pick;
 }
 
+// The heuristic's pick per shape and operand alignment, remembered: evaluating it asks
+// every kernel for its plan, several microseconds of host time that a small layer's launch
+// (5 us on the device) would otherwise wait for.
+std::map<std::tuple<TuneKey, unsigned>, int> g_heuristic_picks;
 Choice choose(const FwdArgs& a) {
+  const std::tuple<TuneKey, unsigned> hk(
+      key_of(a), (unsigned)((reinterpret_cast<uintptr_t>(a.x) & 15) << 4 |
+                            (reinterpret_cast<uintptr_t>(a.y) & 15)));
   {
     std::lock_guard<std::mutex> lk(g_tune_mu);
     auto it = g_tuned.find(key_of(a));
     if (it != g_tuned.end()) return it->second;
+    auto ih = g_heuristic_picks.find(hk);
+    if (ih != g_heuristic_picks.end()) return Choice{ih->second, 0, 0, 0};
   }
-  return Choice{heuristic_variant(a), 0, 0, 0};
+  const int pick = heuristic_variant(a);
+  std::lock_guard<std::mutex> lk(g_tune_mu);
+  if (g_heuristic_picks.size() > 4096) g_heuristic_picks.clear();
+  g_heuristic_picks[hk] = pick;
+  return Choice{pick, 0, 0, 0};
 }
 
 FwdArgs with_tile(const FwdArgs& a, const Choice& c) {
@@ -1946,6 +1960,7 @@ void cp4_tune_clear(void) {
   std::lock_guard<std::mutex> lk(g_tune_mu);
   g_tuned.clear();
   g_tuned_filter.clear();
+  g_heuristic_picks.clear();
 }
 
 cp4_status cp4_device_status(cp4_stream stream, int* detail) {
