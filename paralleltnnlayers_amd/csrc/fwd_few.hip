@@ -367,7 +367,7 @@ bool layout(const FwdArgs& a, int TH, int lgTW, int nw, FewPlan* pl) {
 // vector unit cost one another.  Eight waves on tiles of 512 pixels or more, four on smaller
 // ones; a tuned height / width / schedule (0: eight waves, 2: four) replaces the choice.
 constexpr double kBlockCost = 1.0, kBlockFixed = 0.3, kGroupCost = 4.0, kGroupBlockCost = 2.0,
-                 kTileFixed = 2.0;
+                 kTileFixed = 2.0, kNarrowTileCost = 8.0;
 bool plan_uncached(const FwdArgs& a, FewPlan* best);
 // The plan of the last shape asked for, per thread: a launch asks twice (whether the kernel
 // takes the shape, then with what), a training loop for the same few shapes over and over.
@@ -407,7 +407,8 @@ bool plan_uncached(const FwdArgs& a, FewPlan* best) {
       const long resident = pl.ntiles >= slots ? 16 / nw : (pl.ntiles + cus - 1) / cus;
       const double share = resident * nw > 8 ? resident * nw / 8.0 : 1.0;   // beyond two waves a vector unit
       const double turns = (double)((pl.ntiles + slots - 1) / slots);
-      const double cost = turns * wave_work * share;
+      // (short rows cost more per byte moved: 128-byte pieces at 32 columns, 512 at 128)
+      const double cost = turns * wave_work * share * (1.0 + kNarrowTileCost / pl.TW);
       if (!found || cost < best_cost) {
         best_cost = cost;
         *best = pl;
