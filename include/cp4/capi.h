@@ -342,7 +342,9 @@ cp4_status cp4_conv2d_forward_variant(const cp4_shape* shape, const float* x,
  * each) on the caller's buffers - the producer / consumer variants once per
  * strip height (tile height x width for wide planes) up to 16 rows and with each
  * of the consumers' schedules (role split by the kernel's rule, off, whole pixel
- * groups per wave) - remembers the fastest for this shape for the
+ * groups per wave); the few-channel tiled variant once per tile height, tile
+ * width (32, 64, 128 columns) and workgroup size (schedule 0: eight waves, 2:
+ * four, 1: its own rule) - remembers the fastest for this shape for the
  * rest of the process (a process-wide table behind a mutex; cp4_tune_clear
  * empties it) and reports it.  cp4_tune_backward_data does the same for that
  * pass, cp4_tune_backward_filter chooses between that pass's three variants.
@@ -370,14 +372,16 @@ cp4_status cp4_tuned_choice(const cp4_shape* shape, int backward_data, int* vari
 /* What a launch of `shape` would run with now, for reports and benchmarks: pass 0 =
  * forward, 1 = backward-data, 2 = backward-filter.  `variant` indexes
  * cp4_forward_variant_name (passes 0, 1) or cp4_backward_filter_variant_name (pass 2,
- * for operands and a workspace aligned to 16 bytes); for the whole-row strip kernel
- * `strip_rows` and `workgroups` are the planner's strip height and grid, else 0.
+ * for operands and a workspace aligned to 16 bytes); for the whole-row strip kernels
+ * (32 and 64 ranks) and the few-channel tiled kernel `strip_rows` and `workgroups` are
+ * the planner's strip / tile height and grid, else 0.
  * No counterpart in the reference, whose kernel has one fixed tile
  * (reference/kernels/cp4Conv2dForward.cu:183-198). */
 cp4_status cp4_plan_query(const cp4_shape* shape, int pass, int* variant, int* strip_rows,
                           int* workgroups);
 /* Enters a choice into the table as cp4_tune_forward / cp4_tune_backward_data
  * would (one saved from an earlier process, say), in cp4_tuned_choice's terms.
+ * `tile_cols` is 0, 32, 64, 128 or 256 (which of them a variant takes is its own matter).
  * CP4_ERR_UNSUPPORTED if the variant does not take the shape with that tile. */
 cp4_status cp4_set_tuned_choice(const cp4_shape* shape, int backward_data, int variant,
                                 int tile_rows, int tile_cols, int schedule);
