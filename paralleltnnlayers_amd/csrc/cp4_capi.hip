@@ -746,7 +746,10 @@ size_t filter_workspace(const cp4_shape& s) {
     const cp4_shape t = filter_padded_shape(s);
     const size_t general = cp4::bwd_filter_workspace_bytes(s);
     const size_t padded = filter_pad_layout(s, t).head * sizeof(float) + filter_workspace(t);
-    return padded > general ? padded : general;
+    const size_t dense =
+        cp4::bwd_filter_dense_tiles_supported(s) ? cp4::bwd_filter_dense_tiles_workspace_bytes(s) : 0;
+    const size_t most = padded > general ? padded : general;
+    return most > dense ? most : dense;
   }
   size_t b = cp4::bwd_filter_workspace_bytes(s);
   if (cp4::bwd_filter_mfma_supported(s)) {
@@ -755,6 +758,10 @@ size_t filter_workspace(const cp4_shape& s) {
   }
   if (cp4::bwd_filter_fused_supported(s)) {
     const size_t m = cp4::bwd_filter_fused_workspace_bytes(s);
+    if (m > b) b = m;
+  }
+  if (cp4::bwd_filter_dense_tiles_supported(s)) {
+    const size_t m = cp4::bwd_filter_dense_tiles_workspace_bytes(s);
     if (m > b) b = m;
   }
   if (filter_rank_tiles_supported(s)) {
@@ -1050,6 +1057,7 @@ namespace {
 // matrix-core one, else four launches, else the general kernel.
 struct FilterRoutes {
   bool tiles_ok, mfma_ok, fused_ok;
+  bool dense_ok;      // variant 3: the dense filter gradient over tiles, then the chain rule
 };
 FilterRoutes filter_routes(const cp4_shape& s, bool aligned8, bool aligned16, bool ws256) {
   FilterRoutes r;
@@ -1061,6 +1069,7 @@ FilterRoutes filter_routes(const cp4_shape& s, bool aligned8, bool aligned16, bo
       cp4::bwd_filter_fused_supported(
           filter_rank_tile(s, (s.Rank - 1) / filter_tile_ranks(s) * filter_tile_ranks(s)));
   r.fused_ok = aligned16 && (cp4::bwd_filter_fused_supported(s) || fused_tiles);
+  r.dense_ok = cp4::bwd_filter_dense_tiles_supported(s);
   return r;
 }
 int default_filter_variant(const cp4_shape& s, const FilterRoutes& r) {
@@ -1068,9 +1077,11 @@ int default_filter_variant(const cp4_shape& s, const FilterRoutes& r) {
     std::lock_guard<std::mutex> lk(g_tune_mu);
     auto it = g_tuned_filter.find(key_of(s));
     if (it != g_tuned_filter.end() &&
-        (it->second == 0 || (it->second == 1 && r.mfma_ok) || (it->second == 2 && r.fused_ok)))
+        (it->second == 0 || (it->second == 1 && r.mfma_ok) || (it->second == 2 && r.fused_ok) ||
+         (it->second == 3 && r.dense_ok)))
       return it->second;
   }
+  if (r.dense_ok && cp4::bwd_filter_dense_tiles_preferred(s)) return 3;
   const bool prefer_fused =
       r.fused_ok && (cp4::bwd_filter_fused_preferred(
                          s.Rank > filter_tile_ranks(s) ? filter_rank_tile(s, 0) : s) ||
@@ -1119,13 +1130,20 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
   const FilterRoutes routes = filter_routes(s, (bits & 7) == 0, (bits & 15) == 0,
                                             (reinterpret_cast<uintptr_t>(workspace) & 255) == 0);
   const bool tiles_ok = routes.tiles_ok;
-  if (variant > 2 || (variant == 1 && !routes.mfma_ok) || (variant == 2 && !routes.fused_ok))
+  if (variant > 3 || (variant == 1 && !routes.mfma_ok) || (variant == 2 && !routes.fused_ok) ||
+      (variant == 3 && !routes.dense_ok))
     return fail(CP4_ERR_UNSUPPORTED, "backward-filter variant cannot run this shape");
   cp4::BwdFilterArgs a{};
   a.x = x; a.dy = dy; a.FK = FK; a.FC = FC; a.FH = FH; a.FW = FW;
   a.dFK = dFK; a.dFC = dFC; a.dFH = dFH; a.dFW = dFW; a.workspace = workspace;
   a.N = s.N; a.C = s.C; a.T = s.T; a.H = s.H; a.W = s.W; a.pad = s.pad;
   a.Y = s.Y; a.X = s.X; a.R = s.Rank;
+  // few channels on both sides: the dense-gradient route takes any channel count as it is
+  if (variant < 0 && default_filter_variant(s, routes) == 3) variant = 3;
+  if (variant == 3) {
+    CP4_HIP(cp4::bwd_filter_dense_tiles_launch(a, st));
+    return CP4_OK;
+  }
   if (variant < 0 && filter_pad_route(s) && (bits & 15) == 0 &&
       (reinterpret_cast<uintptr_t>(workspace) & 255) == 0) {
     bool tuned_general = false;
@@ -1777,7 +1795,7 @@ cp4_status cp4_tune_backward_filter(const cp4_shape* shape, const float* x, cons
   if (shape->N == 0) return fail(CP4_ERR_SHAPE, "cannot tune an empty batch");
   int best = -1;
   float best_t = 0.f;
-  for (int v = 0; v < 3; ++v) {
+  for (int v = 0; v < 4; ++v) {
     float us = 0.f;
     rc = time_loop(
         [&] {
@@ -1915,8 +1933,9 @@ cp4_status cp4_tuned_entry(int index, cp4_shape* shape, int* backward_data, int*
 }
 
 const char* cp4_backward_filter_variant_name(int variant) {
-  static const char* const names[3] = {"general_valu", "mfma_four_launches", "mfma_fused_taps"};
-  return variant >= 0 && variant < 3 ? names[variant] : nullptr;
+  static const char* const names[4] = {"general_valu", "mfma_four_launches", "mfma_fused_taps",
+                                       "dense_gradient_tiles"};
+  return variant >= 0 && variant < 4 ? names[variant] : nullptr;
 }
 
 int cp4_tuned_filter_count(void) {
@@ -1948,8 +1967,8 @@ cp4_status cp4_tuned_filter_entry(int index, cp4_shape* shape, int* variant) {
 cp4_status cp4_set_tuned_filter_choice(const cp4_shape* shape, int variant) {
   cp4_status rc = check_shape(shape);
   if (rc != CP4_OK) return rc;
-  if (variant < 0 || variant > 2)
-    return fail(CP4_ERR_UNSUPPORTED, "backward-filter variants are numbered 0, 1 and 2");
+  if (variant < 0 || variant > 3)
+    return fail(CP4_ERR_UNSUPPORTED, "backward-filter variants are numbered 0 to 3");
   // (a choice the shape or the caller's alignment does not allow is ignored at launch)
   std::lock_guard<std::mutex> lk(g_tune_mu);
   g_tuned_filter[key_of(*shape)] = variant;

@@ -172,6 +172,13 @@ bool bwd_filter_fused_supported(const cp4_shape&);
 bool bwd_filter_fused_preferred(const cp4_shape&);
 size_t bwd_filter_fused_workspace_bytes(const cp4_shape&);
 hipError_t bwd_filter_fused_launch(const BwdFilterArgs&, hipStream_t);
+// Few channels on both sides (T * C up to 256, square filters of 1, 3, 5 taps): the dense
+// filter gradient over tiles of pixels, then the chain rule onto the factors (three launches,
+// no [N, R, H, W] intermediates).
+bool bwd_filter_dense_tiles_supported(const cp4_shape&);
+bool bwd_filter_dense_tiles_preferred(const cp4_shape&);
+size_t bwd_filter_dense_tiles_workspace_bytes(const cp4_shape&);
+hipError_t bwd_filter_dense_tiles_launch(const BwdFilterArgs&, hipStream_t);
 // A layer with a stride and zeros of its own before the image (BwdFilterArgs::H, W: the
 // input plane; pad unused; dy on the geometry's Ho x Wo grid).
 bool bwd_filter_mfma_strided_supported(const cp4_shape&, const Geometry&);

@@ -1,0 +1,99 @@
+"""Backward-filter variant 3 (`dense_gradient_tiles`: the dense filter gradient
+dK[k,c,i,j] = sum dy[k,h,w] x[c,h+i-pad,w+j-pad] over tiles of pixels, then the chain rule
+onto the four factors; few channels on both sides) against the CPU oracle's factor-by-factor
+gradients (reference: Cuda_kernels/cp4Conv2dBackwardFilter.cu:64-257), through the C ABI.
+Tolerance: the backward-filter bar, |a-b| <= 1e-3*|b| + 1e-6*max|b| elementwise and
+max|a-b| <= 1e-3*max|b|."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+FACTORS = ("FK", "FC", "FH", "FW")
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+@pytest.fixture(scope="module")
+def cp4():
+    import paralleltnnlayers_amd as p
+    p.lib()
+    assert torch.cuda.is_available()
+    return p
+
+
+def close(got, want, what):
+    scale = float(np.abs(want).max())
+    err = np.abs(got - want)
+    assert np.all(err <= 1e-3 * np.abs(want) + 1e-6 * scale), f"{what}: elementwise {err.max():.3e}"
+    assert err.max() <= 1e-3 * scale, f"{what}: normalised {err.max() / scale:.3e}"
+
+
+# (N, C, H, W, pad, T, Y, R)
+SHAPES = [
+    (2, 3, 64, 200, 1, 1, 3, 16),      # the reference's sweep family: three channels to one
+    (1, 16, 40, 70, 1, 16, 3, 16),     # 256 channel pairs; tiles past the right edge
+    (3, 5, 13, 15, 1, 7, 3, 3),        # ragged channel blocks, odd planes
+    (2, 8, 33, 130, 2, 8, 5, 16),      # 5x5
+    (1, 12, 20, 64, 0, 20, 1, 12),     # 1x1
+    (2, 3, 17, 17, 2, 8, 3, 36),       # pad beyond (Y - 1) / 2, more ranks than channels
+    (1, 1, 100, 20, 1, 1, 3, 16),      # one channel each side
+    (4, 16, 7, 7, 1, 16, 3, 1),        # planes smaller than a tile, rank 1
+    (2, 4, 9, 300, 0, 2, 3, 5),        # no padding with a 3x3 filter
+    (2, 8, 130, 257, 1, 8, 3, 8),      # several tiles per workgroup
+]
+
+
+@pytest.mark.parametrize("dims", SHAPES, ids=lambda d: "x".join(map(str, d)))
+def test_dense_gradient_tiles(cp4, oracle, dims):
+    N, C, H, W, pad, T, Y, R = dims
+    rng = np.random.default_rng(sum(dims))
+    x = (rng.random((N, C, H, W)) * 2 - 1).astype(np.float32)
+    dy = rng.standard_normal((N, T, H, W)).astype(np.float32)
+    fac = [rng.standard_normal((d, R)).astype(np.float32) * np.float32((R * C) ** -0.25)
+           for d in (T, C, Y, Y)]
+    f = [dev(v) for v in fac]
+    assert cp4.backward_filter_variants()[3] == "dense_gradient_tiles"
+    wants = oracle.backward_filter(x, dy, *fac, pad)
+    first = None
+    for rep in range(2):       # bit-reproducible: no atomics anywhere
+        grads = cp4.conv2d_backward_filter(dev(x), dev(dy), *f, pad=pad, variant=3)
+        got = [host(g) for g in grads]
+        for g, w, k in zip(got, wants, FACTORS):
+            close(g, w, f"d{k}")
+        if first is None:
+            first = got
+        else:
+            assert all(np.array_equal(a, b) for a, b in zip(first, got))
+    cp4.device_status()
+
+
+def test_dense_gradient_is_the_default_for_few_channels(cp4):
+    def shape(N, C, H, W, T, R, Y=3):
+        return cp4.capi.Shape(N=N, H=H, W=W, pad=Y // 2, T=T, C=C, Y=Y, X=Y, Rank=R)
+    cp4.tune_clear()
+    name = "dense_gradient_tiles"
+    assert cp4.plan_query(shape(128, 3, 512, 512, 1, 16), "backward_filter")["variant"] == name
+    assert cp4.plan_query(shape(16, 16, 512, 512, 16, 16), "backward_filter")["variant"] == name
+    assert cp4.plan_query(shape(8, 8, 256, 256, 8, 16), "backward_filter")["variant"] == name
+    # many channels, and workload C5: the matrix-core variants
+    assert cp4.plan_query(shape(32, 256, 56, 56, 256, 32), "backward_filter")["variant"] != name
+    assert cp4.plan_query(shape(64, 256, 14, 14, 256, 64), "backward_filter")["variant"] != name
+
+
+def test_dense_gradient_refuses_many_channels(cp4):
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(1, 32, 8, 8, device="cuda", generator=g)
+    dy = torch.randn(1, 32, 8, 8, device="cuda", generator=g)
+    f = [torch.randn(d, 8, device="cuda", generator=g) / 4 for d in (32, 32, 3, 3)]
+    with pytest.raises(cp4.Cp4Error) as ei:
+        cp4.conv2d_backward_filter(x, dy, *f, pad=1, variant=3)
+    assert ei.value.status == cp4.capi.ERR_UNSUPPORTED

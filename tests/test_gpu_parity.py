@@ -69,10 +69,11 @@ def variants_for(cp4, x_shape, f, pad):
 
 def filter_variants(cp4, x, dy, f, pad):
     """Backward-filter variants that accept this shape: -1 (library's choice),
-    0 (general) and, where they qualify, 1 (matrix cores, four launches) and
-    2 (matrix cores, tap step fused into the gradient GEMMs)."""
+    0 (general) and, where they qualify, 1 (matrix cores, four launches),
+    2 (matrix cores, tap step fused into the gradient GEMMs) and 3 (few channels: the
+    dense filter gradient over tiles of pixels, then the chain rule)."""
     out = [-1, 0]
-    for v in (1, 2):
+    for v in (1, 2, 3):
         try:
             cp4.conv2d_backward_filter(x, dy, *f, pad=pad, variant=v)
             out.append(v)
@@ -529,7 +530,8 @@ def test_tuner_table_round_trip(cp4, tmp_path):
         # the backward-filter tuner's own table travels in the same file
         best, _ = cp4.tune_backward_filter(x, dev(a["dy"]), *f, w.pad, warmup=1, profcount=3)
         fnames = cp4.backward_filter_variants()
-        assert fnames == ["general_valu", "mfma_four_launches", "mfma_fused_taps"]
+        assert fnames == ["general_valu", "mfma_four_launches", "mfma_fused_taps",
+                          "dense_gradient_tiles"]
         ftable = cp4.tuned_filter_table()
         assert len(ftable) == 1 and ftable[0]["variant"] == fnames[best]
         table = cp4.tuned_table()
