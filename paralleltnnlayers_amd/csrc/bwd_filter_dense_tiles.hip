@@ -27,7 +27,7 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kCB = 4;                       // input channels per thread
 constexpr int kMaxPairs = 256;               // T * C up to here
-constexpr int kMaxGrid = 512;                // partial sets (two workgroups per compute unit)
+constexpr int kMaxGrid = 1024;               // partial sets (up to four workgroups per compute unit)
 constexpr size_t kLdsLimit = 64 * 1024;
 
 struct DensePlan {
@@ -370,7 +370,12 @@ bool plan(const cp4_shape& s, DensePlan* best) {
       pl.lgtile = __builtin_ctz(TW) + __builtin_ctz(TH);
       pl.chmagic = (unsigned)((0x100000000ull + (unsigned)((TH + FS - 1) * XS) - 1) / (unsigned)((TH + FS - 1) * XS));
       pl.xsmagic = (unsigned)((0x100000000ull + (unsigned)XS - 1) / (unsigned)XS);
-      pl.grid = pl.ntiles < 2 * cus ? pl.ntiles : 2 * cus;
+      // workgroups per compute unit: what the LDS and the registers (two waves per SIMD with
+      // two output channels a thread, three with one) leave room for
+      const int by_lds = (int)(160 * 1024 / (lds > red ? lds : red));
+      int per_cu = KB == 2 || FS >= 5 ? 2 : 3;
+      per_cu = per_cu < by_lds ? per_cu : (by_lds < 1 ? 1 : by_lds);
+      pl.grid = pl.ntiles < per_cu * cus ? pl.ntiles : per_cu * cus;
       if (pl.grid > kMaxGrid) pl.grid = kMaxGrid;
       {
         const size_t per_group = red;                 // S sets of a thread's partial sums
