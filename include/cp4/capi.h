@@ -210,9 +210,11 @@ cp4_status cp4_conv2d_backward_filter_noalloc(const cp4_shape* shape, const floa
  * the gradient GEMMs (square odd filters up to 5x5 with 2 * pad == Y - 1, channel
  * counts multiples of 16, H * W a multiple of 4, W >= 8, 16-byte aligned x / dy /
  * workspace), 3 the dense filter gradient over tiles of pixels followed by the chain
- * rule onto the factors, for few channels on both sides (T * C <= 256, square filters of
- * 1, 3 or 5 taps, pad <= Y - 1; any alignment); CP4_ERR_UNSUPPORTED if the shape does
- * not qualify for 1, 2 or 3. */
+ * rule onto the factors, for few channels on both sides (T * C <= 256 with plain
+ * multiply-adds, or on the matrix cores T <= 64, T * C * Y * X <= 16384 and a tile of
+ * all channels within the LDS, about 80 channels together; square filters of 1, 3 or 5
+ * taps, pad <= Y - 1; any alignment); CP4_ERR_UNSUPPORTED if the shape does not qualify
+ * for 1, 2 or 3. */
 cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const float* x,
                                               const float* dy, const float* FK,
                                               const float* FC, const float* FH,

@@ -9,7 +9,9 @@
 // them through memory (N16 C3 K1 512x512 R16: 67 MB of activations, 1.0 ms).  The dense
 // gradient has K*C*Y*X entries (27 there), needs x and dy once and no intermediate at all.
 //
-//   1. dense_tiles_kernel<FS, KB>: persistent workgroups of 256 threads over tiles of
+//   1. a tile kernel, one of two (use_mfma): dense_mfma_kernel, the sums as a GEMM over the
+//      pixels on the matrix cores, described where it is defined, or
+//      dense_tiles_kernel<FS, KB>: persistent workgroups of 256 threads over tiles of
 //      TH x TW pixels; the x tile with its halo and the dy tile go to LDS (zero outside the
 //      image); a thread owns KB output channels x 4 input channels x FS x FS taps in
 //      registers and a run of consecutive pixels of one row, along which the FS x FS window of
@@ -17,12 +19,17 @@
 //      workgroup's tiles, are added over the threads that share a channel block through LDS in
 //      fixed order, and leave as one partial set per workgroup.
 //   2. dense_reduce_kernel: the partial sets summed in fixed order.
-//   3. dense_fold_kernel: the chain rule, one thread per factor-gradient entry.
-// No atomics: bit-reproducible.  Plain fp32 multiply-adds.
+//   3. dense_fold_kernel: the chain rule, a workgroup per 32 ranks and gradient.
+// No atomics: bit-reproducible.  Plain fp32 multiply-adds, or exact fp32 products from bf16
+// parts on the matrix cores.
 #include "cp4_internal.h"
+#include "split_bf16.h"
 
 namespace cp4 {
 namespace {
+
+using split::f32x16;
+using split::u32x4;
 
 constexpr int kThreads = 256;
 constexpr int kCB = 4;                       // input channels per thread
@@ -203,6 +210,273 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
   }
 }
 
+// ---- the same sums on the matrix cores, for more channels -------------------------------
+// dK as a GEMM whose inner dimension is the pixels: rows = output channels k, columns
+// n = (c, i, j), dK[k][n] = sum_p dy[k][p] * x[c][p + (i, j)], exact fp32 products from three
+// bf16 parts per operand.  The LDS holds x (with its halo) and dy of a tile already split, as
+// three planes of bf16 parts each (a tap's column reads the same x cells shifted: split per
+// use, that work would be FS * FS times as much), in two buffers:
+//   1. the next tile's cells are loaded into registers (four consecutive cells a thread and
+//      slot; the cell a thread loads is the same in every tile, its offset worked out once);
+//   2. the waves take their steps of 16 consecutive pixels of a row of the current tile:
+//      lane (k, half) reads its 8 pixels of dy[k] from the planes (16-byte reads), lane
+//      (n, half) the 8 cells of column n's channel and tap (five dwords from the cell's even
+//      neighbour on, shifted by 16 bits where it is odd), a block's reads issued before the
+//      block before it goes to the matrix cores;
+//   3. the registers are split and written to the other buffer; one barrier per tile.
+// A wave owns up to eight 32 x 32 accumulator blocks for the whole launch: `own` blocks of
+// columns (every nbw-th) x MB blocks of output channels; the 8 / nbw waves that share
+// column blocks take every (8 / nbw)-th step and are added in fixed order at the end.
+constexpr int kMThreads = 512, kMWaves = kMThreads / 64;
+constexpr int kMaxAcc = 6;
+constexpr int kMaxOuts = 16384;              // T * C * Y * X up to here
+constexpr size_t kMLds = 160 * 1024;
+constexpr int kSlots = 6;                    // groups of four cells a thread stages per tile
+
+struct MfmaPlan {
+  int TH, TW, lgTW, tilesX, tilesY, ntiles;
+  int XS, XR, PHXS, DS;   // x: row stride, channel stride, cells of a channel's rows; dy: channel stride
+  int vec, xlead;         // 16-byte loads; columns of x staged before the tile's first (pad, or 4)
+  int nx, nd;             // cells staged: C * XR, T * DS (multiples of 4)
+  int xplane, dplane;     // cells per plane (multiples of 8)
+  int bufbytes;           // one buffer: three planes of x, three of dy
+  int NC, NB, MB;         // columns C * FS * FS; blocks of 32 of them; blocks of 32 output channels
+  int nbw, slices, own;   // waves across column blocks; waves across steps; column blocks a wave
+  int outs, grid;
+  unsigned chmagic, xsmagic, dsmagic;
+  size_t lds_bytes;
+};
+
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ u32x4 funnel(const unsigned (&d)[5], unsigned shift) {
+  u32x4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r[i] = __builtin_amdgcn_alignbit(d[i + 1], d[i], shift);
+  return r;
+}
+// Exact split of 4 floats into bf16 parts.
+__device__ __forceinline__ void split4(const float (&v)[4], u32x2& h, u32x2& m, u32x2& l) {
+#pragma unroll
+  for (int d = 0; d < 2; ++d) {
+    const float a = v[2 * d], b = v[2 * d + 1];
+    h[d] = split::pack_hi16(a, b);
+    const float ra = a - split::trunc_bf16(a), rb = b - split::trunc_bf16(b);
+    m[d] = split::pack_hi16(ra, rb);
+    const float sa = ra - split::trunc_bf16(ra), sb = rb - split::trunc_bf16(rb);
+    l[d] = split::pack_hi16(sa, sb);
+  }
+}
+
+template <int FS, int MB>
+__global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs a, MfmaPlan pl,
+                                                                  float* partial) {
+  constexpr int OWN = kMaxAcc / MB;
+  extern __shared__ float lds[];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int l32 = lane & 31, hi = lane >> 5;
+  const int H = a.H, W = a.W, HW = H * W;
+  const int b = wave & (pl.nbw - 1), sl = wave / pl.nbw;
+  // this lane's column of every column block the wave owns, and its output channel of every
+  // row block (past the last column / channel: the last one's cells, whose sums are not kept)
+  int boff[OWN], aoff[MB];
+#pragma unroll
+  for (int o = 0; o < OWN; ++o) {
+    int n = 32 * (b + o * pl.nbw) + l32;
+    n = n < pl.NC ? n : pl.NC - 1;
+    const int c = n / (FS * FS), tap = n - c * (FS * FS), i = tap / FS, j = tap - i * FS;
+    boff[o] = c * pl.XR + i * pl.XS + j + (pl.xlead - a.pad) + 8 * hi;
+  }
+#pragma unroll
+  for (int m = 0; m < MB; ++m) {
+    int k = 32 * m + l32;
+    k = k < a.T ? k : a.T - 1;
+    aoff[m] = k * pl.DS + 8 * hi;
+  }
+  // column blocks this wave has: b, b + nbw, ... below NB
+  const int nown = (pl.NB - b + pl.nbw - 1) / pl.nbw;
+  f32x16 acc[OWN][MB];
+#pragma unroll
+  for (int o = 0; o < OWN; ++o)
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[o][m][v] = 0.f;
+
+  // Slot q of this thread: the group of four cells g = tid + 512 q of the tile (x's groups,
+  // then dy's): where it goes in the planes, its offset from the tile's first cell in memory,
+  // and its row and column in the tile (-1: padding, zeros).
+  const int xgroups = pl.nx >> 2, groups = xgroups + (pl.nd >> 2);
+  unsigned rel[kSlots];
+  int rc[kSlots];
+#pragma unroll
+  for (int q = 0; q < kSlots; ++q) {
+    const int g = tid + kMThreads * q;
+    if (g < xgroups) {
+      const int e = 4 * g;
+      const int c = (int)__umulhi((unsigned)e, pl.chmagic), r2 = e - c * pl.XR;
+      const int pr = (int)__umulhi((unsigned)r2, pl.xsmagic), pc = r2 - pr * pl.XS;
+      rel[q] = (unsigned)(c * HW + pr * W + pc);
+      rc[q] = r2 < pl.PHXS ? (pr << 16) | pc : -1;
+    } else {
+      const int e = 4 * (g - xgroups);
+      const int k = (int)__umulhi((unsigned)e, pl.dsmagic), r2 = e - k * pl.DS;
+      const int pr = r2 >> pl.lgTW, pc = r2 & (pl.TW - 1);
+      rel[q] = (unsigned)(k * HW + pr * W + pc);
+      rc[q] = g < groups && pr < pl.TH ? (pr << 16) | pc : -1;
+    }
+  }
+
+  const int tiles_per_image = pl.tilesX * pl.tilesY;
+  const int lgcw = pl.lgTW - 4, nsteps = (pl.TH * pl.TW) >> 4;
+  float4 held[kSlots];
+  // Tile t's cells into this thread's registers (zeros outside the image).
+  auto fetch = [&](int t) {
+    const int n = t / tiles_per_image, rem = t - n * tiles_per_image;
+    const int ty = rem / pl.tilesX, tx = rem - ty * pl.tilesX;
+    const int hx = ty * pl.TH - a.pad, wx = tx * pl.TW - pl.xlead;   // x's first staged cell
+    const int hd = ty * pl.TH, wd = tx * pl.TW;                      // dy's
+    const float* xn = a.x + (size_t)n * a.C * HW;
+    const float* dn = a.dy + (size_t)n * a.T * HW;
+#pragma unroll
+    for (int q = 0; q < kSlots; ++q) {
+      const int g = tid + kMThreads * q;
+      const bool isx = g < xgroups;
+      const int h0 = isx ? hx : hd, w0 = isx ? wx : wd;
+      const float* src = isx ? xn : dn;
+      const int h = h0 + (rc[q] >> 16), w = w0 + (rc[q] & 0xffff);
+      const bool row_in = rc[q] >= 0 && (unsigned)h < (unsigned)H;
+      const long at = (long)rel[q] + (long)h0 * W + w0;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (pl.vec) {
+        // rows start at multiples of four columns and W % 4 == 0: four cells are inside
+        // the image together or not at all
+        if (row_in && (unsigned)w < (unsigned)W) v = *reinterpret_cast<const float4*>(src + at);
+      } else if (row_in) {
+        // (unaligned rows, or a width that four does not divide: cell by cell)
+        if ((unsigned)w < (unsigned)W) v.x = src[at];
+        if ((unsigned)(w + 1) < (unsigned)W) v.y = src[at + 1];
+        if ((unsigned)(w + 2) < (unsigned)W) v.z = src[at + 2];
+        if ((unsigned)(w + 3) < (unsigned)W) v.w = src[at + 3];
+      }
+      held[q] = v;
+    }
+  };
+  // The registers, split, into buffer `buf`.
+  auto deposit = [&](char* buf) {
+#pragma unroll
+    for (int q = 0; q < kSlots; ++q) {
+      const int g = tid + kMThreads * q;
+      if (g < groups) {
+        const bool isx = g < xgroups;
+        const int e = isx ? 4 * g : 4 * (g - xgroups);
+        const int plane = isx ? pl.xplane : pl.dplane;
+        char* base = buf + (isx ? 0 : 6 * pl.xplane) + 2 * e;
+        const float v[4] = {held[q].x, held[q].y, held[q].z, held[q].w};
+        u32x2 h, m, l;
+        split4(v, h, m, l);
+        *reinterpret_cast<u32x2*>(base) = h;
+        *reinterpret_cast<u32x2*>(base + 2 * plane) = m;
+        *reinterpret_cast<u32x2*>(base + 4 * plane) = l;
+      }
+    }
+  };
+
+  char* const bufs = reinterpret_cast<char*>(lds);
+  fetch(blockIdx.x);
+  deposit(bufs);
+  __syncthreads();
+  int it = 0;
+  for (int t = blockIdx.x; t < pl.ntiles; t += gridDim.x, ++it) {
+    const bool more = t + (int)gridDim.x < pl.ntiles;
+    if (more) fetch(t + gridDim.x);
+    const char* cur = bufs + (size_t)(it & 1) * pl.bufbytes;
+    const unsigned* xp = reinterpret_cast<const unsigned*>(cur);
+    const char* dp = cur + 6 * pl.xplane;
+    const int xw = pl.xplane >> 1;                     // a plane of x in dwords
+    // ---- this wave's steps ----
+    for (int st = sl; st < nsteps; st += pl.slices) {
+      const int row = st >> lgcw, col0 = (st & ((1 << lgcw) - 1)) << 4;
+      u32x4 ah[MB], am[MB], al[MB];
+#pragma unroll
+      for (int m = 0; m < MB; ++m) {
+        const char* p = dp + 2 * (aoff[m] + (row << pl.lgTW) + col0);
+        ah[m] = *reinterpret_cast<const u32x4*>(p);
+        am[m] = *reinterpret_cast<const u32x4*>(p + 2 * pl.dplane);
+        al[m] = *reinterpret_cast<const u32x4*>(p + 4 * pl.dplane);
+      }
+      // cells off ... off + 7 of each plane: the dwords from off / 2, shifted by its parity
+      // (row strides and steps are even: the parity is that of the lane's column)
+      const int xo = row * pl.XS + col0;
+      unsigned dh[5], dm[5], dl[5];
+      {
+        const unsigned* q = xp + ((boff[0] + xo) >> 1);
+#pragma unroll
+        for (int i = 0; i < 5; ++i) { dh[i] = q[i]; dm[i] = q[xw + i]; dl[i] = q[2 * xw + i]; }
+      }
+#pragma unroll
+      for (int o = 0; o < OWN; ++o) {
+        if (o < nown) {
+          const unsigned shift = (unsigned)(boff[o] & 1) * 16u;
+          const u32x4 bh = funnel(dh, shift), bm = funnel(dm, shift), bl = funnel(dl, shift);
+          if (o + 1 < OWN && o + 1 < nown) {
+            const unsigned* q = xp + ((boff[o + 1 < OWN ? o + 1 : o] + xo) >> 1);
+#pragma unroll
+            for (int i = 0; i < 5; ++i) { dh[i] = q[i]; dm[i] = q[xw + i]; dl[i] = q[2 * xw + i]; }
+          }
+#pragma unroll
+          for (int m = 0; m < MB; ++m)
+            acc[o][m] = split::mfma_split(ah[m], am[m], al[m], bh, bm, bl, acc[o][m]);
+        }
+      }
+    }
+    if (more) deposit(bufs + (size_t)((it + 1) & 1) * pl.bufbytes);
+    __syncthreads();
+  }
+  // ---- the waves that shared column blocks, added in order through LDS ----
+  float* red = lds;                                  // [own block][row block][b][element][lane]
+  for (int s2 = 1; s2 < pl.slices; ++s2) {
+#pragma unroll
+    for (int o = 0; o < OWN; ++o)
+#pragma unroll
+      for (int m = 0; m < MB; ++m) {
+        float* r = red + (((size_t)(o * MB + m) * pl.nbw + b) << 10) + lane;
+        if (sl == s2 && o < pl.own) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) r[v << 6] = acc[o][m][v];
+        }
+      }
+    __syncthreads();
+#pragma unroll
+    for (int o = 0; o < OWN; ++o)
+#pragma unroll
+      for (int m = 0; m < MB; ++m) {
+        const float* r = red + (((size_t)(o * MB + m) * pl.nbw + b) << 10) + lane;
+        if (sl == 0 && o < pl.own) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[o][m][v] += r[v << 6];
+        }
+      }
+    __syncthreads();
+  }
+  if (sl != 0) return;
+  float* out = partial + (size_t)blockIdx.x * pl.outs;
+#pragma unroll
+  for (int o = 0; o < OWN; ++o) {
+    const int n = 32 * (b + o * pl.nbw) + l32;
+    if (o < pl.own && n < pl.NC) {
+#pragma unroll
+      for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int k = 32 * m + 8 * (v >> 2) + 4 * hi + (v & 3);
+          if (k < a.T) out[(size_t)k * pl.NC + n] = acc[o][m][v];
+        }
+    }
+  }
+}
+
 // dK[o] = sum over the partial sets in a fixed order: thread (o, y) adds sets y, y + 8, ...,
 // then the eight partial sums are added in order through LDS (one thread summing all the sets
 // of an entry would wait for several hundred loads one after the other).
@@ -237,10 +511,12 @@ __global__ __launch_bounds__(kRedOuts * kRedSets) void dense_reduce_kernel(const
   }
 }
 
-// The chain rule from dK [T][C][Y][X] onto the factors.  A workgroup takes 32 ranks: dK and
-// the factors' columns for those ranks go to LDS (read from memory inside the sums, every term
-// would wait for a load of its own), then a thread takes (rank, every 32nd row of the four
-// gradients).
+// The chain rule from dK [T][C][Y][X] onto the factors.  A workgroup takes 32 ranks and one of
+// the four gradients (blockIdx.y): dK and the factors' columns for those ranks go to LDS (read
+// from memory inside the sums, every term would wait for a load of its own), then a thread
+// takes a rank and every 32nd row of dFK or dFC, or, per output channel k, of the parts of
+// dFH[i] or dFW[j], which are then added over k in order (a whole dFH row in one thread would
+// be T * C * X terms long, the longest job by far).
 constexpr int kFoldRanks = 32, kFoldRows = 32;
 template <int FS>
 __global__ __launch_bounds__(kFoldRanks * kFoldRows) void dense_fold_kernel(BwdFilterArgs a,
@@ -248,13 +524,15 @@ __global__ __launch_bounds__(kFoldRanks * kFoldRows) void dense_fold_kernel(BwdF
   extern __shared__ float lds[];
   constexpr int Y = FS, X = FS;          // (square filters: the tap loops unroll, their loads overlap)
   const int T = a.T, C = a.C, R = a.R;
-  const int outs = T * C * Y * X, rows = T + C + Y + X;
+  const int outs = T * C * Y * X, frows = T + C + Y + X;
   float* dk = lds;                         // [T][C][Y][X]
   float* fac = lds + outs;                 // [T + C + Y + X][32]: FK, FC, FH, FW rows
+  float* part = fac + frows * kFoldRanks;  // [FS][T][32]: per tap row or column and output channel
   const int tid = threadIdx.y * kFoldRanks + threadIdx.x;
   const int r0 = blockIdx.x * kFoldRanks, r = r0 + threadIdx.x;
+  const int job = blockIdx.y;              // 0 dFK, 1 dFC, 2 dFH, 3 dFW
   for (int e = tid; e < outs; e += kFoldRanks * kFoldRows) dk[e] = dK[e];
-  for (int e = tid; e < rows * kFoldRanks; e += kFoldRanks * kFoldRows) {
+  for (int e = tid; e < frows * kFoldRanks; e += kFoldRanks * kFoldRows) {
     const int row = e / kFoldRanks, rr = r0 + (e % kFoldRanks);
     const float* src = row < T ? a.FK + (size_t)row * R
                      : row < T + C ? a.FC + (size_t)(row - T) * R
@@ -267,11 +545,9 @@ __global__ __launch_bounds__(kFoldRanks * kFoldRows) void dense_fold_kernel(BwdF
   const float* fc = fk + T * kFoldRanks;
   const float* fh = fc + C * kFoldRanks;
   const float* fw = fh + Y * kFoldRanks;
-  if (r >= R) return;
-  for (int row = threadIdx.y; row < rows; row += kFoldRows) {
-    float s = 0.f;
-    if (row < T) {
-      const int k = row;
+  if (job == 0) {
+    for (int k = threadIdx.y; k < T; k += kFoldRows) {
+      float s = 0.f;
 #pragma unroll 4
       for (int c = 0; c < C; ++c) {
         float sc = 0.f;
@@ -284,9 +560,13 @@ __global__ __launch_bounds__(kFoldRanks * kFoldRows) void dense_fold_kernel(BwdF
         }
         s += sc * fc[c * kFoldRanks];
       }
-      a.dFK[(size_t)k * R + r] = s;
-    } else if (row < T + C) {
-      const int c = row - T;
+      if (r < R) a.dFK[(size_t)k * R + r] = s;
+    }
+    return;
+  }
+  if (job == 1) {
+    for (int c = threadIdx.y; c < C; c += kFoldRows) {
+      float s = 0.f;
 #pragma unroll 4
       for (int k = 0; k < T; ++k) {
         float sk = 0.f;
@@ -299,37 +579,40 @@ __global__ __launch_bounds__(kFoldRanks * kFoldRows) void dense_fold_kernel(BwdF
         }
         s += sk * fk[k * kFoldRanks];
       }
-      a.dFC[(size_t)c * R + r] = s;
-    } else if (row < T + C + Y) {
-      const int i = row - T - C;
-      for (int k = 0; k < T; ++k) {
-        float sk = 0.f;
-#pragma unroll 4
-        for (int c = 0; c < C; ++c) {
-          float sc = 0.f;
-#pragma unroll
-          for (int j = 0; j < X; ++j) sc += dk[((k * C + c) * Y + i) * X + j] * fw[j * kFoldRanks];
-          sk += sc * fc[c * kFoldRanks];
-        }
-        s += sk * fk[k * kFoldRanks];
-      }
-      a.dFH[(size_t)i * R + r] = s;
-    } else {
-      const int j = row - T - C - Y;
-      for (int k = 0; k < T; ++k) {
-        float sk = 0.f;
-#pragma unroll 4
-        for (int c = 0; c < C; ++c) {
-          float sc = 0.f;
-#pragma unroll
-          for (int i = 0; i < Y; ++i) sc += dk[((k * C + c) * Y + i) * X + j] * fh[i * kFoldRanks];
-          sk += sc * fc[c * kFoldRanks];
-        }
-        s += sk * fk[k * kFoldRanks];
-      }
-      a.dFW[(size_t)j * R + r] = s;
+      if (r < R) a.dFC[(size_t)c * R + r] = s;
     }
+    return;
   }
+  // the tap row i (dFH) or column j (dFW) and output channel k of q = i * T + k
+  for (int q = threadIdx.y; q < FS * T; q += kFoldRows) {
+    const int ij = q / T, k = q - ij * T;
+    float s = 0.f;
+#pragma unroll 4
+    for (int c = 0; c < C; ++c) {
+      float sc = 0.f;
+      if (job == 2) {
+#pragma unroll
+        for (int j = 0; j < X; ++j) sc += dk[((k * C + c) * Y + ij) * X + j] * fw[j * kFoldRanks];
+      } else {
+#pragma unroll
+        for (int i = 0; i < Y; ++i) sc += dk[((k * C + c) * Y + i) * X + ij] * fh[i * kFoldRanks];
+      }
+      s += sc * fc[c * kFoldRanks];
+    }
+    part[q * kFoldRanks + threadIdx.x] = s * fk[k * kFoldRanks];
+  }
+  __syncthreads();
+  if (threadIdx.y < FS && r < R) {
+    const float* p = part + (size_t)threadIdx.y * T * kFoldRanks + threadIdx.x;
+    float s = 0.f;
+    for (int k = 0; k < T; ++k) s += p[k * kFoldRanks];
+    (job == 2 ? a.dFH : a.dFW)[(size_t)threadIdx.y * R + r] = s;
+  }
+}
+
+size_t fold_lds_bytes(const cp4_shape& s) {
+  return ((size_t)s.T * s.C * s.Y * s.X + (size_t)(s.T + s.C + s.Y + s.X) * kFoldRanks +
+          (size_t)s.Y * s.T * kFoldRanks) * sizeof(float);
 }
 
 int kb_of(const cp4_shape& s) { return s.T >= 2 && s.Y <= 3 ? 2 : 1; }
@@ -412,34 +695,180 @@ hipError_t launch_fs(const BwdFilterArgs& a, const DensePlan& pl, int kb, float*
   return hipGetLastError();
 }
 
+bool mfma_plan(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
+  const int vec = aligned16 && s.W % 4 == 0 ? 1 : 0, xlead = vec ? 4 : (int)s.pad;
+  const int FS = (int)s.Y, T = (int)s.T, C = (int)s.C;
+  const int NC = C * FS * FS, NB = (NC + 31) / 32, MB = (T + 31) / 32;
+  if (MB > 2 || (long)T * NC > kMaxOuts) return false;
+  int nbw = 1;
+  while (nbw <= kMWaves && (NB + nbw - 1) / nbw * MB > kMaxAcc) nbw *= 2;
+  if (nbw > kMWaves) return false;
+  const int slices = kMWaves / nbw, own = (NB + nbw - 1) / nbw;
+  const size_t red = (size_t)own * MB * nbw * 1024 * sizeof(float);
+  const int cus = num_compute_units();
+  bool found = false;
+  double best_cost = 0;
+  for (int TW = 16; TW <= 128; TW *= 2)
+    for (int TH = 1; TH <= 32; TH *= 2) {
+      if (TH * TW / 16 < slices) continue;
+      const int PH = TH + FS - 1;
+      // (a multiple of four: a group of four staged cells stays within a row)
+      const int XS = vec ? TW + 8 : (TW + FS - 1 + 3) / 4 * 4;
+      // a channel's rows, then as many cells as put consecutive channels ten banks of dwords
+      // apart in the bf16 planes: with rows 4 banks apart (XS = 8 mod 64) or any stride, the
+      // taps of the four channels that a step's 32 columns cover then fall into different banks
+      int XR = (PH * XS + 3) / 4 * 4;
+      while (XR % 64 != 20) XR += 4;
+      const int DS = TH * TW + 8;                      // output channels four banks apart
+      const int nx = C * XR, nd = T * DS;
+      if ((nx + nd) / 4 > kSlots * kMThreads) continue;
+      // LDS: two buffers of (x in three planes of bf16 parts | dy likewise); x's planes a few
+      // cells longer: a column's reads end up to two cells past the last
+      const int xplane = (nx + 8 + 7) / 8 * 8, dplane = (nd + 7) / 8 * 8;
+      const int bufbytes = 6 * (xplane + dplane);
+      size_t lds = 2 * (size_t)bufbytes;
+      if (slices > 1 && red > lds) lds = red;
+      if (lds > kMLds) continue;
+      MfmaPlan pl;
+      pl.TH = TH; pl.TW = TW;
+      pl.lgTW = __builtin_ctz(TW);
+      pl.tilesX = ((int)s.W + TW - 1) / TW;
+      pl.tilesY = ((int)s.H + TH - 1) / TH;
+      pl.ntiles = (int)s.N * pl.tilesX * pl.tilesY;
+      pl.XS = XS; pl.XR = XR; pl.PHXS = PH * XS; pl.DS = DS; pl.vec = vec; pl.xlead = xlead;
+      pl.nx = nx; pl.nd = nd; pl.xplane = xplane; pl.dplane = dplane; pl.bufbytes = bufbytes;
+      pl.NC = NC; pl.NB = NB; pl.MB = MB;
+      pl.nbw = nbw; pl.slices = slices; pl.own = own;
+      pl.outs = T * NC;
+      pl.chmagic = (unsigned)((0x100000000ull + (unsigned)XR - 1) / (unsigned)XR);
+      pl.xsmagic = (unsigned)((0x100000000ull + (unsigned)XS - 1) / (unsigned)XS);
+      pl.dsmagic = (unsigned)((0x100000000ull + (unsigned)DS - 1) / (unsigned)DS);
+      pl.lds_bytes = lds;
+      pl.grid = pl.ntiles < cus ? pl.ntiles : cus;
+      // (the partial sets stay within 24 MiB)
+      const long set_bytes = ((long)pl.outs * 4 + 255) / 256 * 256;
+      const long most = (24l << 20) / set_bytes - 1;
+      if (pl.grid > most) pl.grid = (int)most;
+      if (pl.grid > kMaxGrid) pl.grid = kMaxGrid;
+      if (pl.grid < 1) continue;
+      // cells staged per output pixel (halo, pixels past the image's edge), a grid that leaves
+      // compute units idle, and the fixed cost of a tile
+      const double area = (double)pl.tilesX * TW * pl.tilesY * TH / ((double)s.W * s.H);
+      const double halo = (double)XR / ((double)TH * TW);
+      const double staged = ((double)C * halo + T) / (C + T);
+      const double fill = (double)((pl.ntiles + pl.grid - 1) / pl.grid * pl.grid) / pl.ntiles;
+      const double cost = area * fill * (0.5 + 0.5 * staged) * (1.0 + 64.0 / (TH * TW));
+      if (!found || cost < best_cost) {
+        best_cost = cost;
+        *best = pl;
+        found = true;
+      }
+    }
+  return found;
+}
+
+template <int FS>
+hipError_t launch_mfma_fs(const BwdFilterArgs& a, const MfmaPlan& pl, float* partial, hipStream_t st) {
+  auto k1 = dense_mfma_kernel<FS, 1>;
+  auto k2 = dense_mfma_kernel<FS, 2>;
+  auto k = pl.MB == 2 ? k2 : k1;
+  if (pl.lds_bytes > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds_bytes);
+    if (e != hipSuccess) return e;
+  }
+  k<<<pl.grid, kMThreads, pl.lds_bytes, st>>>(a, pl, partial);
+  return hipGetLastError();
+}
+
+template <int FS>
+hipError_t launch_fold(const BwdFilterArgs& a, const float* dK, size_t lds, hipStream_t st) {
+  auto k = dense_fold_kernel<FS>;
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+  }
+  const dim3 fgrid((a.R + kFoldRanks - 1) / kFoldRanks, 4), fblock(kFoldRanks, kFoldRows);
+  k<<<fgrid, fblock, lds, st>>>(a, dK);
+  return hipGetLastError();
+}
+
+cp4_shape shape_of(const BwdFilterArgs& a) {
+  cp4_shape s{};
+  s.N = a.N; s.C = a.C; s.T = a.T; s.H = a.H; s.W = a.W; s.pad = a.pad; s.Y = a.Y; s.X = a.X; s.Rank = a.R;
+  return s;
+}
+
+bool common_ok(const cp4_shape& s) {
+  if (s.Y != s.X || !(s.Y == 1 || s.Y == 3 || s.Y == 5) || s.pad > s.Y - 1) return false;
+  if (s.N == 0 || !fits_int_indexing((int)s.N, (int)s.H, (int)s.W)) return false;
+  return fold_lds_bytes(s) <= 150 * 1024;
+}
+
+bool valu_ok(const cp4_shape& s) {
+  DensePlan pl;
+  return common_ok(s) && (long)s.T * s.C <= kMaxPairs && plan(s, &pl);
+}
+
+bool mfma_ok(const cp4_shape& s) {
+  MfmaPlan pl;
+  return common_ok(s) && mfma_plan(s, false, &pl);
+}
+
+// Which of the two tile kernels.  The matrix cores wherever they can run, except for one to
+// three output channels under a 3x3 or 5x5 filter on large inputs: there a 32-row block of
+// the GEMM is nearly empty and the plain multiply-adds are the faster ones (N16 C32 K1
+// 256x256 3x3: 112 us against 177; N128 C3 K1 512x512: 336 against 515).
+bool use_mfma(const cp4_shape& s) {
+  if (!mfma_ok(s)) return false;
+  if (!valu_ok(s)) return true;
+  const double cells = (double)s.N * s.H * s.W * s.C;
+  return !(s.T <= 3 && s.Y >= 3 && cells >= 3.0e6);
+}
+
 }  // namespace
 
-bool bwd_filter_dense_tiles_supported(const cp4_shape& s) {
-  if (s.Y != s.X || !(s.Y == 1 || s.Y == 3 || s.Y == 5) || s.pad > s.Y - 1) return false;
-  if ((long)s.T * s.C > kMaxPairs || s.N == 0) return false;
-  if (!fits_int_indexing((int)s.N, (int)s.H, (int)s.W)) return false;
-  DensePlan pl;
-  return plan(s, &pl);
-}
+bool bwd_filter_dense_tiles_supported(const cp4_shape& s) { return valu_ok(s) || mfma_ok(s); }
 
 // Partial sets of the tile kernel, then the dense gradient itself.
 size_t bwd_filter_dense_tiles_workspace_bytes(const cp4_shape& s) {
-  const size_t outs = (size_t)s.T * s.C * s.Y * s.X;
-  return (kMaxGrid + 1) * ((outs * sizeof(float) + 255) / 256 * 256);
+  const size_t set = ((size_t)s.T * s.C * s.Y * s.X * sizeof(float) + 255) / 256 * 256;
+  size_t sets = 0;
+  DensePlan dp;
+  MfmaPlan mp;
+  if (valu_ok(s) && plan(s, &dp)) sets = dp.grid;
+  if (mfma_ok(s) && mfma_plan(s, false, &mp) && (size_t)mp.grid > sets) sets = mp.grid;
+  if (mfma_ok(s) && mfma_plan(s, true, &mp) && (size_t)mp.grid > sets) sets = mp.grid;
+  return (sets + 1) * set;
 }
 
-// Where this route is the faster one: two linear time models (us) fitted by least squares to
-// both routes over 378 layers (3 - 32 channels a side, 1x1 / 3x3 / 5x5, ranks 4 and 16, a
-// thousand to a million pixels; the choice they make is 3 % off the better route in the
-// geometric mean).  Here a fixed 18 us plus the final sums and the chain rule (0.05 us per
-// channel pair, 0.008 per multiply-add of a pixel, M = T * C * Y * X), and per million pixels the staging of the tiles (2.7 us per
-// channel staged) and the multiply-adds (0.375 us per channel-block group and tap); the
-// factor-by-factor variants 26 us plus per million pixels 115 us and what grows with the
-// planes (N16 C3 K1 512x512 R16: 1005 us -> 63; N8 C8 K8 256x256 R16: 132 -> 52; N16 C16 K16
-// 512x512 R16: 1058 -> 900; but N1 C16 K16 32x32 R8: 21 against 54).
+// Where this route is the faster one: linear time models (us) fitted by least squares to
+// measured times of this route and of the factor-by-factor variants over some 400 layers each
+// (1 - 64 channels a side, 1x1 / 3x3 / 5x5, ranks 4 and 16, a thousand to a million pixels).
+// With the matrix-core tile kernel: 16 us, 3.1 us per thousand entries of dK (the final sums
+// and the chain rule), and per million pixels 0.83 us per channel staged and 14.4 per 32 x 32
+// block of the GEMM; the factor-by-factor variants 19 us and per million pixels 2.5 us per
+// channel and 0.28 per tap and rank; this route where its model is below 1.2 times theirs
+// (1.3 % off the better route in the geometric mean; always this route 10 % off, never 17 %).
+// With the plain multiply-add tile kernel: a fixed 18 us plus the final sums and the chain
+// rule, and per million pixels the staging of the tiles (2.7 us per channel staged) and the
+// multiply-adds (0.375 us per channel-block group and tap), against 26 us plus per million
+// pixels 115 us and what grows with the planes.
+// (N16 C16 K16 512x512 R16: 1040 us -> 350; N16 C3 K1 512x512 R16: 1005 -> 63; N8 C8 K8
+// 256x256 R16: 132 -> 42; but N1 C16 K16 32x32 R8: 18 against 27.)
 bool bwd_filter_dense_tiles_preferred(const cp4_shape& s) {
   const double mpx = (double)s.N * s.H * s.W / 1.0e6;
   const double taps = (double)s.Y * s.X, macs = (double)s.T * s.C * taps;
+  if (use_mfma(s)) {
+    const double blocks = (double)((s.C * s.Y * s.X + 31) / 32) * ((s.T + 31) / 32);
+    const double dense = 16.03 + 3.143e-3 * macs +
+                         mpx * (-6.15 + 0.829 * (s.C + s.T) + 14.42 * blocks);
+    double planes = 18.79 + mpx * (-10.31 + 2.547 * (s.T + s.C) - 1.559 * s.Rank +
+                                   0.2778 * taps * s.Rank);
+    if (planes < 10.0) planes = 10.0;
+    return dense < 1.2 * planes;
+  }
   const int kb = s.T >= 2 && s.Y <= 3 ? 2 : 1;
   const double groups = (double)((s.T + kb - 1) / kb) * ((s.C + kCB - 1) / kCB);
   const double staged = 1.2 * ((s.C + kCB - 1) / kCB * kCB) + s.T;
@@ -451,34 +880,46 @@ bool bwd_filter_dense_tiles_preferred(const cp4_shape& s) {
 }
 
 hipError_t bwd_filter_dense_tiles_launch(const BwdFilterArgs& a, hipStream_t st) {
-  cp4_shape s{};
-  s.N = a.N; s.C = a.C; s.T = a.T; s.H = a.H; s.W = a.W; s.pad = a.pad; s.Y = a.Y; s.X = a.X; s.Rank = a.R;
-  DensePlan pl;
-  if (!plan(s, &pl)) return hipErrorInvalidValue;
-  const size_t set = ((size_t)pl.outs * sizeof(float) + 255) / 256 * 256 / sizeof(float);
+  const cp4_shape s = shape_of(a);
+  const int outs = a.T * a.C * a.Y * a.X;
+  const size_t set = ((size_t)outs * sizeof(float) + 255) / 256 * 256 / sizeof(float);
   float* ws = static_cast<float*>(a.workspace);
   float* dK = ws;
   float* partial = ws + set;
   hipError_t e;
-  // (the partial sets are pl.outs apart; the padded stride is only what the size allows for)
-  switch (a.Y) {
-    case 1: e = launch_fs<1>(a, pl, kb_of(s), partial, st); break;
-    case 3: e = launch_fs<3>(a, pl, kb_of(s), partial, st); break;
-    default: e = launch_fs<5>(a, pl, kb_of(s), partial, st); break;
+  int sets;
+  // (the partial sets are `outs` apart; the padded stride is only what the size allows for)
+  if (use_mfma(s)) {
+    MfmaPlan pl;
+    const bool aligned16 = ((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.dy)) & 15) == 0;
+    if (!mfma_plan(s, aligned16, &pl) && !mfma_plan(s, false, &pl)) return hipErrorInvalidValue;
+    sets = pl.grid;
+    switch (a.Y) {
+      case 1: e = launch_mfma_fs<1>(a, pl, partial, st); break;
+      case 3: e = launch_mfma_fs<3>(a, pl, partial, st); break;
+      default: e = launch_mfma_fs<5>(a, pl, partial, st); break;
+    }
+  } else {
+    DensePlan pl;
+    if (!valu_ok(s) || !plan(s, &pl)) return hipErrorInvalidValue;
+    sets = pl.grid;
+    switch (a.Y) {
+      case 1: e = launch_fs<1>(a, pl, kb_of(s), partial, st); break;
+      case 3: e = launch_fs<3>(a, pl, kb_of(s), partial, st); break;
+      default: e = launch_fs<5>(a, pl, kb_of(s), partial, st); break;
+    }
   }
   if (e != hipSuccess) return e;
-  dense_reduce_kernel<<<(pl.outs + kRedOuts - 1) / kRedOuts, dim3(kRedOuts, kRedSets), 0, st>>>(
-      partial, dK, pl.outs, pl.grid);
+  dense_reduce_kernel<<<(outs + kRedOuts - 1) / kRedOuts, dim3(kRedOuts, kRedSets), 0, st>>>(
+      partial, dK, outs, sets);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
-  const size_t fold_lds = ((size_t)pl.outs + (size_t)(a.T + a.C + a.Y + a.X) * kFoldRanks) * sizeof(float);
-  const dim3 fgrid((a.R + kFoldRanks - 1) / kFoldRanks), fblock(kFoldRanks, kFoldRows);
+  const size_t fold_lds = fold_lds_bytes(s);
   switch (a.Y) {
-    case 1: dense_fold_kernel<1><<<fgrid, fblock, fold_lds, st>>>(a, dK); break;
-    case 3: dense_fold_kernel<3><<<fgrid, fblock, fold_lds, st>>>(a, dK); break;
-    default: dense_fold_kernel<5><<<fgrid, fblock, fold_lds, st>>>(a, dK); break;
+    case 1: return launch_fold<1>(a, dK, fold_lds, st);
+    case 3: return launch_fold<3>(a, dK, fold_lds, st);
+    default: return launch_fold<5>(a, dK, fold_lds, st);
   }
-  return hipGetLastError();
 }
 
 }  // namespace cp4

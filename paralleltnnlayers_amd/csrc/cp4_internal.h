@@ -172,9 +172,10 @@ bool bwd_filter_fused_supported(const cp4_shape&);
 bool bwd_filter_fused_preferred(const cp4_shape&);
 size_t bwd_filter_fused_workspace_bytes(const cp4_shape&);
 hipError_t bwd_filter_fused_launch(const BwdFilterArgs&, hipStream_t);
-// Few channels on both sides (T * C up to 256, square filters of 1, 3, 5 taps): the dense
-// filter gradient over tiles of pixels, then the chain rule onto the factors (three launches,
-// no [N, R, H, W] intermediates).
+// Few channels on both sides (square filters of 1, 3, 5 taps; T * C up to 256 with plain
+// multiply-adds, or up to 64 output channels and 16384 entries of the dense gradient on the
+// matrix cores): the dense filter gradient over tiles of pixels, then the chain rule onto the
+// factors (three launches, no [N, R, H, W] intermediates).
 bool bwd_filter_dense_tiles_supported(const cp4_shape&);
 bool bwd_filter_dense_tiles_preferred(const cp4_shape&);
 size_t bwd_filter_dense_tiles_workspace_bytes(const cp4_shape&);
