@@ -228,7 +228,8 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
 // columns (every nbw-th) x MB blocks of output channels; the 8 / nbw waves that share
 // column blocks take every (8 / nbw)-th step and are added in fixed order at the end.
 constexpr int kMThreads = 512, kMWaves = kMThreads / 64;
-constexpr int kMaxAcc = 6;
+constexpr int kMaxAcc = 6;                   // 32 x 32 blocks a wave holds
+constexpr int kMaxAcc16 = 12;                // 16 x 16 blocks, with up to 16 output channels
 constexpr int kMaxOuts = 16384;              // T * C * Y * X up to here
 constexpr size_t kMLds = 160 * 1024;
 constexpr int kSlots = 6;                    // groups of four cells a thread stages per tile
@@ -240,7 +241,8 @@ struct MfmaPlan {
   int nx, nd;             // cells staged: C * XR, T * DS (multiples of 4)
   int xplane, dplane;     // cells per plane (multiples of 8)
   int bufbytes;           // one buffer: three planes of x, three of dy
-  int NC, NB, MB;         // columns C * FS * FS; blocks of 32 of them; blocks of 32 output channels
+  int m16;                // up to 16 output channels: 16 x 16 blocks, steps of 32 pixels
+  int NC, NB, MB;         // columns C * FS * FS; blocks of them; blocks of output channels
   int nbw, slices, own;   // waves across column blocks; waves across steps; column blocks a wave
   int outs, grid;
   unsigned chmagic, xsmagic, dsmagic;
@@ -248,6 +250,28 @@ struct MfmaPlan {
 };
 
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// One product of the split: 32 x 32 x 16 (lane: row or column lane % 32, eight of the 16
+// pixels by lane / 32) or 16 x 16 x 32 (lane % 16, eight of 32 pixels by lane / 16).
+__device__ __forceinline__ f32x16 mfma_any(u32x4 a, u32x4 b, f32x16 c) { return split::mfma16(a, b, c); }
+__device__ __forceinline__ f32x4 mfma_any(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(split::bf16x8, a),
+                                                 __builtin_bit_cast(split::bf16x8, b), c, 0, 0, 0);
+}
+template <class Acc>
+__device__ __forceinline__ Acc mfma_split_any(u32x4 ah, u32x4 am, u32x4 al, u32x4 bh, u32x4 bm,
+                                              u32x4 bl, Acc acc) {
+  acc = mfma_any(al, bh, acc);
+  acc = mfma_any(am, bm, acc);
+  acc = mfma_any(ah, bl, acc);
+  acc = mfma_any(am, bh, acc);
+  acc = mfma_any(ah, bm, acc);
+  acc = mfma_any(ah, bh, acc);
+  return acc;
+}
+template <bool M16> struct AccOf { typedef f32x16 type; };
+template <> struct AccOf<true> { typedef f32x4 type; };
 
 __device__ __forceinline__ u32x4 funnel(const unsigned (&d)[5], unsigned shift) {
   u32x4 r;
@@ -268,14 +292,17 @@ __device__ __forceinline__ void split4(const float (&v)[4], u32x2& h, u32x2& m, 
   }
 }
 
-template <int FS, int MB>
+template <int FS, int MB, bool M16>
 __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs a, MfmaPlan pl,
                                                                   float* partial) {
-  constexpr int OWN = kMaxAcc / MB;
+  // blocks of BW x BW entries of dK, steps of 2^SPLG pixels, NV accumulator registers a block
+  constexpr int BW = M16 ? 16 : 32, LGBW = M16 ? 4 : 5, SPLG = M16 ? 5 : 4, NV = M16 ? 4 : 16;
+  constexpr int OWN = M16 ? kMaxAcc16 : kMaxAcc / MB;
+  typedef typename AccOf<M16>::type Acc;
   extern __shared__ float lds[];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-  const int l32 = lane & 31, hi = lane >> 5;
+  const int l32 = lane & (BW - 1), hi = lane >> LGBW;   // row or column of a block; which eight pixels
   const int H = a.H, W = a.W, HW = H * W;
   const int b = wave & (pl.nbw - 1), sl = wave / pl.nbw;
   // this lane's column of every column block the wave owns, and its output channel of every
@@ -283,26 +310,26 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
   int boff[OWN], aoff[MB];
 #pragma unroll
   for (int o = 0; o < OWN; ++o) {
-    int n = 32 * (b + o * pl.nbw) + l32;
+    int n = BW * (b + o * pl.nbw) + l32;
     n = n < pl.NC ? n : pl.NC - 1;
     const int c = n / (FS * FS), tap = n - c * (FS * FS), i = tap / FS, j = tap - i * FS;
     boff[o] = c * pl.XR + i * pl.XS + j + (pl.xlead - a.pad) + 8 * hi;
   }
 #pragma unroll
   for (int m = 0; m < MB; ++m) {
-    int k = 32 * m + l32;
+    int k = BW * m + l32;
     k = k < a.T ? k : a.T - 1;
     aoff[m] = k * pl.DS + 8 * hi;
   }
   // column blocks this wave has: b, b + nbw, ... below NB
   const int nown = (pl.NB - b + pl.nbw - 1) / pl.nbw;
-  f32x16 acc[OWN][MB];
+  Acc acc[OWN][MB];
 #pragma unroll
   for (int o = 0; o < OWN; ++o)
 #pragma unroll
     for (int m = 0; m < MB; ++m)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[o][m][v] = 0.f;
+      for (int v = 0; v < NV; ++v) acc[o][m][v] = 0.f;
 
   // Slot q of this thread: the group of four cells g = tid + 512 q of the tile (x's groups,
   // then dy's): where it goes in the planes, its offset from the tile's first cell in memory,
@@ -329,7 +356,7 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
   }
 
   const int tiles_per_image = pl.tilesX * pl.tilesY;
-  const int lgcw = pl.lgTW - 4, nsteps = (pl.TH * pl.TW) >> 4;
+  const int lgcw = pl.lgTW - SPLG, nsteps = (pl.TH * pl.TW) >> SPLG;
   float4 held[kSlots];
   // Tile t's cells into this thread's registers (zeros outside the image).
   auto fetch = [&](int t) {
@@ -397,7 +424,7 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
     const int xw = pl.xplane >> 1;                     // a plane of x in dwords
     // ---- this wave's steps ----
     for (int st = sl; st < nsteps; st += pl.slices) {
-      const int row = st >> lgcw, col0 = (st & ((1 << lgcw) - 1)) << 4;
+      const int row = st >> lgcw, col0 = (st & ((1 << lgcw) - 1)) << SPLG;
       u32x4 ah[MB], am[MB], al[MB];
 #pragma unroll
       for (int m = 0; m < MB; ++m) {
@@ -427,7 +454,7 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
           }
 #pragma unroll
           for (int m = 0; m < MB; ++m)
-            acc[o][m] = split::mfma_split(ah[m], am[m], al[m], bh, bm, bl, acc[o][m]);
+            acc[o][m] = mfma_split_any(ah[m], am[m], al[m], bh, bm, bl, acc[o][m]);
         }
       }
     }
@@ -441,10 +468,10 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
     for (int o = 0; o < OWN; ++o)
 #pragma unroll
       for (int m = 0; m < MB; ++m) {
-        float* r = red + (((size_t)(o * MB + m) * pl.nbw + b) << 10) + lane;
+        float* r = red + ((size_t)(o * MB + m) * pl.nbw + b) * (NV * 64) + lane;
         if (sl == s2 && o < pl.own) {
 #pragma unroll
-          for (int v = 0; v < 16; ++v) r[v << 6] = acc[o][m][v];
+          for (int v = 0; v < NV; ++v) r[v << 6] = acc[o][m][v];
         }
       }
     __syncthreads();
@@ -452,10 +479,10 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
     for (int o = 0; o < OWN; ++o)
 #pragma unroll
       for (int m = 0; m < MB; ++m) {
-        const float* r = red + (((size_t)(o * MB + m) * pl.nbw + b) << 10) + lane;
+        const float* r = red + ((size_t)(o * MB + m) * pl.nbw + b) * (NV * 64) + lane;
         if (sl == 0 && o < pl.own) {
 #pragma unroll
-          for (int v = 0; v < 16; ++v) acc[o][m][v] += r[v << 6];
+          for (int v = 0; v < NV; ++v) acc[o][m][v] += r[v << 6];
         }
       }
     __syncthreads();
@@ -464,13 +491,15 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
   float* out = partial + (size_t)blockIdx.x * pl.outs;
 #pragma unroll
   for (int o = 0; o < OWN; ++o) {
-    const int n = 32 * (b + o * pl.nbw) + l32;
+    const int n = BW * (b + o * pl.nbw) + l32;
     if (o < pl.own && n < pl.NC) {
 #pragma unroll
       for (int m = 0; m < MB; ++m)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int k = 32 * m + 8 * (v >> 2) + 4 * hi + (v & 3);
+        for (int v = 0; v < NV; ++v) {
+          // (accumulator element v: row 8 * (v / 4) + 4 * (lane / 32) + v % 4 of a 32 x 32 block,
+          //  row 4 * (lane / 16) + v of a 16 x 16 one)
+          const int k = M16 ? 4 * hi + v : 32 * m + 8 * (v >> 2) + 4 * hi + (v & 3);
           if (k < a.T) out[(size_t)k * pl.NC + n] = acc[o][m][v];
         }
     }
@@ -698,19 +727,25 @@ hipError_t launch_fs(const BwdFilterArgs& a, const DensePlan& pl, int kb, float*
 bool mfma_plan(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
   const int vec = aligned16 && s.W % 4 == 0 ? 1 : 0, xlead = vec ? 4 : (int)s.pad;
   const int FS = (int)s.Y, T = (int)s.T, C = (int)s.C;
-  const int NC = C * FS * FS, NB = (NC + 31) / 32, MB = (T + 31) / 32;
+  // up to 16 output channels on up to 600,000 pixels: 16 x 16 blocks, whose rows are all in
+  // use (N32 C16 K16 56x56: 22 -> 19 us); beyond that the fewer, larger steps of the 32 x 32
+  // blocks are the faster ones (N16 C16 K16 512x512: 345 us against 400)
+  const int m16 = T <= 16 && (double)s.N * s.H * s.W <= 6.0e5 ? 1 : 0;
+  const int BW = m16 ? 16 : 32, step = m16 ? 32 : 16;
+  const int NC = C * FS * FS, NB = (NC + BW - 1) / BW, MB = (T + BW - 1) / BW;
   if (MB > 2 || (long)T * NC > kMaxOuts) return false;
+  const int most_own = m16 ? kMaxAcc16 : kMaxAcc / MB;
   int nbw = 1;
-  while (nbw <= kMWaves && (NB + nbw - 1) / nbw * MB > kMaxAcc) nbw *= 2;
+  while (nbw <= kMWaves && (NB + nbw - 1) / nbw > most_own) nbw *= 2;
   if (nbw > kMWaves) return false;
   const int slices = kMWaves / nbw, own = (NB + nbw - 1) / nbw;
-  const size_t red = (size_t)own * MB * nbw * 1024 * sizeof(float);
+  const size_t red = (size_t)own * MB * nbw * (m16 ? 256 : 1024) * sizeof(float);
   const int cus = num_compute_units();
   bool found = false;
   double best_cost = 0;
-  for (int TW = 16; TW <= 128; TW *= 2)
+  for (int TW = step; TW <= 128; TW *= 2)
     for (int TH = 1; TH <= 32; TH *= 2) {
-      if (TH * TW / 16 < slices) continue;
+      if (TH * TW / step < slices) continue;
       const int PH = TH + FS - 1;
       // (a multiple of four: a group of four staged cells stays within a row)
       const int XS = vec ? TW + 8 : (TW + FS - 1 + 3) / 4 * 4;
@@ -737,7 +772,7 @@ bool mfma_plan(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
       pl.ntiles = (int)s.N * pl.tilesX * pl.tilesY;
       pl.XS = XS; pl.XR = XR; pl.PHXS = PH * XS; pl.DS = DS; pl.vec = vec; pl.xlead = xlead;
       pl.nx = nx; pl.nd = nd; pl.xplane = xplane; pl.dplane = dplane; pl.bufbytes = bufbytes;
-      pl.NC = NC; pl.NB = NB; pl.MB = MB;
+      pl.m16 = m16; pl.NC = NC; pl.NB = NB; pl.MB = MB;
       pl.nbw = nbw; pl.slices = slices; pl.own = own;
       pl.outs = T * NC;
       pl.chmagic = (unsigned)((0x100000000ull + (unsigned)XR - 1) / (unsigned)XR);
@@ -769,9 +804,10 @@ bool mfma_plan(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
 
 template <int FS>
 hipError_t launch_mfma_fs(const BwdFilterArgs& a, const MfmaPlan& pl, float* partial, hipStream_t st) {
-  auto k1 = dense_mfma_kernel<FS, 1>;
-  auto k2 = dense_mfma_kernel<FS, 2>;
-  auto k = pl.MB == 2 ? k2 : k1;
+  auto k0 = dense_mfma_kernel<FS, 1, true>;
+  auto k1 = dense_mfma_kernel<FS, 1, false>;
+  auto k2 = dense_mfma_kernel<FS, 2, false>;
+  auto k = pl.m16 ? k0 : (pl.MB == 2 ? k2 : k1);
   if (pl.lds_bytes > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds_bytes);
@@ -846,8 +882,9 @@ size_t bwd_filter_dense_tiles_workspace_bytes(const cp4_shape& s) {
 // Where this route is the faster one: linear time models (us) fitted by least squares to
 // measured times of this route and of the factor-by-factor variants over some 400 layers each
 // (1 - 64 channels a side, 1x1 / 3x3 / 5x5, ranks 4 and 16, a thousand to a million pixels).
-// With the matrix-core tile kernel: 16 us, 3.1 us per thousand entries of dK (the final sums
-// and the chain rule), and per million pixels 0.83 us per channel staged and 14.4 per 32 x 32
+// With the matrix-core tile kernel: 13 us, 2 us per thousand entries of dK (the final sums
+// and the chain rule; both figures lowered by what a workgroup per gradient in the chain
+// rule saved after the fit), and per million pixels 0.83 us per channel staged and 14.4 per 32 x 32
 // block of the GEMM; the factor-by-factor variants 19 us and per million pixels 2.5 us per
 // channel and 0.28 per tap and rank; this route where its model is below 1.2 times theirs
 // (1.3 % off the better route in the geometric mean; always this route 10 % off, never 17 %).
@@ -862,7 +899,7 @@ bool bwd_filter_dense_tiles_preferred(const cp4_shape& s) {
   const double taps = (double)s.Y * s.X, macs = (double)s.T * s.C * taps;
   if (use_mfma(s)) {
     const double blocks = (double)((s.C * s.Y * s.X + 31) / 32) * ((s.T + 31) / 32);
-    const double dense = 16.03 + 3.143e-3 * macs +
+    const double dense = 13.0 + 2.0e-3 * macs +
                          mpx * (-6.15 + 0.829 * (s.C + s.T) + 14.42 * blocks);
     double planes = 18.79 + mpx * (-10.31 + 2.547 * (s.T + s.C) - 1.559 * s.Rank +
                                    0.2778 * taps * s.Rank);

@@ -58,6 +58,8 @@ SHAPES = [
     (3, 16, 70, 132, 1, 16, 3, 16),    # several tiles per workgroup, 16-byte loads, tiles past both edges
     (2, 20, 40, 64, 0, 12, 3, 4),      # no padding with a 3x3 filter
     (1, 6, 9, 16, 2, 64, 3, 5),        # pad beyond (Y - 1) / 2; a plane smaller than a tile
+    (1, 4, 800, 800, 1, 4, 3, 4),      # more than 600,000 pixels: 32 x 32 blocks with four output channels
+    (2, 12, 64, 96, 1, 16, 5, 8),      # 16 x 16 blocks, 5x5: nineteen column blocks over two groups of waves
 ]
 
 
