@@ -436,22 +436,26 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
       // cells off ... off + 7 of each plane: the dwords from off / 2, shifted by its parity
       // (row strides and steps are even: the parity is that of the lane's column)
       const int xo = row * pl.XS + col0;
-      unsigned dh[5], dm[5], dl[5];
+      // (two sets of registers by the block's parity: a block's dwords are read while the
+      //  block before it is in the matrix cores, and nothing is copied between the sets)
+      unsigned dh[2][5], dm[2][5], dl[2][5];
       {
         const unsigned* q = xp + ((boff[0] + xo) >> 1);
 #pragma unroll
-        for (int i = 0; i < 5; ++i) { dh[i] = q[i]; dm[i] = q[xw + i]; dl[i] = q[2 * xw + i]; }
+        for (int i = 0; i < 5; ++i) { dh[0][i] = q[i]; dm[0][i] = q[xw + i]; dl[0][i] = q[2 * xw + i]; }
       }
 #pragma unroll
       for (int o = 0; o < OWN; ++o) {
         if (o < nown) {
-          const unsigned shift = (unsigned)(boff[o] & 1) * 16u;
-          const u32x4 bh = funnel(dh, shift), bm = funnel(dm, shift), bl = funnel(dl, shift);
           if (o + 1 < OWN && o + 1 < nown) {
             const unsigned* q = xp + ((boff[o + 1 < OWN ? o + 1 : o] + xo) >> 1);
 #pragma unroll
-            for (int i = 0; i < 5; ++i) { dh[i] = q[i]; dm[i] = q[xw + i]; dl[i] = q[2 * xw + i]; }
+            for (int i = 0; i < 5; ++i) {
+              dh[(o + 1) & 1][i] = q[i]; dm[(o + 1) & 1][i] = q[xw + i]; dl[(o + 1) & 1][i] = q[2 * xw + i];
+            }
           }
+          const unsigned shift = (unsigned)(boff[o] & 1) * 16u;
+          const u32x4 bh = funnel(dh[o & 1], shift), bm = funnel(dm[o & 1], shift), bl = funnel(dl[o & 1], shift);
 #pragma unroll
           for (int m = 0; m < MB; ++m)
             acc[o][m] = mfma_split_any(ah[m], am[m], al[m], bh, bm, bl, acc[o][m]);
@@ -880,31 +884,37 @@ size_t bwd_filter_dense_tiles_workspace_bytes(const cp4_shape& s) {
 }
 
 // Where this route is the faster one: linear time models (us) fitted by least squares to
-// measured times of this route and of the factor-by-factor variants over some 400 layers each
-// (1 - 64 channels a side, 1x1 / 3x3 / 5x5, ranks 4 and 16, a thousand to a million pixels).
-// With the matrix-core tile kernel: 13 us, 2 us per thousand entries of dK (the final sums
-// and the chain rule; both figures lowered by what a workgroup per gradient in the chain
-// rule saved after the fit), and per million pixels 0.83 us per channel staged and 14.4 per 32 x 32
-// block of the GEMM; the factor-by-factor variants 19 us and per million pixels 2.5 us per
-// channel and 0.28 per tap and rank; this route where its model is below 1.2 times theirs
-// (1.3 % off the better route in the geometric mean; always this route 10 % off, never 17 %).
+// measured times of this route and of what the library runs without it, over 680 layers (1 -
+// 64 channels a side, 1x1 / 3x3 / 5x5, ranks 4, 16 and 64, a thousand to a million pixels).
+// With the matrix-core tile kernel: 14.8 us, 1.9 us per thousand entries of dK (the final
+// sums and the chain rule), and per million pixels 0.89 us per channel staged and 11 per
+// 32 x 32 block of the GEMM; without this route 17.6 us and per million pixels 116 us, 0.72
+// per channel, 5.9 per rank and 0.1 per tap and rank where both channel counts are multiples
+// of 16, and 25.2 us and 124, 0.37 (per channel of the counts rounded up to 16), 5.4 and 0.1
+// where they run on zero-padded copies.  The smaller model picks the route: 0.3 % off the
+// better one in the geometric mean (always this route 5 % off, never 85 %): it loses where
+// both channel counts are multiples of 16 from 32 on under a 3x3 or 5x5 filter.
 // With the plain multiply-add tile kernel: a fixed 18 us plus the final sums and the chain
 // rule, and per million pixels the staging of the tiles (2.7 us per channel staged) and the
 // multiply-adds (0.375 us per channel-block group and tap), against 26 us plus per million
 // pixels 115 us and what grows with the planes.
 // (N16 C16 K16 512x512 R16: 1040 us -> 350; N16 C3 K1 512x512 R16: 1005 -> 63; N8 C8 K8
-// 256x256 R16: 132 -> 42; but N1 C16 K16 32x32 R8: 18 against 27.)
+// 256x256 R16: 132 -> 34; N16 C8 K8 256x256 R4: 210 -> 66; but N8 C32 K32 56x56 R16: 25
+// against 39.)
 bool bwd_filter_dense_tiles_preferred(const cp4_shape& s) {
   const double mpx = (double)s.N * s.H * s.W / 1.0e6;
   const double taps = (double)s.Y * s.X, macs = (double)s.T * s.C * taps;
   if (use_mfma(s)) {
     const double blocks = (double)((s.C * s.Y * s.X + 31) / 32) * ((s.T + 31) / 32);
-    const double dense = 13.0 + 2.0e-3 * macs +
-                         mpx * (-6.15 + 0.829 * (s.C + s.T) + 14.42 * blocks);
-    double planes = 18.79 + mpx * (-10.31 + 2.547 * (s.T + s.C) - 1.559 * s.Rank +
-                                   0.2778 * taps * s.Rank);
-    if (planes < 10.0) planes = 10.0;
-    return dense < 1.2 * planes;
+    const double dense = 14.82 + 1.861e-3 * macs +
+                         mpx * (-6.751 + 0.8939 * (s.C + s.T) + 10.97 * blocks);
+    // (channel counts that are multiples of 16 run as they are, others on zero-padded copies)
+    const bool as_is = s.T % 16 == 0 && s.C % 16 == 0;
+    const double padded = (double)((s.T + 15) / 16 * 16 + (s.C + 15) / 16 * 16);
+    const double planes =
+        as_is ? 17.64 + mpx * (115.6 + 0.7179 * padded + 5.944 * s.Rank + 0.0967 * taps * s.Rank)
+              : 25.24 + mpx * (123.5 + 0.3736 * padded + 5.417 * s.Rank + 0.1013 * taps * s.Rank);
+    return dense < planes;
   }
   const int kb = s.T >= 2 && s.Y <= 3 ? 2 : 1;
   const double groups = (double)((s.T + kb - 1) / kb) * ((s.C + kCB - 1) / kCB);
