@@ -43,6 +43,7 @@ struct DensePlan {
   int G, S;            // channel-block groups; threads (pixel runs) per group
   int L;               // pixels per run
   int XS, XR;          // x tile in LDS: row stride, rows * XS per channel (padded)
+  int vec, xlead;      // 16-byte loads; columns of x staged before the tile's first (pad, or 4)
   int Cp, Tp;          // channel counts padded to their blocks
   int outs;            // T * C * FS * FS
   int lgTW, lgtile;    // log2 of TW and of TH * TW
@@ -90,7 +91,55 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
     // of its own): addresses clamped, values selected, so that no load sits in a branch.
     constexpr int kBatch = 8;
     const float* xn = a.x + (size_t)n * a.C * HW;
+    const float* dn = a.dy + (size_t)n * a.T * HW;
     const int nx = pl.Cp * PH * pl.XS;
+    const int nd = pl.Tp * pl.TH * pl.TW;
+    if (pl.vec) {
+      // Four cells a load (W a multiple of four, x and dy 16-byte aligned): the tile's rows
+      // start four columns before its first, so that a group of four is inside the image
+      // together or not at all; four loads in flight per thread and batch.
+      constexpr int kBatch4 = 4;
+      for (int e0 = 4 * tid; e0 < nx; e0 += 4 * kThreads * kBatch4) {
+        float4 v[kBatch4];
+        int at[kBatch4];
+        bool in[kBatch4];
+#pragma unroll
+        for (int u = 0; u < kBatch4; ++u) {
+          const int e = e0 + 4 * u * kThreads;
+          const int c = (int)__umulhi((unsigned)e, pl.chmagic), r2 = e - c * (PH * pl.XS);
+          const int pr = (int)__umulhi((unsigned)r2, pl.xsmagic), pc = r2 - pr * pl.XS;
+          const int h = h0 - a.pad + pr, w = w0 - 4 + pc;
+          in[u] = e < nx && c < a.C && h >= 0 && h < H && w >= 0 && w < W;
+          at[u] = e < nx ? c * pl.XR + r2 : -1;
+          const int cc = c < a.C ? c : a.C - 1;
+          const int hc = h < 0 ? 0 : (h > H - 1 ? H - 1 : h), wc = w < 0 ? 0 : (w > W - 4 ? W - 4 : w);
+          v[u] = *reinterpret_cast<const float4*>(xn + (size_t)cc * HW + (size_t)hc * W + wc);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch4; ++u)
+          if (at[u] >= 0)
+            *reinterpret_cast<float4*>(X + at[u]) = in[u] ? v[u] : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+      for (int e0 = 4 * tid; e0 < nd; e0 += 4 * kThreads * kBatch4) {
+        float4 v[kBatch4];
+        bool in[kBatch4];
+#pragma unroll
+        for (int u = 0; u < kBatch4; ++u) {
+          const int e = e0 + 4 * u * kThreads;
+          const int k = e >> pl.lgtile, r2 = e & ((1 << pl.lgtile) - 1);
+          const int pr = r2 >> pl.lgTW, pc = r2 & (pl.TW - 1);
+          const int h = h0 + pr, w = w0 + pc;
+          in[u] = e < nd && k < a.T && h < H && w < W;
+          const int kc = k < a.T ? k : a.T - 1, hc = h > H - 1 ? H - 1 : h, wc = w > W - 4 ? W - 4 : w;
+          v[u] = *reinterpret_cast<const float4*>(dn + (size_t)kc * HW + (size_t)hc * W + wc);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch4; ++u)
+          if (e0 + 4 * u * kThreads < nd)
+            *reinterpret_cast<float4*>(D + e0 + 4 * u * kThreads) =
+                in[u] ? v[u] : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    } else {
     for (int e0 = tid; e0 < nx; e0 += kThreads * kBatch) {
       float v[kBatch];
       int at[kBatch];
@@ -111,8 +160,6 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
       for (int u = 0; u < kBatch; ++u)
         if (at[u] >= 0) X[at[u]] = in[u] ? v[u] : 0.f;
     }
-    const float* dn = a.dy + (size_t)n * a.T * HW;
-    const int nd = pl.Tp * pl.TH * pl.TW;
     for (int e0 = tid; e0 < nd; e0 += kThreads * kBatch) {
       float v[kBatch];
       bool in[kBatch];
@@ -130,13 +177,14 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
       for (int u = 0; u < kBatch; ++u)
         if (e0 + u * kThreads < nd) D[e0 + u * kThreads] = in[u] ? v[u] : 0.f;
     }
+    }
     __syncthreads();
     // ---- this thread's runs: every S-th run of the tile ----
     if (active) {
       const int nruns = pl.TH * runs_per_row;
       for (int run = s; run < nruns; run += pl.S) {
         const int row = run / runs_per_row, col0 = (run - row * runs_per_row) * pl.L;
-        const float* xr = X + (size_t)(kCB * cb) * pl.XR + row * pl.XS + col0;
+        const float* xr = X + (size_t)(kCB * cb) * pl.XR + row * pl.XS + col0 + (pl.xlead - a.pad);
         const float* dr = D + (size_t)(KB * kb) * pl.TH * pl.TW + row * pl.TW + col0;
         // window columns col0 + t ... col0 + t + FS - 1; column (t + j) lives in slot (t + j) % FS
         float xw[kCB][FS][FS];
@@ -650,7 +698,8 @@ size_t fold_lds_bytes(const cp4_shape& s) {
 
 int kb_of(const cp4_shape& s) { return s.T >= 2 && s.Y <= 3 ? 2 : 1; }
 
-bool plan(const cp4_shape& s, DensePlan* best) {
+bool plan(const cp4_shape& s, bool aligned16, DensePlan* best) {
+  const int vec = aligned16 && s.W % 4 == 0 && s.W >= 4 ? 1 : 0, xlead = vec ? 4 : (int)s.pad;
   const int FS = (int)s.Y, KB = kb_of(s);
   const int KBLK = ((int)s.T + KB - 1) / KB, CBLK = ((int)s.C + kCB - 1) / kCB;
   const int G = KBLK * CBLK;
@@ -669,8 +718,10 @@ bool plan(const cp4_shape& s, DensePlan* best) {
       // where the tile allows, so that the sliding window pays
       int L = TW;
       while (L > 8 && (long)TH * TW / L < S) L >>= 1;
-      const int XS = TW + FS - 1 + FS;                // room for a run's last steps to read past it
-      const int XR = (TH + FS - 1) * XS + 1;          // odd-ish channel stride against bank conflicts
+      // room for a run's last steps to read past it; with 16-byte loads the columns before
+      // the tile's first, rows and channels multiples of four cells apart
+      const int XS = vec ? (4 + TW + 2 * FS - 1 + 3) / 4 * 4 : TW + FS - 1 + FS;
+      const int XR = (TH + FS - 1) * XS + (vec ? 4 : 1);  // (off a power of two: bank conflicts)
       const size_t lds = ((size_t)Cp * XR + (size_t)Tp * TH * TW + FS) * sizeof(float);
       const size_t red = (size_t)S * KB * kCB * FS * FS * sizeof(float);
       if (lds > kLdsLimit || red > kLdsLimit) continue;
@@ -680,7 +731,7 @@ bool plan(const cp4_shape& s, DensePlan* best) {
       pl.tilesY = ((int)s.H + TH - 1) / TH;
       pl.ntiles = (int)s.N * pl.tilesX * pl.tilesY;
       pl.KBLK = KBLK; pl.CBLK = CBLK; pl.G = G; pl.S = S; pl.L = L;
-      pl.XS = XS; pl.XR = XR; pl.Cp = Cp; pl.Tp = Tp;
+      pl.XS = XS; pl.XR = XR; pl.Cp = Cp; pl.Tp = Tp; pl.vec = vec; pl.xlead = xlead;
       pl.outs = (int)(s.T * s.C * s.Y * s.X);
       pl.lgTW = __builtin_ctz(TW);
       pl.lgtile = __builtin_ctz(TW) + __builtin_ctz(TH);
@@ -848,7 +899,7 @@ bool common_ok(const cp4_shape& s) {
 
 bool valu_ok(const cp4_shape& s) {
   DensePlan pl;
-  return common_ok(s) && (long)s.T * s.C <= kMaxPairs && plan(s, &pl);
+  return common_ok(s) && (long)s.T * s.C <= kMaxPairs && plan(s, false, &pl);
 }
 
 bool mfma_ok(const cp4_shape& s) {
@@ -877,7 +928,8 @@ size_t bwd_filter_dense_tiles_workspace_bytes(const cp4_shape& s) {
   size_t sets = 0;
   DensePlan dp;
   MfmaPlan mp;
-  if (valu_ok(s) && plan(s, &dp)) sets = dp.grid;
+  if (valu_ok(s) && plan(s, false, &dp)) sets = dp.grid;
+  if (valu_ok(s) && plan(s, true, &dp) && (size_t)dp.grid > sets) sets = dp.grid;
   if (mfma_ok(s) && mfma_plan(s, false, &mp) && (size_t)mp.grid > sets) sets = mp.grid;
   if (mfma_ok(s) && mfma_plan(s, true, &mp) && (size_t)mp.grid > sets) sets = mp.grid;
   return (sets + 1) * set;
@@ -936,9 +988,9 @@ hipError_t bwd_filter_dense_tiles_launch(const BwdFilterArgs& a, hipStream_t st)
   hipError_t e;
   int sets;
   // (the partial sets are `outs` apart; the padded stride is only what the size allows for)
+  const bool aligned16 = ((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.dy)) & 15) == 0;
   if (use_mfma(s)) {
     MfmaPlan pl;
-    const bool aligned16 = ((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.dy)) & 15) == 0;
     if (!mfma_plan(s, aligned16, &pl) && !mfma_plan(s, false, &pl)) return hipErrorInvalidValue;
     sets = pl.grid;
     switch (a.Y) {
@@ -948,7 +1000,7 @@ hipError_t bwd_filter_dense_tiles_launch(const BwdFilterArgs& a, hipStream_t st)
     }
   } else {
     DensePlan pl;
-    if (!valu_ok(s) || !plan(s, &pl)) return hipErrorInvalidValue;
+    if (!valu_ok(s) || (!plan(s, aligned16, &pl) && !plan(s, false, &pl))) return hipErrorInvalidValue;
     sets = pl.grid;
     switch (a.Y) {
       case 1: e = launch_fs<1>(a, pl, kb_of(s), partial, st); break;
