@@ -779,7 +779,33 @@ hipError_t launch_fs(const BwdFilterArgs& a, const DensePlan& pl, int kb, float*
   return hipGetLastError();
 }
 
-bool mfma_plan(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
+// LDS bank conflicts of a block's operand reads for a channel stride XR: the 32 lanes that the
+// LDS serves together read dword (c * XR + i * XS + j + shift + 8 * part) / 2 of a plane, with
+// (c, i, j) the lane's column of the GEMM; the worst number of different dwords on one of the 32
+// banks, summed over the column blocks.
+int read_conflicts(int XR, int XS, int FS, int NC, int shift, bool m16) {
+  const int BW = m16 ? 16 : 32, NB = (NC + BW - 1) / BW;
+  int total = 0;
+  for (int nb = 0; nb < NB; ++nb) {
+    int dwords[32];
+    for (int l = 0; l < 32; ++l) {
+      int n = BW * nb + (m16 ? (l & 15) : l);
+      n = n < NC ? n : NC - 1;
+      const int c = n / (FS * FS), tap = n - c * (FS * FS), i = tap / FS, j = tap - i * FS;
+      dwords[l] = (c * XR + i * XS + j + shift + (m16 ? 8 * (l >> 4) : 0)) >> 1;
+    }
+    int count[32] = {0}, worst = 1;
+    for (int l = 0; l < 32; ++l) {
+      bool seen = false;
+      for (int m = 0; m < l; ++m) seen = seen || dwords[m] == dwords[l];
+      if (!seen && ++count[dwords[l] & 31] > worst) worst = count[dwords[l] & 31];
+    }
+    total += worst;
+  }
+  return total;
+}
+
+bool mfma_plan_uncached(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
   const int vec = aligned16 && s.W % 4 == 0 ? 1 : 0, xlead = vec ? 4 : (int)s.pad;
   const int FS = (int)s.Y, T = (int)s.T, C = (int)s.C;
   // up to 16 output channels on up to 600,000 pixels: 16 x 16 blocks, whose rows are all in
@@ -804,11 +830,18 @@ bool mfma_plan(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
       const int PH = TH + FS - 1;
       // (a multiple of four: a group of four staged cells stays within a row)
       const int XS = vec ? TW + 8 : (TW + FS - 1 + 3) / 4 * 4;
-      // a channel's rows, then as many cells as put consecutive channels ten banks of dwords
-      // apart in the bf16 planes: with rows 4 banks apart (XS = 8 mod 64) or any stride, the
-      // taps of the four channels that a step's 32 columns cover then fall into different banks
+      // a channel's rows, then the few cells that leave the operand reads with the fewest
+      // LDS bank conflicts (the taps of the channels that a block's columns cover on
+      // different banks)
       int XR = (PH * XS + 3) / 4 * 4;
-      while (XR % 64 != 20) XR += 4;
+      {
+        int best_xr = XR, fewest = 1 << 30;
+        for (int cand = XR; cand < XR + 64; cand += 4) {
+          const int cf = read_conflicts(cand, XS, FS, NC, xlead - (int)s.pad, m16 != 0);
+          if (cf < fewest) { fewest = cf; best_xr = cand; }
+        }
+        XR = best_xr;
+      }
       const int DS = TH * TW + 8;                      // output channels four banks apart
       const int nx = C * XR, nd = T * DS;
       if ((nx + nd) / 4 > kSlots * kMThreads) continue;
@@ -855,6 +888,29 @@ bool mfma_plan(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
       }
     }
   return found;
+}
+
+// (the search above is a few hundred thousand operations: the last answer is kept per thread)
+bool mfma_plan(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
+  struct Last {
+    bool valid = false, aligned16 = false, found = false;
+    cp4_shape shape;
+    MfmaPlan plan;
+  };
+  thread_local Last both[2];        // (queries alternate between the two alignments)
+  Last& last = both[aligned16 ? 1 : 0];
+  const bool same = last.valid && last.aligned16 == aligned16 && last.shape.N == s.N &&
+                    last.shape.C == s.C && last.shape.T == s.T && last.shape.H == s.H &&
+                    last.shape.W == s.W && last.shape.pad == s.pad && last.shape.Y == s.Y &&
+                    last.shape.X == s.X && last.shape.Rank == s.Rank;
+  if (!same) {
+    last.found = mfma_plan_uncached(s, aligned16, &last.plan);
+    last.shape = s;
+    last.aligned16 = aligned16;
+    last.valid = true;
+  }
+  if (last.found) *best = last.plan;
+  return last.found;
 }
 
 template <int FS>
