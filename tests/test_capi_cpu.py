@@ -156,6 +156,15 @@ def test_plan_query_names_what_a_launch_runs(L):
     capi.set_tuned_filter_choice(small, 1)
     assert capi.plan_query(small, "backward_filter")["variant"] == names[1]
     capi.tune_clear()
+    # few channels on both sides: the dense gradient over tiles and the chain rule, with plain
+    # multiply-adds (three channels to one) or on the matrix cores; not workload C1's 1024 pixels
+    for dims in ((128, 3, 512, 512, 1), (16, 16, 512, 512, 16), (16, 32, 256, 256, 32),
+                 (16, 3, 112, 112, 64), (8, 8, 256, 256, 8)):
+        few = capi.Shape(N=dims[0], H=dims[2], W=dims[3], pad=1, T=dims[4], C=dims[1], Y=3, X=3, Rank=16)
+        assert capi.plan_query(few, "backward_filter")["variant"] == names[3], dims
+        assert L.cp4_conv2d_backward_filter_workspace_bytes(ctypes.byref(few)) >= 2 * 4 * 9 * dims[1] * dims[4]
+    c1 = capi.Shape(N=1, H=32, W=32, pad=1, T=16, C=16, Y=3, X=3, Rank=8)
+    assert capi.plan_query(c1, "backward_filter")["variant"] != names[3]
     v = ctypes.c_int()
     assert L.cp4_plan_query(ctypes.byref(s), 3, ctypes.byref(v), None, None) == capi.ERR_SHAPE
 
