@@ -79,6 +79,8 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
 #pragma unroll
         for (int j = 0; j < FS; ++j) acc[k][c][i][j] = 0.f;
 
+  // the channels that pad x to a multiple of four are zeros for the whole launch
+  for (int e = a.C * pl.XR + tid; e < pl.Cp * pl.XR; e += kThreads) X[e] = 0.f;
   const int tiles_per_image = pl.tilesX * pl.tilesY;
   for (int t = blockIdx.x; t < pl.ntiles; t += gridDim.x) {
     const int n = t / tiles_per_image, rem = t - n * tiles_per_image;
@@ -92,7 +94,7 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
     constexpr int kBatch = 8;
     const float* xn = a.x + (size_t)n * a.C * HW;
     const float* dn = a.dy + (size_t)n * a.T * HW;
-    const int nx = pl.Cp * PH * pl.XS;
+    const int nx = a.C * PH * pl.XS;
     const int nd = pl.Tp * pl.TH * pl.TW;
     if (pl.vec) {
       // Four cells a load (W a multiple of four, x and dy 16-byte aligned): the tile's rows
@@ -830,18 +832,8 @@ bool mfma_plan_uncached(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
       const int PH = TH + FS - 1;
       // (a multiple of four: a group of four staged cells stays within a row)
       const int XS = vec ? TW + 8 : (TW + FS - 1 + 3) / 4 * 4;
-      // a channel's rows, then the few cells that leave the operand reads with the fewest
-      // LDS bank conflicts (the taps of the channels that a block's columns cover on
-      // different banks)
-      int XR = (PH * XS + 3) / 4 * 4;
-      {
-        int best_xr = XR, fewest = 1 << 30;
-        for (int cand = XR; cand < XR + 64; cand += 4) {
-          const int cf = read_conflicts(cand, XS, FS, NC, xlead - (int)s.pad, m16 != 0);
-          if (cf < fewest) { fewest = cf; best_xr = cand; }
-        }
-        XR = best_xr;
-      }
+      // a channel's rows (and up to 60 cells more, chosen below for the tile that wins)
+      const int XR = (PH * XS + 3) / 4 * 4;
       const int DS = TH * TW + 8;                      // output channels four banks apart
       const int nx = C * XR, nd = T * DS;
       if ((nx + nd) / 4 > kSlots * kMThreads) continue;
@@ -877,7 +869,7 @@ bool mfma_plan_uncached(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
       // cells staged per output pixel (halo, pixels past the image's edge), a grid that leaves
       // compute units idle, and the fixed cost of a tile
       const double area = (double)pl.tilesX * TW * pl.tilesY * TH / ((double)s.W * s.H);
-      const double halo = (double)XR / ((double)TH * TW);
+      const double halo = (double)(PH * XS) / ((double)TH * TW);
       const double staged = ((double)C * halo + T) / (C + T);
       const double fill = (double)((pl.ntiles + pl.grid - 1) / pl.grid * pl.grid) / pl.ntiles;
       const double cost = area * fill * (0.5 + 0.5 * staged) * (1.0 + 64.0 / (TH * TW));
@@ -887,30 +879,57 @@ bool mfma_plan_uncached(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
         found = true;
       }
     }
-  return found;
+  if (!found) return false;
+  // The channel stride of the winning tile: a channel's rows, then the few cells that leave
+  // the operand reads with the fewest LDS bank conflicts (the taps of the channels that a
+  // block's columns cover on different banks); what depends on it follows.
+  MfmaPlan& pl = *best;
+  const int XR0 = pl.XR;
+  int fewest = 1 << 30;
+  for (int cand = XR0; cand <= XR0 + 60; cand += 4) {
+    const int nx = C * cand, xplane = (nx + 8 + 7) / 8 * 8;
+    if ((nx + pl.nd) / 4 > kSlots * kMThreads || 12 * (size_t)(xplane + pl.dplane) > kMLds) break;
+    const int cf = read_conflicts(cand, pl.XS, FS, NC, xlead - (int)s.pad, m16 != 0);
+    if (cf < fewest) { fewest = cf; pl.XR = cand; }
+  }
+  pl.nx = C * pl.XR;
+  pl.xplane = (pl.nx + 8 + 7) / 8 * 8;
+  pl.bufbytes = 6 * (pl.xplane + pl.dplane);
+  pl.lds_bytes = 2 * (size_t)pl.bufbytes;
+  if (slices > 1 && red > pl.lds_bytes) pl.lds_bytes = red;
+  pl.chmagic = (unsigned)((0x100000000ull + (unsigned)pl.XR - 1) / (unsigned)pl.XR);
+  return true;
 }
 
-// (the search above is a few hundred thousand operations: the last answer is kept per thread)
+// (the search above is tens of thousands of operations: the last few answers are kept per
+//  thread; a layer's queries alternate between the two alignments and, with odd channel
+//  counts, the layer's zero-padded shape)
 bool mfma_plan(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
-  struct Last {
+  struct Entry {
     bool valid = false, aligned16 = false, found = false;
     cp4_shape shape;
     MfmaPlan plan;
   };
-  thread_local Last both[2];        // (queries alternate between the two alignments)
-  Last& last = both[aligned16 ? 1 : 0];
-  const bool same = last.valid && last.aligned16 == aligned16 && last.shape.N == s.N &&
-                    last.shape.C == s.C && last.shape.T == s.T && last.shape.H == s.H &&
-                    last.shape.W == s.W && last.shape.pad == s.pad && last.shape.Y == s.Y &&
-                    last.shape.X == s.X && last.shape.Rank == s.Rank;
-  if (!same) {
-    last.found = mfma_plan_uncached(s, aligned16, &last.plan);
-    last.shape = s;
-    last.aligned16 = aligned16;
-    last.valid = true;
+  constexpr int kEntries = 32;
+  thread_local Entry cache[kEntries];
+  thread_local int next = 0;
+  for (int i = 0; i < kEntries; ++i) {
+    const Entry& e = cache[i];
+    if (e.valid && e.aligned16 == aligned16 && e.shape.N == s.N && e.shape.C == s.C &&
+        e.shape.T == s.T && e.shape.H == s.H && e.shape.W == s.W && e.shape.pad == s.pad &&
+        e.shape.Y == s.Y && e.shape.X == s.X && e.shape.Rank == s.Rank) {
+      if (e.found) *best = e.plan;
+      return e.found;
+    }
   }
-  if (last.found) *best = last.plan;
-  return last.found;
+  Entry& e = cache[next];
+  next = (next + 1) % kEntries;
+  e.found = mfma_plan_uncached(s, aligned16, &e.plan);
+  e.shape = s;
+  e.aligned16 = aligned16;
+  e.valid = true;
+  if (e.found) *best = e.plan;
+  return e.found;
 }
 
 template <int FS>
