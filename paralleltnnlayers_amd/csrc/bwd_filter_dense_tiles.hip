@@ -268,18 +268,24 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
 // use, that work would be FS * FS times as much), in two buffers:
 //   1. the next tile's cells are loaded into registers (four consecutive cells a thread and
 //      slot; the cell a thread loads is the same in every tile, its offset worked out once);
-//   2. the waves take their steps of 16 consecutive pixels of a row of the current tile:
-//      lane (k, half) reads its 8 pixels of dy[k] from the planes (16-byte reads), lane
-//      (n, half) the 8 cells of column n's channel and tap (five dwords from the cell's even
-//      neighbour on, shifted by 16 bits where it is odd), a block's reads issued before the
-//      block before it goes to the matrix cores;
+//   2. the waves take their steps of 16 (32) consecutive pixels of a row of the current tile:
+//      lane (k, part) reads its 8 pixels of dy[k] from the planes (16-byte reads), lane
+//      (n, part) the 8 cells of column n's channel and tap (five dwords from the cell's even
+//      neighbour on, shifted by 16 bits where it is odd); with 8 waves a block's reads are
+//      issued before the block before it goes to the matrix cores;
 //   3. the registers are split and written to the other buffer; one barrier per tile.
-// A wave owns up to eight 32 x 32 accumulator blocks for the whole launch: `own` blocks of
-// columns (every nbw-th) x MB blocks of output channels; the 8 / nbw waves that share
-// column blocks take every (8 / nbw)-th step and are added in fixed order at the end.
+// A wave owns its accumulator blocks for the whole launch: `own` blocks of columns (every
+// nbw-th) x MB blocks of output channels; the waves that share column blocks take every
+// (waves / nbw)-th step and are added in fixed order at the end.  Two builds: 16 x 16 blocks
+// (v_mfma_f32_16x16x32_bf16, steps of 32 pixels, up to eight blocks a wave) in workgroups of
+// 16 waves for up to 32 output channels, and 32 x 32 blocks (v_mfma_f32_32x32x16_bf16, steps
+// of 16 pixels, up to six blocks) in workgroups of 8 waves.  The first fits 128 registers, four
+// waves per SIMD, which is what covers the latency of a block's chain (LDS reads -> shifts ->
+// six dependent matrix instructions): N16 C16 K16 512x512 takes 205 us on it and 330 on the
+// second (240 registers, two waves per SIMD), whose matrix-core time alone would be 124.
 constexpr int kMThreads = 512, kMWaves = kMThreads / 64;
 constexpr int kMaxAcc = 6;                   // 32 x 32 blocks a wave holds
-constexpr int kMaxAcc16 = 12;                // 16 x 16 blocks, with up to 16 output channels
+constexpr int kMaxAcc16 = 8;                 // 16 x 16 blocks (up to 32 output channels, 16 waves)
 constexpr int kMaxOuts = 16384;              // T * C * Y * X up to here
 constexpr size_t kMLds = 160 * 1024;
 constexpr int kSlots = 6;                    // groups of four cells a thread stages per tile
@@ -291,7 +297,7 @@ struct MfmaPlan {
   int nx, nd;             // cells staged: C * XR, T * DS (multiples of 4)
   int xplane, dplane;     // cells per plane (multiples of 8)
   int bufbytes;           // one buffer: three planes of x, three of dy
-  int m16;                // up to 16 output channels: 16 x 16 blocks, steps of 32 pixels
+  int m16;                // up to 32 output channels: 16 x 16 blocks, steps of 32 pixels, 16 waves
   int NC, NB, MB;         // columns C * FS * FS; blocks of them; blocks of output channels
   int nbw, slices, own;   // waves across column blocks; waves across steps; column blocks a wave
   int outs, grid;
@@ -343,11 +349,13 @@ __device__ __forceinline__ void split4(const float (&v)[4], u32x2& h, u32x2& m, 
 }
 
 template <int FS, int MB, bool M16>
-__global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs a, MfmaPlan pl,
+__global__ __launch_bounds__(M16 ? 1024 : 512, M16 ? 4 : 2) void dense_mfma_kernel(BwdFilterArgs a, MfmaPlan pl,
                                                                   float* partial) {
   // blocks of BW x BW entries of dK, steps of 2^SPLG pixels, NV accumulator registers a block
   constexpr int BW = M16 ? 16 : 32, LGBW = M16 ? 4 : 5, SPLG = M16 ? 5 : 4, NV = M16 ? 4 : 16;
-  constexpr int OWN = M16 ? kMaxAcc16 : kMaxAcc / MB;
+  constexpr int OWN = (M16 ? kMaxAcc16 : kMaxAcc) / MB;
+  // threads: 16 waves where the accumulators are small (four waves per SIMD), else 8
+  constexpr int THREADS = M16 ? 1024 : 512, SLOTS = kSlots * kMThreads / THREADS;
   typedef typename AccOf<M16>::type Acc;
   extern __shared__ float lds[];
   const int tid = threadIdx.x;
@@ -385,11 +393,11 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
   // then dy's): where it goes in the planes, its offset from the tile's first cell in memory,
   // and its row and column in the tile (-1: padding, zeros).
   const int xgroups = pl.nx >> 2, groups = xgroups + (pl.nd >> 2);
-  unsigned rel[kSlots];
-  int rc[kSlots];
+  unsigned rel[SLOTS];
+  int rc[SLOTS];
 #pragma unroll
-  for (int q = 0; q < kSlots; ++q) {
-    const int g = tid + kMThreads * q;
+  for (int q = 0; q < SLOTS; ++q) {
+    const int g = tid + THREADS * q;
     if (g < xgroups) {
       const int e = 4 * g;
       const int c = (int)__umulhi((unsigned)e, pl.chmagic), r2 = e - c * pl.XR;
@@ -407,7 +415,7 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
 
   const int tiles_per_image = pl.tilesX * pl.tilesY;
   const int lgcw = pl.lgTW - SPLG, nsteps = (pl.TH * pl.TW) >> SPLG;
-  float4 held[kSlots];
+  float4 held[SLOTS];
   // Tile t's cells into this thread's registers (zeros outside the image).
   auto fetch = [&](int t) {
     const int n = t / tiles_per_image, rem = t - n * tiles_per_image;
@@ -417,8 +425,8 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
     const float* xn = a.x + (size_t)n * a.C * HW;
     const float* dn = a.dy + (size_t)n * a.T * HW;
 #pragma unroll
-    for (int q = 0; q < kSlots; ++q) {
-      const int g = tid + kMThreads * q;
+    for (int q = 0; q < SLOTS; ++q) {
+      const int g = tid + THREADS * q;
       const bool isx = g < xgroups;
       const int h0 = isx ? hx : hd, w0 = isx ? wx : wd;
       const float* src = isx ? xn : dn;
@@ -443,8 +451,8 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
   // The registers, split, into buffer `buf`.
   auto deposit = [&](char* buf) {
 #pragma unroll
-    for (int q = 0; q < kSlots; ++q) {
-      const int g = tid + kMThreads * q;
+    for (int q = 0; q < SLOTS; ++q) {
+      const int g = tid + THREADS * q;
       if (g < groups) {
         const bool isx = g < xgroups;
         const int e = isx ? 4 * g : 4 * (g - xgroups);
@@ -488,27 +496,45 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
       const int xo = row * pl.XS + col0;
       // (two sets of registers by the block's parity: a block's dwords are read while the
       //  block before it is in the matrix cores, and nothing is copied between the sets)
-      unsigned dh[2][5], dm[2][5], dl[2][5];
-      {
-        const unsigned* q = xp + ((boff[0] + xo) >> 1);
+      if constexpr (!M16) {
+        unsigned dh[2][5], dm[2][5], dl[2][5];
+        {
+          const unsigned* q = xp + ((boff[0] + xo) >> 1);
 #pragma unroll
-        for (int i = 0; i < 5; ++i) { dh[0][i] = q[i]; dm[0][i] = q[xw + i]; dl[0][i] = q[2 * xw + i]; }
-      }
+          for (int i = 0; i < 5; ++i) { dh[0][i] = q[i]; dm[0][i] = q[xw + i]; dl[0][i] = q[2 * xw + i]; }
+        }
 #pragma unroll
-      for (int o = 0; o < OWN; ++o) {
-        if (o < nown) {
-          if (o + 1 < OWN && o + 1 < nown) {
-            const unsigned* q = xp + ((boff[o + 1 < OWN ? o + 1 : o] + xo) >> 1);
+        for (int o = 0; o < OWN; ++o) {
+          if (o < nown) {
+            if (o + 1 < OWN && o + 1 < nown) {
+              const unsigned* q = xp + ((boff[o + 1 < OWN ? o + 1 : o] + xo) >> 1);
 #pragma unroll
-            for (int i = 0; i < 5; ++i) {
-              dh[(o + 1) & 1][i] = q[i]; dm[(o + 1) & 1][i] = q[xw + i]; dl[(o + 1) & 1][i] = q[2 * xw + i];
+              for (int i = 0; i < 5; ++i) {
+                dh[(o + 1) & 1][i] = q[i]; dm[(o + 1) & 1][i] = q[xw + i]; dl[(o + 1) & 1][i] = q[2 * xw + i];
+              }
             }
-          }
-          const unsigned shift = (unsigned)(boff[o] & 1) * 16u;
-          const u32x4 bh = funnel(dh[o & 1], shift), bm = funnel(dm[o & 1], shift), bl = funnel(dl[o & 1], shift);
+            const unsigned shift = (unsigned)(boff[o] & 1) * 16u;
+            const u32x4 bh = funnel(dh[o & 1], shift), bm = funnel(dm[o & 1], shift), bl = funnel(dl[o & 1], shift);
 #pragma unroll
-          for (int m = 0; m < MB; ++m)
-            acc[o][m] = mfma_split_any(ah[m], am[m], al[m], bh, bm, bl, acc[o][m]);
+            for (int m = 0; m < MB; ++m)
+              acc[o][m] = mfma_split_any(ah[m], am[m], al[m], bh, bm, bl, acc[o][m]);
+          }
+        }
+      } else {
+        // (four waves per SIMD cover a block's reads; 128 registers leave no room for a second set)
+#pragma unroll
+        for (int o = 0; o < OWN; ++o) {
+          if (o < nown) {
+            const unsigned* q = xp + ((boff[o] + xo) >> 1);
+            unsigned dh[5], dm[5], dl[5];
+#pragma unroll
+            for (int i = 0; i < 5; ++i) { dh[i] = q[i]; dm[i] = q[xw + i]; dl[i] = q[2 * xw + i]; }
+            const unsigned shift = (unsigned)(boff[o] & 1) * 16u;
+            const u32x4 bh = funnel(dh, shift), bm = funnel(dm, shift), bl = funnel(dl, shift);
+#pragma unroll
+            for (int m = 0; m < MB; ++m)
+              acc[o][m] = mfma_split_any(ah[m], am[m], al[m], bh, bm, bl, acc[o][m]);
+          }
         }
       }
     }
@@ -553,7 +579,7 @@ __global__ __launch_bounds__(kMThreads, 2) void dense_mfma_kernel(BwdFilterArgs 
         for (int v = 0; v < NV; ++v) {
           // (accumulator element v: row 8 * (v / 4) + 4 * (lane / 32) + v % 4 of a 32 x 32 block,
           //  row 4 * (lane / 16) + v of a 16 x 16 one)
-          const int k = M16 ? 4 * hi + v : 32 * m + 8 * (v >> 2) + 4 * hi + (v & 3);
+          const int k = M16 ? 16 * m + 4 * hi + v : 32 * m + 8 * (v >> 2) + 4 * hi + (v & 3);
           if (k < a.T) out[(size_t)k * pl.NC + n] = acc[o][m][v];
         }
     }
@@ -807,25 +833,24 @@ int read_conflicts(int XR, int XS, int FS, int NC, int shift, bool m16) {
   return total;
 }
 
-bool mfma_plan_uncached(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
+bool mfma_plan_blocks(const cp4_shape& s, bool aligned16, int m16, MfmaPlan* best) {
   const int vec = aligned16 && s.W % 4 == 0 ? 1 : 0, xlead = vec ? 4 : (int)s.pad;
   const int FS = (int)s.Y, T = (int)s.T, C = (int)s.C;
-  // up to 16 output channels on up to 600,000 pixels: 16 x 16 blocks, whose rows are all in
-  // use (N32 C16 K16 56x56: 22 -> 19 us); beyond that the fewer, larger steps of the 32 x 32
-  // blocks are the faster ones (N16 C16 K16 512x512: 345 us against 400)
-  const int m16 = T <= 16 && (double)s.N * s.H * s.W <= 6.0e5 ? 1 : 0;
   const int BW = m16 ? 16 : 32, step = m16 ? 32 : 16;
   const int NC = C * FS * FS, NB = (NC + BW - 1) / BW, MB = (T + BW - 1) / BW;
   if (MB > 2 || (long)T * NC > kMaxOuts) return false;
-  const int most_own = m16 ? kMaxAcc16 : kMaxAcc / MB;
-  int nbw = 1;
-  while (nbw <= kMWaves && (NB + nbw - 1) / nbw > most_own) nbw *= 2;
-  if (nbw > kMWaves) return false;
-  const int slices = kMWaves / nbw, own = (NB + nbw - 1) / nbw;
-  const size_t red = (size_t)own * MB * nbw * (m16 ? 256 : 1024) * sizeof(float);
+  const int most_own = (m16 ? kMaxAcc16 : kMaxAcc) / MB;
+  const int waves = m16 ? 16 : kMWaves;
   const int cus = num_compute_units();
   bool found = false;
   double best_cost = 0;
+  // waves across the column blocks: as few as hold them all, or more (fewer waves then share
+  // a tile's steps, which lets smaller tiles in where the LDS is short; groups of waves
+  // without a block of their own idle)
+  for (int nbw = 1; nbw <= waves; nbw *= 2) {
+    if ((NB + nbw - 1) / nbw > most_own) continue;
+    const int slices = waves / nbw, own = (NB + nbw - 1) / nbw;
+    const size_t red = (size_t)own * MB * nbw * (m16 ? 256 : 1024) * sizeof(float);
   for (int TW = step; TW <= 128; TW *= 2)
     for (int TH = 1; TH <= 32; TH *= 2) {
       if (TH * TW / step < slices) continue;
@@ -872,13 +897,15 @@ bool mfma_plan_uncached(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
       const double halo = (double)(PH * XS) / ((double)TH * TW);
       const double staged = ((double)C * halo + T) / (C + T);
       const double fill = (double)((pl.ntiles + pl.grid - 1) / pl.grid * pl.grid) / pl.ntiles;
-      const double cost = area * fill * (0.5 + 0.5 * staged) * (1.0 + 64.0 / (TH * TW));
+      const double busy = (double)own * nbw / NB;      // (block slots per block)
+      const double cost = area * fill * (0.5 + 0.5 * staged) * (1.0 + 64.0 / (TH * TW)) * busy;
       if (!found || cost < best_cost) {
         best_cost = cost;
         *best = pl;
         found = true;
       }
     }
+  }
   if (!found) return false;
   // The channel stride of the winning tile: a channel's rows, then the few cells that leave
   // the operand reads with the fewest LDS bank conflicts (the taps of the channels that a
@@ -896,9 +923,18 @@ bool mfma_plan_uncached(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
   pl.xplane = (pl.nx + 8 + 7) / 8 * 8;
   pl.bufbytes = 6 * (pl.xplane + pl.dplane);
   pl.lds_bytes = 2 * (size_t)pl.bufbytes;
-  if (slices > 1 && red > pl.lds_bytes) pl.lds_bytes = red;
+  const size_t red = (size_t)pl.own * MB * pl.nbw * (m16 ? 256 : 1024) * sizeof(float);
+  if (pl.slices > 1 && red > pl.lds_bytes) pl.lds_bytes = red;
   pl.chmagic = (unsigned)((0x100000000ull + (unsigned)pl.XR - 1) / (unsigned)pl.XR);
   return true;
+}
+
+// Up to 32 output channels: 16 x 16 blocks (all rows in use with up to 16 channels) on 16
+// waves, whose accumulators are small enough for four waves per SIMD (N16 C16 K16 512x512:
+// 330 -> 204 us); else, or where no tile of those fits, 32 x 32 blocks on 8 waves.
+bool mfma_plan_uncached(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
+  if (s.T <= 32 && mfma_plan_blocks(s, aligned16, 1, best)) return true;
+  return mfma_plan_blocks(s, aligned16, 0, best);
 }
 
 // (the search above is tens of thousands of operations: the last few answers are kept per
@@ -935,15 +971,16 @@ bool mfma_plan(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
 template <int FS>
 hipError_t launch_mfma_fs(const BwdFilterArgs& a, const MfmaPlan& pl, float* partial, hipStream_t st) {
   auto k0 = dense_mfma_kernel<FS, 1, true>;
+  auto k02 = dense_mfma_kernel<FS, 2, true>;
   auto k1 = dense_mfma_kernel<FS, 1, false>;
   auto k2 = dense_mfma_kernel<FS, 2, false>;
-  auto k = pl.m16 ? k0 : (pl.MB == 2 ? k2 : k1);
+  auto k = pl.m16 ? (pl.MB == 2 ? k02 : k0) : (pl.MB == 2 ? k2 : k1);
   if (pl.lds_bytes > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds_bytes);
     if (e != hipSuccess) return e;
   }
-  k<<<pl.grid, kMThreads, pl.lds_bytes, st>>>(a, pl, partial);
+  k<<<pl.grid, pl.m16 ? 1024 : kMThreads, pl.lds_bytes, st>>>(a, pl, partial);
   return hipGetLastError();
 }
 
@@ -1013,28 +1050,28 @@ size_t bwd_filter_dense_tiles_workspace_bytes(const cp4_shape& s) {
 // Where this route is the faster one: linear time models (us) fitted by least squares to
 // measured times of this route and of what the library runs without it, over 680 layers (1 -
 // 64 channels a side, 1x1 / 3x3 / 5x5, ranks 4, 16 and 64, a thousand to a million pixels).
-// With the matrix-core tile kernel: 14.8 us, 1.9 us per thousand entries of dK (the final
-// sums and the chain rule), and per million pixels 0.89 us per channel staged and 11 per
+// With the matrix-core tile kernel: 14.9 us, 1.7 us per thousand entries of dK (the final
+// sums and the chain rule), and per million pixels 0.68 us per channel staged and 8.8 per
 // 32 x 32 block of the GEMM; without this route 17.6 us and per million pixels 116 us, 0.72
 // per channel, 5.9 per rank and 0.1 per tap and rank where both channel counts are multiples
 // of 16, and 25.2 us and 124, 0.37 (per channel of the counts rounded up to 16), 5.4 and 0.1
 // where they run on zero-padded copies.  The smaller model picks the route: 0.3 % off the
-// better one in the geometric mean (always this route 5 % off, never 85 %): it loses where
+// better one in the geometric mean (always this route 4 % off, never 96 %): it loses where
 // both channel counts are multiples of 16 from 32 on under a 3x3 or 5x5 filter.
 // With the plain multiply-add tile kernel: a fixed 18 us plus the final sums and the chain
 // rule, and per million pixels the staging of the tiles (2.7 us per channel staged) and the
 // multiply-adds (0.375 us per channel-block group and tap), against 26 us plus per million
 // pixels 115 us and what grows with the planes.
-// (N16 C16 K16 512x512 R16: 1040 us -> 350; N16 C3 K1 512x512 R16: 1005 -> 63; N8 C8 K8
-// 256x256 R16: 132 -> 34; N16 C8 K8 256x256 R4: 210 -> 66; but N8 C32 K32 56x56 R16: 25
-// against 39.)
+// (N16 C16 K16 512x512 R16: 1040 us -> 215; N16 C3 K1 512x512 R16: 1005 -> 63; N8 C8 K8
+// 256x256 R16: 132 -> 32; N16 C8 K8 256x256 R4: 210 -> 60; but N8 C32 K32 56x56 R16: 25
+// against 33.)
 bool bwd_filter_dense_tiles_preferred(const cp4_shape& s) {
   const double mpx = (double)s.N * s.H * s.W / 1.0e6;
   const double taps = (double)s.Y * s.X, macs = (double)s.T * s.C * taps;
   if (use_mfma(s)) {
     const double blocks = (double)((s.C * s.Y * s.X + 31) / 32) * ((s.T + 31) / 32);
-    const double dense = 14.82 + 1.861e-3 * macs +
-                         mpx * (-6.751 + 0.8939 * (s.C + s.T) + 10.97 * blocks);
+    const double dense = 14.86 + 1.7325e-3 * macs +
+                         mpx * (-4.73 + 0.6821 * (s.C + s.T) + 8.835 * blocks);
     // (channel counts that are multiples of 16 run as they are, others on zero-padded copies)
     const bool as_is = s.T % 16 == 0 && s.C % 16 == 0;
     const double padded = (double)((s.T + 15) / 16 * 16 + (s.C + 15) / 16 * 16);

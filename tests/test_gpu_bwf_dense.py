@@ -53,13 +53,16 @@ SHAPES = [
     (2, 32, 31, 45, 1, 32, 3, 16),     # nine column blocks over two groups of waves; odd width: cell-by-cell loads
     (1, 40, 20, 36, 1, 40, 3, 8),      # two blocks of output channels, the second ragged
     (2, 24, 30, 32, 2, 24, 5, 8),      # 5x5, nineteen column blocks
-    (1, 48, 17, 40, 0, 32, 1, 16),     # 1x1 with 80 channels in all
+    (1, 48, 17, 40, 0, 32, 1, 16),     # 1x1 with 80 channels in all: waves across more column blocks than there are
+    (1, 64, 17, 40, 0, 64, 1, 16),     # 1x1 with 64 channels a side: 32 x 32 blocks, two blocks of output channels
     (1, 50, 20, 20, 1, 33, 3, 16),     # ragged on both sides
     (3, 16, 70, 132, 1, 16, 3, 16),    # several tiles per workgroup, 16-byte loads, tiles past both edges
     (2, 20, 40, 64, 0, 12, 3, 4),      # no padding with a 3x3 filter
     (1, 6, 9, 16, 2, 64, 3, 5),        # pad beyond (Y - 1) / 2; a plane smaller than a tile
-    (1, 4, 800, 800, 1, 4, 3, 4),      # more than 600,000 pixels: 32 x 32 blocks with four output channels
-    (2, 12, 64, 96, 1, 16, 5, 8),      # 16 x 16 blocks, 5x5: nineteen column blocks over two groups of waves
+    (1, 4, 800, 800, 1, 4, 3, 4),      # 640,000 pixels, four channels a side
+    (2, 12, 64, 96, 1, 16, 5, 8),      # 16 x 16 blocks, 5x5: nineteen column blocks over four groups of waves
+    (2, 16, 24, 40, 1, 32, 3, 8),      # 16 x 16 blocks, two blocks of output channels
+    (1, 20, 30, 44, 1, 25, 3, 6),      # the same, ragged on both sides
 ]
 
 
