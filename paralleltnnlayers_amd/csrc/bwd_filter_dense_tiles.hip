@@ -300,6 +300,7 @@ struct MfmaPlan {
   int m16;                // up to 32 output channels: 16 x 16 blocks, steps of 32 pixels, 16 waves
   int NC, NB, MB;         // columns C * FS * FS; blocks of them; blocks of output channels
   int nbw, slices, own;   // waves across column blocks; waves across steps; column blocks a wave
+  int rgroups;            // groups of waves across blocks of output channels (MB blocks each)
   int outs, grid;
   unsigned chmagic, xsmagic, dsmagic;
   size_t lds_bytes;
@@ -362,7 +363,10 @@ __global__ __launch_bounds__(M16 ? 1024 : 512, M16 ? 4 : 2) void dense_mfma_kern
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int l32 = lane & (BW - 1), hi = lane >> LGBW;   // row or column of a block; which eight pixels
   const int H = a.H, W = a.W, HW = H * W;
-  const int b = wave & (pl.nbw - 1), sl = wave / pl.nbw;
+  // wave = (row group, step slice, column-block lane): a row group takes MB blocks of output
+  // channels (more than MB blocks in all: two groups of waves, each with its own rows)
+  const int b = wave & (pl.nbw - 1), rest = wave / pl.nbw;
+  const int sl = rest % pl.slices, rg = rest / pl.slices;
   // this lane's column of every column block the wave owns, and its output channel of every
   // row block (past the last column / channel: the last one's cells, whose sums are not kept)
   int boff[OWN], aoff[MB];
@@ -375,7 +379,7 @@ __global__ __launch_bounds__(M16 ? 1024 : 512, M16 ? 4 : 2) void dense_mfma_kern
   }
 #pragma unroll
   for (int m = 0; m < MB; ++m) {
-    int k = BW * m + l32;
+    int k = BW * (MB * rg + m) + l32;
     k = k < a.T ? k : a.T - 1;
     aoff[m] = k * pl.DS + 8 * hi;
   }
@@ -548,7 +552,7 @@ __global__ __launch_bounds__(M16 ? 1024 : 512, M16 ? 4 : 2) void dense_mfma_kern
     for (int o = 0; o < OWN; ++o)
 #pragma unroll
       for (int m = 0; m < MB; ++m) {
-        float* r = red + ((size_t)(o * MB + m) * pl.nbw + b) * (NV * 64) + lane;
+        float* r = red + ((size_t)((rg * OWN + o) * MB + m) * pl.nbw + b) * (NV * 64) + lane;
         if (sl == s2 && o < pl.own) {
 #pragma unroll
           for (int v = 0; v < NV; ++v) r[v << 6] = acc[o][m][v];
@@ -559,7 +563,7 @@ __global__ __launch_bounds__(M16 ? 1024 : 512, M16 ? 4 : 2) void dense_mfma_kern
     for (int o = 0; o < OWN; ++o)
 #pragma unroll
       for (int m = 0; m < MB; ++m) {
-        const float* r = red + ((size_t)(o * MB + m) * pl.nbw + b) * (NV * 64) + lane;
+        const float* r = red + ((size_t)((rg * OWN + o) * MB + m) * pl.nbw + b) * (NV * 64) + lane;
         if (sl == 0 && o < pl.own) {
 #pragma unroll
           for (int v = 0; v < NV; ++v) acc[o][m][v] += r[v << 6];
@@ -579,7 +583,8 @@ __global__ __launch_bounds__(M16 ? 1024 : 512, M16 ? 4 : 2) void dense_mfma_kern
         for (int v = 0; v < NV; ++v) {
           // (accumulator element v: row 8 * (v / 4) + 4 * (lane / 32) + v % 4 of a 32 x 32 block,
           //  row 4 * (lane / 16) + v of a 16 x 16 one)
-          const int k = M16 ? 16 * m + 4 * hi + v : 32 * m + 8 * (v >> 2) + 4 * hi + (v & 3);
+          const int k = M16 ? 16 * (MB * rg + m) + 4 * hi + v
+                            : 32 * (MB * rg + m) + 8 * (v >> 2) + 4 * hi + (v & 3);
           if (k < a.T) out[(size_t)k * pl.NC + n] = acc[o][m][v];
         }
     }
@@ -837,10 +842,13 @@ bool mfma_plan_blocks(const cp4_shape& s, bool aligned16, int m16, MfmaPlan* bes
   const int vec = aligned16 && s.W % 4 == 0 ? 1 : 0, xlead = vec ? 4 : (int)s.pad;
   const int FS = (int)s.Y, T = (int)s.T, C = (int)s.C;
   const int BW = m16 ? 16 : 32, step = m16 ? 32 : 16;
-  const int NC = C * FS * FS, NB = (NC + BW - 1) / BW, MB = (T + BW - 1) / BW;
-  if (MB > 2 || (long)T * NC > kMaxOuts) return false;
+  const int NC = C * FS * FS, NB = (NC + BW - 1) / BW, MBall = (T + BW - 1) / BW;
+  // (a wave takes up to two blocks of output channels; with 16 x 16 blocks, 33 - 64 output
+  //  channels go over two groups of waves)
+  const int rgroups = MBall > 2 ? 2 : 1, MB = MBall > 2 ? 2 : MBall;
+  if (MBall > 2 * rgroups || (!m16 && rgroups > 1) || (long)T * NC > kMaxOuts) return false;
   const int most_own = (m16 ? kMaxAcc16 : kMaxAcc) / MB;
-  const int waves = m16 ? 16 : kMWaves;
+  const int waves = (m16 ? 16 : kMWaves) / rgroups;   // per row group
   const int cus = num_compute_units();
   bool found = false;
   double best_cost = 0;
@@ -850,7 +858,7 @@ bool mfma_plan_blocks(const cp4_shape& s, bool aligned16, int m16, MfmaPlan* bes
   for (int nbw = 1; nbw <= waves; nbw *= 2) {
     if ((NB + nbw - 1) / nbw > most_own) continue;
     const int slices = waves / nbw, own = (NB + nbw - 1) / nbw;
-    const size_t red = (size_t)own * MB * nbw * (m16 ? 256 : 1024) * sizeof(float);
+    const size_t red = (size_t)rgroups * (m16 ? kMaxAcc16 : kMaxAcc) * nbw * (m16 ? 256 : 1024) * sizeof(float);
   for (int TW = step; TW <= 128; TW *= 2)
     for (int TH = 1; TH <= 32; TH *= 2) {
       if (TH * TW / step < slices) continue;
@@ -878,7 +886,7 @@ bool mfma_plan_blocks(const cp4_shape& s, bool aligned16, int m16, MfmaPlan* bes
       pl.XS = XS; pl.XR = XR; pl.PHXS = PH * XS; pl.DS = DS; pl.vec = vec; pl.xlead = xlead;
       pl.nx = nx; pl.nd = nd; pl.xplane = xplane; pl.dplane = dplane; pl.bufbytes = bufbytes;
       pl.m16 = m16; pl.NC = NC; pl.NB = NB; pl.MB = MB;
-      pl.nbw = nbw; pl.slices = slices; pl.own = own;
+      pl.nbw = nbw; pl.slices = slices; pl.own = own; pl.rgroups = rgroups;
       pl.outs = T * NC;
       pl.chmagic = (unsigned)((0x100000000ull + (unsigned)XR - 1) / (unsigned)XR);
       pl.xsmagic = (unsigned)((0x100000000ull + (unsigned)XS - 1) / (unsigned)XS);
@@ -923,17 +931,17 @@ bool mfma_plan_blocks(const cp4_shape& s, bool aligned16, int m16, MfmaPlan* bes
   pl.xplane = (pl.nx + 8 + 7) / 8 * 8;
   pl.bufbytes = 6 * (pl.xplane + pl.dplane);
   pl.lds_bytes = 2 * (size_t)pl.bufbytes;
-  const size_t red = (size_t)pl.own * MB * pl.nbw * (m16 ? 256 : 1024) * sizeof(float);
+  const size_t red = (size_t)rgroups * (m16 ? kMaxAcc16 : kMaxAcc) * pl.nbw * (m16 ? 256 : 1024) * sizeof(float);
   if (pl.slices > 1 && red > pl.lds_bytes) pl.lds_bytes = red;
   pl.chmagic = (unsigned)((0x100000000ull + (unsigned)pl.XR - 1) / (unsigned)pl.XR);
   return true;
 }
 
-// Up to 32 output channels: 16 x 16 blocks (all rows in use with up to 16 channels) on 16
-// waves, whose accumulators are small enough for four waves per SIMD (N16 C16 K16 512x512:
-// 330 -> 204 us); else, or where no tile of those fits, 32 x 32 blocks on 8 waves.
+// 16 x 16 blocks (all rows in use with up to 16 channels) on 16 waves, whose accumulators are
+// small enough for four waves per SIMD (N16 C16 K16 512x512: 330 -> 204 us); where no tile of
+// those fits, 32 x 32 blocks on 8 waves.
 bool mfma_plan_uncached(const cp4_shape& s, bool aligned16, MfmaPlan* best) {
-  if (s.T <= 32 && mfma_plan_blocks(s, aligned16, 1, best)) return true;
+  if (mfma_plan_blocks(s, aligned16, 1, best)) return true;
   return mfma_plan_blocks(s, aligned16, 0, best);
 }
 
