@@ -212,7 +212,8 @@ cp4_status cp4_conv2d_backward_filter_noalloc(const cp4_shape* shape, const floa
  * workspace), 3 the dense filter gradient over tiles of pixels followed by the chain
  * rule onto the factors, for few channels on both sides (T * C <= 256 with plain
  * multiply-adds, or on the matrix cores T <= 64, T * C * Y * X <= 16384 and a tile of
- * all channels within the LDS, about 80 channels together; square filters of 1, 3 or 5
+ * all channels within the LDS: 64 + 64 channels under a 1x1 filter, about 80 together
+ * under 3x3; square filters of 1, 3 or 5
  * taps, pad <= Y - 1; any alignment); CP4_ERR_UNSUPPORTED if the shape does not qualify
  * for 1, 2 or 3. */
 cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const float* x,

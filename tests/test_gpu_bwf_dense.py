@@ -63,6 +63,9 @@ SHAPES = [
     (2, 12, 64, 96, 1, 16, 5, 8),      # 16 x 16 blocks, 5x5: nineteen column blocks over four groups of waves
     (2, 16, 24, 40, 1, 32, 3, 8),      # 16 x 16 blocks, two blocks of output channels
     (1, 20, 30, 44, 1, 25, 3, 6),      # the same, ragged on both sides
+    (2, 4, 1, 1, 0, 4, 1, 3),          # planes of one pixel
+    (1, 3, 2, 3, 2, 2, 3, 2),          # planes narrower than four pixels, pad 2
+    (300, 6, 5, 8, 1, 6, 3, 4),        # more images than workgroups
 ]
 
 
