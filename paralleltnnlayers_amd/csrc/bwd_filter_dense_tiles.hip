@@ -1027,15 +1027,17 @@ bool mfma_ok(const cp4_shape& s) {
   return common_ok(s) && mfma_plan(s, false, &pl);
 }
 
-// Which of the two tile kernels.  The matrix cores wherever they can run, except for one to
-// three output channels under a 3x3 or 5x5 filter on large inputs: there a 32-row block of
-// the GEMM is nearly empty and the plain multiply-adds are the faster ones (N16 C32 K1
-// 256x256 3x3: 112 us against 177; N128 C3 K1 512x512: 336 against 515).
+// Which of the two tile kernels.  The matrix cores wherever they can run, except for one or
+// two output channels under a 3x3 filter on large inputs: there a block of the GEMM is nearly
+// empty and the plain multiply-adds are the faster ones (N128 C3 K1 512x512: 236 us against
+// 370; N16 C32 K1 256x256: 90 against 104; but N32 C16 K3 256x256: 143 against 106, and under
+// a 5x5 filter, whose 25 taps a thread take the plain kernel to 256 registers, N128 C3 K1
+// 512x512: 1330 against 664).
 bool use_mfma(const cp4_shape& s) {
   if (!mfma_ok(s)) return false;
   if (!valu_ok(s)) return true;
   const double cells = (double)s.N * s.H * s.W * s.C;
-  return !(s.T <= 3 && s.Y >= 3 && cells >= 3.0e6);
+  return !(s.T <= 2 && s.Y == 3 && cells >= 3.0e6);
 }
 
 }  // namespace
