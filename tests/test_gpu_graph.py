@@ -19,8 +19,11 @@ def cp4():
     return p
 
 
-# (N, C, H, W, T, Y, R): matrix-core kernels / general kernels / channels above 256
-SHAPES = [(2, 64, 28, 28, 64, 3, 16), (3, 5, 9, 9, 7, 3, 3), (1, 320, 14, 14, 64, 3, 32)]
+# (N, C, H, W, T, Y, R): matrix-core kernels / odd channel counts (backward-filter by the dense
+# gradient) / channels above 256 / few channels on a wide plane (the few-channel forward kernel,
+# backward-filter by the dense gradient over several tiles per workgroup)
+SHAPES = [(2, 64, 28, 28, 64, 3, 16), (3, 5, 9, 9, 7, 3, 3), (1, 320, 14, 14, 64, 3, 32),
+          (4, 16, 192, 320, 16, 3, 16)]
 
 
 @pytest.mark.parametrize("dims", SHAPES, ids=lambda d: "x".join(map(str, d)))
