@@ -54,6 +54,25 @@ struct DensePlan {
   size_t lds_bytes;
 };
 
+// A workgroup's tiles.  Workgroups go to the chip's eight dies in turn (blockIdx & 7), each die
+// with an L2 of its own: a die takes one contiguous eighth of the tiles and its workgroups
+// stride through it, so that tiles which share halo rows and columns run on the same die at
+// about the same time (tile t, t + 1 on neighbouring dies: every halo cell is fetched once
+// per die that needs it, 1.7 - 1.9 times the input in all).
+struct TileRange {
+  int first, end, step;
+};
+__device__ __forceinline__ TileRange tiles_of_workgroup(int ntiles) {
+  const int dies = gridDim.x < 8 ? (int)gridDim.x : 8;            // (fewer than eight workgroups: a range each)
+  const int die = blockIdx.x % dies, slot = blockIdx.x / dies;
+  const int on_die = ((int)gridDim.x - die + dies - 1) / dies;     // workgroups on this die
+  TileRange r;
+  r.first = (int)((long)ntiles * die / dies) + slot;
+  r.end = (int)((long)ntiles * (die + 1) / dies);
+  r.step = on_die;
+  return r;
+}
+
 template <int FS, int KB>
 __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, DensePlan pl,
                                                                float* partial) {
@@ -82,7 +101,8 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
   // the channels that pad x to a multiple of four are zeros for the whole launch
   for (int e = a.C * pl.XR + tid; e < pl.Cp * pl.XR; e += kThreads) X[e] = 0.f;
   const int tiles_per_image = pl.tilesX * pl.tilesY;
-  for (int t = blockIdx.x; t < pl.ntiles; t += gridDim.x) {
+  const TileRange tr = tiles_of_workgroup(pl.ntiles);
+  for (int t = tr.first; t < tr.end; t += tr.step) {
     const int n = t / tiles_per_image, rem = t - n * tiles_per_image;
     const int ty = rem / pl.tilesX, tx = rem - ty * pl.tilesX;
     const int h0 = ty * pl.TH, w0 = tx * pl.TW;
@@ -473,13 +493,16 @@ __global__ __launch_bounds__(M16 ? 1024 : 512, M16 ? 4 : 2) void dense_mfma_kern
   };
 
   char* const bufs = reinterpret_cast<char*>(lds);
-  fetch(blockIdx.x);
-  deposit(bufs);
+  const TileRange tr = tiles_of_workgroup(pl.ntiles);
+  if (tr.first < tr.end) {
+    fetch(tr.first);
+    deposit(bufs);
+  }
   __syncthreads();
   int it = 0;
-  for (int t = blockIdx.x; t < pl.ntiles; t += gridDim.x, ++it) {
-    const bool more = t + (int)gridDim.x < pl.ntiles;
-    if (more) fetch(t + gridDim.x);
+  for (int t = tr.first; t < tr.end; t += tr.step, ++it) {
+    const bool more = t + tr.step < tr.end;
+    if (more) fetch(t + tr.step);
     const char* cur = bufs + (size_t)(it & 1) * pl.bufbytes;
     const unsigned* xp = reinterpret_cast<const unsigned*>(cur);
     const char* dp = cur + 6 * pl.xplane;
