@@ -224,6 +224,15 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
                                               size_t workspace_bytes, int variant,
                                               cp4_stream stream);
 
+/* Variant 3 has two tile kernels and picks one by the shape (one or two output channels
+ * under a 3x3 filter on large inputs: plain multiply-adds; else the matrix cores).
+ * cp4_set_backward_filter_tile_kernel overrides that for every later launch of the process
+ * where both can run the shape: 0 plain multiply-adds, 1 matrix cores, anything else the
+ * library's choice again.  For A/B measurements and for tests that run both kernels on the
+ * same inputs; no counterpart in the reference (cp4Conv2dBackwardFilter.cu has one kernel
+ * sequence). */
+void cp4_set_backward_filter_tile_kernel(int which);
+
 /* Replaces cp4_conv2d_backward_filter_full_gpu
  * (Cuda_kernels/cp4Conv2dBackwardFilter.cuh:7-11, .cu:23-59): dense filter
  * gradient dK[T,C,Y,X]; accumulate != 0 adds into dK as the reference does. */

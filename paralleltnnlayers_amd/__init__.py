@@ -16,7 +16,7 @@ from .capi import (Shape, Geometry, geometry, conv2d_forward_ex, conv2d_backward
                    time_forward, time_forward_sets, time_backward_data, time_backward_filter,
                    tune_forward, tune_backward_data, tune_backward_filter, tuned_choice, plan_query,
                    set_tuned_choice, tuned_table, tuned_filter_table, set_tuned_filter_choice,
-                   backward_filter_variants, save_tuned, load_tuned, tune_clear, device_status, device_status_detail, set_spin_limit,
+                   backward_filter_variants, save_tuned, load_tuned, tune_clear, device_status, device_status_detail, set_spin_limit, set_backward_filter_tile_kernel,
                    forward_variants, default_variant, recompose, count_exceeding,
                    random_uniform, time_copy, cp3_shape_for, cp3_expand_factors,
                    cp3_fold_gradients, cp3_conv2d_forward, cp3_conv2d_backward_data,

@@ -149,6 +149,8 @@ def lib():
     L.cp4_device_status.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
     L.cp4_set_spin_limit.argtypes = [ctypes.c_int]
     L.cp4_set_spin_limit.restype = None
+    L.cp4_set_backward_filter_tile_kernel.argtypes = [ctypes.c_int]
+    L.cp4_set_backward_filter_tile_kernel.restype = None
     L.cp4_recompose.argtypes = [_S, _F, _F, _F, _F, _F, ctypes.c_void_p]
     L.cp3_expand_factors.argtypes = [_S] + [_F] * 7 + [ctypes.c_void_p]
     L.cp3_fold_gradients.argtypes = [_S] + [_F] * 6 + [ctypes.c_void_p]
@@ -735,6 +737,12 @@ def device_status_detail(stream=None):
 def set_spin_limit(polls):
     """Polls after which an in-kernel wait gives up (0: the default); fault injection."""
     lib().cp4_set_spin_limit(int(polls))
+
+
+def set_backward_filter_tile_kernel(which):
+    """Backward-filter variant 3: 0 the plain multiply-add tile kernel, 1 the matrix-core one
+    (wherever both can run the shape), anything else the library's choice."""
+    lib().cp4_set_backward_filter_tile_kernel(int(which))
 
 
 def recompose(FK, FC, FH, FW, stream=None):

@@ -23,6 +23,7 @@
 // No atomics: bit-reproducible.  Plain fp32 multiply-adds, or exact fp32 products from bf16
 // parts on the matrix cores.
 #include "cp4_internal.h"
+#include <atomic>
 #include "split_bf16.h"
 
 namespace cp4 {
@@ -1056,9 +1057,13 @@ bool mfma_ok(const cp4_shape& s) {
 // 370; N16 C32 K1 256x256: 90 against 104; but N32 C16 K3 256x256: 143 against 106, and under
 // a 5x5 filter, whose 25 taps a thread take the plain kernel to 256 registers, N128 C3 K1
 // 512x512: 1330 against 664).
+std::atomic<int> g_forced_tile_kernel{-1};
+
 bool use_mfma(const cp4_shape& s) {
   if (!mfma_ok(s)) return false;
   if (!valu_ok(s)) return true;
+  const int forced = g_forced_tile_kernel.load();
+  if (forced >= 0) return forced == 1;
   const double cells = (double)s.N * s.H * s.W * s.C;
   return !(s.T <= 2 && s.Y == 3 && cells >= 3.0e6);
 }
@@ -1066,6 +1071,10 @@ bool use_mfma(const cp4_shape& s) {
 }  // namespace
 
 bool bwd_filter_dense_tiles_supported(const cp4_shape& s) { return valu_ok(s) || mfma_ok(s); }
+
+void bwd_filter_dense_tiles_force_kernel(int which) {
+  g_forced_tile_kernel.store(which == 0 || which == 1 ? which : -1);
+}
 
 // Partial sets of the tile kernel, then the dense gradient itself.
 size_t bwd_filter_dense_tiles_workspace_bytes(const cp4_shape& s) {

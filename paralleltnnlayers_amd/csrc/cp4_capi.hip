@@ -1988,6 +1988,10 @@ cp4_status cp4_device_status(cp4_stream stream, int* detail) {
 
 void cp4_set_spin_limit(int polls) { g_spin_limit.store(polls > 0 ? polls : 0); }
 
+void cp4_set_backward_filter_tile_kernel(int which) {
+  cp4::bwd_filter_dense_tiles_force_kernel(which);
+}
+
 cp4_status cp4_set_device(int ordinal) {
   CP4_HIP(hipSetDevice(ordinal));
   return CP4_OK;

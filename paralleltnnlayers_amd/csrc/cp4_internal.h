@@ -180,6 +180,9 @@ bool bwd_filter_dense_tiles_supported(const cp4_shape&);
 bool bwd_filter_dense_tiles_preferred(const cp4_shape&);
 size_t bwd_filter_dense_tiles_workspace_bytes(const cp4_shape&);
 hipError_t bwd_filter_dense_tiles_launch(const BwdFilterArgs&, hipStream_t);
+// 0: the plain multiply-add tile kernel, 1: the matrix-core one, wherever both can run the
+// shape; anything else: the route's own choice.
+void bwd_filter_dense_tiles_force_kernel(int which);
 // A layer with a stride and zeros of its own before the image (BwdFilterArgs::H, W: the
 // input plane; pad unused; dy on the geometry's Ho x Wo grid).
 bool bwd_filter_mfma_strided_supported(const cp4_shape&, const Geometry&);

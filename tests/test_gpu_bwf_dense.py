@@ -66,6 +66,8 @@ SHAPES = [
     (2, 4, 1, 1, 0, 4, 1, 3),          # planes of one pixel
     (1, 3, 2, 3, 2, 2, 3, 2),          # planes narrower than four pixels, pad 2
     (300, 6, 5, 8, 1, 6, 3, 4),        # more images than workgroups
+    (4, 3, 512, 512, 1, 1, 3, 16),     # three channels to one on a million pixels: plain multiply-adds by choice
+    (1, 8, 701, 603, 1, 2, 3, 4),      # the same kernel with cell-by-cell loads (odd width)
 ]
 
 
@@ -80,16 +82,23 @@ def test_dense_gradient_tiles(cp4, oracle, dims):
     f = [dev(v) for v in fac]
     assert cp4.backward_filter_variants()[3] == "dense_gradient_tiles"
     wants = oracle.backward_filter(x, dy, *fac, pad)
-    first = None
-    for rep in range(2):       # bit-reproducible: no atomics anywhere
-        grads = cp4.conv2d_backward_filter(dev(x), dev(dy), *f, pad=pad, variant=3)
-        got = [host(g) for g in grads]
-        for g, w, k in zip(got, wants, FACTORS):
-            close(g, w, f"d{k}")
-        if first is None:
-            first = got
-        else:
-            assert all(np.array_equal(a, b) for a, b in zip(first, got))
+    # the route's own tile kernel, then each of the two where it can run the shape
+    # (0: plain multiply-adds, T * C <= 256; 1: matrix cores)
+    try:
+        for which in (-1, 0, 1):
+            cp4.set_backward_filter_tile_kernel(which)
+            first = None
+            for rep in range(2):       # bit-reproducible: no atomics anywhere
+                grads = cp4.conv2d_backward_filter(dev(x), dev(dy), *f, pad=pad, variant=3)
+                got = [host(g) for g in grads]
+                for g, w, k in zip(got, wants, FACTORS):
+                    close(g, w, f"d{k}, tile kernel {which}")
+                if first is None:
+                    first = got
+                else:
+                    assert all(np.array_equal(a, b) for a, b in zip(first, got))
+    finally:
+        cp4.set_backward_filter_tile_kernel(-1)
     cp4.device_status()
 
 
