@@ -43,13 +43,15 @@ struct DensePlan {
   int KBLK, CBLK;      // blocks of KB output channels / 4 input channels
   int G, S;            // channel-block groups; threads (pixel runs) per group
   int L;               // pixels per run
-  int XS, XR;          // x tile in LDS: row stride, rows * XS per channel (padded)
+  int XS, XR;          // x tile in LDS: row stride (odd), rows * XS per channel
+  int XSg, DRS;        // columns staged per row of x; row stride of the dy tile (odd)
+  int skew;            // runs to lanes: four runs of a row, then the next row (see the kernel)
   int vec, xlead;      // 16-byte loads; columns of x staged before the tile's first (pad, or 4)
   int Cp, Tp;          // channel counts padded to their blocks
   int outs;            // T * C * FS * FS
   int lgTW, lgtile;    // log2 of TW and of TH * TW
-  unsigned chmagic;    // ceil(2^32 / ((TH + FS - 1) * XS))
-  unsigned xsmagic;    // ceil(2^32 / XS)
+  unsigned chmagic;    // ceil(2^32 / ((TH + FS - 1) * XSg))
+  unsigned xsmagic;    // ceil(2^32 / XSg)
   int gbatch;          // groups whose partial sums the LDS holds at a time in the final sum
   int grid;
   size_t lds_bytes;
@@ -79,7 +81,8 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
                                                                float* partial) {
   extern __shared__ float lds[];
   float* X = lds;                                    // [Cp][TH + FS - 1][XS]
-  float* D = lds + (size_t)pl.Cp * pl.XR;            // [Tp][TH][TW]
+  float* D = lds + (size_t)pl.Cp * pl.XR;            // [Tp][TH][DRS]
+  const int DK = pl.TH * pl.DRS;                     // an output channel's tile
   const int tid = threadIdx.x;
   const int H = a.H, W = a.W, HW = H * W;
   const int PH = pl.TH + FS - 1, PW = pl.TW + FS - 1;
@@ -115,7 +118,7 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
     constexpr int kBatch = 8;
     const float* xn = a.x + (size_t)n * a.C * HW;
     const float* dn = a.dy + (size_t)n * a.T * HW;
-    const int nx = a.C * PH * pl.XS;
+    const int nx = a.C * PH * pl.XSg;
     const int nd = pl.Tp * pl.TH * pl.TW;
     if (pl.vec) {
       // Four cells a load (W a multiple of four, x and dy 16-byte aligned): the tile's rows
@@ -129,38 +132,43 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
 #pragma unroll
         for (int u = 0; u < kBatch4; ++u) {
           const int e = e0 + 4 * u * kThreads;
-          const int c = (int)__umulhi((unsigned)e, pl.chmagic), r2 = e - c * (PH * pl.XS);
-          const int pr = (int)__umulhi((unsigned)r2, pl.xsmagic), pc = r2 - pr * pl.XS;
+          const int c = (int)__umulhi((unsigned)e, pl.chmagic), r2 = e - c * (PH * pl.XSg);
+          const int pr = (int)__umulhi((unsigned)r2, pl.xsmagic), pc = r2 - pr * pl.XSg;
           const int h = h0 - a.pad + pr, w = w0 - 4 + pc;
           in[u] = e < nx && c < a.C && h >= 0 && h < H && w >= 0 && w < W;
-          at[u] = e < nx ? c * pl.XR + r2 : -1;
+          at[u] = e < nx ? c * pl.XR + pr * pl.XS + pc : -1;
           const int cc = c < a.C ? c : a.C - 1;
           const int hc = h < 0 ? 0 : (h > H - 1 ? H - 1 : h), wc = w < 0 ? 0 : (w > W - 4 ? W - 4 : w);
           v[u] = *reinterpret_cast<const float4*>(xn + (size_t)cc * HW + (size_t)hc * W + wc);
         }
 #pragma unroll
         for (int u = 0; u < kBatch4; ++u)
-          if (at[u] >= 0)
-            *reinterpret_cast<float4*>(X + at[u]) = in[u] ? v[u] : make_float4(0.f, 0.f, 0.f, 0.f);
+          if (at[u] >= 0) {              // (rows an odd number of cells apart: four 4-byte stores)
+            const float4 w4 = in[u] ? v[u] : make_float4(0.f, 0.f, 0.f, 0.f);
+            X[at[u]] = w4.x; X[at[u] + 1] = w4.y; X[at[u] + 2] = w4.z; X[at[u] + 3] = w4.w;
+          }
       }
       for (int e0 = 4 * tid; e0 < nd; e0 += 4 * kThreads * kBatch4) {
         float4 v[kBatch4];
         bool in[kBatch4];
+        int at[kBatch4];
 #pragma unroll
         for (int u = 0; u < kBatch4; ++u) {
           const int e = e0 + 4 * u * kThreads;
           const int k = e >> pl.lgtile, r2 = e & ((1 << pl.lgtile) - 1);
           const int pr = r2 >> pl.lgTW, pc = r2 & (pl.TW - 1);
           const int h = h0 + pr, w = w0 + pc;
+          at[u] = e < nd ? k * DK + pr * pl.DRS + pc : -1;
           in[u] = e < nd && k < a.T && h < H && w < W;
           const int kc = k < a.T ? k : a.T - 1, hc = h > H - 1 ? H - 1 : h, wc = w > W - 4 ? W - 4 : w;
           v[u] = *reinterpret_cast<const float4*>(dn + (size_t)kc * HW + (size_t)hc * W + wc);
         }
 #pragma unroll
         for (int u = 0; u < kBatch4; ++u)
-          if (e0 + 4 * u * kThreads < nd)
-            *reinterpret_cast<float4*>(D + e0 + 4 * u * kThreads) =
-                in[u] ? v[u] : make_float4(0.f, 0.f, 0.f, 0.f);
+          if (at[u] >= 0) {
+            const float4 w4 = in[u] ? v[u] : make_float4(0.f, 0.f, 0.f, 0.f);
+            D[at[u]] = w4.x; D[at[u] + 1] = w4.y; D[at[u] + 2] = w4.z; D[at[u] + 3] = w4.w;
+          }
       }
     } else {
     for (int e0 = tid; e0 < nx; e0 += kThreads * kBatch) {
@@ -170,11 +178,11 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
         const int e = e0 + u * kThreads;
-        const int c = (int)__umulhi((unsigned)e, pl.chmagic), r2 = e - c * (PH * pl.XS);
-        const int pr = (int)__umulhi((unsigned)r2, pl.xsmagic), pc = r2 - pr * pl.XS;
+        const int c = (int)__umulhi((unsigned)e, pl.chmagic), r2 = e - c * (PH * pl.XSg);
+        const int pr = (int)__umulhi((unsigned)r2, pl.xsmagic), pc = r2 - pr * pl.XSg;
         const int h = h0 - a.pad + pr, w = w0 - a.pad + pc;
         in[u] = e < nx && c < a.C && pc < PW && h >= 0 && h < H && w >= 0 && w < W;
-        at[u] = e < nx ? c * pl.XR + r2 : -1;
+        at[u] = e < nx ? c * pl.XR + pr * pl.XS + pc : -1;
         const int cc = c < a.C ? c : a.C - 1;
         const int hc = h < 0 ? 0 : (h > H - 1 ? H - 1 : h), wc = w < 0 ? 0 : (w > W - 1 ? W - 1 : w);
         v[u] = xn[(size_t)cc * HW + (size_t)hc * W + wc];
@@ -186,19 +194,21 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
     for (int e0 = tid; e0 < nd; e0 += kThreads * kBatch) {
       float v[kBatch];
       bool in[kBatch];
+      int at[kBatch];
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
         const int e = e0 + u * kThreads;
         const int k = e >> pl.lgtile, r2 = e & ((1 << pl.lgtile) - 1);
         const int pr = r2 >> pl.lgTW, pc = r2 & (pl.TW - 1);
         const int h = h0 + pr, w = w0 + pc;
+        at[u] = e < nd ? k * DK + pr * pl.DRS + pc : -1;
         in[u] = e < nd && k < a.T && h < H && w < W;
         const int kc = k < a.T ? k : a.T - 1, hc = h > H - 1 ? H - 1 : h, wc = w > W - 1 ? W - 1 : w;
         v[u] = dn[(size_t)kc * HW + (size_t)hc * W + wc];
       }
 #pragma unroll
       for (int u = 0; u < kBatch; ++u)
-        if (e0 + u * kThreads < nd) D[e0 + u * kThreads] = in[u] ? v[u] : 0.f;
+        if (at[u] >= 0) D[at[u]] = in[u] ? v[u] : 0.f;
     }
     }
     __syncthreads();
@@ -206,9 +216,21 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
     if (active) {
       const int nruns = pl.TH * runs_per_row;
       for (int run = s; run < nruns; run += pl.S) {
-        const int row = run / runs_per_row, col0 = (run - row * runs_per_row) * pl.L;
+        // Runs to lanes: in row-major order 16 lanes of a row would read cells L apart, a
+        // few LDS banks only.  With `skew`, consecutive lanes take four runs of a row and then
+        // the next row: rows are an odd number of cells apart, so 32 lanes (8 rows x 4 runs of
+        // 8 cells) read 32 different banks.
+        int row, col0;
+        if (pl.skew) {
+          const int quad = run >> 2;
+          row = quad & (pl.TH - 1);
+          col0 = (((quad >> (pl.lgtile - pl.lgTW)) << 2) + (run & 3)) * pl.L;
+        } else {
+          row = run / runs_per_row;
+          col0 = (run - row * runs_per_row) * pl.L;
+        }
         const float* xr = X + (size_t)(kCB * cb) * pl.XR + row * pl.XS + col0 + (pl.xlead - a.pad);
-        const float* dr = D + (size_t)(KB * kb) * pl.TH * pl.TW + row * pl.TW + col0;
+        const float* dr = D + (size_t)(KB * kb) * DK + row * pl.DRS + col0;
         // window columns col0 + t ... col0 + t + FS - 1; column (t + j) lives in slot (t + j) % FS
         float xw[kCB][FS][FS];
 #pragma unroll
@@ -231,7 +253,7 @@ __global__ __launch_bounds__(kThreads) void dense_tiles_kernel(BwdFilterArgs a, 
                 xw[c][i][(tt + FS - 1) % FS] = xr[(size_t)c * pl.XR + i * pl.XS + tcol + FS - 1];
             float d[KB];
 #pragma unroll
-            for (int k = 0; k < KB; ++k) d[k] = live ? dr[(size_t)k * pl.TH * pl.TW + tcol] : 0.f;
+            for (int k = 0; k < KB; ++k) d[k] = live ? dr[(size_t)k * DK + tcol] : 0.f;
 #pragma unroll
             for (int k = 0; k < KB; ++k)
 #pragma unroll
@@ -777,9 +799,12 @@ bool plan(const cp4_shape& s, bool aligned16, DensePlan* best) {
       while (L > 8 && (long)TH * TW / L < S) L >>= 1;
       // room for a run's last steps to read past it; with 16-byte loads the columns before
       // the tile's first, rows and channels multiples of four cells apart
-      const int XS = vec ? (4 + TW + 2 * FS - 1 + 3) / 4 * 4 : TW + FS - 1 + FS;
-      const int XR = (TH + FS - 1) * XS + (vec ? 4 : 1);  // (off a power of two: bank conflicts)
-      const size_t lds = ((size_t)Cp * XR + (size_t)Tp * TH * TW + FS) * sizeof(float);
+      // (in LDS the rows of both tiles are an odd number of cells apart: lanes on consecutive
+      //  rows then read different banks)
+      const int XSg = vec ? (4 + TW + 2 * FS - 1 + 3) / 4 * 4 : TW + FS - 1 + FS;
+      const int XS = XSg | 1, DRS = TW + 1;
+      const int XR = (TH + FS - 1) * XS;
+      const size_t lds = ((size_t)Cp * XR + (size_t)Tp * TH * DRS + FS) * sizeof(float);
       const size_t red = (size_t)S * KB * kCB * FS * FS * sizeof(float);
       if (lds > kLdsLimit || red > kLdsLimit) continue;
       DensePlan pl;
@@ -789,11 +814,13 @@ bool plan(const cp4_shape& s, bool aligned16, DensePlan* best) {
       pl.ntiles = (int)s.N * pl.tilesX * pl.tilesY;
       pl.KBLK = KBLK; pl.CBLK = CBLK; pl.G = G; pl.S = S; pl.L = L;
       pl.XS = XS; pl.XR = XR; pl.Cp = Cp; pl.Tp = Tp; pl.vec = vec; pl.xlead = xlead;
+      pl.XSg = XSg; pl.DRS = DRS;
+      pl.skew = (TW / L) % 4 == 0 && TH >= 2 ? 1 : 0;
       pl.outs = (int)(s.T * s.C * s.Y * s.X);
       pl.lgTW = __builtin_ctz(TW);
       pl.lgtile = __builtin_ctz(TW) + __builtin_ctz(TH);
-      pl.chmagic = (unsigned)((0x100000000ull + (unsigned)((TH + FS - 1) * XS) - 1) / (unsigned)((TH + FS - 1) * XS));
-      pl.xsmagic = (unsigned)((0x100000000ull + (unsigned)XS - 1) / (unsigned)XS);
+      pl.chmagic = (unsigned)((0x100000000ull + (unsigned)((TH + FS - 1) * XSg) - 1) / (unsigned)((TH + FS - 1) * XSg));
+      pl.xsmagic = (unsigned)((0x100000000ull + (unsigned)XSg - 1) / (unsigned)XSg);
       // workgroups per compute unit: what the LDS and the registers (two waves per SIMD with
       // two output channels a thread, three with one) leave room for
       const int by_lds = (int)(160 * 1024 / (lds > red ? lds : red));
@@ -1052,11 +1079,11 @@ bool mfma_ok(const cp4_shape& s) {
 }
 
 // Which of the two tile kernels.  The matrix cores wherever they can run, except for one or
-// two output channels under a 3x3 filter on large inputs: there a block of the GEMM is nearly
-// empty and the plain multiply-adds are the faster ones (N128 C3 K1 512x512: 236 us against
-// 370; N16 C32 K1 256x256: 90 against 104; but N32 C16 K3 256x256: 143 against 106, and under
-// a 5x5 filter, whose 25 taps a thread take the plain kernel to 256 registers, N128 C3 K1
-// 512x512: 1330 against 664).
+// two output channels under a 3x3 or 5x5 filter on large inputs: there a block of the GEMM is
+// nearly empty and the plain multiply-adds are the faster ones (N128 C3 K1 512x512: 173 us
+// against 360; N32 C16 K2 256x256: 79 against 97; N16 C16 K1 256x256 5x5: 85 against 124;
+// but N32 C16 K3 256x256: 97 either way, N16 C16 K3 256x256 5x5: 175 against 128, and
+// N8 C8 K2 256x256: 32 against 30).
 std::atomic<int> g_forced_tile_kernel{-1};
 
 bool use_mfma(const cp4_shape& s) {
@@ -1065,7 +1092,7 @@ bool use_mfma(const cp4_shape& s) {
   const int forced = g_forced_tile_kernel.load();
   if (forced >= 0) return forced == 1;
   const double cells = (double)s.N * s.H * s.W * s.C;
-  return !(s.T <= 2 && s.Y == 3 && cells >= 3.0e6);
+  return !(s.T <= 2 && s.Y >= 3 && cells >= 1.0e7);
 }
 
 }  // namespace

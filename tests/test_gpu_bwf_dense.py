@@ -66,8 +66,8 @@ SHAPES = [
     (2, 4, 1, 1, 0, 4, 1, 3),          # planes of one pixel
     (1, 3, 2, 3, 2, 2, 3, 2),          # planes narrower than four pixels, pad 2
     (300, 6, 5, 8, 1, 6, 3, 4),        # more images than workgroups
-    (4, 3, 512, 512, 1, 1, 3, 16),     # three channels to one on a million pixels: plain multiply-adds by choice
-    (1, 8, 701, 603, 1, 2, 3, 4),      # the same kernel with cell-by-cell loads (odd width)
+    (4, 3, 512, 512, 1, 1, 3, 16),     # three channels to one on a million pixels
+    (1, 24, 701, 603, 1, 2, 3, 4),     # plain multiply-adds by choice (ten million cells), cell-by-cell loads (odd width)
 ]
 
 
