@@ -637,36 +637,39 @@ __global__ __launch_bounds__(M16 ? 1024 : 512, M16 ? 4 : 2) void dense_mfma_kern
   }
 }
 
-// dK[o] = sum over the partial sets in a fixed order: thread (o, y) adds sets y, y + 8, ...,
-// then the eight partial sums are added in order through LDS (one thread summing all the sets
-// of an entry would wait for several hundred loads one after the other).
-constexpr int kRedOuts = 32, kRedSets = 8;
-__global__ __launch_bounds__(kRedOuts * kRedSets) void dense_reduce_kernel(const float* partial,
-                                                                           float* dK, int outs,
-                                                                           int sets) {
-  __shared__ float part[kRedSets][kRedOuts];
+// dK[o] = sum over the partial sets in a fixed order: thread (o, y) adds sets y, y + LANES, ...,
+// then the LANES partial sums are added in order through LDS (one thread summing all the sets
+// of an entry would wait for several hundred loads one after the other).  Eight lanes of sets
+// where dK has many entries, 32 where it has few (27 entries for three channels to one: a
+// single workgroup, whose threads then wait for 24 loads each instead of 96).
+constexpr int kRedOuts = 32;
+template <int LANES>
+__global__ __launch_bounds__(kRedOuts * LANES) void dense_reduce_kernel(const float* partial,
+                                                                        float* dK, int outs,
+                                                                        int sets) {
+  __shared__ float part[LANES][kRedOuts];
   const int o = blockIdx.x * kRedOuts + threadIdx.x, y = threadIdx.y;
   float s = 0.f;
   if (o < outs) {
     int w = y;
-    for (; w + 3 * kRedSets < sets; w += 4 * kRedSets) {
+    for (; w + 3 * LANES < sets; w += 4 * LANES) {
       const float v0 = partial[(size_t)w * outs + o];
-      const float v1 = partial[(size_t)(w + kRedSets) * outs + o];
-      const float v2 = partial[(size_t)(w + 2 * kRedSets) * outs + o];
-      const float v3 = partial[(size_t)(w + 3 * kRedSets) * outs + o];
+      const float v1 = partial[(size_t)(w + LANES) * outs + o];
+      const float v2 = partial[(size_t)(w + 2 * LANES) * outs + o];
+      const float v3 = partial[(size_t)(w + 3 * LANES) * outs + o];
       s += v0;
       s += v1;
       s += v2;
       s += v3;
     }
-    for (; w < sets; w += kRedSets) s += partial[(size_t)w * outs + o];
+    for (; w < sets; w += LANES) s += partial[(size_t)w * outs + o];
   }
   part[y][threadIdx.x] = s;
   __syncthreads();
   if (y == 0 && o < outs) {
     float t = part[0][threadIdx.x];
 #pragma unroll
-    for (int i = 1; i < kRedSets; ++i) t += part[i][threadIdx.x];
+    for (int i = 1; i < LANES; ++i) t += part[i][threadIdx.x];
     dK[o] = t;
   }
 }
@@ -1190,8 +1193,12 @@ hipError_t bwd_filter_dense_tiles_launch(const BwdFilterArgs& a, hipStream_t st)
     }
   }
   if (e != hipSuccess) return e;
-  dense_reduce_kernel<<<(outs + kRedOuts - 1) / kRedOuts, dim3(kRedOuts, kRedSets), 0, st>>>(
-      partial, dK, outs, sets);
+  if (outs <= 512)
+    dense_reduce_kernel<32><<<(outs + kRedOuts - 1) / kRedOuts, dim3(kRedOuts, 32), 0, st>>>(
+        partial, dK, outs, sets);
+  else
+    dense_reduce_kernel<8><<<(outs + kRedOuts - 1) / kRedOuts, dim3(kRedOuts, 8), 0, st>>>(
+        partial, dK, outs, sets);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
   const size_t fold_lds = fold_lds_bytes(s);
