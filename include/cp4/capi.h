@@ -225,7 +225,8 @@ cp4_status cp4_conv2d_backward_filter_variant(const cp4_shape* shape, const floa
                                               cp4_stream stream);
 
 /* Variant 3 has two tile kernels and picks one by the shape (one or two output channels
- * under a 3x3 filter on large inputs: plain multiply-adds; else the matrix cores).
+ * under a 3x3 or 5x5 filter on inputs of ten million cells or more: plain multiply-adds;
+ * else the matrix cores).
  * cp4_set_backward_filter_tile_kernel overrides that for every later launch of the process
  * where both can run the shape: 0 plain multiply-adds, 1 matrix cores, anything else the
  * library's choice again.  For A/B measurements and for tests that run both kernels on the
