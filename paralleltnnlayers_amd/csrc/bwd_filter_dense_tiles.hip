@@ -694,14 +694,44 @@ __global__ __launch_bounds__(kFoldRanks * kFoldRows) void dense_fold_kernel(BwdF
   const int tid = threadIdx.y * kFoldRanks + threadIdx.x;
   const int r0 = blockIdx.x * kFoldRanks, r = r0 + threadIdx.x;
   const int job = blockIdx.y;              // 0 dFK, 1 dFC, 2 dFH, 3 dFW
-  for (int e = tid; e < outs; e += kFoldRanks * kFoldRows) dk[e] = dK[e];
-  for (int e = tid; e < frows * kFoldRanks; e += kFoldRanks * kFoldRows) {
-    const int row = e / kFoldRanks, rr = r0 + (e % kFoldRanks);
-    const float* src = row < T ? a.FK + (size_t)row * R
-                     : row < T + C ? a.FC + (size_t)(row - T) * R
-                     : row < T + C + Y ? a.FH + (size_t)(row - T - C) * R
-                                       : a.FW + (size_t)(row - T - C - Y) * R;
-    fac[e] = rr < R ? src[rr] : 0.f;
+  // (dK in 16-byte pieces with four loads in flight a thread, the factors' columns with
+  //  eight: one after the other, these loads were a third of the kernel's time)
+  constexpr int kThreadsFold = kFoldRanks * kFoldRows;
+  {
+    const int quads = outs >> 2;
+    const float4* src = reinterpret_cast<const float4*>(dK);
+    float4* dst = reinterpret_cast<float4*>(dk);
+    for (int e0 = tid; e0 < quads; e0 += 4 * kThreadsFold) {
+      float4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int e = e0 + u * kThreadsFold;
+        v[u] = src[e < quads ? e : quads - 1];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (e0 + u * kThreadsFold < quads) dst[e0 + u * kThreadsFold] = v[u];
+    }
+    for (int e = 4 * quads + tid; e < outs; e += kThreadsFold) dk[e] = dK[e];
+  }
+  for (int e0 = tid; e0 < frows * kFoldRanks; e0 += 8 * kThreadsFold) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      int e = e0 + u * kThreadsFold;
+      e = e < frows * kFoldRanks ? e : frows * kFoldRanks - 1;
+      const int row = e / kFoldRanks, rr = r0 + (e % kFoldRanks);
+      const float* src = row < T ? a.FK + (size_t)row * R
+                       : row < T + C ? a.FC + (size_t)(row - T) * R
+                       : row < T + C + Y ? a.FH + (size_t)(row - T - C) * R
+                                         : a.FW + (size_t)(row - T - C - Y) * R;
+      v[u] = src[rr < R ? rr : R - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int e = e0 + u * kThreadsFold;
+      if (e < frows * kFoldRanks) fac[e] = r0 + (e % kFoldRanks) < R ? v[u] : 0.f;
+    }
   }
   __syncthreads();
   const float* fk = fac + threadIdx.x;                   // row stride kFoldRanks
